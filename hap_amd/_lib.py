@@ -1,0 +1,52 @@
+"""ctypes binding of libhapmi.so.  There is no fallback: if the library is
+missing or a call fails, an exception is raised."""
+from __future__ import annotations
+
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_PATH = os.path.join(_HERE, "libhapmi.so")
+_lib = None
+
+F32, BF16 = 0, 1
+ACT_NONE, ACT_RELU, ACT_GELU = 0, 1, 2
+MAX_RANKS = 64
+
+
+class HapmiError(RuntimeError):
+    pass
+
+
+class GemmArgs(ctypes.Structure):
+    _fields_ = [
+        ("A", ctypes.c_void_p), ("B", ctypes.c_void_p), ("C", ctypes.c_void_p), ("bias", ctypes.c_void_p),
+        ("M", ctypes.c_int64), ("N", ctypes.c_int64), ("K", ctypes.c_int64),
+        ("lda", ctypes.c_int64), ("ldb", ctypes.c_int64), ("ldc", ctypes.c_int64),
+        ("transA", ctypes.c_int), ("transB", ctypes.c_int),
+        ("in_dtype", ctypes.c_int), ("out_dtype", ctypes.c_int),
+        ("accumulate", ctypes.c_int), ("act", ctypes.c_int),
+        ("alpha", ctypes.c_float),
+        ("batch1", ctypes.c_int64), ("batch2", ctypes.c_int64),
+        ("strideA1", ctypes.c_int64), ("strideA2", ctypes.c_int64),
+        ("strideB1", ctypes.c_int64), ("strideB2", ctypes.c_int64),
+        ("strideC1", ctypes.c_int64), ("strideC2", ctypes.c_int64),
+    ]
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_PATH):
+            raise HapmiError(f"{_PATH} is missing: build it with `python -m hap_amd.build` "
+                             "(there is no fallback path)")
+        _lib = ctypes.CDLL(_PATH)
+        _lib.hapmi_last_error.restype = ctypes.c_char_p
+        _lib.hapmi_sharding_round.argtypes = [ctypes.c_int64, ctypes.POINTER(ctypes.c_double), ctypes.c_int64,
+                                              ctypes.POINTER(ctypes.c_int64)]
+    return _lib
+
+
+def check(rc: int) -> None:
+    if rc != 0:
+        raise HapmiError(f"libhapmi error {rc}: {lib().hapmi_last_error().decode()}")

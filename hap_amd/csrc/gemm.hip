@@ -1,0 +1,436 @@
+// MFMA GEMM for gfx950: C = alpha * op(A) * op(B) (+ bias) (act) (+ C), float32 accumulation.
+//
+// One kernel template serves bf16 (v_mfma_f32_32x32x16_bf16) and float32
+// (v_mfma_f32_32x32x2_f32) inputs.  Both operands are staged in LDS as
+// [row][k] with k contiguous, so the register fragment of either type is one
+// 16-byte LDS read; an operand whose reduction dimension is the slow one in
+// memory (dgrad's weight, both operands of wgrad) is transposed in registers on
+// its way into LDS.  Ragged M / N / K are handled by guarded edge loads and
+// stores; the interior of every tile runs unguarded 16-byte accesses.
+//
+// The MFMA "A" operand is fed from op(B) rows (n) and the "B" operand from op(A)
+// rows (m): each lane then holds 4 consecutive n of one m in its accumulators
+// and the epilogue issues 8/16-byte stores along the contiguous dimension of C.
+#include "common.h"
+#include <vector>
+#include <mutex>
+
+namespace {
+
+template <typename TI> struct Mma;
+template <> struct Mma<bf16_t> {
+    static constexpr int EPV = 8;
+    __device__ __forceinline__ static void run(f32x16 &acc, const Vec16<bf16_t> &a, const Vec16<bf16_t> &b) {
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, b.v, acc, 0, 0, 0);
+    }
+};
+template <> struct Mma<float> {
+    static constexpr int EPV = 4;
+    __device__ __forceinline__ static void run(f32x16 &acc, const Vec16<float> &a, const Vec16<float> &b) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.v[i], b.v[i], acc, 0, 0, 0);
+    }
+};
+
+struct GemmParams {
+    const void *A, *B;
+    void *C;
+    const float *bias;
+    int64_t M, N, K;
+    int64_t lda, ldb, ldc;
+    int64_t batch2;
+    int64_t sA1, sA2, sB1, sB2, sC1, sC2;
+    float alpha;
+    int accumulate, act;
+    int tiles_m, tiles_n;
+};
+
+__device__ __forceinline__ float apply_act(float v, int act) {
+    if (act == HAPMI_ACT_RELU) return v > 0.f ? v : 0.f;
+    if (act == HAPMI_ACT_GELU) return 0.5f * v * (1.0f + erff(v * 0.70710678118654752f));
+    return v;
+}
+
+// Loads one operand tile [ROWS][BK] (row = m or n index, k = reduction index) from global memory into
+// registers.  KMAJOR: memory is [row][k] (k contiguous); otherwise memory is [k][row] (row contiguous).
+template <typename TI, int ROWS, int BK, int THREADS, bool KMAJOR> struct TileLoader {
+    static constexpr int EPV = 16 / sizeof(TI);
+    // KMAJOR: vectors along k; thread -> (row, kvec)
+    static constexpr int KV = BK / EPV;                         // vectors per row
+    static constexpr int ROWS_PER_PASS = THREADS / KV;
+    static constexpr int PASSES_K = ROWS / ROWS_PER_PASS;
+    // !KMAJOR: 4(k) x EPV(row) blocks; thread -> (kgroup, rowvec)
+    static constexpr int RV = ROWS / EPV;                       // row-vectors per k line
+    static constexpr int BLOCKS = (BK / 4) * RV;
+    static constexpr int PASSES_T = BLOCKS / THREADS;
+    static constexpr int NV = KMAJOR ? PASSES_K : PASSES_T * 4;
+    static_assert(KMAJOR ? (ROWS % ROWS_PER_PASS == 0 && PASSES_K >= 1) : (BLOCKS % THREADS == 0 && PASSES_T >= 1),
+                  "tile does not divide over the block");
+
+    Vec16<TI> v[NV];
+
+    __device__ __forceinline__ static Vec16<TI> guarded(const TI *p, int64_t n_valid) {
+        Vec16<TI> r;
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) r.set(e, (e < n_valid) ? ld_f(p, e) : 0.f);
+        return r;
+    }
+
+    // base: pointer to element (row0, k0) of the operand; rows_left / k_left: valid extent from there
+    __device__ __forceinline__ void load(const TI *base, int64_t ld, int64_t rows_left, int64_t k_left) {
+        const int t = threadIdx.x;
+        if (KMAJOR) {
+            const int kv = t % KV, r0 = t / KV;
+#pragma unroll
+            for (int p = 0; p < PASSES_K; ++p) {
+                const int row = r0 + p * ROWS_PER_PASS;
+                const int64_t kk = (int64_t)kv * EPV;
+                const TI *src = base + (int64_t)row * ld + kk;
+                if (row < rows_left && kk + EPV <= k_left) v[p] = *(const Vec16<TI> *)src;
+                else if (row < rows_left && kk < k_left) v[p] = guarded(src, k_left - kk);
+                else v[p] = guarded(src, 0);
+            }
+        } else {
+#pragma unroll
+            for (int p = 0; p < PASSES_T; ++p) {
+                const int blk = t + p * THREADS;
+                const int rv = blk % RV, kg = blk / RV;
+                const int64_t rr = (int64_t)rv * EPV;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int64_t kk = (int64_t)kg * 4 + q;
+                    const TI *src = base + kk * ld + rr;
+                    if (kk < k_left && rr + EPV <= rows_left) v[p * 4 + q] = *(const Vec16<TI> *)src;
+                    else if (kk < k_left && rr < rows_left) v[p * 4 + q] = guarded(src, rows_left - rr);
+                    else v[p * 4 + q] = guarded(src, 0);
+                }
+            }
+        }
+    }
+
+    // LDS tile is [ROWS][LDK] elements, k contiguous
+    template <int LDK> __device__ __forceinline__ void store(TI *lds) const {
+        const int t = threadIdx.x;
+        if (KMAJOR) {
+            const int kv = t % KV, r0 = t / KV;
+#pragma unroll
+            for (int p = 0; p < PASSES_K; ++p)
+                *(Vec16<TI> *)(lds + (r0 + p * ROWS_PER_PASS) * LDK + kv * EPV) = v[p];
+        } else {
+            typedef TI quad_t __attribute__((ext_vector_type(4)));
+#pragma unroll
+            for (int p = 0; p < PASSES_T; ++p) {
+                const int blk = t + p * THREADS;
+                const int rv = blk % RV, kg = blk / RV;
+#pragma unroll
+                for (int e = 0; e < EPV; ++e) {
+                    quad_t q4;
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) q4[q] = v[p * 4 + q].v[e];
+                    *(quad_t *)(lds + (rv * EPV + e) * LDK + kg * 4) = q4;
+                }
+            }
+        }
+    }
+};
+
+template <typename TI, typename TO, int BM, int BN, int WAVES_M, int WAVES_N, bool A_KMAJOR, bool B_KMAJOR>
+__global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_kernel(GemmParams p) {
+    constexpr int THREADS = WAVES_M * WAVES_N * 64;
+    constexpr int EPV = 16 / sizeof(TI);
+    constexpr int BK = 128 / sizeof(TI);              // 128 bytes of k per LDS row
+    constexpr int LDK = BK + EPV;                     // +16 bytes: conflict-free 16-byte fragment reads
+    constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
+    constexpr int TM = WTM / 32, TN = WTN / 32;
+    constexpr int KSTEPS = BK / (2 * EPV);            // fragment pairs (one per lane half) per tile
+
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    TI *As = (TI *)smem;                              // [2][BM][LDK]
+    TI *Bs = As + 2 * BM * LDK;                       // [2][BN][LDK]
+
+    // tile mapping: blocks go round-robin over the 8 XCDs; give each XCD a contiguous range of tiles and
+    // walk it in columns of 8 m-tiles so that concurrently running tiles share A rows / B columns in L2
+    int bid = blockIdx.x;
+    const int nblk = gridDim.x;
+    if (nblk % 8 == 0) bid = (bid % 8) * (nblk / 8) + bid / 8;
+    constexpr int GROUP = 8;
+    const int per_group = GROUP * p.tiles_n;
+    const int g = bid / per_group;
+    const int gm0 = g * GROUP;
+    const int gsz = (p.tiles_m - gm0) < GROUP ? (p.tiles_m - gm0) : GROUP;
+    const int tm = gm0 + (bid % per_group) % gsz;
+    const int tn = (bid % per_group) / gsz;
+
+    const int64_t z1 = blockIdx.z / p.batch2, z2 = blockIdx.z % p.batch2;
+    const TI *A = (const TI *)p.A + z1 * p.sA1 + z2 * p.sA2;
+    const TI *B = (const TI *)p.B + z1 * p.sB1 + z2 * p.sB2;
+    TO *C = (TO *)p.C + z1 * p.sC1 + z2 * p.sC2;
+
+    const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
+    const int64_t m_left = p.M - m0, n_left = p.N - n0;
+
+    const TI *a_base = A_KMAJOR ? A + m0 * p.lda : A + m0;     // element (m0, k=0)
+    const TI *b_base = B_KMAJOR ? B + n0 * p.ldb : B + n0;
+    const int64_t a_kstep = A_KMAJOR ? (int64_t)BK : (int64_t)BK * p.lda;
+    const int64_t b_kstep = B_KMAJOR ? (int64_t)BK : (int64_t)BK * p.ldb;
+
+    TileLoader<TI, BM, BK, THREADS, A_KMAJOR> la;
+    TileLoader<TI, BN, BK, THREADS, B_KMAJOR> lb;
+
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int wm = (wave % WAVES_M) * WTM, wn = (wave / WAVES_M) * WTN;
+    const int frow = lane & 31, fk = (lane >> 5) * EPV;
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    const int nk = (int)((p.K + BK - 1) / BK);
+    la.load(a_base, p.lda, m_left, p.K);
+    lb.load(b_base, p.ldb, n_left, p.K);
+    la.template store<LDK>(As);
+    lb.template store<LDK>(Bs);
+    __syncthreads();
+
+    for (int kt = 0; kt < nk; ++kt) {
+        const int cur = kt & 1;
+        if (kt + 1 < nk) {
+            const int64_t k_left = p.K - (int64_t)(kt + 1) * BK;
+            la.load(a_base + (int64_t)(kt + 1) * a_kstep, p.lda, m_left, k_left);
+            lb.load(b_base + (int64_t)(kt + 1) * b_kstep, p.ldb, n_left, k_left);
+        }
+        const TI *as = As + cur * BM * LDK + wm * LDK;
+        const TI *bs = Bs + cur * BN * LDK + wn * LDK;
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) {
+            Vec16<TI> fa[TM], fb[TN];
+#pragma unroll
+            for (int i = 0; i < TM; ++i) fa[i] = *(const Vec16<TI> *)(as + (i * 32 + frow) * LDK + ks * 2 * EPV + fk);
+#pragma unroll
+            for (int j = 0; j < TN; ++j) fb[j] = *(const Vec16<TI> *)(bs + (j * 32 + frow) * LDK + ks * 2 * EPV + fk);
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j) Mma<TI>::run(acc[i][j], fb[j], fa[i]);
+        }
+        if (kt + 1 < nk) {
+            la.template store<LDK>(As + (cur ^ 1) * BM * LDK);
+            lb.template store<LDK>(Bs + (cur ^ 1) * BN * LDK);
+        }
+        __syncthreads();
+    }
+
+    // epilogue: acc[i][j][r] is C[m, n] with m = wm + i*32 + lane%32, n = wn + j*32 + (r/4)*8 + (lane/32)*4 + r%4
+    const int64_t mrow_base = m0 + wm + (lane & 31);
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+        const int64_t m = mrow_base + i * 32;
+        if (m >= p.M) continue;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int64_t n = n0 + wn + j * 32 + q * 8 + (lane >> 5) * 4;
+                if (n >= p.N) continue;
+                float v[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = acc[i][j][q * 4 + e] * p.alpha;
+                TO *dst = C + m * p.ldc + n;
+                const bool full = (n + 4 <= p.N);
+                if (p.bias) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (full || n + e < p.N) v[e] += p.bias[n + e];
+                }
+                if (p.act != HAPMI_ACT_NONE) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] = apply_act(v[e], p.act);
+                }
+                if (full && ((p.ldc & 3) == 0)) {
+                    typedef TO out4_t __attribute__((ext_vector_type(4)));
+                    if (p.accumulate) {
+                        const out4_t old = *(const out4_t *)dst;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) v[e] += (float)old[e];
+                    }
+                    out4_t o;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) o[e] = (TO)v[e];
+                    *(out4_t *)dst = o;
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        if (n + e < p.N) {
+                            float x = v[e];
+                            if (p.accumulate) x += (float)dst[e];
+                            dst[e] = (TO)x;
+                        }
+                    }
+                }
+            }
+        }
+    }
+}
+
+template <typename TI, int BM, int BN> constexpr size_t gemm_smem() {
+    constexpr int EPV = 16 / sizeof(TI);
+    constexpr int BK = 128 / sizeof(TI);
+    return (size_t)2 * (BM + BN) * (BK + EPV) * sizeof(TI);
+}
+
+// ---- instrumentation: HIP events around every launch --------------------------------------------
+struct ProfState {
+    std::mutex mu;
+    bool on = false;
+    std::vector<hipEvent_t> pool;          // events not in use
+    std::vector<std::pair<hipEvent_t, hipEvent_t>> pending;
+    double flops = 0.0;
+    int64_t launches = 0;
+};
+ProfState g_prof;
+
+hipEvent_t prof_event() {
+    if (!g_prof.pool.empty()) {
+        hipEvent_t e = g_prof.pool.back();
+        g_prof.pool.pop_back();
+        return e;
+    }
+    hipEvent_t e;
+    if (hipEventCreate(&e) != hipSuccess) return nullptr;
+    return e;
+}
+
+template <typename TI, typename TO, int BM, int BN, int WM, int WN>
+int launch_cfg(const GemmParams &p, int transA, int transB, int64_t batch, hipStream_t st) {
+    GemmParams q = p;
+    q.tiles_m = (int)hapmi_cdiv(p.M, BM);
+    q.tiles_n = (int)hapmi_cdiv(p.N, BN);
+    dim3 grid((unsigned)(q.tiles_m * q.tiles_n), 1, (unsigned)batch), block(WM * WN * 64);
+    const size_t smem = gemm_smem<TI, BM, BN>();
+#define HAPMI_GEMM_LAUNCH(AK, BK_)                                                                        \
+    do {                                                                                                  \
+        auto kern = gemm_kernel<TI, TO, BM, BN, WM, WN, AK, BK_>;                                         \
+        if (smem > 64 * 1024) {                                                                           \
+            static bool raised = false;                                                                   \
+            if (!raised) {                                                                                \
+                if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,   \
+                                        (int)smem) != hipSuccess)                                         \
+                    return hapmi_set_error(HAPMI_ELAUNCH, "gemm: cannot raise the LDS limit to %zu", smem); \
+                raised = true;                                                                            \
+            }                                                                                             \
+        }                                                                                                 \
+        hipLaunchKernelGGL(kern, grid, block, smem, st, q);                                               \
+    } while (0)
+    if (!transA && transB) HAPMI_GEMM_LAUNCH(true, true);
+    else if (!transA && !transB) HAPMI_GEMM_LAUNCH(true, false);
+    else if (transA && !transB) HAPMI_GEMM_LAUNCH(false, false);
+    else HAPMI_GEMM_LAUNCH(false, true);
+#undef HAPMI_GEMM_LAUNCH
+    return HAPMI_OK;
+}
+
+template <typename TI, typename TO>
+int launch_typed(const GemmParams &p, int transA, int transB, int64_t batch, hipStream_t st) {
+    // big tiles when they still give every CU at least ~2 tiles of work, else smaller ones
+    const int64_t t256 = hapmi_cdiv(p.M, 256) * hapmi_cdiv(p.N, 128) * batch;
+    if (t256 >= 256 * 2 && p.M >= 256 && p.N >= 128) return launch_cfg<TI, TO, 256, 128, 2, 2>(p, transA, transB, batch, st);
+    return launch_cfg<TI, TO, 128, 128, 2, 2>(p, transA, transB, batch, st);
+}
+
+}  // namespace
+
+extern "C" int hapmi_gemm(const hapmi_gemm_args *a, hapmi_stream_t stream) {
+    HAPMI_REQUIRE(a, HAPMI_EINVAL, "gemm: null argument block");
+    HAPMI_REQUIRE(hapmi_dtype_ok(a->in_dtype) && hapmi_dtype_ok(a->out_dtype), HAPMI_EINVAL, "gemm: bad dtype");
+    HAPMI_REQUIRE(a->M >= 0 && a->N >= 0 && a->K >= 0 && a->batch1 >= 1 && a->batch2 >= 1, HAPMI_EINVAL,
+                  "gemm: bad shape M=%lld N=%lld K=%lld", (long long)a->M, (long long)a->N, (long long)a->K);
+    if (a->M == 0 || a->N == 0) return HAPMI_OK;
+    HAPMI_REQUIRE(a->A && a->B && a->C, HAPMI_EINVAL, "gemm: null pointer");
+    HAPMI_REQUIRE(a->act == HAPMI_ACT_NONE || a->act == HAPMI_ACT_RELU || a->act == HAPMI_ACT_GELU, HAPMI_EINVAL,
+                  "gemm: unknown activation %d", a->act);
+    const int64_t epv = a->in_dtype == HAPMI_F32 ? 4 : 8;
+    const int64_t a_cols = a->transA ? a->M : a->K, b_cols = a->transB ? a->K : a->N;
+    HAPMI_REQUIRE(a->lda >= a_cols && a->ldb >= b_cols && a->ldc >= a->N, HAPMI_EINVAL,
+                  "gemm: leading dimension below the row length (lda=%lld ldb=%lld ldc=%lld)", (long long)a->lda,
+                  (long long)a->ldb, (long long)a->ldc);
+    HAPMI_REQUIRE(((uintptr_t)a->A % 16) == 0 && ((uintptr_t)a->B % 16) == 0 && a->lda % epv == 0 &&
+                      a->ldb % epv == 0 && a->strideA1 % epv == 0 && a->strideA2 % epv == 0 &&
+                      a->strideB1 % epv == 0 && a->strideB2 % epv == 0,
+                  HAPMI_EALIGN, "gemm: A/B pointers, leading dimensions and batch strides must be 16-byte multiples");
+    const int64_t osz = hapmi_elem_size(a->out_dtype);
+    HAPMI_REQUIRE(((uintptr_t)a->C % (4 * osz)) == 0 && (a->strideC1 % 4) == 0 && (a->strideC2 % 4) == 0, HAPMI_EALIGN,
+                  "gemm: C pointer and batch strides must be multiples of 4 elements");
+    const int64_t batch = a->batch1 * a->batch2;
+    HAPMI_REQUIRE(batch <= 65535, HAPMI_ELIMIT, "gemm: batch %lld above 65535", (long long)batch);
+    HAPMI_REQUIRE(hapmi_cdiv(a->M, 128) * hapmi_cdiv(a->N, 128) < (1ll << 31), HAPMI_ELIMIT, "gemm: too many tiles");
+
+    GemmParams p;
+    p.A = a->A; p.B = a->B; p.C = a->C; p.bias = (const float *)a->bias;
+    p.M = a->M; p.N = a->N; p.K = a->K;
+    p.lda = a->lda; p.ldb = a->ldb; p.ldc = a->ldc;
+    p.batch2 = a->batch2;
+    p.sA1 = a->strideA1; p.sA2 = a->strideA2; p.sB1 = a->strideB1; p.sB2 = a->strideB2;
+    p.sC1 = a->strideC1; p.sC2 = a->strideC2;
+    p.alpha = a->alpha; p.accumulate = a->accumulate; p.act = a->act;
+    p.tiles_m = p.tiles_n = 0;
+
+    hipStream_t st = (hipStream_t)stream;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    bool prof = false;
+    {
+        std::lock_guard<std::mutex> lk(g_prof.mu);
+        prof = g_prof.on;
+        if (prof) {
+            e0 = prof_event();
+            e1 = prof_event();
+            prof = e0 && e1;
+        }
+    }
+    if (prof) hipEventRecord(e0, st);
+    int rc;
+    if (a->in_dtype == HAPMI_BF16 && a->out_dtype == HAPMI_BF16) rc = launch_typed<bf16_t, bf16_t>(p, a->transA, a->transB, batch, st);
+    else if (a->in_dtype == HAPMI_BF16) rc = launch_typed<bf16_t, float>(p, a->transA, a->transB, batch, st);
+    else if (a->out_dtype == HAPMI_F32) rc = launch_typed<float, float>(p, a->transA, a->transB, batch, st);
+    else rc = launch_typed<float, bf16_t>(p, a->transA, a->transB, batch, st);
+    if (prof) {
+        hipEventRecord(e1, st);
+        std::lock_guard<std::mutex> lk(g_prof.mu);
+        g_prof.pending.emplace_back(e0, e1);
+        g_prof.flops += 2.0 * (double)a->M * (double)a->N * (double)a->K * (double)batch;
+        g_prof.launches += 1;
+    }
+    if (rc) return rc;
+    HAPMI_CHECK_LAUNCH("gemm");
+    return HAPMI_OK;
+}
+
+extern "C" int hapmi_prof_gemm_enable(int on) {
+    std::lock_guard<std::mutex> lk(g_prof.mu);
+    g_prof.on = on != 0;
+    return HAPMI_OK;
+}
+
+extern "C" int hapmi_prof_gemm_collect(double *ms, int64_t *launches, double *flops) {
+    std::lock_guard<std::mutex> lk(g_prof.mu);
+    double total = 0.0;
+    for (auto &pr : g_prof.pending) {
+        if (hipEventSynchronize(pr.second) != hipSuccess) return hapmi_set_error(HAPMI_ELAUNCH, "prof: event sync failed");
+        float t = 0.f;
+        if (hipEventElapsedTime(&t, pr.first, pr.second) != hipSuccess)
+            return hapmi_set_error(HAPMI_ELAUNCH, "prof: elapsed time failed");
+        total += t;
+        g_prof.pool.push_back(pr.first);
+        g_prof.pool.push_back(pr.second);
+    }
+    g_prof.pending.clear();
+    if (ms) *ms = total;
+    if (launches) *launches = g_prof.launches;
+    if (flops) *flops = g_prof.flops;
+    g_prof.flops = 0.0;
+    g_prof.launches = 0;
+    return HAPMI_OK;
+}

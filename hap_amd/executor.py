@@ -1,0 +1,1026 @@
+"""Executor of one device's SPMD program on MI355X.
+
+``compile_program(graph_module, ...)`` walks the ``torch.fx`` graph that HAP's
+synthesizer emits (node forms: /root/reference/hap.rs:991-2324, 2466-2746) ONCE
+and turns it into two static lists of kernel launches -- forward and backward
+-- over buffers that are allocated up front.  A training step is then a fixed
+sequence of HIP kernel launches through the C ABI of libhapmi.so (no autograd
+graph, no allocation, no host synchronisation), which is also what a HIP graph
+can capture.  The reference runs the same graph through PyTorch eager +
+autograd (/root/reference/worker.py:44-76).
+
+Fusions done while walking the graph (results equal the unfused program):
+``operator.add`` + ``F.layer_norm`` -> one kernel; ``transpose`` around
+``F.multi_head_attention_forward`` -> folded into strides; ``F.dropout(p=0)``
+-> alias; ``all_to_all`` + ``F.relu`` -> activation inside the concat;
+``torch.log_softmax`` + ``transpose`` + ``F.nll_loss`` -> one kernel that also
+writes d(logits); ``top_2_gating`` + ``dynamic_slice`` + the four einsums ->
+index-form gather / grouped GEMM / weighted gather; ``conv2d`` (kernel = stride)
++ ``flatten`` + ``transpose`` -> patch rows + GEMM; ``append_cls_token`` +
+``operator.add(pos_embed)`` -> one kernel.
+
+bf16 mode: float32 master parameters in one flat buffer, a bf16 shadow of it
+that the GEMMs read, bf16 activations and activation gradients, float32
+parameter gradients / statistics / loss / gate probabilities.
+"""
+from __future__ import annotations
+
+import math
+import operator
+from typing import Callable, Dict, List, Optional
+
+import torch
+import torch.fx
+import torch.nn.functional as F
+
+from . import collectives, models, ops
+from .wire import SilentWire, Wire
+
+_EPS = 1e-5
+
+
+class Val:
+    """Compile-time description of a program value."""
+
+    def __init__(self, kind: str, t: Optional[torch.Tensor] = None, shape=None, **kw):
+        self.kind = kind            # 'tensor' | 'param' | 'input' | lazy kinds
+        self.t = t                  # storage (static buffer) for materialised values
+        self.shape = tuple(shape) if shape is not None else (tuple(t.shape) if t is not None else None)
+        self.ld = kw.pop("ld", None)        # row stride when the last dim is padded in storage
+        self.grad: Optional[torch.Tensor] = None
+        self.needs_grad = kw.pop("needs_grad", False)
+        self.meta = kw
+
+
+def _round_up(n, m):
+    return (n + m - 1) // m * m
+
+
+class ShardExecutor:
+    def __init__(self, gm: torch.fx.GraphModule, example_inputs, dtype: str = "fp32", wire: Optional[Wire] = None,
+                 rank: int = 0, world_size: int = 1, device: str = "cuda:0"):
+        """``example_inputs``: the program's inputs (global batch) as tensors or shapes; activations are
+        sized from them.  ``rank`` / ``world_size`` are only needed by all_reduce / replicate, whose node
+        forms do not carry them (collectives.py:86, 182)."""
+        if dtype not in ("fp32", "bf16"):
+            raise ValueError("dtype must be 'fp32' or 'bf16'")
+        if not torch.cuda.is_available():
+            raise ops._lib.HapmiError("no GPU visible: the shard executor has no CPU path")
+        ops.init()
+        self.gm = gm
+        self.dev = torch.device(device)
+        self.cdt = torch.float32 if dtype == "fp32" else torch.bfloat16
+        self.dtype = dtype
+        self.epv = 4 if dtype == "fp32" else 8
+        self.wire = wire if wire is not None else SilentWire()
+        self.fwd: List[Callable[[], None]] = []
+        self.bwd: List[Callable[[], None]] = []
+        self._tape: List[Callable[[], None]] = []      # backward emitters, run in reverse at compile time
+        self.env: Dict[torch.fx.Node, object] = {}
+        self.inputs: List[dict] = []
+        self.loss: Optional[torch.Tensor] = None
+        self._opt = None
+        self._step_count = 0
+        self._shadow_stale = False
+        self._example_inputs = [a if isinstance(a, torch.Tensor) else torch.empty(tuple(a), device="meta")
+                                for a in example_inputs]
+        self.rank_hint, self.world_hint = rank, world_size
+        self._param_reduce: List[Callable[[], None]] = []
+        self._prepare_params()
+        self._compile()
+        self._finish_param_reduce()
+
+    # ------------------------------------------------------------------ parameters
+    def _prepare_params(self):
+        """Parameters the program reads go into one flat float32 master buffer (views replace
+        ``p.data``), with flat float32 gradients and, in bf16 mode, a flat bf16 shadow."""
+        used = []
+        for node in self.gm.graph.nodes:
+            if node.op == "get_attr" and node.target not in used:
+                used.append(node.target)
+        self.param_names, self.buffers = [], {}
+        metas = []
+        off = 0
+        for name in used:
+            obj = self._fetch(name)
+            if isinstance(obj, torch.nn.Parameter):
+                n = obj.numel()
+                metas.append((name, obj, off, n))
+                off += _round_up(n, 64)        # keep every view 256-byte aligned
+                self.param_names.append(name)
+            else:
+                self.buffers[name] = obj
+        self.n_flat = off
+        self.master = torch.zeros(max(off, 4), dtype=torch.float32, device=self.dev)
+        self.flat_grad = torch.zeros_like(self.master)
+        self.shadow = torch.zeros(max(off, 4), dtype=torch.bfloat16, device=self.dev) if self.dtype == "bf16" else None
+        self.params: Dict[str, dict] = {}
+        for name, p, o, n in metas:
+            view = self.master[o:o + n].view(p.shape)
+            view.copy_(p.data.to(self.dev, torch.float32))
+            p.data = view
+            g = self.flat_grad[o:o + n].view(p.shape)
+            p.grad = g
+            sh = self.shadow[o:o + n].view(p.shape) if self.shadow is not None else None
+            self.params[name] = dict(param=p, master=view, grad=g, shadow=sh, offset=o, numel=n)
+        if self.shadow is not None:
+            ops.cast(self.master, self.shadow)
+
+    def _fetch(self, target: str):
+        obj = self.gm
+        for atom in target.split("."):
+            obj = getattr(obj, atom)
+        return obj
+
+    # ------------------------------------------------------------------ small helpers
+    def _new(self, shape, dtype=None):
+        return torch.empty(tuple(shape), dtype=dtype or self.cdt, device=self.dev)
+
+    def _val(self, x):
+        return self.env[x] if isinstance(x, torch.fx.Node) else x
+
+    def _grad_slot(self, v: Val):
+        """Buffer that the next contribution to d(v) goes into and whether it must accumulate."""
+        if v.grad is None:
+            v.grad = self._new(v.t.shape if v.t is not None else v.shape)
+            return v.grad, False
+        return v.grad, True
+
+    def _param_grad_slot(self, v: Val):
+        first = not v.meta.get("grad_written", False)
+        v.meta["grad_written"] = True
+        return v.meta["grad"], not first
+
+    def _unsupported(self, node, why):
+        raise ValueError(f"node {node.name} ({node.target}): {why}")
+
+    # ------------------------------------------------------------------ compile
+    def _compile(self):
+        handlers = {
+            F.embedding: self._embedding, operator.mul: self._mul, operator.add: self._add,
+            torch.transpose: self._transpose, F.multi_head_attention_forward: self._mha,
+            operator.getitem: self._getitem, F.dropout: self._dropout, F.layer_norm: self._layer_norm,
+            F.linear: self._linear, F.relu: self._activation, F.gelu: self._activation,
+            torch.log_softmax: self._log_softmax, F.nll_loss: self._nll_loss,
+            F.conv2d: self._conv2d, torch.flatten: self._flatten,
+            models.append_cls_token: self._append_cls, models.get_cls_token: self._get_cls,
+            models.new_segment: self._alias, models.top_2_gating: self._gating, torch.einsum: self._einsum,
+            collectives.replicate: self._replicate, collectives.all_gather: self._all_gather,
+            collectives.reduce_scatter: self._reduce_scatter, collectives.all_to_all: self._all_to_all,
+            collectives.all_reduce: self._all_reduce, collectives.dynamic_slice: self._dynamic_slice,
+        }
+        for node in self.gm.graph.nodes:
+            if node.op == "placeholder":
+                self.env[node] = Val("input", name=node.name, index=len(self.inputs))
+                self.inputs.append(dict(name=node.name, buf=None, offset=None, length=None))
+            elif node.op == "get_attr":
+                self.env[node] = self._get_attr(node)
+            elif node.op == "call_method":
+                if node.target != "split":
+                    self._unsupported(node, "only Tensor.split is emitted for inputs")
+                src = self._val(node.args[0])
+                if src.kind != "input" or node.args[2] != 0:
+                    self._unsupported(node, "split is only supported on a program input along dim 0")
+                self.env[node] = Val("input_split", src=src, lengths=list(node.args[1]))
+            elif node.op == "call_function":
+                h = handlers.get(node.target)
+                if h is None:
+                    self._unsupported(node, "this op has no handler")
+                self.env[node] = h(node)
+            elif node.op == "output":
+                out = self._val(node.args[0])
+                if out.kind != "loss":
+                    self._unsupported(node, "the program output must be the nll_loss scalar")
+                self.loss = out.t
+        for emit in reversed(self._tape):
+            emit()
+        self._tape = []
+
+    # ------------------------------------------------------------------ leaves
+    def _get_attr(self, node):
+        name = node.target
+        if name in self.params:
+            rec = self.params[name]
+            t = rec["shadow"] if self.dtype == "bf16" else rec["master"]
+            return Val("param", t, name=name, master=rec["master"], grad=rec["grad"], needs_grad=True)
+        buf = self.buffers[name]
+        keep_f32 = name.endswith("src_mask")
+        t = buf.detach().to(self.dev, torch.float32 if keep_f32 else self.cdt).contiguous()
+        return Val("tensor", t, name=name)
+
+    def _alias(self, node):
+        return self._val(node.args[0])
+
+    def _replicate(self, node):
+        v = self._val(node.args[0])
+        if v.kind == "param":
+            v.meta["replicated_tag"] = node.name
+        return v
+
+    def _getitem(self, node):
+        src, idx = self._val(node.args[0]), node.args[1]
+        if src.kind == "input_split":
+            L = src.meta["lengths"]
+            return Val("input_slice", src=src.meta["src"], offset=sum(L[:idx]), length=L[idx])
+        if src.kind == "mha":
+            if idx == 0:
+                return src.meta["out"]
+            return Val("dead", why="head-averaged attention probabilities are never consumed by the program")
+        if src.kind == "gating":
+            return Val("routing", which="dispatch" if idx == 0 else "combine", gating=src, e_lo=0, E_loc=src.meta["E"])
+        self._unsupported(node, f"getitem on a {src.kind} value")
+
+    # ------------------------------------------------------------------ ops
+    def _embedding(self, node):
+        ids_v, table = self._val(node.args[0]), self._val(node.args[1])
+        ids = self._input_buffer(ids_v, torch.int64)
+        d = table.t.shape[1]
+        out = Val("tensor", self._new(tuple(ids.shape) + (d,)), needs_grad=True)
+        self.fwd.append(lambda: ops.embedding_fwd(ids, table.t, None, out.t, 1, 1.0))
+
+        def emit():
+            if out.grad is None:
+                return
+            g, acc = self._param_grad_slot(table)
+            if not acc:
+                self.bwd.append(lambda: ops.fill_zero(g))
+            self.bwd.append(lambda: ops.embedding_bwd(ids, out.grad, g, 1.0))
+        self._tape.append(emit)
+        return out
+
+    def _input_buffer(self, v: Val, dtype) -> torch.Tensor:
+        if v.kind not in ("input", "input_slice"):
+            raise ValueError("expected a program input")
+        src = v if v.kind == "input" else v.meta["src"]
+        rec = self.inputs[src.meta["index"]]
+        if rec["buf"] is None:
+            full = self._example_inputs[src.meta["index"]]
+            off = v.meta.get("offset") if v.kind == "input_slice" else None
+            length = v.meta.get("length") if v.kind == "input_slice" else full.shape[0]
+            rec.update(offset=off, length=length)
+            rec["buf"] = torch.empty((length,) + tuple(full.shape[1:]), dtype=dtype, device=self.dev)
+        return rec["buf"]
+
+    def _mul(self, node):
+        a, s = self._val(node.args[0]), node.args[1]
+        if not isinstance(s, (int, float)):
+            self._unsupported(node, "only multiplication by a number is supported")
+        out = Val("tensor", self._new(a.t.shape), needs_grad=a.needs_grad)
+        self.fwd.append(lambda: ops.scale(a.t, float(s), out.t))
+
+        def emit():
+            if out.grad is None or not a.needs_grad:
+                return
+            g, acc = self._grad_slot(a)
+            if acc:
+                tmp = self._new(a.t.shape)
+                self.bwd.append(lambda: (ops.scale(out.grad, float(s), tmp), ops.add(g, tmp, g)))
+            else:
+                self.bwd.append(lambda: ops.scale(out.grad, float(s), g))
+        self._tape.append(emit)
+        return out
+
+    def _add(self, node):
+        a, b = self._val(node.args[0]), self._val(node.args[1])
+        users = list(node.users)
+        if a.kind == "cls_appended" or b.kind == "cls_appended":
+            return self._append_cls_pos(node, a if a.kind == "cls_appended" else b, b if a.kind == "cls_appended" else a)
+        if a.t is None or b.t is None:
+            self._unsupported(node, "operands must be materialised tensors")
+        if tuple(a.t.shape) == tuple(b.t.shape):
+            if len(users) == 1 and users[0].target is F.layer_norm:
+                return Val("sum", None, shape=a.t.shape, a=a, b=b, needs_grad=True)
+            out = Val("tensor", self._new(a.t.shape), needs_grad=a.needs_grad or b.needs_grad)
+            self.fwd.append(lambda: ops.add(a.t, b.t, out.t))
+
+            def emit():
+                if out.grad is None:
+                    return
+                for v in (a, b):
+                    if v.needs_grad:
+                        self._accumulate_into(v, out.grad)
+            self._tape.append(emit)
+            return out
+        # broadcast over the leading dimension: [b, S, d] + [1, S, d]
+        big, small = (a, b) if a.t.numel() >= b.t.numel() else (b, a)
+        if small.t.shape[0] != 1 or tuple(small.t.shape[1:]) != tuple(big.t.shape[1:]):
+            self._unsupported(node, f"broadcast of {tuple(small.t.shape)} onto {tuple(big.t.shape)} is not supported")
+        width = big.t.shape[-1]
+        b_rows = small.t.numel() // width
+        rows = big.t.numel() // width
+        out = Val("tensor", self._new(big.t.shape), needs_grad=big.needs_grad or small.needs_grad)
+        self.fwd.append(lambda: ops.add_bcast_rows(big.t, small.t, out.t, rows, b_rows, width))
+
+        def emit():
+            if out.grad is None:
+                return
+            if big.needs_grad:
+                self._accumulate_into(big, out.grad)
+            if small.kind == "param":
+                g, acc = self._param_grad_slot(small)
+                n = small.t.numel()
+                self.bwd.append(lambda: ops.colsum(out.grad, g, big.t.shape[0], n, n, acc))
+        self._tape.append(emit)
+        return out
+
+    def _accumulate_into(self, v: Val, src: torch.Tensor):
+        """d(v) += src; when d(v) does not exist yet it ALIASES src.  Safe because every reader of an
+        aliased gradient (the backward of its single producer) is enqueued before any later accumulation
+        into the other owner: accumulating contributions come from consumers that precede that producer in
+        program order, hence follow it in backward order."""
+        if v.grad is None:
+            v.grad = src
+        else:
+            g = v.grad
+            self.bwd.append(lambda: ops.add(g, src, g))
+
+    def _transpose(self, node):
+        v, d0, d1 = self._val(node.args[0]), node.args[1], node.args[2]
+        dims = tuple(sorted((d0, d1)))
+        if v.kind == "transposed" and v.meta["dims"] == dims:
+            return v.meta["src"]
+        if v.kind == "logprobs" and dims == (1, 2):
+            return Val("logprobs", src=v.meta["src"], transposed=True)
+        if v.kind == "conv_flat" and dims == (1, 2):
+            return v.meta["tokens"]
+        if v.t is None:
+            self._unsupported(node, f"transpose of a {v.kind} value")
+        return Val("transposed", None, src=v, dims=dims, needs_grad=v.needs_grad)
+
+    def _dropout(self, node):
+        if float(node.args[1]) != 0.0:
+            self._unsupported(node, "dropout with p > 0 is not implemented (parity runs use p = 0)")
+        return self._val(node.args[0])
+
+    def _layer_norm(self, node):
+        v, shape = self._val(node.args[0]), tuple(node.args[1])
+        if len(node.args) > 2 or node.kwargs:
+            self._unsupported(node, "the program emits layer_norm without affine parameters")
+        if v.kind == "sum":
+            a, b = v.meta["a"], v.meta["b"]
+            x, res, ref_shape = a.t, b.t, a.t.shape
+        else:
+            a, b, x, res, ref_shape = v, None, v.t, None, v.t.shape
+        if len(shape) != 1 or shape[0] != ref_shape[-1]:
+            self._unsupported(node, "layer_norm over the last dimension only")
+        rows = x.numel() // shape[0]
+        out = Val("tensor", self._new(ref_shape), needs_grad=True)
+        rstd = self._new((rows,), torch.float32)
+        self.fwd.append(lambda: ops.add_layernorm_fwd(x, res, out.t, rstd, _EPS))
+
+        def emit():
+            if out.grad is None:
+                return
+            targets = [v for v in (a, b) if v is not None and v.needs_grad]
+            if not targets:
+                return
+            dx = self._new(ref_shape)
+            self.bwd.append(lambda: ops.layernorm_bwd(out.grad, out.t, rstd, None, dx))
+            for v in targets:                   # the residual add passes the same gradient to both operands
+                self._accumulate_into(v, dx)
+        self._tape.append(emit)
+        return out
+
+    # ---- linear ---------------------------------------------------------------------------------
+    def _linear(self, node):
+        x, w, b = self._val(node.args[0]), self._val(node.args[1]), self._val(node.args[2])
+        if w.kind != "param" or (b is not None and b.kind != "param"):
+            self._unsupported(node, "weight and bias must be parameters")
+        if x.kind == "cls_view":
+            xt, lda, lead = x.meta["src"].t, x.meta["row_stride"], (x.meta["src"].t.shape[0],)
+        elif x.t is not None:
+            xt, lda, lead = x.t, x.ld or x.t.shape[-1], tuple(x.t.shape[:-1])
+        else:
+            self._unsupported(node, f"linear on a {x.kind} value")
+        N, K = w.t.shape
+        M = 1
+        for s in lead:
+            M *= s
+        ldc = _round_up(N, self.epv)
+        store = self._new(lead + (ldc,))
+        out = Val("tensor", store, shape=lead + (N,), ld=ldc if ldc != N else None, needs_grad=True)
+        bias = b.meta["master"] if b is not None else None
+        self.fwd.append(lambda: ops.gemm(xt, w.t, store, M, N, K, transB=True, lda=lda, ldc=ldc, bias=bias))
+
+        def emit():
+            if out.grad is None:
+                return
+            dy = out.grad
+            gw, accw = self._param_grad_slot(w)
+            self.bwd.append(lambda: ops.gemm(dy, xt, gw, N, K, M, transA=True, lda=ldc, ldb=lda, accumulate=accw))
+            if b is not None:
+                gb, accb = self._param_grad_slot(b)
+                self.bwd.append(lambda: ops.colsum(dy, gb, M, N, ldc, accb))
+            if x.kind == "cls_view":
+                src = x.meta["src"]
+                if src.grad is None:
+                    src.grad = self._new(src.t.shape)
+                    g = src.grad
+                    self.bwd.append(lambda: ops.fill_zero(g))
+                g = src.grad
+                self.bwd.append(lambda: ops.gemm(dy, w.t, g, M, K, N, lda=ldc, ldc=lda, accumulate=True))
+            elif x.needs_grad:
+                g, acc = self._grad_slot(x)
+                self.bwd.append(lambda: ops.gemm(dy, w.t, g, M, K, N, lda=ldc, ldc=lda, accumulate=acc))
+        self._tape.append(emit)
+        return out
+
+    def _activation(self, node):
+        x = self._val(node.args[0])
+        kind = "relu" if node.target is F.relu else "gelu"
+        if node.target is F.gelu and (len(node.args) > 1 or node.kwargs.get("approximate", "none") != "none"):
+            self._unsupported(node, "only the erf form of gelu is implemented")
+        if x.meta.get("fused_act") == kind:
+            return x                                    # already applied by the producer
+        if x.t is None or x.ld is not None:
+            self._unsupported(node, f"activation on a {x.kind} value")
+        out = Val("tensor", self._new(x.t.shape), needs_grad=x.needs_grad)
+        self.fwd.append(lambda: ops.act_fwd(x.t, out.t, kind))
+
+        def emit():
+            if out.grad is None or not x.needs_grad:
+                return
+            ref = out.t if kind == "relu" else x.t
+            if x.grad is None:
+                x.grad = self._new(x.t.shape)
+                g = x.grad
+                self.bwd.append(lambda: ops.act_bwd(out.grad, ref, g, kind))
+            else:
+                tmp, g = self._new(x.t.shape), x.grad
+                self.bwd.append(lambda: (ops.act_bwd(out.grad, ref, tmp, kind), ops.add(g, tmp, g)))
+        self._tape.append(emit)
+        return out
+
+    def _wants_fused_relu(self, node):
+        users = list(node.users)
+        return len(users) == 1 and users[0].target is F.relu
+
+    def _relu_backward_through(self, out: Val):
+        """For a producer that applied relu itself: d(pre-activation) = d(out) * (out > 0), in place."""
+        g = out.grad
+        self.bwd.append(lambda: ops.act_bwd(g, out.t, g, "relu"))
+
+    # ---- attention ------------------------------------------------------------------------------
+    def _mha(self, node):
+        kw = {k: self._val(v) for k, v in node.kwargs.items()}
+        q = kw["query"]
+        if not (kw["key"] is q and kw["value"] is q):
+            self._unsupported(node, "self-attention only (query, key and value must be one tensor)")
+        if q.kind != "transposed" or q.meta["dims"] != (0, 1):
+            self._unsupported(node, "expects the (L, N, E) view produced by transpose(0, 1) of a batch-first tensor")
+        if kw.get("bias_k") is not None or kw.get("bias_v") is not None or kw.get("add_zero_attn"):
+            self._unsupported(node, "bias_k / bias_v / add_zero_attn are not supported")
+        if float(kw.get("dropout_p", 0.0)) != 0.0:
+            self._unsupported(node, "attention dropout with p > 0 is not implemented")
+        x = q.meta["src"]
+        b, S, E = x.t.shape
+        H = kw["num_heads"]
+        if kw["embed_dim_to_check"] != E or E % H:
+            self._unsupported(node, "embed_dim mismatch")
+        hd = E // H
+        if hd % self.epv:
+            self._unsupported(node, f"head_dim {hd} must be a multiple of {self.epv}")
+        w_in, b_in, w_out, b_out = kw["in_proj_weight"], kw["in_proj_bias"], kw["out_proj_weight"], kw["out_proj_bias"]
+        mask = kw.get("attn_mask")
+        mask_t = None
+        if mask is not None:
+            if tuple(mask.t.shape) != (S, S) or mask.t.dtype != torch.float32:
+                self._unsupported(node, "attn_mask must be a float32 [L, S] additive mask")
+            mask_t = mask.t
+        scale = 1.0 / math.sqrt(hd)
+        Sp = _round_up(S, self.epv)
+        qkv = self._new((b, S, 3 * E))
+        P = self._new((b, H, S, Sp))
+        ctx = self._new((b, S, E))
+        o = self._new((b, S, E))
+        out_bsd = Val("tensor", o, needs_grad=True)
+        out = Val("transposed", None, src=out_bsd, dims=(0, 1), needs_grad=True)
+        M = b * S
+        sQ, sP = (S * 3 * E, hd), (H * S * Sp, S * Sp)
+
+        def forward():
+            ops.gemm(x.t, w_in.t, qkv, M, 3 * E, E, transB=True, bias=b_in.meta["master"])
+            ops.gemm(qkv, qkv, P, S, S, hd, transB=True, lda=3 * E, ldb=3 * E, ldc=Sp, alpha=scale, batch1=b, batch2=H,
+                     strideA=sQ, strideB=sQ, strideC=sP, offB=E)
+            ops.softmax_fwd(P, mask_t, P, b * H * S, S, Sp, S)
+            ops.gemm(P, qkv, ctx, S, hd, S, lda=Sp, ldb=3 * E, ldc=E, batch1=b, batch2=H, strideA=sP, strideB=sQ,
+                     strideC=(S * E, hd), offB=2 * E)
+            ops.gemm(ctx, w_out.t, o, M, E, E, transB=True, bias=b_out.meta["master"])
+        self.fwd.append(forward)
+
+        def emit():
+            if out_bsd.grad is None:
+                return
+            do = out_bsd.grad
+            dctx = self._new((b, S, E))
+            dP = self._new((b, H, S, Sp))
+            dqkv = self._new((b, S, 3 * E))
+            gwo, acc_wo = self._param_grad_slot(w_out)
+            gbo, acc_bo = self._param_grad_slot(b_out)
+            gwi, acc_wi = self._param_grad_slot(w_in)
+            gbi, acc_bi = self._param_grad_slot(b_in)
+            gx, acc_x = self._grad_slot(x) if x.needs_grad else (None, False)
+
+            def backward():
+                ops.gemm(do, ctx, gwo, E, E, M, transA=True, accumulate=acc_wo)
+                ops.colsum(do, gbo, M, E, E, acc_bo)
+                ops.gemm(do, w_out.t, dctx, M, E, E)
+                # dP = dctx V^T ; dV = P^T dctx
+                ops.gemm(dctx, qkv, dP, S, S, hd, transB=True, lda=E, ldb=3 * E, ldc=Sp, batch1=b, batch2=H,
+                         strideA=(S * E, hd), strideB=sQ, strideC=sP, offB=2 * E)
+                ops.gemm(P, dctx, dqkv, S, hd, S, transA=True, lda=Sp, ldb=E, ldc=3 * E, batch1=b, batch2=H,
+                         strideA=sP, strideB=(S * E, hd), strideC=sQ, offC=2 * E)
+                ops.softmax_bwd(dP, P, dP, b * H * S, S, Sp)
+                # dQ = scale dS K ; dK = scale dS^T Q
+                ops.gemm(dP, qkv, dqkv, S, hd, S, lda=Sp, ldb=3 * E, ldc=3 * E, alpha=scale, batch1=b, batch2=H,
+                         strideA=sP, strideB=sQ, strideC=sQ, offB=E)
+                ops.gemm(dP, qkv, dqkv, S, hd, S, transA=True, lda=Sp, ldb=3 * E, ldc=3 * E, alpha=scale, batch1=b,
+                         batch2=H, strideA=sP, strideB=sQ, strideC=sQ, offC=E)
+                ops.gemm(dqkv, x.t, gwi, 3 * E, E, M, transA=True, accumulate=acc_wi)
+                ops.colsum(dqkv, gbi, M, 3 * E, 3 * E, acc_bi)
+                if gx is not None:
+                    ops.gemm(dqkv, w_in.t, gx, M, E, 3 * E, accumulate=acc_x)
+            self.bwd.append(backward)
+        self._tape.append(emit)
+        return Val("mha", None, out=out)
+
+    # ---- loss -----------------------------------------------------------------------------------
+    def _log_softmax(self, node):
+        v, dim = self._val(node.args[0]), node.args[1]
+        nd = len(v.shape)
+        if dim < 0:
+            dim += nd
+        if v.t is None or dim != nd - 1:
+            self._unsupported(node, "log_softmax over the last dimension of a materialised tensor only")
+        for u in node.users:
+            if u.target not in (torch.transpose, F.nll_loss):
+                self._unsupported(node, "log-probabilities may only feed transpose / nll_loss")
+        return Val("logprobs", src=v, transposed=False)
+
+    def _nll_loss(self, node):
+        lp, y = self._val(node.args[0]), self._val(node.args[1])
+        if node.kwargs.get("reduction") != "sum" or lp.kind != "logprobs":
+            self._unsupported(node, "expects nll_loss(log_softmax(...), target, reduction='sum')")
+        logits = lp.meta["src"]
+        nd = len(logits.shape)
+        if (nd == 3) != bool(lp.meta["transposed"]):
+            self._unsupported(node, "class dimension must be dim 1 of the nll_loss input")
+        V = logits.shape[-1]
+        ld = logits.ld or V
+        rows = logits.t.numel() // ld
+        tgt = self._input_buffer(y, torch.int64)
+        row_loss = self._new((rows,), torch.float32)
+        loss = self._new((1,), torch.float32)
+        ignore = node.kwargs.get("ignore_index", -100)
+
+        def forward():
+            # writes d(loss)/d(logits) over the logits: the backward pass starts from it
+            ops.logsoftmax_nll(logits.t, tgt, row_loss, logits.t, rows, V, ld, ignore, 1.0)
+            ops.sum_f32(row_loss, loss)
+        self.fwd.append(forward)
+        logits.grad = logits.t
+        return Val("loss", loss)
+
+    # ---- ViT leaves -----------------------------------------------------------------------------
+    def _conv2d(self, node):
+        x, w, b = self._val(node.args[0]), self._val(node.args[1]), self._val(node.args[2])
+        stride, padding, dilation, groups = node.args[3], node.args[4], node.args[5], node.args[6]
+        d, C, ph, pw = w.t.shape
+        if tuple(stride) != (ph, pw) or tuple(padding) != (0, 0) or tuple(dilation) != (1, 1) or groups != 1:
+            self._unsupported(node, "only the patch-embedding form (kernel = stride, no padding) is supported")
+        img = self._input_buffer(x, torch.float32)
+        n, _, Hh, Ww = img.shape
+        gh, gw = Hh // ph, Ww // pw
+        Kc = C * ph * pw
+        if Kc % self.epv:
+            self._unsupported(node, "C*ph*pw must be a multiple of the vector width")
+        cols = self._new((n * gh * gw, Kc))
+        tokens = Val("tensor", self._new((n, gh * gw, d)), needs_grad=True)
+        M = n * gh * gw
+
+        def forward():
+            ops.patchify(img, cols, n, C, gh, gw, ph, pw)
+            ops.gemm(cols, w.t, tokens.t, M, d, Kc, transB=True, bias=b.meta["master"])
+        self.fwd.append(forward)
+
+        def emit():
+            if tokens.grad is None:
+                return
+            gw_, accw = self._param_grad_slot(w)
+            gb_, accb = self._param_grad_slot(b)
+            dy = tokens.grad
+            self.bwd.append(lambda: (ops.gemm(dy, cols, gw_, d, Kc, M, transA=True, accumulate=accw),
+                                     ops.colsum(dy, gb_, M, d, d, accb)))
+        self._tape.append(emit)
+        return Val("conv_out", None, tokens=tokens, shape=(n, d, gh, gw))
+
+    def _flatten(self, node):
+        v = self._val(node.args[0])
+        if v.kind != "conv_out" or node.args[1] != 2 or node.args[2] != -1:
+            self._unsupported(node, "flatten(2, -1) of the patch convolution only")
+        return Val("conv_flat", None, tokens=v.meta["tokens"])
+
+    def _append_cls(self, node):
+        x, cls = self._val(node.args[0]), self._val(node.args[1])
+        users = list(node.users)
+        if not (len(users) == 1 and users[0].target is operator.add):
+            self._unsupported(node, "append_cls_token must be followed by the position-embedding add")
+        return Val("cls_appended", None, x=x, cls=cls)
+
+    def _append_cls_pos(self, node, ac: Val, pos: Val):
+        x, cls = ac.meta["x"], ac.meta["cls"]
+        n, T, d = x.t.shape
+        if tuple(pos.t.shape) != (1, T + 1, d):
+            self._unsupported(node, "position embedding must be [1, T+1, d]")
+        out = Val("tensor", self._new((n, T + 1, d)), needs_grad=True)
+        self.fwd.append(lambda: ops.append_cls_pos(x.t, cls.t, pos.t, out.t, n, T, d))
+
+        def emit():
+            if out.grad is None:
+                return
+            g = out.grad
+            if pos.kind == "param":
+                gp, accp = self._param_grad_slot(pos)
+                self.bwd.append(lambda: ops.colsum(g, gp, n, (T + 1) * d, (T + 1) * d, accp))
+            if cls.kind == "param":
+                gc, accc = self._param_grad_slot(cls)
+                self.bwd.append(lambda: ops.colsum(g, gc, n, d, (T + 1) * d, accc))
+            if x.needs_grad:
+                if x.grad is None:
+                    x.grad = self._new(x.t.shape)
+                    gx = x.grad
+                    self.bwd.append(lambda: ops.slice_rows(g, 1, 1, T, gx))
+                else:
+                    tmp, gx = self._new(x.t.shape), x.grad
+                    self.bwd.append(lambda: (ops.slice_rows(g, 1, 1, T, tmp), ops.add(gx, tmp, gx)))
+        self._tape.append(emit)
+        return out
+
+    def _get_cls(self, node):
+        v = self._val(node.args[0])
+        n, T, d = v.t.shape
+        return Val("cls_view", None, src=v, row_stride=T * d, shape=(n, d), needs_grad=v.needs_grad)
+
+    # ---- collectives (device-local halves + wire) ---------------------------------------------
+    def _peers(self, tag, direction, rank, W, shape, reduction, dtype=None):
+        out = {}
+        for src in range(W):
+            if src != rank:
+                out[src] = self.wire.recv(tag, direction, src, shape, dtype or self.cdt, self.dev, reduction=reduction)
+        return out
+
+    def _emit_gather(self, tag, direction, x_t, dim, L, rank, sink: List[Callable]):
+        """pad own shard -> [wire] -> cut pads and concatenate.  Returns the full tensor."""
+        m, W = max(L), len(L)
+        pshape = ops._with_dim(x_t.shape, dim, m)
+        own = self._new(pshape)
+        peers = self._peers(tag, direction, rank, W, pshape, False)
+        slices = [own if s == rank else peers[s] for s in range(W)]
+        full = self._new(ops._with_dim(x_t.shape, dim, sum(L)))
+        sink.append(lambda: (ops.pad_rows(x_t, dim, m, own), ops.unpad_concat(slices, L, dim, full)))
+        return full
+
+    def _emit_scatter(self, tag, direction, full_t, dim, L, rank, sink: List[Callable], out_t=None):
+        """split + pad -> [wire] -> rank-ordered float32 sum of the pieces for this rank, pad cut off."""
+        m, W = max(L), len(L)
+        pshape = ops._with_dim(full_t.shape, dim, m)
+        sent = [self._new(pshape) for _ in range(W)]
+        peers = self._peers(tag, direction, rank, W, pshape, True)
+        contribs = [sent[rank] if s == rank else peers[s] for s in range(W)]
+        contribs = [c for c in contribs if c is not None]
+        out = out_t if out_t is not None else self._new(ops._with_dim(full_t.shape, dim, L[rank]))
+        sink.append(lambda: (ops.split_pad(full_t, L, dim, m, sent), ops.ragged_reduce(contribs, dim, 0, L[rank], out)))
+        return out
+
+    def _all_gather(self, node):
+        x, dim, L, rank = self._val(node.args[0]), node.args[1], list(node.args[2]), node.args[3]
+        if x.t is None or x.ld is not None:
+            self._unsupported(node, f"all_gather of a {x.kind} value")
+        full = self._emit_gather(node.name, "fwd", x.t, dim, L, rank, self.fwd)
+        out = Val("tensor", full, needs_grad=x.needs_grad)
+
+        def emit():
+            if out.grad is None or not x.needs_grad:
+                return
+            if x.grad is None:
+                x.grad = self._emit_scatter(node.name, "bwd", out.grad, dim, L, rank, self.bwd)
+            else:
+                part = self._emit_scatter(node.name, "bwd", out.grad, dim, L, rank, self.bwd)
+                g = x.grad
+                self.bwd.append(lambda: ops.add(g, part, g))
+        self._tape.append(emit)
+        return out
+
+    def _reduce_scatter(self, node):
+        x, dim, L, rank = self._val(node.args[0]), node.args[1], list(node.args[2]), node.args[3]
+        if x.t is None or x.ld is not None:
+            self._unsupported(node, f"reduce_scatter of a {x.kind} value")
+        piece = self._emit_scatter(node.name, "fwd", x.t, dim, L, rank, self.fwd)
+        out = Val("tensor", piece, needs_grad=x.needs_grad)
+
+        def emit():
+            if out.grad is None or not x.needs_grad:
+                return
+            full = self._emit_gather(node.name, "bwd", out.grad, dim, L, rank, self.bwd)
+            self._accumulate_into(x, full)
+        self._tape.append(emit)
+        return out
+
+    def _emit_exchange(self, tag, direction, x_t, split_dim, cat_dim, split_L, cat_L, rank, sink, act=None):
+        W = len(split_L)
+        pieces = [self._new(ops._with_dim(x_t.shape, split_dim, l)) for l in split_L]
+        own = pieces[rank]
+        parts = []
+        for src in range(W):
+            if src == rank:
+                parts.append(own)
+            else:
+                shape = ops._with_dim(own.shape, cat_dim, cat_L[src])
+                parts.append(self.wire.recv(tag, direction, src, shape, self.cdt, self.dev, reduction=False))
+        out = self._new(ops._with_dim(own.shape, cat_dim, sum(cat_L)))
+        sink.append(lambda: (ops.split_rows(x_t, split_L, split_dim, pieces), ops.concat_rows(parts, cat_dim, out, act)))
+        return out
+
+    def _all_to_all(self, node):
+        x, sd, cd = self._val(node.args[0]), node.args[1], node.args[2]
+        sL, cL, rank = list(node.args[3]), list(node.args[4]), node.args[5]
+        if x.t is None or x.ld is not None:
+            self._unsupported(node, f"all_to_all of a {x.kind} value")
+        fuse = self._wants_fused_relu(node)
+        t = self._emit_exchange(node.name, "fwd", x.t, sd, cd, sL, cL, rank, self.fwd, "relu" if fuse else None)
+        out = Val("tensor", t, needs_grad=x.needs_grad)
+        if fuse:
+            out.meta["fused_act"] = "relu"
+
+        def emit():
+            if out.grad is None or not x.needs_grad:
+                return
+            if fuse:
+                self._relu_backward_through(out)
+            g = self._emit_exchange(node.name, "bwd", out.grad, cd, sd, cL, sL, rank, self.bwd)
+            self._accumulate_into(x, g)
+        self._tape.append(emit)
+        return out
+
+    def _emit_sum(self, tag, direction, x_t, rank, W, sink, out_t=None):
+        peers = self._peers(tag, direction, rank, W, x_t.shape, True)
+        contribs = [x_t if s == rank else peers[s] for s in range(W)]
+        contribs = [c.view(1, -1) for c in contribs if c is not None]
+        out = out_t if out_t is not None else self._new(x_t.shape, x_t.dtype)
+        n = x_t.numel()
+        sink.append(lambda: ops.ragged_reduce(contribs, 1, 0, n, out.view(1, -1)))
+        return out
+
+    def _all_reduce(self, node):
+        x = self._val(node.args[0])
+        if x.t is None or x.ld is not None:
+            self._unsupported(node, f"all_reduce of a {x.kind} value")
+        rank, W = self.rank_hint, self.world_hint
+        t = self._emit_sum(node.name, "fwd", x.t, rank, W, self.fwd)
+        out = Val("tensor", t, needs_grad=x.needs_grad)
+
+        def emit():
+            if out.grad is None or not x.needs_grad:
+                return
+            g = self._emit_sum(node.name, "bwd", out.grad, rank, W, self.bwd)
+            self._accumulate_into(x, g)
+        self._tape.append(emit)
+        return out
+
+    def _dynamic_slice(self, node):
+        v, dim, L, rank = self._val(node.args[0]), node.args[1], list(node.args[2]), node.args[3]
+        if v.kind == "routing" and dim == 2:
+            return Val("routing", which=v.meta["which"], gating=v.meta["gating"], e_lo=sum(L[:rank]), E_loc=L[rank])
+        if v.t is None or v.ld is not None:
+            self._unsupported(node, f"dynamic_slice of a {v.kind} value")
+        off = sum(L[:rank])
+        out = Val("tensor", self._new(ops._with_dim(v.t.shape, dim, L[rank])), needs_grad=v.needs_grad)
+        self.fwd.append(lambda: ops.slice_rows(v.t, dim, off, L[rank], out.t))
+
+        def emit():
+            if out.grad is None or not v.needs_grad:
+                return
+            full = self._new(v.t.shape)
+            self.bwd.append(lambda: (ops.fill_zero(full), ops.place_rows(out.grad, full, dim, off)))
+            self._accumulate_into(v, full)
+        self._tape.append(emit)
+        return out
+
+    # ---- mixture of experts -----------------------------------------------------------------------
+    def _gating(self, node):
+        x, E, C, wg = self._val(node.args[0]), node.args[1], node.args[2], self._val(node.args[3])
+        if x.t is None or wg.kind != "param":
+            self._unsupported(node, "gating expects a materialised input and a parameter")
+        B, S, d = x.t.shape
+        if E % self.epv:
+            self._unsupported(node, f"n_expert must be a multiple of {self.epv}")
+        logits = self._new((B, S, E), torch.float32)
+        r = dict(probs=self._new((B, S, E), torch.float32), index=self._new((B, S, 2), torch.int32),
+                 slot=self._new((B, S, 2), torch.int32), gate=self._new((B, S, 2), torch.float32),
+                 token_of_slot=self._new((B, E, C), torch.int32))
+        dgate = self._new((B, S, 2), torch.float32)
+        self.fwd.append(lambda: (ops.gemm(x.t, wg.t, logits, B * S, E, d), ops.top2_gate_into(logits, C, r)))
+        v = Val("gating", None, x=x, E=E, C=C, r=r, dgate=dgate, dgate_used=False)
+
+        def emit():
+            if not v.meta["dgate_used"]:
+                return
+            dlogits = self._new((B, S, E), torch.float32)
+            dl = self._new((B, S, E)) if self.cdt != torch.float32 else dlogits
+            gw, accw = self._param_grad_slot(wg)
+            gx, accx = self._grad_slot(x) if x.needs_grad else (None, False)
+
+            def backward():
+                ops.top2_gate_bwd(r, dgate, dlogits)
+                if dl is not dlogits:
+                    ops.cast(dlogits, dl)
+                ops.gemm(x.t, dl, gw, d, E, B * S, transA=True, accumulate=accw)
+                if gx is not None:
+                    ops.gemm(dl, wg.t, gx, B * S, d, E, transB=True, accumulate=accx)
+            self.bwd.append(backward)
+        self._tape.append(emit)
+        return v
+
+    def _einsum(self, node):
+        code, a, b = node.args[0], self._val(node.args[1]), self._val(node.args[2])
+        if code == "bsd,bsec->becd":
+            return self._moe_dispatch(node, a, b)
+        if code == "edh,becd->bech":
+            return self._expert_gemm(node, a, b, first=True)
+        if code == "ehd,bech->becd":
+            return self._expert_gemm(node, a, b, first=False)
+        if code == "becd,bsec->bsd":
+            return self._moe_combine(node, a, b)
+        self._unsupported(node, f"einsum code {code!r} has no handler")
+
+    def _moe_dispatch(self, node, x: Val, route: Val):
+        if route.kind != "routing" or route.meta["which"] != "dispatch" or x.t is None:
+            self._unsupported(node, "expects (tokens, dispatch tensor of top_2_gating)")
+        gv = route.meta["gating"]
+        r, E, C = gv.meta["r"], gv.meta["E"], gv.meta["C"]
+        e_lo, E_loc = route.meta["e_lo"], route.meta["E_loc"]
+        B, S, d = x.t.shape
+        out = Val("expert", self._new((E_loc, B, C, d)), shape=(B, E_loc, C, d), needs_grad=True)
+        self.fwd.append(lambda: ops.moe_dispatch(x.t, r, out.t, E, C, e_lo, E_loc))
+
+        def emit():
+            if out.grad is None or not x.needs_grad:
+                return
+            gx, acc = self._grad_slot(x)
+            self.bwd.append(lambda: ops.moe_dispatch_bwd(out.grad, r, gx, C, e_lo, E_loc, acc))
+        self._tape.append(emit)
+        return out
+
+    def _expert_gemm(self, node, w: Val, x: Val, first: bool):
+        if w.kind != "param" or x.kind != "expert":
+            self._unsupported(node, "expects (expert weights, expert-major activations)")
+        E_loc, K, N = w.t.shape
+        El, B, C, Kx = x.t.shape
+        if El != E_loc or Kx != K:
+            self._unsupported(node, "expert weight / activation shapes do not match")
+        M = B * C
+        fuse = self._wants_fused_relu(node)
+        out = Val("expert", self._new((E_loc, B, C, N)), shape=(B, E_loc, C, N), needs_grad=True)
+        if fuse:
+            out.meta["fused_act"] = "relu"
+        self.fwd.append(lambda: ops.gemm(x.t, w.t, out.t, M, N, K, batch1=E_loc, strideA=(M * K, 0), strideB=(K * N, 0),
+                                         strideC=(M * N, 0), act="relu" if fuse else None))
+
+        def emit():
+            if out.grad is None:
+                return
+            if fuse:
+                self._relu_backward_through(out)
+            dy = out.grad
+            gw, accw = self._param_grad_slot(w)
+            self.bwd.append(lambda: ops.gemm(x.t, dy, gw, K, N, M, transA=True, lda=K, ldb=N, batch1=E_loc,
+                                             strideA=(M * K, 0), strideB=(M * N, 0), strideC=(K * N, 0),
+                                             accumulate=accw))
+            if x.needs_grad:
+                gx, accx = self._grad_slot(x)
+                self.bwd.append(lambda: ops.gemm(dy, w.t, gx, M, K, N, transB=True, batch1=E_loc, strideA=(M * N, 0),
+                                                 strideB=(K * N, 0), strideC=(M * K, 0), accumulate=accx))
+        self._tape.append(emit)
+        return out
+
+    def _moe_combine(self, node, eo: Val, route: Val):
+        if route.kind != "routing" or route.meta["which"] != "combine" or eo.kind != "expert":
+            self._unsupported(node, "expects (expert outputs, combine tensor of top_2_gating)")
+        gv = route.meta["gating"]
+        r, E, C = gv.meta["r"], gv.meta["E"], gv.meta["C"]
+        e_lo, E_loc = route.meta["e_lo"], route.meta["E_loc"]
+        _, B, _, d = eo.t.shape
+        S = r["index"].shape[1]
+        out = Val("tensor", self._new((B, S, d)), needs_grad=True)
+        self.fwd.append(lambda: ops.moe_combine(eo.t, r, out.t, C, e_lo, E_loc))
+
+        def emit():
+            if out.grad is None:
+                return
+            if eo.grad is not None:
+                self._unsupported(node, "expert outputs feed one combine only")
+            eo.grad = self._new(eo.t.shape)
+            gv.meta["dgate_used"] = True
+            g, dgate = eo.grad, gv.meta["dgate"]
+            self.bwd.append(lambda: ops.moe_combine_bwd(out.grad, eo.t, r, g, dgate, E, C, e_lo, E_loc))
+        self._tape.append(emit)
+        return out
+
+    # ------------------------------------------------------------------ running
+    def load_inputs(self, *args):
+        for rec, a in zip(self.inputs, args):
+            if rec["buf"] is None:
+                continue
+            src = a if rec["offset"] is None else a.narrow(0, rec["offset"], rec["length"])
+            rec["buf"].copy_(src, non_blocking=True)
+
+    def refresh_shadow(self):
+        if self.shadow is not None:
+            ops.cast(self.master, self.shadow)
+        self._shadow_stale = False
+
+    def forward(self, *args) -> torch.Tensor:
+        if args:
+            self.load_inputs(*args)
+        if self._shadow_stale:
+            self.refresh_shadow()
+        for f in self.fwd:
+            f()
+        return self.loss[0]
+
+    def backward(self):
+        for f in self.bwd:
+            f()
+        self._reduce_replicated_grads()
+
+    def _reduce_replicated_grads(self):
+        for f in self._param_reduce:
+            f()
+
+    # ------------------------------------------------------------------ optimizer (worker.py:47, 74-76)
+    def configure_optimizer(self, kind: str = "adam", lr: float = 5e-4, betas=(0.9, 0.999), eps: float = 1e-8,
+                            clip_grad_norm: Optional[float] = None):
+        if kind not in ("adam", "sgd"):
+            raise ValueError("optimizer must be 'adam' or 'sgd'")
+        self._opt = dict(kind=kind, lr=lr, betas=betas, eps=eps, clip=clip_grad_norm)
+        if kind == "adam":
+            self.exp_avg = torch.zeros_like(self.master)
+            self.exp_avg_sq = torch.zeros_like(self.master)
+        if clip_grad_norm is not None:
+            self._sumsq = torch.zeros(1, dtype=torch.float32, device=self.dev)
+            self._coef = torch.ones(1, dtype=torch.float32, device=self.dev)
+        self._step_count = 0
+
+    def step(self):
+        o = self._opt
+        if o is None:
+            raise RuntimeError("configure_optimizer() first")
+        coef = None
+        if o["clip"] is not None:
+            ops.fill_zero(self._sumsq)
+            ops.sumsq(self.flat_grad, self._sumsq)
+            ops.clip_coef(self._sumsq, o["clip"], self._coef)
+            coef = self._coef
+        self._step_count += 1
+        if o["kind"] == "sgd":
+            ops.sgd_step(self.master, self.flat_grad, self.shadow, o["lr"], coef)
+        else:
+            ops.adam_step(self.master, self.flat_grad, self.exp_avg, self.exp_avg_sq, self.shadow, o["lr"],
+                          o["betas"][0], o["betas"][1], o["eps"], self._step_count, coef)
+
+    def train_step(self, *args) -> torch.Tensor:
+        loss = self.forward(*args)
+        self.backward()
+        self.step()
+        return loss
+
+    def mark_params_dirty(self):
+        """Call after parameters were changed from outside (e.g. by a torch.optim optimizer)."""
+        self._shadow_stale = True
+
+
+def compile_program(gm: torch.fx.GraphModule, example_inputs, dtype: str = "fp32", wire: Optional[Wire] = None,
+                    rank: int = 0, world_size: int = 1, device: str = "cuda:0") -> ShardExecutor:
+    """Compile the emitted program for the global-batch shapes of ``example_inputs`` (tensors or shapes)."""
+    return ShardExecutor(gm, example_inputs, dtype=dtype, wire=wire, rank=rank, world_size=world_size, device=device)
+
+
+def _finish_param_reduce(self: ShardExecutor):
+    """collectives.replicate backward (collectives.py:176-180): sum the replicated parameters'
+    gradients with what the peers send, in rank order, in place."""
+    for node in self.gm.graph.nodes:
+        if node.op == "call_function" and node.target is collectives.replicate:
+            v = self.env[node]
+            if v.kind != "param" or not v.meta.get("grad_written"):
+                continue
+            g = v.meta["grad"]
+            peers = self._peers(node.name, "bwd", self.rank_hint, self.world_hint, g.shape, True, torch.float32)
+            contribs = [g if s == self.rank_hint else peers.get(s) for s in range(self.world_hint)]
+            contribs = [c for c in contribs if c is not None]
+            if len(contribs) > 1:
+                flat = [c.reshape(1, -1) for c in contribs]
+                n = g.numel()
+                self._param_reduce.append(lambda flat=flat, n=n, g=g: ops.ragged_reduce(flat, 1, 0, n, g.view(1, -1)))
+
+
+ShardExecutor._finish_param_reduce = _finish_param_reduce

@@ -1,0 +1,474 @@
+"""Tensor-level wrappers over the C ABI of libhapmi.so.
+
+Every function takes torch tensors that live on the GPU, passes raw device
+pointers to the library and enqueues on torch's current stream.  CPU tensors
+are refused: there is no fallback path.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import List, Optional, Sequence
+
+import torch
+
+from . import _lib
+from ._lib import ACT_GELU, ACT_NONE, ACT_RELU, BF16, F32, GemmArgs, check, lib
+
+_ACT = {None: ACT_NONE, "none": ACT_NONE, "relu": ACT_RELU, "gelu": ACT_GELU}
+
+
+def dtype_code(t) -> int:
+    dt = t if isinstance(t, torch.dtype) else t.dtype
+    if dt == torch.float32:
+        return F32
+    if dt == torch.bfloat16:
+        return BF16
+    raise TypeError(f"dtype {dt} is not handled by the HIP kernels (float32 / bfloat16 only)")
+
+
+def _dev(*tensors):
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise _lib.HapmiError("the HIP kernels take GPU tensors only; got a CPU tensor (no CPU fallback exists)")
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _i64(vals: Sequence[int]):
+    return (ctypes.c_int64 * len(vals))(*[int(v) for v in vals])
+
+
+def _ptrs(tensors: Sequence[Optional[torch.Tensor]]):
+    return (ctypes.c_void_p * len(tensors))(*[t.data_ptr() if t is not None else 0 for t in tensors])
+
+
+def init():
+    check(lib().hapmi_init())
+
+
+# ---------------------------------------------------------------------------
+# layout helpers: a tensor sharded on `dim` is [outer, len, inner]
+# ---------------------------------------------------------------------------
+
+def _oli(shape, dim):
+    outer = 1
+    for s in shape[:dim]:
+        outer *= s
+    inner = 1
+    for s in shape[dim + 1:]:
+        inner *= s
+    return outer, shape[dim], inner
+
+
+def _with_dim(shape, dim, n):
+    return tuple(shape[:dim]) + (n,) + tuple(shape[dim + 1:])
+
+
+def pad_rows(src: torch.Tensor, dim: int, padded_len: int, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """collectives.padded: copy ``src`` into the head of a buffer whose ``dim`` is ``padded_len`` long."""
+    _dev(src, out)
+    assert src.is_contiguous()
+    outer, length, inner = _oli(src.shape, dim)
+    if out is None:
+        out = torch.empty(_with_dim(src.shape, dim, padded_len), dtype=src.dtype, device=src.device)
+    check(lib().hapmi_pad_rows(_ptr(src), _ptr(out), outer, length, padded_len, inner * src.element_size(), _stream()))
+    return out
+
+
+def unpad_concat(slices: Sequence[torch.Tensor], lengths: Sequence[int], dim: int,
+                 out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    _dev(*slices, out)
+    ref = slices[0]
+    outer, padded_len, inner = _oli(ref.shape, dim)
+    if out is None:
+        out = torch.empty(_with_dim(ref.shape, dim, sum(lengths)), dtype=ref.dtype, device=ref.device)
+    check(lib().hapmi_unpad_concat(_ptrs(slices), _i64(lengths), len(lengths), _ptr(out), outer, padded_len,
+                                   inner * ref.element_size(), _stream()))
+    return out
+
+
+def split_pad(src: torch.Tensor, lengths: Sequence[int], dim: int, padded_len: int,
+              outs: Optional[Sequence[torch.Tensor]] = None) -> List[torch.Tensor]:
+    _dev(src)
+    assert src.is_contiguous()
+    outer, total, inner = _oli(src.shape, dim)
+    assert total == sum(lengths)
+    if outs is None:
+        outs = [torch.empty(_with_dim(src.shape, dim, padded_len), dtype=src.dtype, device=src.device) for _ in lengths]
+    check(lib().hapmi_split_pad(_ptr(src), _ptrs(outs), _i64(lengths), len(lengths), outer, padded_len,
+                                inner * src.element_size(), _stream()))
+    return list(outs)
+
+
+def slice_rows(src: torch.Tensor, dim: int, offset: int, length: int, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    _dev(src, out)
+    assert src.is_contiguous()
+    outer, src_len, inner = _oli(src.shape, dim)
+    if out is None:
+        out = torch.empty(_with_dim(src.shape, dim, length), dtype=src.dtype, device=src.device)
+    check(lib().hapmi_slice_rows(_ptr(src), _ptr(out), outer, src_len, offset, length, inner * src.element_size(), _stream()))
+    return out
+
+
+def place_rows(src: torch.Tensor, dst: torch.Tensor, dim: int, offset: int) -> torch.Tensor:
+    _dev(src, dst)
+    outer, length, inner = _oli(src.shape, dim)
+    check(lib().hapmi_place_rows(_ptr(src), _ptr(dst), outer, dst.shape[dim], offset, length,
+                                 inner * src.element_size(), _stream()))
+    return dst
+
+
+def split_rows(src: torch.Tensor, lengths: Sequence[int], dim: int,
+               outs: Optional[Sequence[Optional[torch.Tensor]]] = None) -> List[torch.Tensor]:
+    _dev(src)
+    assert src.is_contiguous()
+    outer, total, inner = _oli(src.shape, dim)
+    assert total == sum(lengths)
+    if outs is None:
+        outs = [torch.empty(_with_dim(src.shape, dim, l), dtype=src.dtype, device=src.device) for l in lengths]
+    check(lib().hapmi_split_rows(_ptr(src), _ptrs(outs), _i64(lengths), len(lengths), outer,
+                                 inner * src.element_size(), _stream()))
+    return list(outs)
+
+
+def concat_rows(pieces: Sequence[torch.Tensor], dim: int, out: Optional[torch.Tensor] = None,
+                act: Optional[str] = None) -> torch.Tensor:
+    _dev(*pieces, out)
+    ref = pieces[0]
+    lengths = [p.shape[dim] for p in pieces]
+    outer, _, inner = _oli(ref.shape, dim)
+    if out is None:
+        out = torch.empty(_with_dim(ref.shape, dim, sum(lengths)), dtype=ref.dtype, device=ref.device)
+    check(lib().hapmi_concat_rows(_ptrs(pieces), _i64(lengths), len(lengths), _ptr(out), outer,
+                                  inner * ref.element_size(), _ACT[act], dtype_code(ref), _stream()))
+    return out
+
+
+def ragged_reduce(contribs: Sequence[torch.Tensor], dim: int, offset: int, length: int,
+                  out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out = sum_w contribs[w].narrow(dim, offset, length) in rank order, float32 accumulation."""
+    _dev(*contribs, out)
+    ref = contribs[0]
+    outer, src_len, inner = _oli(ref.shape, dim)
+    if out is None:
+        out = torch.empty(_with_dim(ref.shape, dim, length), dtype=ref.dtype, device=ref.device)
+    check(lib().hapmi_ragged_reduce(_ptrs(contribs), len(contribs), _ptr(out), outer, src_len, offset, length, inner,
+                                    dtype_code(ref), _stream()))
+    return out
+
+
+# ---------------------------------------------------------------------------
+# GEMM
+# ---------------------------------------------------------------------------
+
+def gemm(A: torch.Tensor, B: torch.Tensor, C: torch.Tensor, M: int, N: int, K: int, *, transA=False, transB=False,
+         lda=None, ldb=None, ldc=None, bias: Optional[torch.Tensor] = None, accumulate=False, act=None, alpha=1.0,
+         batch1=1, batch2=1, strideA=(0, 0), strideB=(0, 0), strideC=(0, 0),
+         offA=0, offB=0, offC=0):
+    """C = alpha * op(A) @ op(B) (+bias)(act)(+C).  Offsets and strides are in elements."""
+    _dev(A, B, C, bias)
+    if A.dtype != B.dtype:
+        raise TypeError("gemm operands must share a dtype")
+    a = GemmArgs()
+    a.A = A.data_ptr() + offA * A.element_size()
+    a.B = B.data_ptr() + offB * B.element_size()
+    a.C = C.data_ptr() + offC * C.element_size()
+    a.bias = bias.data_ptr() if bias is not None else 0
+    if bias is not None and bias.dtype != torch.float32:
+        raise TypeError("gemm bias must be float32")
+    a.M, a.N, a.K = M, N, K
+    a.lda = lda if lda is not None else (M if transA else K)
+    a.ldb = ldb if ldb is not None else (K if transB else N)
+    a.ldc = ldc if ldc is not None else N
+    a.transA, a.transB = int(transA), int(transB)
+    a.in_dtype, a.out_dtype = dtype_code(A), dtype_code(C)
+    a.accumulate, a.act, a.alpha = int(accumulate), _ACT[act], float(alpha)
+    a.batch1, a.batch2 = batch1, batch2
+    a.strideA1, a.strideA2 = strideA
+    a.strideB1, a.strideB2 = strideB
+    a.strideC1, a.strideC2 = strideC
+    check(lib().hapmi_gemm(ctypes.byref(a), _stream()))
+    return C
+
+
+def linear(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, out_dtype=None, act=None) -> torch.Tensor:
+    """F.linear on a [..., K] input with a [N, K] weight."""
+    K = x.shape[-1]
+    M = x.numel() // K
+    N = w.shape[0]
+    out = torch.empty(x.shape[:-1] + (N,), dtype=out_dtype or x.dtype, device=x.device)
+    gemm(x, w, out, M, N, K, transB=True, bias=bias, act=act)
+    return out
+
+
+# ---------------------------------------------------------------------------
+# row-wise
+# ---------------------------------------------------------------------------
+
+def add_layernorm_fwd(x, res, y, rstd, eps=1e-5):
+    _dev(x, res, y, rstd)
+    width = x.shape[-1]
+    rows = x.numel() // width
+    check(lib().hapmi_add_layernorm_fwd(_ptr(x), _ptr(res), _ptr(y), _ptr(rstd), rows, width,
+                                        ctypes.c_float(eps), dtype_code(x), _stream()))
+
+
+def layernorm_bwd(dy, y, rstd, dx_add, dx):
+    _dev(dy, y, rstd, dx_add, dx)
+    width = y.shape[-1]
+    rows = y.numel() // width
+    check(lib().hapmi_layernorm_bwd(_ptr(dy), _ptr(y), _ptr(rstd), _ptr(dx_add), _ptr(dx), rows, width,
+                                    dtype_code(y), _stream()))
+
+
+def softmax_fwd(x, mask, p, rows, width, ld, mask_rows=1):
+    _dev(x, mask, p)
+    check(lib().hapmi_softmax_fwd(_ptr(x), _ptr(mask), _ptr(p), rows, width, ld, mask_rows, dtype_code(x), _stream()))
+
+
+def softmax_bwd(dp, p, ds, rows, width, ld):
+    _dev(dp, p, ds)
+    check(lib().hapmi_softmax_bwd(_ptr(dp), _ptr(p), _ptr(ds), rows, width, ld, dtype_code(p), _stream()))
+
+
+def logsoftmax_nll(logits, targets, row_loss, dlogits, rows, width, ld, ignore_index=-100, grad_scale=1.0):
+    _dev(logits, targets, row_loss, dlogits)
+    if targets.dtype != torch.int64:
+        raise TypeError("targets must be int64")
+    check(lib().hapmi_logsoftmax_nll(_ptr(logits), _ptr(targets), ignore_index, _ptr(row_loss), _ptr(dlogits), rows,
+                                     width, ld, ctypes.c_float(grad_scale), dtype_code(logits), _stream()))
+
+
+def sum_f32(x, out):
+    _dev(x, out)
+    check(lib().hapmi_sum_f32(_ptr(x), x.numel(), _ptr(out), _stream()))
+
+
+# ---------------------------------------------------------------------------
+# elementwise
+# ---------------------------------------------------------------------------
+
+def act_fwd(x, y, act):
+    _dev(x, y)
+    check(lib().hapmi_act_fwd(_ptr(x), _ptr(y), x.numel(), _ACT[act], dtype_code(x), _stream()))
+
+
+def act_bwd(dy, ref, dx, act):
+    _dev(dy, ref, dx)
+    check(lib().hapmi_act_bwd(_ptr(dy), _ptr(ref), _ptr(dx), dy.numel(), _ACT[act], dtype_code(dy), _stream()))
+
+
+def add(a, b, out):
+    _dev(a, b, out)
+    check(lib().hapmi_add(_ptr(a), _ptr(b), _ptr(out), a.numel(), dtype_code(a), _stream()))
+
+
+def scale(a, s, out):
+    _dev(a, out)
+    check(lib().hapmi_scale(_ptr(a), ctypes.c_float(s), _ptr(out), a.numel(), dtype_code(a), _stream()))
+
+
+def add_bcast_rows(a, b, out, rows, b_rows, width):
+    _dev(a, b, out)
+    check(lib().hapmi_add_bcast_rows(_ptr(a), _ptr(b), _ptr(out), rows, b_rows, width, dtype_code(a), _stream()))
+
+
+def colsum(x, out, M, N, ldx=None, accumulate=False):
+    _dev(x, out)
+    check(lib().hapmi_colsum(_ptr(x), _ptr(out), M, N, ldx if ldx is not None else N, int(accumulate),
+                             dtype_code(x), _stream()))
+
+
+def fill_zero(t):
+    _dev(t)
+    check(lib().hapmi_fill_zero(_ptr(t), t.numel() * t.element_size(), _stream()))
+
+
+def cast(src, dst):
+    _dev(src, dst)
+    check(lib().hapmi_cast(_ptr(src), dtype_code(src), _ptr(dst), dtype_code(dst), src.numel(), _stream()))
+
+
+def embedding_fwd(ids, table, pe, out, S, scale_=1.0):
+    _dev(ids, table, pe, out)
+    check(lib().hapmi_embedding_fwd(_ptr(ids), _ptr(table), _ptr(pe), _ptr(out), ids.numel(), table.shape[1], S,
+                                    table.shape[0], ctypes.c_float(scale_), dtype_code(table), _stream()))
+
+
+def embedding_bwd(ids, dout, dtable, scale_=1.0):
+    _dev(ids, dout, dtable)
+    check(lib().hapmi_embedding_bwd(_ptr(ids), _ptr(dout), _ptr(dtable), ids.numel(), dtable.shape[1],
+                                    dtable.shape[0], ctypes.c_float(scale_), dtype_code(dout), _stream()))
+
+
+def patchify(x, cols, b, C, gh, gw, ph, pw):
+    _dev(x, cols)
+    check(lib().hapmi_patchify(_ptr(x), _ptr(cols), b, C, gh, gw, ph, pw, dtype_code(cols), _stream()))
+
+
+def append_cls_pos(patches, cls, pos, out, b, T, d):
+    _dev(patches, cls, pos, out)
+    check(lib().hapmi_append_cls_pos(_ptr(patches), _ptr(cls), _ptr(pos), _ptr(out), b, T, d, dtype_code(out), _stream()))
+
+
+# ---------------------------------------------------------------------------
+# optimizer
+# ---------------------------------------------------------------------------
+
+def sgd_step(param, grad, shadow, lr, grad_scale=None):
+    _dev(param, grad, shadow, grad_scale)
+    check(lib().hapmi_sgd_step(_ptr(param), _ptr(grad), _ptr(shadow), param.numel(), ctypes.c_float(lr),
+                               _ptr(grad_scale), _stream()))
+
+
+def adam_step(param, grad, exp_avg, exp_avg_sq, shadow, lr, beta1, beta2, eps, step, grad_scale=None):
+    _dev(param, grad, exp_avg, exp_avg_sq, shadow, grad_scale)
+    bc1 = 1.0 - beta1 ** step
+    bc2 = 1.0 - beta2 ** step
+    check(lib().hapmi_adam_step(_ptr(param), _ptr(grad), _ptr(exp_avg), _ptr(exp_avg_sq), _ptr(shadow), param.numel(),
+                                ctypes.c_float(lr), ctypes.c_float(beta1), ctypes.c_float(beta2), ctypes.c_float(eps),
+                                ctypes.c_float(bc1), ctypes.c_float(bc2), _ptr(grad_scale), _stream()))
+
+
+def sumsq(g, out):
+    _dev(g, out)
+    check(lib().hapmi_sumsq(_ptr(g), g.numel(), _ptr(out), _stream()))
+
+
+def clip_coef(sumsq_t, max_norm, coef):
+    _dev(sumsq_t, coef)
+    check(lib().hapmi_clip_coef(_ptr(sumsq_t), ctypes.c_float(max_norm), _ptr(coef), _stream()))
+
+
+# ---------------------------------------------------------------------------
+# MoE
+# ---------------------------------------------------------------------------
+
+def top2_gate(logits, capacity):
+    """logits [B,S,E] float32 -> dict(probs, index, slot, gate, token_of_slot)."""
+    _dev(logits)
+    B, S, E = logits.shape
+    dev = logits.device
+    r = dict(probs=torch.empty(B, S, E, dtype=torch.float32, device=dev),
+             index=torch.empty(B, S, 2, dtype=torch.int32, device=dev),
+             slot=torch.empty(B, S, 2, dtype=torch.int32, device=dev),
+             gate=torch.empty(B, S, 2, dtype=torch.float32, device=dev),
+             token_of_slot=torch.empty(B, E, capacity, dtype=torch.int32, device=dev))
+    top2_gate_into(logits, capacity, r)
+    return r
+
+
+def top2_gate_into(logits, capacity, r):
+    B, S, E = logits.shape
+    check(lib().hapmi_top2_gate(_ptr(logits), _ptr(r["probs"]), _ptr(r["index"]), _ptr(r["slot"]), _ptr(r["gate"]),
+                                _ptr(r["token_of_slot"]), B, S, E, capacity, _stream()))
+
+
+def top2_gate_bwd(r, dgate, dlogits):
+    B, S, E = r["probs"].shape
+    check(lib().hapmi_top2_gate_bwd(_ptr(r["probs"]), _ptr(r["index"]), _ptr(r["slot"]), _ptr(dgate), _ptr(dlogits),
+                                    B, S, E, _stream()))
+
+
+def top2_densify(r, E, C):
+    B, S, _ = r["index"].shape
+    dev = r["index"].device
+    dispatch = torch.empty(B, S, E, C, dtype=torch.float32, device=dev)
+    combine = torch.empty(B, S, E, C, dtype=torch.float32, device=dev)
+    check(lib().hapmi_top2_densify(_ptr(r["index"]), _ptr(r["slot"]), _ptr(r["gate"]), _ptr(dispatch), _ptr(combine),
+                                   B, S, E, C, _stream()))
+    return dispatch, combine
+
+
+def moe_dispatch(x, r, expert_in, E, C, e_lo, E_loc):
+    B, S, d = x.shape
+    check(lib().hapmi_moe_dispatch(_ptr(x), _ptr(r["token_of_slot"]), _ptr(expert_in), B, S, E, C, d, e_lo, E_loc,
+                                   dtype_code(x), _stream()))
+
+
+def moe_combine(expert_out, r, out, C, e_lo, E_loc):
+    B, S, d = out.shape
+    check(lib().hapmi_moe_combine(_ptr(expert_out), _ptr(r["index"]), _ptr(r["slot"]), _ptr(r["gate"]), _ptr(out),
+                                  B, S, C, d, e_lo, E_loc, dtype_code(out), _stream()))
+
+
+def moe_combine_bwd(dout, expert_out, r, d_expert_out, dgate, E, C, e_lo, E_loc):
+    B, S, d = dout.shape
+    check(lib().hapmi_moe_combine_bwd(_ptr(dout), _ptr(expert_out), _ptr(r["index"]), _ptr(r["slot"]), _ptr(r["gate"]),
+                                      _ptr(r["token_of_slot"]), _ptr(d_expert_out), _ptr(dgate), B, S, E, C, d, e_lo,
+                                      E_loc, dtype_code(dout), _stream()))
+
+
+def moe_dispatch_bwd(d_expert_in, r, dx, C, e_lo, E_loc, accumulate):
+    B, S, d = dx.shape
+    check(lib().hapmi_moe_dispatch_bwd(_ptr(d_expert_in), _ptr(r["index"]), _ptr(r["slot"]), _ptr(r["gate"]), _ptr(dx),
+                                       B, S, C, d, e_lo, E_loc, int(accumulate), dtype_code(dx), _stream()))
+
+
+# ---------------------------------------------------------------------------
+# leaf ops with autograd, for direct (eager) use of the emitted graph's callables
+# ---------------------------------------------------------------------------
+
+class _AppendCls(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, cls_token):
+        _dev(x, cls_token)
+        b, T, d = x.shape
+        out = torch.empty(b, T + 1, d, dtype=x.dtype, device=x.device)
+        zeros = torch.zeros(T + 1, d, dtype=x.dtype, device=x.device)
+        append_cls_pos(x.contiguous(), cls_token.contiguous(), zeros, out, b, T, d)
+        return out
+
+    @staticmethod
+    def backward(ctx, g):
+        g = g.contiguous()
+        b, T1, d = g.shape
+        dx = slice_rows(g, 1, 1, T1 - 1)
+        dcls = torch.empty(d, dtype=torch.float32, device=g.device)
+        colsum(g, dcls, b, d, ldx=T1 * d)
+        return dx, dcls.to(g.dtype).view(1, 1, d)
+
+
+def append_cls_token(x, cls_token):
+    return _AppendCls.apply(x, cls_token)
+
+
+class _GetCls(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x):
+        _dev(x)
+        ctx.shape = x.shape
+        b, T, d = x.shape
+        return slice_rows(x.contiguous().view(b, T, d), 1, 0, 1).view(b, d)
+
+    @staticmethod
+    def backward(ctx, g):
+        b, T, d = ctx.shape
+        dx = torch.empty(b, T, d, dtype=g.dtype, device=g.device)
+        fill_zero(dx)
+        place_rows(g.contiguous().view(b, 1, d), dx, 1, 0)
+        return dx
+
+
+def get_cls_token(x):
+    return _GetCls.apply(x)
+
+
+def top_2_gating_dense(gate_input, n_expert, capacity, gate_weight):
+    """Dense (dispatch, combine) [B,S,E,C] from the index-form gate kernel (forward only)."""
+    _dev(gate_input, gate_weight)
+    B, S, d = gate_input.shape
+    x = gate_input.contiguous()
+    w = gate_weight.contiguous().to(x.dtype)
+    logits = torch.empty(B, S, n_expert, dtype=torch.float32, device=x.device)
+    if n_expert % 4 != 0:
+        raise _lib.HapmiError("top_2_gating: n_expert must be a multiple of 4")
+    gemm(x, w, logits, B * S, n_expert, d)
+    r = top2_gate(logits, capacity)
+    return top2_densify(r, n_expert, capacity)

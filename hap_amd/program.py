@@ -1,0 +1,211 @@
+"""Generator of the per-device SPMD program as a ``torch.fx`` graph.
+
+The reference obtains this graph from its synthesizer (``hap.main``,
+/root/reference/hap.rs:81-188); the search and the LP are outside this
+package, so the graph is generated directly for fixed, legal plans.  Every
+node uses the form the reference's code generator emits, so an executor for
+these graphs is an executor for the synthesizer's output:
+
+* inputs       placeholder -> ``.split(lengths, dim)`` -> ``getitem(rank)``  (hap.rs:2504-2520)
+* parameters   replicated: ``get_attr`` -> ``collectives.replicate``          (hap.rs:2561-2568)
+               sharded: ``get_attr`` of a tensor sliced in place             (hap.rs:2588-2596, 36-47)
+* ops          ``F.linear(x, w, b)`` (1032), ``torch.transpose(x, a, b)`` (1213),
+               ``F.multi_head_attention_forward(**kw)`` + 2 getitems (1301-1327),
+               ``F.relu(x, inplace=..)`` (1417), ``F.dropout(x, p)`` (1464),
+               ``operator.add`` (1515), ``operator.mul(x, num)`` (1563),
+               ``F.layer_norm(x, shape)`` (1653), ``F.conv2d(x, w, b, stride, padding, (1, 1), 1)`` (1723),
+               ``torch.flatten(x, start, -1)`` (1779), ``torch.log_softmax(x, dim)`` (1829),
+               ``F.nll_loss(x, y, reduction=..)`` (1881), ``F.embedding(ids, table)`` (2041),
+               ``models.append_cls_token`` (2093), ``models.get_cls_token`` (2141),
+               ``models.top_2_gating(x, E, C, wg)`` + 2 getitems (2201-2203),
+               ``torch.einsum(code, a, b)`` (2273)
+* collectives  ``all_gather(t, dim, L, rank)`` (2641), ``dynamic_slice`` (2662),
+               ``reduce_scatter`` (2680), ``all_reduce(t)`` (2701),
+               ``all_to_all(t, split_dim, cat_dim, split_L, cat_L, rank)`` (2723-2730)
+* output       the device's partial loss (hap.rs:2602-2615)
+
+Plans (each step is a legal Hoare triple of hap.rs:2786-3419):
+``ffn="column"``  batch-sharded attention, all_gather, column-sharded FFN1 on
+                  the replicated rows, all_to_all, batch-sharded FFN2;
+``ffn="batch"``   pure uneven data parallelism;
+MoE layers        gating on replicated tokens, experts sharded over the
+                  expert dimension, combine -> reduce_scatter / all_reduce.
+"""
+from __future__ import annotations
+
+import math
+import operator
+from typing import List, Optional
+
+import torch
+import torch.fx
+import torch.nn as nn
+import torch.nn.functional as F
+
+from . import collectives, models
+from .sharding import ShardingPlan, shard_inplace
+
+
+class _Emitter:
+    def __init__(self, module: nn.Module, plan: ShardingPlan):
+        self.g = torch.fx.Graph()
+        self.module = module
+        self.plan = plan
+        self.rank = plan.rank
+        self._attr_cache = {}
+
+    # inputs -------------------------------------------------------------
+    def sharded_input(self, name: str, full_length: int, dim: int = 0):
+        ph = self.g.placeholder(name)
+        chunks = self.g.call_method("split", (ph, self.plan.lengths(full_length), dim))
+        return self.g.call_function(operator.getitem, (chunks, self.rank))
+
+    def whole_input(self, name: str):
+        return self.g.placeholder(name)
+
+    # parameters ---------------------------------------------------------
+    def replicated(self, target: str):
+        if target not in self._attr_cache:
+            attr = self.g.get_attr(target)
+            self._attr_cache[target] = self.g.call_function(collectives.replicate, (attr,))
+        return self._attr_cache[target]
+
+    def sharded(self, target: str, full_length: int, dim: int):
+        if target not in self._attr_cache:
+            shard_inplace(self.module, target, self.plan.lengths(full_length), dim, self.rank)
+            self._attr_cache[target] = self.g.get_attr(target)
+        return self._attr_cache[target]
+
+    def call(self, fn, *args, **kwargs):
+        return self.g.call_function(fn, tuple(args), kwargs or None)
+
+
+def _attention(e: _Emitter, h, prefix: str, emsize: int, nheads: int, p: float, mask):
+    t = e.call(torch.transpose, h, 0, 1)
+    kw = dict(query=t, key=t, value=t,
+              in_proj_weight=e.replicated(prefix + "self_attn.in_proj_weight"),
+              in_proj_bias=e.replicated(prefix + "self_attn.in_proj_bias"),
+              out_proj_weight=e.replicated(prefix + "self_attn.out_proj.weight"),
+              out_proj_bias=e.replicated(prefix + "self_attn.out_proj.bias"))
+    if mask is not None:
+        kw["attn_mask"] = mask
+    kw.update(embed_dim_to_check=emsize, num_heads=nheads, bias_k=None, bias_v=None,
+              add_zero_attn=False, dropout_p=p)
+    both = e.g.call_function(F.multi_head_attention_forward, (), kw)
+    out = e.call(operator.getitem, both, 0)
+    e.call(operator.getitem, both, 1)            # head-averaged probabilities: bound, never consumed
+    out = e.call(torch.transpose, out, 0, 1)
+    out = e.call(F.dropout, out, p)
+    s = e.call(operator.add, h, out)
+    return e.call(F.layer_norm, s, (emsize,))
+
+
+def _activation(e: _Emitter, x, activation: str):
+    if activation == "relu":
+        return e.g.call_function(F.relu, (x,), {"inplace": False})
+    if activation == "gelu":
+        return e.call(F.gelu, x)
+    raise ValueError(f"activation {activation!r} has no handler")
+
+
+def _dense_ffn(e: _Emitter, h1, prefix: str, emsize: int, nhid: int, B: int, p: float,
+               activation: str, batch_sharded: bool):
+    plan = e.plan
+    if plan.ffn == "column" and batch_sharded:
+        L_B, L_F = plan.lengths(B), plan.lengths(nhid)
+        full = e.call(collectives.all_gather, h1, 0, L_B, e.rank)
+        u = e.call(F.linear, full, e.sharded(prefix + "linear1.weight", nhid, 0),
+                   e.sharded(prefix + "linear1.bias", nhid, 0))
+        u = e.call(collectives.all_to_all, u, 0, 2, L_B, L_F, e.rank)
+    else:
+        u = e.call(F.linear, h1, e.replicated(prefix + "linear1.weight"), e.replicated(prefix + "linear1.bias"))
+    u = _activation(e, u, activation)
+    u = e.call(F.dropout, u, p)
+    o = e.call(F.linear, u, e.replicated(prefix + "linear2.weight"), e.replicated(prefix + "linear2.bias"))
+    o = e.call(F.dropout, o, p)
+    s = e.call(operator.add, h1, o)
+    return e.call(F.layer_norm, s, (emsize,))
+
+
+def _moe_ffn(e: _Emitter, h1, prefix: str, emsize: int, n_expert: int, capacity: int, B: int,
+             batch_sharded: bool):
+    L_E = e.plan.lengths(n_expert)
+    if batch_sharded:
+        L_B = e.plan.lengths(B)
+        tokens = e.call(collectives.all_gather, h1, 0, L_B, e.rank)
+    else:
+        tokens = h1
+    gating = e.call(models.top_2_gating, tokens, n_expert, capacity, e.replicated(prefix + "gate_weight"))
+    dispatch = e.call(operator.getitem, gating, 0)
+    combine = e.call(operator.getitem, gating, 1)
+    dispatch = e.call(collectives.dynamic_slice, dispatch, 2, L_E, e.rank)
+    combine = e.call(collectives.dynamic_slice, combine, 2, L_E, e.rank)
+    w1 = e.sharded(prefix + "w1", n_expert, 0)
+    w2 = e.sharded(prefix + "w2", n_expert, 0)
+    x = e.call(torch.einsum, "bsd,bsec->becd", tokens, dispatch)
+    x = e.call(torch.einsum, "edh,becd->bech", w1, x)
+    x = e.g.call_function(F.relu, (x,), {"inplace": False})
+    x = e.call(torch.einsum, "ehd,bech->becd", w2, x)
+    partial = e.call(torch.einsum, "becd,bsec->bsd", x, combine)
+    if batch_sharded:
+        o = e.call(collectives.reduce_scatter, partial, 0, L_B, e.rank)
+    else:
+        o = e.call(collectives.all_reduce, partial)
+    s = e.call(operator.add, h1, o)
+    return e.call(F.layer_norm, s, (emsize,))
+
+
+def build_program(model: nn.Module, plan: ShardingPlan, global_batch: int,
+                  activation: str = "relu", batch_sharded: bool = True) -> torch.fx.GraphModule:
+    """Slice ``model``'s parameters in place for ``plan.rank`` and return the
+    rank's program.  ``batch_sharded=False`` keeps the batch replicated (every
+    op on the whole batch; only expert weights are sharded)."""
+    e = _Emitter(model, plan)
+    B = global_batch
+    p = float(model.dropout_p)
+    d = model.emsize
+
+    if model.family == "lm":
+        if batch_sharded:
+            x = e.sharded_input("x", B)
+            y = e.sharded_input("y", B)
+        else:
+            x, y = e.whole_input("x"), e.whole_input("y")
+        h = e.call(F.embedding, x, e.replicated("encoder.weight"))
+        h = e.call(operator.mul, h, math.sqrt(d))
+        h = e.call(operator.add, h, e.g.get_attr("pe"))          # [1,S,d]: size-1 dim, never split
+        mask = e.replicated("src_mask") if getattr(model, "src_mask", None) is not None else None
+    elif model.family == "vit":
+        x = e.sharded_input("x", B)
+        y = e.sharded_input("y", B)
+        pe = model.patch_embed
+        c = e.call(F.conv2d, x, e.replicated("patch_embed.proj.weight"), e.replicated("patch_embed.proj.bias"),
+                   tuple(pe.patch_size), (0, 0), (1, 1), 1)
+        c = e.call(torch.flatten, c, 2, -1)
+        c = e.call(torch.transpose, c, 1, 2)
+        c = e.call(models.append_cls_token, c, e.replicated("cls_token"))
+        h = e.call(operator.add, c, e.replicated("pos_embed"))
+        mask = None
+    else:
+        raise ValueError(f"model family {model.family!r} has no handler")
+
+    for i, layer in enumerate(model.layers):
+        prefix = f"layers.{i}."
+        h1 = _attention(e, h, prefix, d, model.nheads, p, mask)
+        if isinstance(layer, models.Top2TransformerEncoderLayer):
+            h = _moe_ffn(e, h1, prefix, d, layer.n_expert, layer.capacity, B, batch_sharded)
+        else:
+            h = _dense_ffn(e, h1, prefix, d, model.nhid, B, p, activation, batch_sharded)
+
+    if model.family == "lm":
+        logits = e.call(F.linear, h, e.replicated("decoder.weight"), e.replicated("decoder.bias"))
+        lp = e.call(torch.log_softmax, logits, 2)
+        lp = e.call(torch.transpose, lp, 1, 2)
+    else:
+        c = e.call(models.get_cls_token, h)
+        logits = e.call(F.linear, c, e.replicated("decoder.weight"), e.replicated("decoder.bias"))
+        lp = e.call(torch.log_softmax, logits, 1)
+    loss = e.g.call_function(F.nll_loss, (lp, y), {"reduction": "sum"})
+    e.g.output(loss)
+    e.g.lint()
+    return torch.fx.GraphModule(model, e.g)

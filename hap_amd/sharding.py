@@ -1,0 +1,64 @@
+"""Integer shard lengths and in-place parameter slicing.
+
+``sharding_round`` is the layout contract of the whole program: every split,
+pad and concat extent is derived from it (/root/reference/hap.rs:3536-3559,
+exported to Python at hap.rs:211-218 as a function that overwrites the ratio
+list with the integer lengths).  The arithmetic runs in the native library
+(``hapmi_sharding_round``); there is no Python fallback.
+
+``shard_inplace`` follows split_param_or_buffer (hap.rs:36-47).
+"""
+from __future__ import annotations
+
+import ctypes
+from dataclasses import dataclass, field
+from typing import List, Sequence
+
+import torch
+
+from . import _lib
+
+
+def sharding_lengths(full_length: int, ratios: Sequence[float]) -> List[int]:
+    """Integer lengths for ``full_length`` units under ``ratios`` (pure)."""
+    n = len(ratios)
+    r = (ctypes.c_double * n)(*[float(x) for x in ratios])
+    out = (ctypes.c_int64 * n)()
+    _lib.check(_lib.lib().hapmi_sharding_round(int(full_length), r, n, out))
+    return [int(v) for v in out]
+
+
+def sharding_round(full_length: int, ratios: list) -> None:
+    """Drop-in for ``hap.sharding_round``: overwrites ``ratios`` in place with
+    the integer lengths (hap.rs:211-218)."""
+    lengths = sharding_lengths(full_length, ratios)
+    for i, v in enumerate(lengths):
+        ratios[i] = v
+
+
+def shard_inplace(module: torch.nn.Module, target: str, lengths: Sequence[int], dim: int, rank: int) -> None:
+    """``p.data = torch.split(p.data, lengths, dim)[rank]``; a dimension of
+    size 1 is left alone (the broadcast hack, hap.rs:44-45)."""
+    try:
+        p = module.get_parameter(target)
+    except AttributeError:
+        p = module.get_buffer(target)
+    if p.data.shape[dim] == 1:
+        return
+    p.data = torch.split(p.data, list(lengths), dim)[rank].contiguous()
+
+
+@dataclass
+class ShardingPlan:
+    """Per-segment device ratios plus this device's rank (hap.rs:865, 178-180)."""
+    ratios: List[List[float]]
+    rank: int
+    ffn: str = "column"          # "column": FFN1 column-sharded (plan P1); "batch": pure DP (plan P2)
+    segment: int = 0
+
+    @property
+    def world_size(self) -> int:
+        return len(self.ratios[0])
+
+    def lengths(self, full_length: int, segment: int = 0) -> List[int]:
+        return sharding_lengths(full_length, self.ratios[min(segment, len(self.ratios) - 1)])

@@ -1,0 +1,80 @@
+"""Stand-ins for the wire half of the uneven collectives.
+
+This package executes ONE device's share of the SPMD program; no data crosses
+the device.  Every ``collectives.*`` call is therefore: local preparation
+kernel -> wire -> local completion kernel, and the wire is one of the objects
+below.  They hand out what the peers would have sent as static GPU tensors.
+
+* ``SilentWire``     peers send nothing to reductions and zeros to gathers.
+* ``SyntheticWire``  peers send seeded N(0, scale) data of the right shape
+                     (generated on the CPU, uploaded once).
+* ``ReplayWire``     peers send what a recorded run of all ranks sent
+                     (``log[(tag, direction)][src][dst]`` CPU tensors).
+
+With more than one GPU the wire would be RCCL point-to-point sends of the
+exact (unpadded) extents; that transport is not part of this package.
+"""
+from __future__ import annotations
+
+from typing import Dict, Optional, Tuple
+
+import torch
+
+
+class Wire:
+    """``recv(tag, direction, src, shape, dtype, device)`` returns the tensor that rank
+    ``src`` sent to this rank at collective ``tag`` (``direction`` 'fwd' or 'bwd'), or
+    None when that peer contributes nothing."""
+
+    def recv(self, tag: str, direction: str, src: int, shape, dtype, device) -> Optional[torch.Tensor]:
+        raise NotImplementedError
+
+
+class SilentWire(Wire):
+    def __init__(self, gather_fill: float = 0.0):
+        self.gather_fill = gather_fill
+        self._cache: Dict[Tuple, torch.Tensor] = {}
+
+    def recv(self, tag, direction, src, shape, dtype, device, reduction: bool = False):
+        if reduction:
+            return None
+        key = (tuple(shape), dtype)
+        if key not in self._cache:
+            self._cache[key] = torch.full(tuple(shape), self.gather_fill, dtype=dtype, device=device)
+        return self._cache[key]
+
+
+class SyntheticWire(Wire):
+    def __init__(self, seed: int = 0, scale: float = 1.0, grad_scale: float = 1e-3, reduce_params: bool = False):
+        self.gen = torch.Generator().manual_seed(seed)
+        self.scale, self.grad_scale = scale, grad_scale
+        self.reduce_params = reduce_params
+        self._cache: Dict[Tuple, torch.Tensor] = {}
+
+    def recv(self, tag, direction, src, shape, dtype, device, reduction: bool = False):
+        if tag.startswith("replicate") and not self.reduce_params:
+            return None
+        key = (tag, direction, src)
+        if key not in self._cache:
+            s = self.scale if direction == "fwd" else self.grad_scale
+            t = torch.randn(tuple(shape), generator=self.gen, dtype=torch.float32) * s
+            self._cache[key] = t.to(dtype).to(device)
+        return self._cache[key]
+
+
+class ReplayWire(Wire):
+    def __init__(self, log: dict, rank: int):
+        self.log, self.rank = log, rank
+        self._cache: Dict[Tuple, torch.Tensor] = {}
+
+    def recv(self, tag, direction, src, shape, dtype, device, reduction: bool = False):
+        key = (tag, direction, src)
+        if key not in self._cache:
+            if (tag, direction) not in self.log:
+                raise KeyError(f"no recorded message for collective {tag!r} ({direction})")
+            t = self.log[(tag, direction)][src][self.rank]
+            if tuple(t.shape) != tuple(shape):
+                raise ValueError(f"recorded message for {tag!r} ({direction}) from rank {src} has shape "
+                                 f"{tuple(t.shape)}, the program expects {tuple(shape)}")
+            self._cache[key] = t.detach().to(dtype).contiguous().to(device)
+        return self._cache[key]

@@ -1,0 +1,243 @@
+/*
+ * libhapmi -- flat C ABI of the MI355X (gfx950) kernels that execute one
+ * device's shard of a HAP SPMD program.
+ *
+ * The reference (alibaba/hap) has no native kernels and no FFI for this path:
+ * its emitted torch.fx graph calls PyTorch ops (cuBLAS/cuDNN below them) and
+ * collectives.py.  Each entry point below therefore cites the reference NODE
+ * FORM (the call the synthesizer emits, /root/reference/hap.rs) or the
+ * Python function (/root/reference/collectives.py, models.py) it replaces.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless its name ends in _host;
+ *     the caller owns all memory, nothing is allocated or freed here;
+ *   - all work is enqueued on `stream` (a hipStream_t passed as void*); no
+ *     entry point synchronises with the host;
+ *   - return value 0 = success, negative = HAPMI_E* code; hapmi_last_error()
+ *     returns a thread-local message for the last failure;
+ *   - tensors are row-major and contiguous unless a leading dimension (ld*)
+ *     or stride is given; `dtype` is HAPMI_F32 or HAPMI_BF16.
+ */
+#ifndef HAPMI_H
+#define HAPMI_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void *hapmi_stream_t;
+
+enum { HAPMI_F32 = 0, HAPMI_BF16 = 1 };
+enum { HAPMI_ACT_NONE = 0, HAPMI_ACT_RELU = 1, HAPMI_ACT_GELU = 2 };
+enum {
+    HAPMI_OK = 0,
+    HAPMI_EINVAL = -1,   /* bad shape / argument            */
+    HAPMI_EALIGN = -2,   /* pointer or stride not aligned   */
+    HAPMI_EARCH = -3,    /* device is not gfx950            */
+    HAPMI_ELAUNCH = -4,  /* HIP reported a launch error     */
+    HAPMI_ELIMIT = -5    /* size beyond a documented limit  */
+};
+#define HAPMI_MAX_RANKS 64
+
+/* ---- host side ------------------------------------------------------- */
+int hapmi_init(void);
+const char *hapmi_last_error(void);
+int hapmi_version(void);
+
+/* hap.rs:3536-3559 sharding_round (exported to Python at hap.rs:211-218):
+ * integer shard lengths for `full_length` units under `ratios`. Host only. */
+int hapmi_sharding_round(int64_t full_length, const double *ratios_host, int64_t n_ranks,
+                         int64_t *lengths_host);
+
+/* ---- uneven-collective local halves (collectives.py) ------------------
+ * A tensor is seen as [outer, len, inner] with the sharded dimension in the
+ * middle; `inner_bytes` = inner * element size.                           */
+
+/* collectives.py:9-12 padded(): dst[outer, padded_len, inner] <- src[outer, len, inner];
+ * the tail rows are left untouched (the reference leaves them uninitialised). */
+int hapmi_pad_rows(const void *src, void *dst, int64_t outer, int64_t len, int64_t padded_len,
+                   int64_t inner_bytes, hapmi_stream_t stream);
+
+/* collectives.py:20 / :102: cut the pad off W padded slices [outer, padded_len, inner]
+ * and concatenate them along the sharded dimension into dst[outer, sum(lengths), inner]. */
+int hapmi_unpad_concat(const void *const *slices_host, const int64_t *lengths_host, int n_ranks, void *dst,
+                       int64_t outer, int64_t padded_len, int64_t inner_bytes, hapmi_stream_t stream);
+
+/* collectives.py:24-25 / :92-93: split src[outer, sum(lengths), inner] along the
+ * sharded dimension and pad every piece into its own [outer, padded_len, inner] buffer. */
+int hapmi_split_pad(const void *src, void *const *slices_host, const int64_t *lengths_host, int n_ranks,
+                    int64_t outer, int64_t padded_len, int64_t inner_bytes, hapmi_stream_t stream);
+
+/* collectives.py:146-148 dynamic_slice, and the slice-off-pad of :28 / :96:
+ * dst[outer, len, inner] <- src[outer, src_len, inner][:, offset:offset+len, :]. */
+int hapmi_slice_rows(const void *src, void *dst, int64_t outer, int64_t src_len, int64_t offset, int64_t len,
+                     int64_t inner_bytes, hapmi_stream_t stream);
+
+/* inverse of hapmi_slice_rows: dst[:, offset:offset+len, :] <- src (rest of dst untouched). */
+int hapmi_place_rows(const void *src, void *dst, int64_t outer, int64_t dst_len, int64_t offset, int64_t len,
+                     int64_t inner_bytes, hapmi_stream_t stream);
+
+/* collectives.py:156-158 / :163-165: split src[outer, sum(lengths), inner] into W
+ * contiguous unpadded pieces (the all_to_all send buffers). */
+int hapmi_split_rows(const void *src, void *const *pieces_host, const int64_t *lengths_host, int n_ranks,
+                     int64_t outer, int64_t inner_bytes, hapmi_stream_t stream);
+
+/* collectives.py:159 / :166: concatenate W contiguous pieces [outer, lengths[i], inner]
+ * into dst[outer, sum(lengths), inner]; `act` != NONE applies the activation to
+ * every element on the way (dtype needed then). */
+int hapmi_concat_rows(const void *const *pieces_host, const int64_t *lengths_host, int n_ranks, void *dst,
+                      int64_t outer, int64_t inner_bytes, int act, int dtype, hapmi_stream_t stream);
+
+/* the local sum of dist.reduce_scatter / dist.all_reduce (collectives.py:27, :95, :77):
+ * dst[outer, len, inner] = sum_w contribs[w][outer, src_len, inner][:, offset:offset+len, :]
+ * accumulated in float32 in rank order. */
+int hapmi_ragged_reduce(const void *const *contribs_host, int n_ranks, void *dst, int64_t outer, int64_t src_len,
+                        int64_t offset, int64_t len, int64_t inner, int dtype, hapmi_stream_t stream);
+
+/* ---- GEMM: F.linear (hap.rs:1032) and the expert einsums (hap.rs:2273) --
+ * C[z] = op(A[z]) * op(B[z]) (+ bias[N]) (act) (+ C[z] if accumulate)
+ * op(A) is [M,K]: transA=0 -> A stored [M,K] (lda), transA=1 -> A stored [K,M];
+ * op(B) is [K,N]: transB=0 -> B stored [K,N] (ldb), transB=1 -> B stored [N,K].
+ * z = z1 * batch2 + z2 addresses X + z1*strideX1 + z2*strideX2 (elements).
+ * Accumulation is float32; in/out element types are given separately. */
+typedef struct {
+    const void *A, *B;
+    void *C;
+    const void *bias;            /* float32[N] or NULL */
+    int64_t M, N, K;
+    int64_t lda, ldb, ldc;
+    int transA, transB;
+    int in_dtype, out_dtype;
+    int accumulate;              /* 1: C += result (C read in out_dtype) */
+    int act;
+    float alpha;                 /* result scaled before bias */
+    int64_t batch1, batch2;      /* >= 1 */
+    int64_t strideA1, strideA2, strideB1, strideB2, strideC1, strideC2;
+} hapmi_gemm_args;
+int hapmi_gemm(const hapmi_gemm_args *args_host, hapmi_stream_t stream);
+
+/* ---- row-wise kernels ------------------------------------------------- */
+/* operator.add + F.layer_norm(x, (width,)) without affine, eps (hap.rs:1515, 1653):
+ * y = LN(x + res); res may be NULL; rstd[rows] (float32) is kept for backward. */
+int hapmi_add_layernorm_fwd(const void *x, const void *res, void *y, float *rstd, int64_t rows, int64_t width,
+                            float eps, int dtype, hapmi_stream_t stream);
+/* dx = rstd * (dy - mean(dy) - y * mean(dy * y)) (+ dx_add if not NULL) */
+int hapmi_layernorm_bwd(const void *dy, const void *y, const float *rstd, const void *dx_add, void *dx,
+                        int64_t rows, int64_t width, int dtype, hapmi_stream_t stream);
+
+/* softmax over the last dimension of [rows, width] (row stride ld elements, the same for
+ * input and output) with an optional additive float32 mask[mask_rows, width] (contiguous;
+ * row r uses mask row r % mask_rows), in place allowed:
+ * the explicit attention path of torch's multi_head_attention_forward (hap.rs:1301). */
+int hapmi_softmax_fwd(const void *x, const float *mask, void *p, int64_t rows, int64_t width, int64_t ld,
+                      int64_t mask_rows, int dtype, hapmi_stream_t stream);
+/* ds = p * (dp - sum(dp * p)) */
+int hapmi_softmax_bwd(const void *dp, const void *p, void *ds, int64_t rows, int64_t width, int64_t ld, int dtype,
+                      hapmi_stream_t stream);
+
+/* torch.log_softmax + F.nll_loss(reduction='sum', ignore_index) (hap.rs:1829, 1881) and their
+ * backward in one pass: row_loss[rows] float32, dlogits = (softmax - onehot) * grad_scale for
+ * counted rows and 0 for ignored rows; dlogits may alias logits; rows of both are ld elements apart. */
+int hapmi_logsoftmax_nll(const void *logits, const int64_t *targets, int64_t ignore_index, float *row_loss,
+                         void *dlogits, int64_t rows, int64_t width, int64_t ld, float grad_scale, int dtype,
+                         hapmi_stream_t stream);
+/* out[0] = sum of x[0..n) in a fixed order (deterministic) */
+int hapmi_sum_f32(const float *x, int64_t n, float *out, hapmi_stream_t stream);
+
+/* ---- elementwise ------------------------------------------------------- */
+/* F.relu (hap.rs:1417) / F.gelu */
+int hapmi_act_fwd(const void *x, void *y, int64_t n, int act, int dtype, hapmi_stream_t stream);
+/* relu: ref = y (output); gelu: ref = x (input) */
+int hapmi_act_bwd(const void *dy, const void *ref, void *dx, int64_t n, int act, int dtype, hapmi_stream_t stream);
+/* out = a + b (operator.add, hap.rs:1515; also gradient accumulation) */
+int hapmi_add(const void *a, const void *b, void *out, int64_t n, int dtype, hapmi_stream_t stream);
+/* out = a * s (operator.mul with a number, hap.rs:1563) */
+int hapmi_scale(const void *a, float s, void *out, int64_t n, int dtype, hapmi_stream_t stream);
+/* out[r, :] = a[r, :] + b[r % b_rows, :] (broadcast add of pe / pos_embed, hap.rs:3821-3837) */
+int hapmi_add_bcast_rows(const void *a, const void *b, void *out, int64_t rows, int64_t b_rows, int64_t width,
+                         int dtype, hapmi_stream_t stream);
+/* column sums: out[N] (float32) (+)= sum_m x[m, :]; bias gradient of F.linear; also sums over samples */
+int hapmi_colsum(const void *x, float *out, int64_t M, int64_t N, int64_t ldx, int accumulate, int dtype,
+                 hapmi_stream_t stream);
+int hapmi_fill_zero(void *p, int64_t bytes, hapmi_stream_t stream);
+int hapmi_cast(const void *src, int src_dtype, void *dst, int dst_dtype, int64_t n, hapmi_stream_t stream);
+
+/* F.embedding (hap.rs:2041) fused with `* scale` and `+ pe[S, d]` (models.py:79-81):
+ * out[t, :] = table[ids[t], :] * scale + pe[t % S, :]   (pe may be NULL) */
+int hapmi_embedding_fwd(const int64_t *ids, const void *table, const void *pe, void *out, int64_t n_tokens,
+                        int64_t d, int64_t S, int64_t vocab, float scale, int dtype, hapmi_stream_t stream);
+/* dtable[ids[t], :] += dout[t, :] * scale   (float32 atomics; dtable zeroed by the caller) */
+int hapmi_embedding_bwd(const int64_t *ids, const void *dout, float *dtable, int64_t n_tokens, int64_t d,
+                        int64_t vocab, float scale, int dtype, hapmi_stream_t stream);
+
+/* ---- ViT leaves -------------------------------------------------------- */
+/* F.conv2d with kernel = stride, no padding (hap.rs:1723) as patch rows for a GEMM:
+ * cols[b * gh * gw, C * ph * pw] <- x[b, C, gh*ph, gw*pw] (float32 in, `dtype` out) */
+int hapmi_patchify(const float *x, void *cols, int64_t b, int64_t C, int64_t gh, int64_t gw, int64_t ph,
+                   int64_t pw, int dtype, hapmi_stream_t stream);
+/* models.append_cls_token (models.py:443-445) fused with `+ pos_embed` (models.py:167):
+ * out[b, 0, :] = cls + pos[0]; out[b, 1 + t, :] = patches[b, t, :] + pos[1 + t] */
+int hapmi_append_cls_pos(const void *patches, const void *cls, const void *pos, void *out, int64_t b, int64_t T,
+                         int64_t d, int dtype, hapmi_stream_t stream);
+
+/* ---- MoE: models.top_2_gating (models.py:477-502) in index form --------
+ * logits[B, S, E] float32 -> probs[B, S, E] float32, index[B, S, 2] int32,
+ * slot[B, S, 2] int32 (0 = dropped, usable slots 1..C-1; a choice whose gate is exactly 0
+ * counts as dropped, as models.py:500 derives dispatch from combine > 0), gate[B, S, 2] float32,
+ * token_of_slot[B, E, C] int32 (-1 = empty). */
+int hapmi_top2_gate(const float *logits, float *probs, int32_t *index, int32_t *slot, float *gate,
+                    int32_t *token_of_slot, int64_t B, int64_t S, int64_t E, int64_t C, hapmi_stream_t stream);
+/* dlogits = softmax backward of the two kept gate gradients */
+int hapmi_top2_gate_bwd(const float *probs, const int32_t *index, const int32_t *slot, const float *dgate,
+                        float *dlogits, int64_t B, int64_t S, int64_t E, hapmi_stream_t stream);
+/* dense [B, S, E, C] tensors exactly as models.py:495-500 lays them out */
+int hapmi_top2_densify(const int32_t *index, const int32_t *slot, const float *gate, float *dispatch,
+                       float *combine, int64_t B, int64_t S, int64_t E, int64_t C, hapmi_stream_t stream);
+/* einsum "bsd,bsec->becd" with the local expert range [e_lo, e_lo + E_loc) (hap.rs:2273,
+ * models.py:356) as a row gather; expert-major output expert_in[E_loc, B, C, d] */
+int hapmi_moe_dispatch(const void *x, const int32_t *token_of_slot, void *expert_in, int64_t B, int64_t S,
+                       int64_t E, int64_t C, int64_t d, int64_t e_lo, int64_t E_loc, int dtype,
+                       hapmi_stream_t stream);
+/* einsum "becd,bsec->bsd" (models.py:364) as a weighted row gather:
+ * out[b, s, :] = sum_k gate_k * expert_out[e_k - e_lo, b, slot_k, :] over kept local choices */
+int hapmi_moe_combine(const void *expert_out, const int32_t *index, const int32_t *slot, const float *gate,
+                      void *out, int64_t B, int64_t S, int64_t C, int64_t d, int64_t e_lo, int64_t E_loc,
+                      int dtype, hapmi_stream_t stream);
+/* backward of combine: d_expert_out[e, b, c, :] = gate * dout[b, token, :] (0 for empty slots);
+ * dgate[b, s, k] = <dout[b, s, :], expert_out[e_k - e_lo, b, slot_k, :]> (0 if not kept / not local) */
+int hapmi_moe_combine_bwd(const void *dout, const void *expert_out, const int32_t *index, const int32_t *slot,
+                          const float *gate, const int32_t *token_of_slot, void *d_expert_out, float *dgate,
+                          int64_t B, int64_t S, int64_t E, int64_t C, int64_t d, int64_t e_lo, int64_t E_loc,
+                          int dtype, hapmi_stream_t stream);
+/* backward of dispatch: dx[b, s, :] (+)= sum_k d_expert_in[e_k - e_lo, b, slot_k, :] */
+int hapmi_moe_dispatch_bwd(const void *d_expert_in, const int32_t *index, const int32_t *slot, const float *gate,
+                           void *dx, int64_t B, int64_t S, int64_t C, int64_t d, int64_t e_lo, int64_t E_loc,
+                           int accumulate, int dtype, hapmi_stream_t stream);
+
+/* ---- optimizer (worker.py:47, 74-76; profiler.py:18) --------------------
+ * Flat float32 master parameters and gradients; `shadow` (bf16 copy of the
+ * updated parameters) may be NULL; `grad_scale_dev` (device float, e.g. the
+ * clipping coefficient) may be NULL. */
+int hapmi_sgd_step(float *param, const float *grad, void *shadow, int64_t n, float lr,
+                   const float *grad_scale_dev, hapmi_stream_t stream);
+int hapmi_adam_step(float *param, const float *grad, float *exp_avg, float *exp_avg_sq, void *shadow, int64_t n,
+                    float lr, float beta1, float beta2, float eps, float bias_corr1, float bias_corr2,
+                    const float *grad_scale_dev, hapmi_stream_t stream);
+/* out[0] += sum g^2 (float32 atomics over block partials; out zeroed by the caller) */
+int hapmi_sumsq(const float *g, int64_t n, float *out, hapmi_stream_t stream);
+/* torch.nn.utils.clip_grad_norm_ coefficient (worker.py:74): coef = min(1, max_norm / (sqrt(sumsq) + 1e-6)) */
+int hapmi_clip_coef(const float *sumsq, float max_norm, float *coef, hapmi_stream_t stream);
+
+/* ---- instrumentation ---------------------------------------------------
+ * When enabled, every hapmi_gemm launch is bracketed by HIP events on its own
+ * stream; hapmi_prof_gemm_collect synchronises those events and returns the
+ * summed kernel time (ms), launch count and algorithmic FLOPs since enable. */
+int hapmi_prof_gemm_enable(int on);
+int hapmi_prof_gemm_collect(double *ms_host, int64_t *launches_host, double *flops_host);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HAPMI_H */

@@ -1,0 +1,299 @@
+"""CPU restatements of the reference leaf functions.  TEST INFRASTRUCTURE ONLY.
+
+Everything here runs on the CPU with stock PyTorch / numpy and is used solely
+as the checker for the HIP path (tests/, smoke(), bench.py's cpu_baseline).
+
+Functions and the reference lines they follow:
+
+* ``sharding_round``       -- /root/reference/hap.rs:3536-3559 (C restatement in
+  oracle/sharding_round.c, loaded through ctypes).
+* ``positional_encoding``  -- /root/reference/models.py:504-509.
+* ``top_2_gating``         -- /root/reference/models.py:477-502.
+* ``JointWorld`` collectives -- /root/reference/collectives.py:6-29 (padded,
+  AllGather), 73-84 (AllReduce), 88-103 (ReduceScatter), 146-148
+  (dynamic_slice), 152-166 (AllToAll), 171-180 (Replicate).
+
+The reference's arithmetic lives in PyTorch (environment.yml pins 1.13.1); the
+oracle calls the same public PyTorch routines on the CPU.
+
+Pins (see tests/test_oracle_*.py): sharding_round -- hand-derived known
+answers + invariants; positional_encoding -- closed form at chosen points;
+top_2_gating -- hand-worked routing vector, per-token brute force, slot
+invariants; collectives -- the ones-tensor expectations the reference keeps in
+collectives.py:195-323, round-trip identities.  Tie order of equal gate
+probabilities inside torch.topk is unspecified by PyTorch: parity unpinned for
+exact ties (they do not occur for the seeded continuous inputs used).
+"""
+from __future__ import annotations
+
+import ctypes
+import math
+import os
+from typing import List, Sequence
+
+import numpy as np
+import torch
+import torch.nn.functional as F
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_liboracle = None
+
+
+def _lib():
+    global _liboracle
+    if _liboracle is None:
+        path = os.path.join(_HERE, "liboracle.so")
+        if not os.path.exists(path):
+            import subprocess
+            subprocess.check_call(["make", "-C", _HERE, "liboracle.so"])
+        _liboracle = ctypes.CDLL(path)
+        _liboracle.oracle_sharding_round.restype = ctypes.c_int
+        _liboracle.oracle_sharding_round.argtypes = [
+            ctypes.c_int64, ctypes.POINTER(ctypes.c_double), ctypes.c_int64,
+            ctypes.POINTER(ctypes.c_int64)]
+    return _liboracle
+
+
+def sharding_round(full_length: int, ratios: Sequence[float]) -> List[int]:
+    """hap.rs:3536-3559.  Returns the integer lengths (does not mutate)."""
+    n = len(ratios)
+    r = (ctypes.c_double * n)(*[float(x) for x in ratios])
+    out = (ctypes.c_int64 * n)()
+    rc = _lib().oracle_sharding_round(int(full_length), r, n, out)
+    if rc != 0:
+        raise AssertionError("truncated lengths exceed full_length (hap.rs:3543)")
+    return [int(v) for v in out]
+
+
+def positional_encoding(seqlen: int, emsize: int) -> np.ndarray:
+    """models.py:504-509: angle = pos / 10000^(2*(j//2)/emsize); even columns
+    take sin, odd columns cos; float64."""
+    pos = np.arange(seqlen, dtype=np.float64)[:, None]
+    j = np.arange(emsize)[None, :]
+    angle = pos / np.power(10000.0, 2.0 * (j // 2) / emsize)
+    out = np.empty_like(angle)
+    out[:, 0::2] = np.sin(angle[:, 0::2])
+    out[:, 1::2] = np.cos(angle[:, 1::2])
+    return out
+
+
+# --------------------------------------------------------------------------
+# top-2 gating
+# --------------------------------------------------------------------------
+
+def top_2_gating(gate_input, n_expert: int, capacity: int, gate_weight, train: bool = True):
+    """models.py:477-502, dense form: returns (dispatch, combine), each
+    [B, S, E, C]; dispatch is float32, combine carries the gate dtype."""
+    logits = gate_input @ gate_weight                                  # :478
+    probs = torch.softmax(logits, dim=2)                               # :479
+    gate, index = probs.topk(2, dim=2)                                 # :481  [B,S,2]
+    chosen = F.one_hot(index, n_expert)                                # :483  [B,S,2,E] int64
+    pos = chosen.cumsum(dim=1) * chosen                                # :485  1-based, per choice
+    first_sum = pos[:, :, 0, :].sum(dim=1, keepdim=True)               # :486  sum of positions (n(n+1)/2)
+    pos = torch.stack([pos[:, :, 0, :], pos[:, :, 1, :] + first_sum], dim=2) * chosen   # :487-488
+    fits = pos < capacity                                              # :490-491
+    kept = chosen * fits
+    pos = pos * fits
+    kept_flag = kept.sum(dim=3)                                        # :493  [B,S,2]
+    weight = (gate * kept_flag)[:, :, :, None, None]                   # :496
+    combine = (weight * F.one_hot(index, n_expert)[..., None]          # :497
+               * F.one_hot(pos, capacity)).sum(dim=2)                  # :498
+    dispatch = (combine > 0).to(torch.float32)                         # :500
+    return dispatch, combine
+
+
+def top_2_gating_sparse(logits: torch.Tensor, capacity: int):
+    """Per-token brute force over fp32 logits [B,S,E] (pure Python loops; small
+    inputs only).  Returns (index[B,S,2] int64, slot[B,S,2] int64 with 0 =
+    dropped, gate[B,S,2] float)."""
+    B, S, E = logits.shape
+    probs = torch.softmax(logits, dim=2)
+    index = torch.zeros(B, S, 2, dtype=torch.int64)
+    slot = torch.zeros(B, S, 2, dtype=torch.int64)
+    gate = torch.zeros(B, S, 2, dtype=probs.dtype)
+    for b in range(B):
+        seen0 = [0] * E
+        for s in range(S):
+            row = probs[b, s].tolist()
+            order = sorted(range(E), key=lambda e: (-row[e], e))
+            index[b, s, 0], index[b, s, 1] = order[0], order[1]
+            gate[b, s, 0], gate[b, s, 1] = probs[b, s, order[0]], probs[b, s, order[1]]
+            seen0[order[0]] += 1
+            p = seen0[order[0]]
+            slot[b, s, 0] = p if p < capacity else 0
+        offset = [n * (n + 1) // 2 for n in seen0]
+        seen1 = [0] * E
+        for s in range(S):
+            e = int(index[b, s, 1])
+            seen1[e] += 1
+            p = seen1[e] + offset[e]
+            slot[b, s, 1] = p if p < capacity else 0
+    return index, slot, gate
+
+
+def densify(index, slot, gate, n_expert: int, capacity: int):
+    """Sparse routing -> dense (dispatch, combine) as the reference lays them out."""
+    B, S, _ = index.shape
+    combine = torch.zeros(B, S, n_expert, capacity, dtype=gate.dtype)
+    for b in range(B):
+        for s in range(S):
+            for k in range(2):
+                c = int(slot[b, s, k])
+                if c > 0:
+                    combine[b, s, int(index[b, s, k]), c] += gate[b, s, k]
+    return (combine > 0).to(torch.float32), combine
+
+
+# --------------------------------------------------------------------------
+# uneven collectives over an in-memory world of W ranks
+# --------------------------------------------------------------------------
+
+def _padded(t: torch.Tensor, dim: int, length: int) -> torch.Tensor:
+    """collectives.py:9-12.  The reference leaves the tail uninitialised
+    (torch.empty); the oracle poisons it with NaN so that any read of it shows."""
+    if t.shape[dim] == length:
+        return t
+    shape = list(t.shape)
+    shape[dim] = length - t.shape[dim]
+    tail = torch.full(shape, float("nan"), dtype=t.dtype)
+    return torch.cat([t, tail], dim=dim)
+
+
+def _accumulate(parts: Sequence[torch.Tensor]) -> torch.Tensor:
+    """Elementwise sum over ranks in rank order with float32 accumulation."""
+    acc = parts[0].float().clone()
+    for p in parts[1:]:
+        acc = acc + p.float()
+    return acc.to(parts[0].dtype)
+
+
+class JointWorld:
+    """All W ranks of the SPMD program live in one process; each collective is
+    one autograd node over the W per-rank tensors, so one backward pass yields
+    every rank's gradients.  ``log[(tag, 'fwd'|'bwd')]`` records what went over
+    the wire: ``log[key][src][dst]`` is the message rank ``src`` sent to ``dst``."""
+
+    def __init__(self, world_size: int):
+        self.W = world_size
+        self.log = {}
+
+    # -- all_gather: collectives.py:14-29 --------------------------------
+    def all_gather(self, tag, xs, dim, L):
+        world = self
+
+        class Fn(torch.autograd.Function):
+            @staticmethod
+            def forward(ctx, *xs):
+                m = max(L)
+                sent = [_padded(x, dim, m).contiguous() for x in xs]                    # :19
+                world.log[(tag, "fwd")] = [[sent[src] for _ in range(world.W)] for src in range(world.W)]
+                out = torch.cat([s.split([l, m - l], dim=dim)[0] for s, l in zip(sent, L)], dim=dim)  # :20
+                return tuple(out.clone() for _ in range(world.W))
+
+            @staticmethod
+            def backward(ctx, *gs):
+                m = max(L)
+                sent = [[_padded(p, dim, m).contiguous() for p in torch.split(g.contiguous(), L, dim=dim)]
+                        for g in gs]                                                       # :24-25
+                world.log[(tag, "bwd")] = sent
+                outs = []
+                for r in range(world.W):
+                    red = _accumulate([sent[src][r] for src in range(world.W)])            # :27
+                    outs.append(red.split([L[r], m - L[r]], dim=dim)[0])                   # :28
+                return tuple(outs)
+
+        return list(Fn.apply(*xs))
+
+    # -- reduce_scatter: collectives.py:88-103 ---------------------------
+    def reduce_scatter(self, tag, xs, dim, L):
+        world = self
+
+        class Fn(torch.autograd.Function):
+            @staticmethod
+            def forward(ctx, *xs):
+                m = max(L)
+                sent = [[_padded(p, dim, m).contiguous() for p in torch.split(x.contiguous(), L, dim=dim)]
+                        for x in xs]                                                       # :92-93
+                world.log[(tag, "fwd")] = sent
+                outs = []
+                for r in range(world.W):
+                    red = _accumulate([sent[src][r] for src in range(world.W)])            # :95
+                    outs.append(red.split([L[r], m - L[r]], dim=dim)[0].clone())           # :96
+                return tuple(outs)
+
+            @staticmethod
+            def backward(ctx, *gs):
+                m = max(L)
+                sent = [_padded(g.contiguous(), dim, m).contiguous() for g in gs]          # :101
+                world.log[(tag, "bwd")] = [[sent[src] for _ in range(world.W)] for src in range(world.W)]
+                grad = torch.cat([s.split([l, m - l], dim=dim)[0] for s, l in zip(sent, L)], dim=dim)  # :102
+                return tuple(grad.clone() for _ in range(world.W))
+
+        return list(Fn.apply(*xs))
+
+    # -- all_to_all: collectives.py:152-166 ------------------------------
+    def all_to_all(self, tag, xs, split_dim, cat_dim, split_L, cat_L):
+        world = self
+
+        class Fn(torch.autograd.Function):
+            @staticmethod
+            def forward(ctx, *xs):
+                sent = [[p.contiguous() for p in torch.split(x.contiguous(), split_L, dim=split_dim)]
+                        for x in xs]                                                       # :156-158
+                world.log[(tag, "fwd")] = sent
+                return tuple(torch.cat([sent[src][r] for src in range(world.W)], dim=cat_dim)  # :159
+                             for r in range(world.W))
+
+            @staticmethod
+            def backward(ctx, *gs):
+                sent = [[p.contiguous() for p in torch.split(g.contiguous(), cat_L, dim=cat_dim)]
+                        for g in gs]                                                       # :163-165
+                world.log[(tag, "bwd")] = sent
+                return tuple(torch.cat([sent[src][r] for src in range(world.W)], dim=split_dim)  # :166
+                             for r in range(world.W))
+
+        return list(Fn.apply(*xs))
+
+    # -- all_reduce: collectives.py:73-84 --------------------------------
+    def all_reduce(self, tag, xs):
+        world = self
+
+        class Fn(torch.autograd.Function):
+            @staticmethod
+            def forward(ctx, *xs):
+                sent = [x.contiguous() for x in xs]
+                world.log[(tag, "fwd")] = [[sent[src] for _ in range(world.W)] for src in range(world.W)]
+                total = _accumulate(sent)
+                return tuple(total.clone() for _ in range(world.W))
+
+            @staticmethod
+            def backward(ctx, *gs):
+                sent = [g.clone() for g in gs]
+                world.log[(tag, "bwd")] = [[sent[src] for _ in range(world.W)] for src in range(world.W)]
+                total = _accumulate(sent)
+                return tuple(total.clone() for _ in range(world.W))
+
+        return list(Fn.apply(*xs))
+
+    # -- replicate: collectives.py:171-180 -------------------------------
+    def replicate(self, tag, xs):
+        world = self
+
+        class Fn(torch.autograd.Function):
+            @staticmethod
+            def forward(ctx, *xs):
+                return tuple(x.view_as(x) for x in xs)
+
+            @staticmethod
+            def backward(ctx, *gs):
+                sent = [g.contiguous() for g in gs]
+                world.log[(tag, "bwd")] = [[sent[src] for _ in range(world.W)] for src in range(world.W)]
+                total = _accumulate(sent)
+                return tuple(total.clone() for _ in range(world.W))
+
+        return list(Fn.apply(*xs))
+
+    # -- dynamic_slice: collectives.py:146-148 (local, no wire) ----------
+    @staticmethod
+    def dynamic_slice(x, dim, L, rank):
+        return torch.split(x, L, dim=dim)[rank].contiguous()

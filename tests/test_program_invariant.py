@@ -1,0 +1,88 @@
+"""Pins the program generator: the sum over ranks of the per-rank partial losses and gradients of the SPMD
+program equals the unsharded model built from stock torch.nn (models.py:65-88, 90-118, 147-177, 301-366),
+all on the CPU in float32."""
+import copy
+
+import pytest
+import torch
+
+from helpers import (RATIOS4, RATIOS_E, joint_cpu, lm_batch, make_lm, make_moe, make_vit, rel_err, vit_batch)
+from oracle import single_device
+import hap_amd
+
+
+def _single(model, x, y):
+    m = copy.deepcopy(model)
+    m.train()
+    loss = single_device.forward(m, x, y)
+    loss.backward()
+    return loss.detach(), dict(m.named_parameters())
+
+
+def _check(model, run, x, y, sharded):
+    loss1, p1 = _single(model, x, y)
+    losses = run.step(x, y)
+    torch.testing.assert_close(sum(l.double() for l in losses).float(), loss1, rtol=1e-5, atol=1e-5)
+    W = run.W
+    for name, ref_p in p1.items():
+        if ref_p.grad is None:
+            continue
+        held = [dict(p.named_parameters()).get(name) for p in run.programs]
+        if any(h is None or h.grad is None for h in held):
+            assert ".norm" in name, name       # LayerNorm affine parameters are never read by the program
+            continue
+        grads = [h.grad for h in held]
+        if name in sharded:
+            dim, L = sharded[name]
+            want = torch.split(ref_p.grad, L, dim)
+            for r in range(W):
+                assert rel_err(grads[r], want[r]) < 2e-5, (name, r)
+        else:
+            for r in range(W):                 # replicate.backward all-reduces: every rank holds the full gradient
+                assert rel_err(grads[r], ref_p.grad) < 2e-5, (name, r)
+
+
+@pytest.mark.parametrize("ffn", ["column", "batch"])
+def test_lm_spmd_equals_single_device(ffn):
+    model = make_lm()
+    B = 8
+    x, y = lm_batch(B, 16, 97)
+    run = joint_cpu(model, RATIOS4, B, ffn=ffn)
+    L_F = hap_amd.sharding_lengths(64, RATIOS4)
+    sharded = {}
+    if ffn == "column":
+        for i in range(2):
+            sharded[f"layers.{i}.linear1.weight"] = (0, L_F)
+            sharded[f"layers.{i}.linear1.bias"] = (0, L_F)
+    _check(model, run, x, y, sharded)
+
+
+def test_mlm_targets_with_ignore_index():
+    model = make_lm(causal=False)
+    x, y = lm_batch(8, 16, 97, mlm=True)
+    _check(model, joint_cpu(model, RATIOS4, 8), x, y, {
+        f"layers.{i}.linear1.{k}": (0, hap_amd.sharding_lengths(64, RATIOS4)) for i in range(2) for k in ("weight", "bias")})
+
+
+def test_vit_spmd_equals_single_device():
+    model = make_vit()
+    x, y = vit_batch(8, 16, 10)
+    _check(model, joint_cpu(model, RATIOS4, 8, ffn="batch"), x, y, {})
+
+
+@pytest.mark.parametrize("batch_sharded", [True, False])
+def test_moe_spmd_equals_single_device(batch_sharded):
+    model = make_moe()
+    B = 16 if batch_sharded else 4
+    x, y = lm_batch(B, 16, 61)
+    L_E = hap_amd.sharding_lengths(8, RATIOS_E)
+    run = joint_cpu(model, RATIOS_E, B, ffn="batch", batch_sharded=batch_sharded)
+    sharded = {"layers.1.w1": (0, L_E), "layers.1.w2": (0, L_E)}
+    if not batch_sharded:
+        # every rank computes the whole batch: the W partial losses are W copies of the full loss
+        loss1, _ = _single(model, x, y)
+        losses = run.forward(x, y)
+        for l in losses:
+            torch.testing.assert_close(l, loss1, rtol=1e-5, atol=1e-5)
+        return
+    _check(model, run, x, y, sharded)
