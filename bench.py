@@ -1,0 +1,222 @@
+#!/usr/bin/env python3
+"""Throughput of one GPU's uneven shard: fwd + bwd + optimizer step of the generated SPMD program.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload bert|lm|vit|moe|ragged]
+
+Default workload (N = 1): BASELINE config 2 -- BERT-large-style encoder, bf16 compute with float32 master
+weights, 24 layers, d 1024, 16 heads, FFN 4096 column-split to a local 1536 slice, seq 512, local batch 12
+of 32, vocab 30522, 15 % masked-LM targets, Adam.  Inputs are synthetic (seeded), resident in HBM before the
+timed region; the peers' halves of the collectives come from a seeded synthetic wire.
+Prints ONE JSON line.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+RATIOS = [.375, .375, .125, .125]
+RATIOS_E = [.3125, .3125, .1875, .1875]
+PEAK = {"bf16": 2500.0, "fp32": 157.3}        # dense MFMA TFLOP/s, MI355X
+HBM_PEAK = 8000.0                              # GB/s
+
+WORKLOADS = {
+    # name: (description, dtype)
+    "bert": ("BERT-large uneven shard: 24L d1024 h16 FFN 1536/4096 seq512 batch 12/32 vocab30522 MLM Adam", "bf16"),
+    "lm": ("2-layer post-LN LM: d512 h8 FFN 768/2048 seq128 batch 3/8 vocab33280 SGD", "fp32"),
+    "vit": ("ViT-L/16: 24L d1024 h16 FFN4096 197 tokens batch 48/128 1000 classes Adam", "bf16"),
+    "moe": ("MoE LM: 12L d768 h12 16 experts (5 local) top-2 C=80 seq512 batch 16 vocab33280 Adam", "bf16"),
+}
+
+
+def build_workload(name, layers_override=None):
+    import torch
+    import hap_amd
+    from hap_amd import models
+    g = torch.Generator().manual_seed(39)
+    if name == "bert":
+        L = layers_override or 24
+        B, S, V = 32, 512, 30522
+        model = models.RTransformer(V, S, 1024, 16, 4096, 0.0, nlayers=L, causal=False)
+        x = torch.randint(0, V, (B, S), generator=g)
+        masked = torch.rand(B, S, generator=g) < 0.15
+        y = torch.where(masked, x, torch.full_like(x, -100))
+        plan = hap_amd.ShardingPlan([RATIOS], 0, ffn="column")
+        meta = dict(local_batch=12, global_batch=B, seq_len=S, opt=dict(kind="adam", lr=5e-4), batch_sharded=True,
+                    ratios=RATIOS)
+    elif name == "lm":
+        L = layers_override or 2
+        B, S, V = 8, 128, 33280
+        model = models.RTransformer(V, S, 512, 8, 2048, 0.0, nlayers=L, causal=True)
+        ids = torch.randint(0, V, (B, S + 1), generator=g)
+        x, y = ids[:, :-1].contiguous(), ids[:, 1:].contiguous()
+        plan = hap_amd.ShardingPlan([RATIOS], 0, ffn="column")
+        meta = dict(local_batch=3, global_batch=B, seq_len=S, opt=dict(kind="sgd", lr=1e-3), batch_sharded=True,
+                    ratios=RATIOS)
+    elif name == "vit":
+        L = layers_override or 24
+        B = 128
+        model = models.VTransformer(1000, 196, 1024, 16, 4096, 0.0, nlayers=L, img_size=(224, 224), patch_size=(16, 16))
+        x = torch.randn(B, 3, 224, 224, generator=g)
+        y = torch.randint(0, 1000, (B,), generator=g)
+        plan = hap_amd.ShardingPlan([RATIOS], 0, ffn="batch")
+        meta = dict(local_batch=48, global_batch=B, seq_len=197, opt=dict(kind="adam", lr=5e-4), batch_sharded=True,
+                    ratios=RATIOS)
+    elif name == "moe":
+        L = layers_override or 12
+        B, S, V = 16, 512, 33280
+        model = models.RMoE(V, S, 768, 12, 3072, 0.0, 16, 80, L, causal=True)
+        ids = torch.randint(0, V, (B, S + 1), generator=g)
+        x, y = ids[:, :-1].contiguous(), ids[:, 1:].contiguous()
+        plan = hap_amd.ShardingPlan([RATIOS_E], 0, ffn="batch")
+        meta = dict(local_batch=16, global_batch=B, seq_len=S, opt=dict(kind="adam", lr=5e-4), batch_sharded=False,
+                    ratios=RATIOS_E)
+    else:
+        raise SystemExit(f"unknown workload {name}")
+    models.init_normal_(model, 0.02, 39)
+    gm = hap_amd.build_program(model, plan, meta["global_batch"], batch_sharded=meta["batch_sharded"])
+    return gm, x, y, meta
+
+
+def cpu_baseline(name, meta, budget_s=25.0):
+    """The CPU oracle (stock PyTorch eager + autograd + torch.optim on the same generated graph, float32 as in
+    the reference) timed on this host for a bounded sample: the same shard with 1 and 2 layers, extrapolated
+    linearly to the full depth."""
+    import torch
+    from oracle.cpu_executor import PeerlessCPURun
+    cores = os.cpu_count() or 1
+    cores = min(cores, 16)
+    torch.set_num_threads(cores)
+    full_layers = {"bert": 24, "lm": 2, "vit": 24, "moe": 12}[name]
+    sample_layers = [2] if name in ("lm",) else ([2, 4] if name == "moe" else [1, 2])
+    times = {}
+    for L in sample_layers:
+        gm, x, y, _ = build_workload(name, layers_override=L)
+        run = PeerlessCPURun(gm, 0, "fp32")
+        o = meta["opt"]
+        opt = (torch.optim.Adam if o["kind"] == "adam" else torch.optim.SGD)(gm.parameters(), lr=o["lr"])
+        run.step(x, y, [opt])                     # warm-up
+        t0 = time.perf_counter()
+        n = 0
+        while n < 2 or (time.perf_counter() - t0 < budget_s / (2 * len(sample_layers)) and n < 5):
+            run.step(x, y, [opt])
+            n += 1
+        times[L] = (time.perf_counter() - t0) / n
+    if len(times) == 2:
+        a, b = sample_layers
+        per_layer = (times[b] - times[a]) / (b - a)
+        t_full = times[a] + per_layer * (full_layers - a)
+        sample = (f"fp32 CPU oracle, same shard at {a} and {b} layers ({times[a]:.2f}s, {times[b]:.2f}s per step), "
+                  f"extrapolated linearly to {full_layers} layers")
+    else:
+        t_full = times[sample_layers[0]]
+        sample = f"fp32 CPU oracle, full workload, {t_full:.3f}s per step"
+    return dict(value=meta["local_batch"] / t_full, unit="samples/s", cores=cores, kind="port", sample=sample)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="bert", choices=list(WORKLOADS) + ["ragged"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--graph", action="store_true", help="replay the step from a captured HIP graph")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        raise SystemExit("bench.py: this build executes ONE device's shard; no collective crosses the device, "
+                         "so only --gpus 1 is measured")
+    if args.workload == "ragged":
+        from hap_amd import ragged_bench
+        print(json.dumps(ragged_bench.run(args.steps, args.warmup, not args.no_cpu_baseline)))
+        return
+
+    import torch
+    import hap_amd
+    from hap_amd import ops
+    from hap_amd._lib import lib
+
+    desc, dtype = WORKLOADS[args.workload]
+    gm, x, y, meta = build_workload(args.workload)
+    wire = hap_amd.SyntheticWire(seed=39, scale=1.0, grad_scale=1e-3, share_shapes=True)
+    ex = hap_amd.compile_program(gm, [x, y], dtype=dtype, wire=wire, rank=0, world_size=len(meta["ratios"]))
+    ex.configure_optimizer(**meta["opt"])
+    ex.load_inputs(x, y)                              # inputs resident in HBM before the timed region
+    torch.cuda.synchronize()
+
+    def one_step():
+        ex.forward()
+        ex.backward()
+        ex.step()
+
+    graph = None
+    for _ in range(args.warmup):
+        one_step()
+    torch.cuda.synchronize()
+    if args.graph:
+        graph = torch.cuda.CUDAGraph()
+        side = torch.cuda.Stream()
+        with torch.cuda.stream(side):
+            one_step()
+            torch.cuda.synchronize()
+            with torch.cuda.graph(graph, stream=side):
+                one_step()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+
+    lib().hapmi_prof_gemm_enable(0 if graph is not None else 1)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        if graph is not None:
+            graph.replay()
+        else:
+            one_step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    loss = float(ex.loss[0].item())
+
+    import ctypes
+    ms, n_launch, flops = ctypes.c_double(), ctypes.c_int64(), ctypes.c_double()
+    if graph is None:
+        lib().hapmi_prof_gemm_collect(ctypes.byref(ms), ctypes.byref(n_launch), ctypes.byref(flops))
+        lib().hapmi_prof_gemm_enable(0)
+    else:
+        # kernel durations cannot be bracketed inside a replayed graph: profile the same launches eagerly
+        lib().hapmi_prof_gemm_enable(1)
+        for _ in range(3):
+            one_step()
+        torch.cuda.synchronize()
+        lib().hapmi_prof_gemm_collect(ctypes.byref(ms), ctypes.byref(n_launch), ctypes.byref(flops))
+        lib().hapmi_prof_gemm_enable(0)
+    achieved = flops.value / (ms.value * 1e-3) / 1e12 if ms.value > 0 else 0.0
+    peak = PEAK[dtype]
+    ms_per_step = dt / args.steps * 1e3
+    result = {
+        "metric": "samples/sec of one GPU's uneven shard (fwd+bwd+step)",
+        "value": meta["local_batch"] * args.steps / dt,
+        "unit": "samples/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": dtype, "data": "synthetic",
+        "config": {"workload": desc, "local_batch": meta["local_batch"], "global_batch": meta["global_batch"],
+                   "seq_len": meta["seq_len"], "launch": "hip-graph" if graph is not None else "eager",
+                   "final_loss": loss},
+        "roofline": {"bound": "mfma", "kernel": "gemm_kernel (all GEMM launches of the step)",
+                     "achieved": achieved, "peak": peak, "unit": "TFLOP/s", "frac": achieved / peak,
+                     "launches_per_step": n_launch.value / max(1, args.steps if graph is None else 3),
+                     "gemm_ms_per_step": ms.value / max(1, args.steps if graph is None else 3), "traffic": None},
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(args.workload, meta)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -34,16 +34,47 @@ class GemmArgs(ctypes.Structure):
     ]
 
 
+_HEADER = os.path.join(_HERE, "..", "include", "hapmi.h")
+_SCALARS = {"int64_t": ctypes.c_int64, "int": ctypes.c_int, "float": ctypes.c_float, "double": ctypes.c_double,
+            "hapmi_stream_t": ctypes.c_void_p}
+
+
+def _prototypes():
+    """(name, [ctypes argument types]) for every ``int hapmi_*(...)`` declared in include/hapmi.h.  Without
+    explicit argument types ctypes would pass Python ints as 32-bit C ints, which is wrong for the int64_t
+    parameters (those that travel on the stack keep garbage in their upper half)."""
+    import re
+    text = open(_HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    out = []
+    for m in re.finditer(r"\bint\s+(hapmi_[a-z0-9_]+)\s*\(([^)]*)\)\s*;", text):
+        name, params = m.group(1), m.group(2).strip()
+        types = []
+        if params and params != "void":
+            for prm in params.split(","):
+                prm = " ".join(prm.split())
+                if "*" in prm:
+                    types.append(ctypes.c_void_p)
+                else:
+                    base = prm.rsplit(" ", 1)[0].replace("const ", "").strip()
+                    types.append(_SCALARS[base])
+        out.append((name, types))
+    return out
+
+
 def lib() -> ctypes.CDLL:
     global _lib
     if _lib is None:
         if not os.path.exists(_PATH):
             raise HapmiError(f"{_PATH} is missing: build it with `python -m hap_amd.build` "
                              "(there is no fallback path)")
-        _lib = ctypes.CDLL(_PATH)
-        _lib.hapmi_last_error.restype = ctypes.c_char_p
-        _lib.hapmi_sharding_round.argtypes = [ctypes.c_int64, ctypes.POINTER(ctypes.c_double), ctypes.c_int64,
-                                              ctypes.POINTER(ctypes.c_int64)]
+        handle = ctypes.CDLL(_PATH)
+        handle.hapmi_last_error.restype = ctypes.c_char_p
+        for name, types in _prototypes():
+            fn = getattr(handle, name)
+            fn.argtypes = types
+            fn.restype = ctypes.c_int
+        _lib = handle
     return _lib
 
 

@@ -51,6 +51,7 @@ __global__ __launch_bounds__(GATE_THREADS) void top2_gate_kernel(const float *lo
                             p1 = pe; i1 = e;
                         }
                     }
+                    if (i1 < 0) i1 = (i0 + 1) % E;      // only with NaN logits; gate stays -1, so the choice is dropped
                     index[tok * 2 + 0] = i0;
                     index[tok * 2 + 1] = i1;
                     gate[tok * 2 + 0] = p0;
@@ -140,7 +141,7 @@ __global__ __launch_bounds__(256) void moe_dispatch_kernel(const T *x, const int
     const int el = (int)(row / ((int64_t)C * B));
     const int tok = token_of_slot[((int64_t)b * E + e_lo + el) * C + c];
     Vec16<T> *dst = (Vec16<T> *)(expert_in + row * d);
-    if (tok >= 0) {
+    if (tok >= 0 && tok < S) {
         const Vec16<T> *src = (const Vec16<T> *)(x + ((int64_t)b * S + tok) * d);
         for (int i = lane; i < d / EPV; i += 64) dst[i] = src[i];
     } else {
@@ -166,7 +167,7 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const T *src, const in
 #pragma unroll
     for (int k = 0; k < 2; ++k) {
         const int e = index[tok * 2 + k] - e_lo, sl = slot[tok * 2 + k];
-        if (sl > 0 && e >= 0 && e < E_loc) {
+        if (sl > 0 && sl < C && e >= 0 && e < E_loc) {
             rows[k] = (const Vec16<T> *)(src + (((int64_t)e * B + b) * C + sl) * d);
             w[k] = WEIGHTED ? gate[tok * 2 + k] : 1.0f;
         }
@@ -212,7 +213,7 @@ __global__ __launch_bounds__(256) void moe_combine_bwd_rows_kernel(const T *dout
     Vec16<T> *dst = (Vec16<T> *)(d_expert_out + row * d);
     float w = 0.f;
     const Vec16<T> *src = nullptr;
-    if (tok >= 0) {
+    if (tok >= 0 && tok < S) {
         const int64_t t = (int64_t)b * S + tok;
         w = (index[t * 2] == e_lo + el) ? gate[t * 2] : gate[t * 2 + 1];
         src = (const Vec16<T> *)(dout + t * d);
@@ -246,7 +247,7 @@ __global__ __launch_bounds__(256) void moe_combine_bwd_gate_kernel(const T *dout
     for (int k = 0; k < 2; ++k) {
         const int e = index[tok * 2 + k] - e_lo, sl = slot[tok * 2 + k];
         float acc = 0.f;
-        if (sl > 0 && e >= 0 && e < E_loc) {
+        if (sl > 0 && sl < C && e >= 0 && e < E_loc) {
             const Vec16<T> *r = (const Vec16<T> *)(expert_out + (((int64_t)e * B + b) * C + sl) * d);
             for (int i = lane; i < d / EPV; i += 64) {
                 const Vec16<T> a = g[i], v = r[i];

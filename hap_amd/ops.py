@@ -52,6 +52,22 @@ def init():
     check(lib().hapmi_init())
 
 
+def _need(t: Optional[torch.Tensor], n_elems: int, what: str, offset: int = 0):
+    """Host-side bounds check: the kernel will touch elements [offset, offset + n_elems) of ``t``."""
+    if t is None:
+        return
+    if offset < 0 or n_elems < 0 or offset + n_elems > t.numel():
+        raise _lib.HapmiError(f"{what}: the kernel would access elements [{offset}, {offset + n_elems}) of a buffer "
+                              f"that holds {t.numel()}")
+    if not t.is_contiguous():
+        raise _lib.HapmiError(f"{what}: buffer must be contiguous")
+
+
+def _span(rows: int, cols: int, ld: int) -> int:
+    """Elements spanned by a [rows, cols] block with row stride ld."""
+    return 0 if rows <= 0 or cols <= 0 else (rows - 1) * ld + cols
+
+
 # ---------------------------------------------------------------------------
 # layout helpers: a tensor sharded on `dim` is [outer, len, inner]
 # ---------------------------------------------------------------------------
@@ -77,6 +93,9 @@ def pad_rows(src: torch.Tensor, dim: int, padded_len: int, out: Optional[torch.T
     outer, length, inner = _oli(src.shape, dim)
     if out is None:
         out = torch.empty(_with_dim(src.shape, dim, padded_len), dtype=src.dtype, device=src.device)
+    _need(out, outer * padded_len * inner, "pad_rows dst")
+    if out.dtype != src.dtype:
+        raise TypeError("pad_rows: dtype mismatch")
     check(lib().hapmi_pad_rows(_ptr(src), _ptr(out), outer, length, padded_len, inner * src.element_size(), _stream()))
     return out
 
@@ -88,6 +107,13 @@ def unpad_concat(slices: Sequence[torch.Tensor], lengths: Sequence[int], dim: in
     outer, padded_len, inner = _oli(ref.shape, dim)
     if out is None:
         out = torch.empty(_with_dim(ref.shape, dim, sum(lengths)), dtype=ref.dtype, device=ref.device)
+    for sl in slices:
+        _need(sl, outer * padded_len * inner, "unpad_concat slice")
+        if sl.dtype != ref.dtype:
+            raise TypeError("unpad_concat: dtype mismatch")
+    _need(out, outer * sum(lengths) * inner, "unpad_concat dst")
+    if out.numel() == 0:
+        return out
     check(lib().hapmi_unpad_concat(_ptrs(slices), _i64(lengths), len(lengths), _ptr(out), outer, padded_len,
                                    inner * ref.element_size(), _stream()))
     return out
@@ -101,6 +127,11 @@ def split_pad(src: torch.Tensor, lengths: Sequence[int], dim: int, padded_len: i
     assert total == sum(lengths)
     if outs is None:
         outs = [torch.empty(_with_dim(src.shape, dim, padded_len), dtype=src.dtype, device=src.device) for _ in lengths]
+    for o in outs:
+        _dev(o)
+        _need(o, outer * padded_len * inner, "split_pad slice")
+    if src.numel() == 0:
+        return list(outs)
     check(lib().hapmi_split_pad(_ptr(src), _ptrs(outs), _i64(lengths), len(lengths), outer, padded_len,
                                 inner * src.element_size(), _stream()))
     return list(outs)
@@ -112,6 +143,9 @@ def slice_rows(src: torch.Tensor, dim: int, offset: int, length: int, out: Optio
     outer, src_len, inner = _oli(src.shape, dim)
     if out is None:
         out = torch.empty(_with_dim(src.shape, dim, length), dtype=src.dtype, device=src.device)
+    _need(out, outer * length * inner, "slice_rows dst")
+    if out.numel() == 0:
+        return out
     check(lib().hapmi_slice_rows(_ptr(src), _ptr(out), outer, src_len, offset, length, inner * src.element_size(), _stream()))
     return out
 
@@ -119,6 +153,11 @@ def slice_rows(src: torch.Tensor, dim: int, offset: int, length: int, out: Optio
 def place_rows(src: torch.Tensor, dst: torch.Tensor, dim: int, offset: int) -> torch.Tensor:
     _dev(src, dst)
     outer, length, inner = _oli(src.shape, dim)
+    o2, dst_len, i2 = _oli(dst.shape, dim)
+    if (o2, i2) != (outer, inner) or not src.is_contiguous() or not dst.is_contiguous() or src.dtype != dst.dtype:
+        raise _lib.HapmiError("place_rows: source and destination do not agree outside the sliced dimension")
+    if src.numel() == 0:
+        return dst
     check(lib().hapmi_place_rows(_ptr(src), _ptr(dst), outer, dst.shape[dim], offset, length,
                                  inner * src.element_size(), _stream()))
     return dst
@@ -132,6 +171,12 @@ def split_rows(src: torch.Tensor, lengths: Sequence[int], dim: int,
     assert total == sum(lengths)
     if outs is None:
         outs = [torch.empty(_with_dim(src.shape, dim, l), dtype=src.dtype, device=src.device) for l in lengths]
+    for o, l in zip(outs, lengths):
+        if o is not None:
+            _dev(o)
+            _need(o, outer * l * inner, "split_rows piece")
+    if src.numel() == 0:
+        return list(outs)
     check(lib().hapmi_split_rows(_ptr(src), _ptrs(outs), _i64(lengths), len(lengths), outer,
                                  inner * src.element_size(), _stream()))
     return list(outs)
@@ -145,8 +190,15 @@ def concat_rows(pieces: Sequence[torch.Tensor], dim: int, out: Optional[torch.Te
     outer, _, inner = _oli(ref.shape, dim)
     if out is None:
         out = torch.empty(_with_dim(ref.shape, dim, sum(lengths)), dtype=ref.dtype, device=ref.device)
+    for p_, l in zip(pieces, lengths):
+        _need(p_, outer * l * inner, "concat_rows piece")
+        if p_.dtype != ref.dtype:
+            raise TypeError("concat_rows: dtype mismatch")
+    _need(out, outer * sum(lengths) * inner, "concat_rows dst")
+    if out.numel() == 0:
+        return out
     check(lib().hapmi_concat_rows(_ptrs(pieces), _i64(lengths), len(lengths), _ptr(out), outer,
-                                  inner * ref.element_size(), _ACT[act], dtype_code(ref), _stream()))
+                                  inner * ref.element_size(), _ACT[act], dtype_code(ref) if _ACT[act] else 0, _stream()))
     return out
 
 
@@ -158,6 +210,15 @@ def ragged_reduce(contribs: Sequence[torch.Tensor], dim: int, offset: int, lengt
     outer, src_len, inner = _oli(ref.shape, dim)
     if out is None:
         out = torch.empty(_with_dim(ref.shape, dim, length), dtype=ref.dtype, device=ref.device)
+    for c in contribs:
+        _need(c, outer * src_len * inner, "ragged_reduce contribution")
+        if c.dtype != ref.dtype:
+            raise TypeError("ragged_reduce: dtype mismatch")
+    _need(out, outer * length * inner, "ragged_reduce dst")
+    if out.dtype != ref.dtype:
+        raise TypeError("ragged_reduce: dtype mismatch")
+    if out.numel() == 0:
+        return out
     check(lib().hapmi_ragged_reduce(_ptrs(contribs), len(contribs), _ptr(out), outer, src_len, offset, length, inner,
                                     dtype_code(ref), _stream()))
     return out
@@ -193,6 +254,13 @@ def gemm(A: torch.Tensor, B: torch.Tensor, C: torch.Tensor, M: int, N: int, K: i
     a.strideA1, a.strideA2 = strideA
     a.strideB1, a.strideB2 = strideB
     a.strideC1, a.strideC2 = strideC
+    zb = lambda st: (batch1 - 1) * st[0] + (batch2 - 1) * st[1]
+    _need(A, _span(K if transA else M, M if transA else K, a.lda) + zb(strideA), "gemm A", offA)
+    _need(B, _span(N if transB else K, K if transB else N, a.ldb) + zb(strideB), "gemm B", offB)
+    _need(C, _span(M, N, a.ldc) + zb(strideC), "gemm C", offC)
+    _need(bias, N, "gemm bias")
+    if min(strideA + strideB + strideC) < 0:
+        raise _lib.HapmiError("gemm: negative batch stride")
     check(lib().hapmi_gemm(ctypes.byref(a), _stream()))
     return C
 
@@ -215,6 +283,11 @@ def add_layernorm_fwd(x, res, y, rstd, eps=1e-5):
     _dev(x, res, y, rstd)
     width = x.shape[-1]
     rows = x.numel() // width
+    for t_ in (x, res, y):
+        _need(t_, rows * width, "add_layernorm_fwd")
+        if t_ is not None and t_.dtype != x.dtype:
+            raise TypeError("add_layernorm_fwd: dtype mismatch")
+    _need(rstd, rows, "add_layernorm_fwd rstd")
     check(lib().hapmi_add_layernorm_fwd(_ptr(x), _ptr(res), _ptr(y), _ptr(rstd), rows, width,
                                         ctypes.c_float(eps), dtype_code(x), _stream()))
 
@@ -223,17 +296,31 @@ def layernorm_bwd(dy, y, rstd, dx_add, dx):
     _dev(dy, y, rstd, dx_add, dx)
     width = y.shape[-1]
     rows = y.numel() // width
+    for t_ in (dy, y, dx_add, dx):
+        _need(t_, rows * width, "layernorm_bwd")
+        if t_ is not None and t_.dtype != y.dtype:
+            raise TypeError("layernorm_bwd: dtype mismatch")
+    _need(rstd, rows, "layernorm_bwd rstd")
     check(lib().hapmi_layernorm_bwd(_ptr(dy), _ptr(y), _ptr(rstd), _ptr(dx_add), _ptr(dx), rows, width,
                                     dtype_code(y), _stream()))
 
 
 def softmax_fwd(x, mask, p, rows, width, ld, mask_rows=1):
     _dev(x, mask, p)
+    _need(x, _span(rows, width, ld), "softmax_fwd x")
+    _need(p, _span(rows, width, ld), "softmax_fwd p")
+    _need(mask, mask_rows * width, "softmax_fwd mask")
+    if p.dtype != x.dtype or (mask is not None and mask.dtype != torch.float32):
+        raise TypeError("softmax_fwd: dtype mismatch")
     check(lib().hapmi_softmax_fwd(_ptr(x), _ptr(mask), _ptr(p), rows, width, ld, mask_rows, dtype_code(x), _stream()))
 
 
 def softmax_bwd(dp, p, ds, rows, width, ld):
     _dev(dp, p, ds)
+    for t_ in (dp, p, ds):
+        _need(t_, _span(rows, width, ld), "softmax_bwd")
+        if t_.dtype != p.dtype:
+            raise TypeError("softmax_bwd: dtype mismatch")
     check(lib().hapmi_softmax_bwd(_ptr(dp), _ptr(p), _ptr(ds), rows, width, ld, dtype_code(p), _stream()))
 
 
@@ -241,12 +328,20 @@ def logsoftmax_nll(logits, targets, row_loss, dlogits, rows, width, ld, ignore_i
     _dev(logits, targets, row_loss, dlogits)
     if targets.dtype != torch.int64:
         raise TypeError("targets must be int64")
+    _need(logits, _span(rows, width, ld), "logsoftmax_nll logits")
+    _need(dlogits, _span(rows, width, ld), "logsoftmax_nll dlogits")
+    _need(targets, rows, "logsoftmax_nll targets")
+    _need(row_loss, rows, "logsoftmax_nll row_loss")
+    if row_loss.dtype != torch.float32 or (dlogits is not None and dlogits.dtype != logits.dtype):
+        raise TypeError("logsoftmax_nll: dtype mismatch")
     check(lib().hapmi_logsoftmax_nll(_ptr(logits), _ptr(targets), ignore_index, _ptr(row_loss), _ptr(dlogits), rows,
                                      width, ld, ctypes.c_float(grad_scale), dtype_code(logits), _stream()))
 
 
 def sum_f32(x, out):
     _dev(x, out)
+    if x.dtype != torch.float32 or out.dtype != torch.float32 or out.numel() < 1:
+        raise TypeError("sum_f32: float32 buffers expected")
     check(lib().hapmi_sum_f32(_ptr(x), x.numel(), _ptr(out), _stream()))
 
 
@@ -256,31 +351,54 @@ def sum_f32(x, out):
 
 def act_fwd(x, y, act):
     _dev(x, y)
+    _need(y, x.numel(), "act_fwd")
+    if y.dtype != x.dtype or not x.is_contiguous():
+        raise TypeError("act_fwd: dtype / layout mismatch")
     check(lib().hapmi_act_fwd(_ptr(x), _ptr(y), x.numel(), _ACT[act], dtype_code(x), _stream()))
 
 
 def act_bwd(dy, ref, dx, act):
     _dev(dy, ref, dx)
+    _need(ref, dy.numel(), "act_bwd")
+    _need(dx, dy.numel(), "act_bwd")
+    if ref.dtype != dy.dtype or dx.dtype != dy.dtype:
+        raise TypeError("act_bwd: dtype mismatch")
     check(lib().hapmi_act_bwd(_ptr(dy), _ptr(ref), _ptr(dx), dy.numel(), _ACT[act], dtype_code(dy), _stream()))
 
 
 def add(a, b, out):
     _dev(a, b, out)
+    _need(b, a.numel(), "add")
+    _need(out, a.numel(), "add")
+    if b.dtype != a.dtype or out.dtype != a.dtype:
+        raise TypeError("add: dtype mismatch")
     check(lib().hapmi_add(_ptr(a), _ptr(b), _ptr(out), a.numel(), dtype_code(a), _stream()))
 
 
 def scale(a, s, out):
     _dev(a, out)
+    _need(out, a.numel(), "scale")
+    if out.dtype != a.dtype:
+        raise TypeError("scale: dtype mismatch")
     check(lib().hapmi_scale(_ptr(a), ctypes.c_float(s), _ptr(out), a.numel(), dtype_code(a), _stream()))
 
 
 def add_bcast_rows(a, b, out, rows, b_rows, width):
     _dev(a, b, out)
+    _need(a, rows * width, "add_bcast_rows")
+    _need(out, rows * width, "add_bcast_rows")
+    _need(b, b_rows * width, "add_bcast_rows")
+    if b.dtype != a.dtype or out.dtype != a.dtype:
+        raise TypeError("add_bcast_rows: dtype mismatch")
     check(lib().hapmi_add_bcast_rows(_ptr(a), _ptr(b), _ptr(out), rows, b_rows, width, dtype_code(a), _stream()))
 
 
 def colsum(x, out, M, N, ldx=None, accumulate=False):
     _dev(x, out)
+    _need(x, _span(M, N, ldx if ldx is not None else N), "colsum x")
+    _need(out, N, "colsum out")
+    if out.dtype != torch.float32:
+        raise TypeError("colsum: float32 output expected")
     check(lib().hapmi_colsum(_ptr(x), _ptr(out), M, N, ldx if ldx is not None else N, int(accumulate),
                              dtype_code(x), _stream()))
 
@@ -292,28 +410,46 @@ def fill_zero(t):
 
 def cast(src, dst):
     _dev(src, dst)
+    _need(dst, src.numel(), "cast")
     check(lib().hapmi_cast(_ptr(src), dtype_code(src), _ptr(dst), dtype_code(dst), src.numel(), _stream()))
 
 
 def embedding_fwd(ids, table, pe, out, S, scale_=1.0):
     _dev(ids, table, pe, out)
+    _need(out, ids.numel() * table.shape[1], "embedding_fwd out")
+    _need(pe, S * table.shape[1], "embedding_fwd pe")
+    if ids.dtype != torch.int64 or out.dtype != table.dtype or (pe is not None and pe.dtype != table.dtype):
+        raise TypeError("embedding_fwd: dtype mismatch")
     check(lib().hapmi_embedding_fwd(_ptr(ids), _ptr(table), _ptr(pe), _ptr(out), ids.numel(), table.shape[1], S,
                                     table.shape[0], ctypes.c_float(scale_), dtype_code(table), _stream()))
 
 
 def embedding_bwd(ids, dout, dtable, scale_=1.0):
     _dev(ids, dout, dtable)
+    _need(dout, ids.numel() * dtable.shape[1], "embedding_bwd dout")
+    if ids.dtype != torch.int64 or dtable.dtype != torch.float32 or not dtable.is_contiguous():
+        raise TypeError("embedding_bwd: dtype mismatch")
     check(lib().hapmi_embedding_bwd(_ptr(ids), _ptr(dout), _ptr(dtable), ids.numel(), dtable.shape[1],
                                     dtable.shape[0], ctypes.c_float(scale_), dtype_code(dout), _stream()))
 
 
 def patchify(x, cols, b, C, gh, gw, ph, pw):
     _dev(x, cols)
+    _need(x, b * C * gh * ph * gw * pw, "patchify x")
+    _need(cols, b * C * gh * ph * gw * pw, "patchify cols")
+    if x.dtype != torch.float32:
+        raise TypeError("patchify: float32 images expected")
     check(lib().hapmi_patchify(_ptr(x), _ptr(cols), b, C, gh, gw, ph, pw, dtype_code(cols), _stream()))
 
 
 def append_cls_pos(patches, cls, pos, out, b, T, d):
     _dev(patches, cls, pos, out)
+    _need(patches, b * T * d, "append_cls_pos patches")
+    _need(cls, d, "append_cls_pos cls")
+    _need(pos, (T + 1) * d, "append_cls_pos pos")
+    _need(out, b * (T + 1) * d, "append_cls_pos out")
+    if not (patches.dtype == cls.dtype == pos.dtype == out.dtype):
+        raise TypeError("append_cls_pos: dtype mismatch")
     check(lib().hapmi_append_cls_pos(_ptr(patches), _ptr(cls), _ptr(pos), _ptr(out), b, T, d, dtype_code(out), _stream()))
 
 
@@ -323,6 +459,10 @@ def append_cls_pos(patches, cls, pos, out, b, T, d):
 
 def sgd_step(param, grad, shadow, lr, grad_scale=None):
     _dev(param, grad, shadow, grad_scale)
+    _need(grad, param.numel(), "sgd_step grad")
+    _need(shadow, param.numel(), "sgd_step shadow")
+    if param.dtype != torch.float32 or grad.dtype != torch.float32 or (shadow is not None and shadow.dtype != torch.bfloat16):
+        raise TypeError("sgd_step: dtype mismatch")
     check(lib().hapmi_sgd_step(_ptr(param), _ptr(grad), _ptr(shadow), param.numel(), ctypes.c_float(lr),
                                _ptr(grad_scale), _stream()))
 
@@ -331,6 +471,13 @@ def adam_step(param, grad, exp_avg, exp_avg_sq, shadow, lr, beta1, beta2, eps, s
     _dev(param, grad, exp_avg, exp_avg_sq, shadow, grad_scale)
     bc1 = 1.0 - beta1 ** step
     bc2 = 1.0 - beta2 ** step
+    for t_ in (grad, exp_avg, exp_avg_sq):
+        _need(t_, param.numel(), "adam_step")
+        if t_.dtype != torch.float32:
+            raise TypeError("adam_step: float32 state expected")
+    _need(shadow, param.numel(), "adam_step shadow")
+    if param.dtype != torch.float32 or (shadow is not None and shadow.dtype != torch.bfloat16):
+        raise TypeError("adam_step: dtype mismatch")
     check(lib().hapmi_adam_step(_ptr(param), _ptr(grad), _ptr(exp_avg), _ptr(exp_avg_sq), _ptr(shadow), param.numel(),
                                 ctypes.c_float(lr), ctypes.c_float(beta1), ctypes.c_float(beta2), ctypes.c_float(eps),
                                 ctypes.c_float(bc1), ctypes.c_float(bc2), _ptr(grad_scale), _stream()))
@@ -364,14 +511,39 @@ def top2_gate(logits, capacity):
     return r
 
 
+def _check_routing(r, B, S, E=None, C=None):
+    _dev(*r.values())
+    _need(r["index"], B * S * 2, "routing index")
+    _need(r["slot"], B * S * 2, "routing slot")
+    _need(r["gate"], B * S * 2, "routing gate")
+    if r["index"].dtype != torch.int32 or r["slot"].dtype != torch.int32 or r["gate"].dtype != torch.float32:
+        raise TypeError("routing tensors must be int32 / int32 / float32")
+    if E is not None:
+        _need(r["probs"], B * S * E, "routing probs")
+        if C is not None:
+            _need(r["token_of_slot"], B * E * C, "routing token_of_slot")
+            if r["token_of_slot"].dtype != torch.int32:
+                raise TypeError("token_of_slot must be int32")
+
+
 def top2_gate_into(logits, capacity, r):
     B, S, E = logits.shape
+    _dev(logits)
+    if logits.dtype != torch.float32 or not logits.is_contiguous():
+        raise TypeError("top2_gate: contiguous float32 logits expected")
+    _check_routing(r, B, S, E, capacity)
     check(lib().hapmi_top2_gate(_ptr(logits), _ptr(r["probs"]), _ptr(r["index"]), _ptr(r["slot"]), _ptr(r["gate"]),
                                 _ptr(r["token_of_slot"]), B, S, E, capacity, _stream()))
 
 
 def top2_gate_bwd(r, dgate, dlogits):
     B, S, E = r["probs"].shape
+    _check_routing(r, B, S, E)
+    _dev(dgate, dlogits)
+    _need(dgate, B * S * 2, "top2_gate_bwd dgate")
+    _need(dlogits, B * S * E, "top2_gate_bwd dlogits")
+    if dgate.dtype != torch.float32 or dlogits.dtype != torch.float32:
+        raise TypeError("top2_gate_bwd: float32 expected")
     check(lib().hapmi_top2_gate_bwd(_ptr(r["probs"]), _ptr(r["index"]), _ptr(r["slot"]), _ptr(dgate), _ptr(dlogits),
                                     B, S, E, _stream()))
 
@@ -381,6 +553,7 @@ def top2_densify(r, E, C):
     dev = r["index"].device
     dispatch = torch.empty(B, S, E, C, dtype=torch.float32, device=dev)
     combine = torch.empty(B, S, E, C, dtype=torch.float32, device=dev)
+    _check_routing(r, B, S)
     check(lib().hapmi_top2_densify(_ptr(r["index"]), _ptr(r["slot"]), _ptr(r["gate"]), _ptr(dispatch), _ptr(combine),
                                    B, S, E, C, _stream()))
     return dispatch, combine
@@ -388,18 +561,35 @@ def top2_densify(r, E, C):
 
 def moe_dispatch(x, r, expert_in, E, C, e_lo, E_loc):
     B, S, d = x.shape
+    _dev(x, expert_in)
+    _check_routing(r, B, S, E, C)
+    _need(expert_in, E_loc * B * C * d, "moe_dispatch expert_in")
+    if expert_in.dtype != x.dtype or not x.is_contiguous():
+        raise TypeError("moe_dispatch: dtype / layout mismatch")
     check(lib().hapmi_moe_dispatch(_ptr(x), _ptr(r["token_of_slot"]), _ptr(expert_in), B, S, E, C, d, e_lo, E_loc,
                                    dtype_code(x), _stream()))
 
 
 def moe_combine(expert_out, r, out, C, e_lo, E_loc):
     B, S, d = out.shape
+    _dev(expert_out, out)
+    _check_routing(r, B, S)
+    _need(expert_out, E_loc * B * C * d, "moe_combine expert_out")
+    if expert_out.dtype != out.dtype or not out.is_contiguous():
+        raise TypeError("moe_combine: dtype / layout mismatch")
     check(lib().hapmi_moe_combine(_ptr(expert_out), _ptr(r["index"]), _ptr(r["slot"]), _ptr(r["gate"]), _ptr(out),
                                   B, S, C, d, e_lo, E_loc, dtype_code(out), _stream()))
 
 
 def moe_combine_bwd(dout, expert_out, r, d_expert_out, dgate, E, C, e_lo, E_loc):
     B, S, d = dout.shape
+    _dev(dout, expert_out, d_expert_out, dgate)
+    _check_routing(r, B, S, E, C)
+    _need(expert_out, E_loc * B * C * d, "moe_combine_bwd expert_out")
+    _need(d_expert_out, E_loc * B * C * d, "moe_combine_bwd d_expert_out")
+    _need(dgate, B * S * 2, "moe_combine_bwd dgate")
+    if not (expert_out.dtype == d_expert_out.dtype == dout.dtype) or dgate.dtype != torch.float32:
+        raise TypeError("moe_combine_bwd: dtype mismatch")
     check(lib().hapmi_moe_combine_bwd(_ptr(dout), _ptr(expert_out), _ptr(r["index"]), _ptr(r["slot"]), _ptr(r["gate"]),
                                       _ptr(r["token_of_slot"]), _ptr(d_expert_out), _ptr(dgate), B, S, E, C, d, e_lo,
                                       E_loc, dtype_code(dout), _stream()))
@@ -407,6 +597,11 @@ def moe_combine_bwd(dout, expert_out, r, d_expert_out, dgate, E, C, e_lo, E_loc)
 
 def moe_dispatch_bwd(d_expert_in, r, dx, C, e_lo, E_loc, accumulate):
     B, S, d = dx.shape
+    _dev(d_expert_in, dx)
+    _check_routing(r, B, S)
+    _need(d_expert_in, E_loc * B * C * d, "moe_dispatch_bwd d_expert_in")
+    if d_expert_in.dtype != dx.dtype or not dx.is_contiguous():
+        raise TypeError("moe_dispatch_bwd: dtype / layout mismatch")
     check(lib().hapmi_moe_dispatch_bwd(_ptr(d_expert_in), _ptr(r["index"]), _ptr(r["slot"]), _ptr(r["gate"]), _ptr(dx),
                                        B, S, C, d, e_lo, E_loc, int(accumulate), dtype_code(dx), _stream()))
 

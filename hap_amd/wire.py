@@ -45,16 +45,20 @@ class SilentWire(Wire):
 
 
 class SyntheticWire(Wire):
-    def __init__(self, seed: int = 0, scale: float = 1.0, grad_scale: float = 1e-3, reduce_params: bool = False):
+    def __init__(self, seed: int = 0, scale: float = 1.0, grad_scale: float = 1e-3, reduce_params: bool = False,
+                 share_shapes: bool = False):
+        """``share_shapes``: messages of equal shape, direction and sender reuse one buffer (a benchmark with
+        many identical layers then needs one set of peer buffers instead of one per layer)."""
         self.gen = torch.Generator().manual_seed(seed)
         self.scale, self.grad_scale = scale, grad_scale
         self.reduce_params = reduce_params
+        self.share_shapes = share_shapes
         self._cache: Dict[Tuple, torch.Tensor] = {}
 
     def recv(self, tag, direction, src, shape, dtype, device, reduction: bool = False):
         if tag.startswith("replicate") and not self.reduce_params:
             return None
-        key = (tag, direction, src)
+        key = (direction, src, tuple(shape), dtype) if self.share_shapes else (tag, direction, src)
         if key not in self._cache:
             s = self.scale if direction == "fwd" else self.grad_scale
             t = torch.randn(tuple(shape), generator=self.gen, dtype=torch.float32) * s

@@ -69,6 +69,8 @@ class JointCPURun:
         if t is product_collectives.dynamic_slice:
             return self.world.dynamic_slice(*args)
         if self.dtype == "bf16":
+            if t is F.conv2d:                           # images arrive as float32; the patch GEMM runs in bf16
+                return F.conv2d(args[0].to(torch.bfloat16), *args[1:], **kwargs)
             if t is torch.log_softmax:
                 return torch.log_softmax(args[0].float(), *args[1:], **kwargs)
             if t is torch.einsum and any(a.dtype == torch.float32 for a in args[1:]):

@@ -1,0 +1,246 @@
+"""Single-kernel parity through the C ABI against stock PyTorch on the CPU (the library routines the emitted
+program calls in the reference: F.linear, F.layer_norm, softmax, log_softmax + nll_loss, F.embedding, relu,
+torch.optim).  Tolerances: float32 rtol 1e-4; bfloat16 rtol 2e-2 (inputs are rounded to bf16 on both sides)."""
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from hap_amd import ops
+from helpers import rel_err
+
+pytestmark = pytest.mark.gpu
+DT = [torch.float32, torch.bfloat16]
+TOL = {torch.float32: 1e-4, torch.bfloat16: 2e-2}
+
+
+def close(got, want, dtype, scale=1.0):
+    got, want = got.float().cpu(), want.float()
+    tol = TOL[dtype] * scale
+    assert rel_err(got, want) < tol, rel_err(got, want)
+    torch.testing.assert_close(got, want, rtol=tol, atol=tol * max(want.abs().max().item(), 1e-6))
+
+
+GEMM_SHAPES = [(128, 128, 64), (384, 768, 512), (100, 52, 72), (257, 136, 200), (33, 1000, 96), (64, 16, 768),
+               (512, 264, 1096)]
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("tA,tB", [(0, 1), (0, 0), (1, 0), (1, 1)])
+@pytest.mark.parametrize("M,N,K", GEMM_SHAPES)
+def test_gemm_layouts_and_ragged_edges(cuda, dtype, tA, tB, M, N, K):
+    g = torch.Generator().manual_seed(M + N + K)
+    epv = 4 if dtype == torch.float32 else 8
+    if (tA and M % epv) or ((not tA) and K % epv) or (tB and K % epv) or ((not tB) and N % epv):
+        pytest.skip("leading dimension must be a multiple of the vector width")
+    A = torch.randn((K, M) if tA else (M, K), generator=g).to(dtype)
+    B = torch.randn((N, K) if tB else (K, N), generator=g).to(dtype)
+    bias = torch.randn(N, generator=g)
+    ldc = (N + 3) // 4 * 4
+    C = torch.zeros(M, ldc, dtype=dtype, device=cuda)
+    ops.gemm(A.to(cuda), B.to(cuda), C, M, N, K, transA=bool(tA), transB=bool(tB), ldc=ldc, bias=bias.to(cuda))
+    opA = A.double().t() if tA else A.double()
+    opB = B.double().t() if tB else B.double()
+    want = opA @ opB + bias.double()
+    close(C[:, :N], want, dtype, scale=2.0)
+    assert (C[:, N:] == 0).all()
+
+
+@pytest.mark.parametrize("dtype", DT)
+def test_gemm_epilogue_accumulate_alpha_act_batch(cuda, dtype):
+    g = torch.Generator().manual_seed(2)
+    b1, b2, M, N, K = 3, 2, 40, 24, 64
+    A = torch.randn(b1, b2, M, K, generator=g).to(dtype)
+    B = torch.randn(b1, b2, K, N, generator=g).to(dtype)
+    C0 = torch.randn(b1, b2, M, N, generator=g)
+    C = C0.clone().to(cuda)                                   # float32 output from either input type
+    ops.gemm(A.to(cuda), B.to(cuda), C, M, N, K, alpha=0.5, accumulate=True, batch1=b1, batch2=b2,
+             strideA=(b2 * M * K, M * K), strideB=(b2 * K * N, K * N), strideC=(b2 * M * N, M * N))
+    close(C, C0.double() + 0.5 * (A.double() @ B.double()), dtype, scale=2.0)
+    for act, fn in (("relu", torch.relu), ("gelu", F.gelu)):
+        out = torch.empty(M, N, dtype=dtype, device=cuda)
+        ops.gemm(A[0, 0].to(cuda), B[0, 0].to(cuda), out, M, N, K, act=act)
+        close(out, fn(A[0, 0].double() @ B[0, 0].double()), dtype, scale=2.0)
+
+
+def test_gemm_refuses_misaligned(cuda):
+    from hap_amd._lib import HapmiError
+    a = torch.zeros(8, 10, dtype=torch.bfloat16, device=cuda)
+    with pytest.raises(HapmiError):
+        ops.gemm(a, a, torch.zeros(8, 8, dtype=torch.bfloat16, device=cuda), 8, 8, 10, transB=True)
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("rows,width", [(384, 512), (37, 768), (5, 1024), (9, 100), (3, 2048)])
+def test_add_layernorm_forward_backward(cuda, dtype, rows, width):
+    g = torch.Generator().manual_seed(rows)
+    x, r = torch.randn(rows, width, generator=g).to(dtype), torch.randn(rows, width, generator=g).to(dtype)
+    dy = torch.randn(rows, width, generator=g).to(dtype)
+    y = torch.empty(rows, width, dtype=dtype, device=cuda)
+    rstd = torch.empty(rows, dtype=torch.float32, device=cuda)
+    ops.add_layernorm_fwd(x.to(cuda), r.to(cuda), y, rstd)
+    s = (x + r).double().requires_grad_(True)                 # the sum is rounded to the storage type first
+    want = F.layer_norm(s, (width,))
+    close(y, want.detach(), dtype)
+    dx = torch.empty_like(y)
+    ops.layernorm_bwd(dy.to(cuda), y, rstd, None, dx)
+    want.backward(dy.double())
+    close(dx, s.grad, dtype, scale=2.0)
+    dx2 = torch.empty_like(y)
+    ops.layernorm_bwd(dy.to(cuda), y, rstd, dy.to(cuda), dx2)
+    close(dx2, s.grad + dy.double(), dtype, scale=2.0)
+    # without a residual
+    ops.add_layernorm_fwd(x.to(cuda), None, y, rstd)
+    close(y, F.layer_norm(x.double(), (width,)), dtype)
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("S,ld", [(128, 128), (197, 200), (16, 16), (512, 512)])
+def test_softmax_with_mask_forward_backward(cuda, dtype, S, ld):
+    g = torch.Generator().manual_seed(S)
+    rows = 3 * S
+    x = torch.randn(rows, ld, generator=g).to(dtype)
+    mask = torch.triu(torch.full((S, S), float("-inf")), diagonal=1)
+    p = x.clone().to(cuda)
+    ops.softmax_fwd(p, mask.to(cuda), p, rows, S, ld, S)
+    want = torch.softmax(x[:, :S].double().view(3, S, S) + mask.double(), dim=-1).view(rows, S)
+    close(p[:, :S], want, dtype)
+    assert torch.equal(p[:, S:].cpu(), x[:, S:])              # pad columns untouched
+    assert (p[:, :S].cpu().view(3, S, S).triu(1) == 0).all()   # causal: nothing above the diagonal
+    dp = torch.randn(rows, ld, generator=g).to(dtype)
+    ds = dp.clone().to(cuda)
+    ops.softmax_bwd(ds, p, ds, rows, S, ld)
+    pw = p[:, :S].double().cpu()
+    wantd = pw * (dp[:, :S].double() - (dp[:, :S].double() * pw).sum(-1, keepdim=True))
+    close(ds[:, :S], wantd, dtype, scale=2.0)
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("rows,V,ld", [(24, 33280, 33280), (17, 30522, 30528), (8, 1000, 1000), (5, 97, 100)])
+def test_logsoftmax_nll_and_gradient(cuda, dtype, rows, V, ld):
+    g = torch.Generator().manual_seed(V)
+    logits = (torch.randn(rows, ld, generator=g) * 3).to(dtype)
+    tgt = torch.randint(0, V, (rows,), generator=g)
+    tgt[::3] = -100
+    row_loss = torch.empty(rows, dtype=torch.float32, device=cuda)
+    loss = torch.empty(1, dtype=torch.float32, device=cuda)
+    buf = logits.clone().to(cuda)
+    ops.logsoftmax_nll(buf, tgt.to(cuda), row_loss, buf, rows, V, ld)
+    ops.sum_f32(row_loss, loss)
+    x = logits[:, :V].double().requires_grad_(True)
+    want = F.nll_loss(torch.log_softmax(x, dim=1), tgt, reduction="sum")
+    want.backward()
+    assert abs(loss.item() - want.item()) <= 1e-5 * abs(want.item())
+    close(buf[:, :V], x.grad, dtype)
+    assert (buf[::3, :V] == 0).all()
+
+
+@pytest.mark.parametrize("dtype", DT)
+def test_embedding_forward_backward(cuda, dtype):
+    g = torch.Generator().manual_seed(1)
+    V, d, n, S = 211, 48, 60, 20
+    table = torch.randn(V, d, generator=g).to(dtype)
+    pe = torch.randn(S, d, generator=g).to(dtype)
+    ids = torch.randint(0, V, (n,), generator=g)
+    ids[5] = ids[6] = ids[7]                                    # collisions in the scatter-add
+    out = torch.empty(n, d, dtype=dtype, device=cuda)
+    ops.embedding_fwd(ids.to(cuda), table.to(cuda), pe.to(cuda), out, S, math.sqrt(d))
+    want = (F.embedding(ids, table) * math.sqrt(d)).float() + pe.float()[torch.arange(n) % S]
+    close(out, want, dtype)
+    plain = torch.empty(n, d, dtype=dtype, device=cuda)
+    ops.embedding_fwd(ids.to(cuda), table.to(cuda), None, plain, 1, 1.0)
+    assert torch.equal(plain.cpu(), F.embedding(ids, table))       # a pure row gather is exact
+    dout = torch.randn(n, d, generator=g).to(dtype)
+    dt = torch.zeros(V, d, dtype=torch.float32, device=cuda)
+    ops.embedding_bwd(ids.to(cuda), dout.to(cuda), dt, 1.0)
+    wantg = torch.zeros(V, d, dtype=torch.float64).index_add_(0, ids, dout.double())
+    close(dt, wantg, torch.float32)
+
+
+@pytest.mark.parametrize("dtype", DT)
+def test_elementwise_and_reductions(cuda, dtype):
+    g = torch.Generator().manual_seed(4)
+    n = 4099
+    a, b = torch.randn(n, generator=g).to(dtype), torch.randn(n, generator=g).to(dtype)
+    da, db = a.to(cuda), b.to(cuda)
+    out = torch.empty_like(da)
+    ops.add(da, db, out)
+    assert torch.equal(out.cpu(), a + b)
+    ops.scale(da, 1.5, out)
+    assert torch.equal(out.cpu(), (a.float() * 1.5).to(dtype))
+    ops.act_fwd(da, out, "relu")
+    assert torch.equal(out.cpu(), torch.relu(a))
+    y = out.clone()
+    ops.act_bwd(db, y, out, "relu")
+    assert torch.equal(out.cpu(), torch.where(a > 0, b, torch.zeros_like(b)))
+    ops.act_fwd(da, out, "gelu")
+    close(out, F.gelu(a.double()), dtype)
+    ops.act_bwd(db, da, out, "gelu")
+    ad = a.double().requires_grad_(True)
+    F.gelu(ad).backward(b.double())
+    close(out, ad.grad, dtype)
+    x = torch.randn(300, 72, generator=g).to(dtype)
+    cs = torch.empty(72, dtype=torch.float32, device=cuda)
+    ops.colsum(x.to(cuda), cs, 300, 72)
+    close(cs, x.double().sum(0), torch.float32)
+    ops.colsum(x.to(cuda), cs, 300, 72, accumulate=True)
+    close(cs, 2 * x.double().sum(0), torch.float32)
+    big, small = torch.randn(6, 5, 8, generator=g).to(dtype), torch.randn(1, 5, 8, generator=g).to(dtype)
+    o3 = torch.empty(6, 5, 8, dtype=dtype, device=cuda)
+    ops.add_bcast_rows(big.to(cuda), small.to(cuda), o3, 30, 5, 8)
+    assert torch.equal(o3.cpu(), big + small)
+
+
+def test_patchify_and_cls_pos(cuda):
+    g = torch.Generator().manual_seed(6)
+    b, C, gh, gw, ph, pw, d = 3, 3, 4, 5, 4, 2, 16
+    x = torch.randn(b, C, gh * ph, gw * pw, generator=g)
+    w = torch.randn(d, C, ph, pw, generator=g)
+    cols = torch.empty(b * gh * gw, C * ph * pw, dtype=torch.float32, device=cuda)
+    ops.patchify(x.to(cuda), cols, b, C, gh, gw, ph, pw)
+    got = cols.cpu() @ w.view(d, -1).t()
+    want = torch.flatten(F.conv2d(x, w, None, (ph, pw)), 2).transpose(1, 2).reshape(b * gh * gw, d)
+    torch.testing.assert_close(got, want, rtol=1e-5, atol=1e-5)
+    T = gh * gw
+    patches, cls, pos = torch.randn(b, T, d, generator=g), torch.randn(1, 1, d, generator=g), torch.randn(1, T + 1, d, generator=g)
+    out = torch.empty(b, T + 1, d, device=cuda)
+    ops.append_cls_pos(patches.to(cuda), cls.to(cuda), pos.to(cuda), out, b, T, d)
+    assert torch.equal(out.cpu(), torch.cat((cls.expand(b, -1, -1), patches), dim=1) + pos)
+
+
+def test_optimizers_match_torch(cuda):
+    g = torch.Generator().manual_seed(8)
+    n = 1003
+    p0 = torch.randn(n, generator=g)
+    grads = [torch.randn(n, generator=g) for _ in range(3)]
+    # SGD
+    ref = p0.clone().requires_grad_(True)
+    opt = torch.optim.SGD([ref], lr=1e-3)
+    p = p0.clone().to(cuda)
+    for gr in grads:
+        ref.grad = gr.clone()
+        opt.step()
+        ops.sgd_step(p, gr.to(cuda), None, 1e-3)
+    torch.testing.assert_close(p.cpu(), ref.detach(), rtol=1e-6, atol=1e-7)
+    # Adam with a bf16 shadow
+    ref = p0.clone().requires_grad_(True)
+    opt = torch.optim.Adam([ref], lr=5e-4)
+    p, m, v = p0.clone().to(cuda), torch.zeros(n, device=cuda), torch.zeros(n, device=cuda)
+    sh = torch.empty(n, dtype=torch.bfloat16, device=cuda)
+    for i, gr in enumerate(grads):
+        ref.grad = gr.clone()
+        opt.step()
+        ops.adam_step(p, gr.to(cuda), m, v, sh, 5e-4, 0.9, 0.999, 1e-8, i + 1)
+    torch.testing.assert_close(p.cpu(), ref.detach(), rtol=1e-5, atol=1e-7)
+    assert torch.equal(sh.cpu(), p.cpu().bfloat16())
+    # first Adam step is -lr * sign(g) up to eps
+    p1, m1, v1 = torch.zeros(n, device=cuda), torch.zeros(n, device=cuda), torch.zeros(n, device=cuda)
+    ops.adam_step(p1, grads[0].to(cuda), m1, v1, None, 5e-4, 0.9, 0.999, 1e-8, 1)
+    torch.testing.assert_close(p1.cpu(), -5e-4 * torch.sign(grads[0]), rtol=1e-4, atol=1e-9)
+    # gradient clipping coefficient (clip_grad_norm_)
+    ss, coef = torch.zeros(1, device=cuda), torch.zeros(1, device=cuda)
+    ops.sumsq(grads[0].to(cuda), ss)
+    ops.clip_coef(ss, 0.5, coef)
+    want = min(1.0, 0.5 / (grads[0].norm().item() + 1e-6))
+    assert abs(coef.item() - want) < 1e-6 * want

@@ -1,0 +1,145 @@
+"""End-to-end parity of the compiled shard program on the GPU against stock-PyTorch CPU execution of the same
+generated graph (all ranks on the CPU; the GPU runs one rank with the peers' messages replayed).
+Loss, every parameter gradient and the updated parameters are compared:
+float32: rtol 1e-4 (norm-wise and element-wise with atol = rtol * max|ref|);
+bfloat16: rtol 2e-2 norm-wise on losses, gradients and updated weights."""
+import copy
+
+import pytest
+import torch
+
+import hap_amd
+from helpers import (RATIOS4, RATIOS_E, joint_cpu, lm_batch, make_lm, make_moe, make_vit, rel_err, vit_batch)
+
+pytestmark = pytest.mark.gpu
+
+
+def _gpu_rank(model, ratios, rank, B, x, y, log, dtype, opt, **kw):
+    m = copy.deepcopy(model)
+    plan = hap_amd.ShardingPlan([list(ratios)], rank, ffn=kw.get("ffn", "column"))
+    gm = hap_amd.build_program(m, plan, B, activation=kw.get("activation", "relu"),
+                               batch_sharded=kw.get("batch_sharded", True))
+    ex = hap_amd.compile_program(gm, [x, y], dtype=dtype, wire=hap_amd.ReplayWire(log, rank), rank=rank,
+                                 world_size=len(ratios))
+    ex.configure_optimizer(**opt)
+    loss = ex.forward(x, y)
+    ex.backward()
+    grads = {n: rec["grad"].clone().cpu() for n, rec in ex.params.items()}
+    ex.step()
+    torch.cuda.synchronize()
+    params = {n: rec["master"].clone().cpu() for n, rec in ex.params.items()}
+    return loss.item(), grads, params, ex
+
+
+def _compare(model, ratios, B, x, y, dtype, ranks, opt, **kw):
+    run = joint_cpu(model, ratios, B, dtype, **kw)
+    if opt["kind"] == "sgd":
+        optims = [torch.optim.SGD(p.parameters(), lr=opt["lr"]) for p in run.programs]
+    else:
+        optims = [torch.optim.Adam(p.parameters(), lr=opt["lr"]) for p in run.programs]
+    initial = [{n: p.detach().clone() for n, p in prog.named_parameters()} for prog in run.programs]
+    losses = run.step(x, y, None)
+    ref_grads = [{n: p.grad.clone() for n, p in prog.named_parameters() if p.grad is not None} for prog in run.programs]
+    for o in optims:
+        o.step()
+    tol = 1e-4 if dtype == "fp32" else 2e-2
+    ex_initial = {r: [(n, p.detach().clone()) for n, p in initial[r].items()] for r in ranks}
+    for r in ranks:
+        loss, grads, params, ex = _gpu_rank(model, ratios, r, B, x, y, run.world.log, dtype, opt, **kw)
+        want = losses[r].float().item()
+        assert abs(loss - want) <= tol * abs(want), (r, loss, want)
+        assert set(grads) == set(ref_grads[r]), set(grads) ^ set(ref_grads[r])
+        for n, g in grads.items():
+            ref = ref_grads[r][n].float()
+            assert g.shape == ref.shape, n
+            err = rel_err(g, ref)
+            assert err < tol * (1 if dtype == "fp32" else 1.5), (r, n, err)
+            if dtype == "fp32":
+                torch.testing.assert_close(g, ref, rtol=tol, atol=tol * ref.abs().max().item())
+        ref_params = dict(run.programs[r].named_parameters())
+        for n, p in params.items():
+            assert rel_err(p, ref_params[n].detach()) < tol, (r, n)
+    return run
+
+
+SGD = dict(kind="sgd", lr=1e-3)
+ADAM = dict(kind="adam", lr=5e-4)
+
+
+@pytest.mark.parametrize("ffn", ["column", "batch"])
+def test_lm_fp32_small(cuda, ffn):
+    model = make_lm()
+    x, y = lm_batch(8, 16, 97)
+    _compare(model, RATIOS4, 8, x, y, "fp32", [0, 3], SGD, ffn=ffn)
+
+
+def test_config1_full_size_fp32(cuda):
+    """BASELINE config 1: 2-layer post-LN LM, d 512, 8 heads, FFN 2048 -> 768 local, seq 128, 3 of 8, vocab 33280."""
+    model = make_lm(vocab=33280, S=128, d=512, H=8, F=2048, layers=2, seed=39)
+    x, y = lm_batch(8, 128, 33280, seed=39)
+    _compare(model, RATIOS4, 8, x, y, "fp32", [0], SGD)
+
+
+def test_lm_bf16_mlm_adam(cuda):
+    model = make_lm(vocab=1003, S=32, d=64, H=4, F=128, layers=2, causal=False)
+    x, y = lm_batch(8, 32, 1003, mlm=True)
+    _compare(model, RATIOS4, 8, x, y, "bf16", [0, 2], ADAM)
+
+
+def test_lm_gelu_fp32(cuda):
+    model = make_lm()
+    x, y = lm_batch(8, 16, 97)
+    _compare(model, RATIOS4, 8, x, y, "fp32", [1], SGD, activation="gelu")
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+def test_vit(cuda, dtype):
+    model = make_vit(img=32, patch=8, d=64, F=128)
+    x, y = vit_batch(8, 32, 10)
+    _compare(model, RATIOS4, 8, x, y, dtype, [0, 3], ADAM, ffn="batch")
+
+
+@pytest.mark.parametrize("batch_sharded", [True, False])
+def test_moe_fp32(cuda, batch_sharded):
+    model = make_moe()
+    B = 16 if batch_sharded else 4
+    x, y = lm_batch(B, 16, 61)
+    _compare(model, RATIOS_E, B, x, y, "fp32", [0, 2], ADAM, ffn="batch", batch_sharded=batch_sharded)
+
+
+def test_moe_bf16_routing_matches(cuda):
+    model = make_moe(d=64, F=96, std=0.3)
+    x, y = lm_batch(4, 16, 61)
+    run = _compare(model, RATIOS_E, 4, x, y, "bf16", [0], ADAM, ffn="batch", batch_sharded=False)
+
+
+def test_module_facade_is_a_drop_in(cuda):
+    """worker.py:59-76 usage: loss = dmodel(x, y); loss.backward(); torch optimizer step."""
+    model = make_lm()
+    x, y = lm_batch(8, 16, 97)
+    run = joint_cpu(model, RATIOS4, 8)
+    ref_opt = torch.optim.Adam(run.programs[0].parameters(), lr=5e-4)
+    losses = run.step(x, y, [ref_opt])
+    m = copy.deepcopy(model)
+    gm = hap_amd.build_program(m, hap_amd.ShardingPlan([RATIOS4], 0), 8)
+    dmodel = hap_amd.compile(gm, [x, y], wire=hap_amd.ReplayWire(run.world.log, 0), rank=0, world_size=4)
+    opt = torch.optim.Adam(dmodel.parameters(), lr=5e-4)
+    dmodel.zero_grad()
+    loss = dmodel(x, y)
+    loss.backward()
+    opt.step()
+    assert abs(loss.item() - losses[0].item()) < 1e-4 * abs(losses[0].item())
+    ref_params = dict(run.programs[0].named_parameters())
+    for n, rec in dmodel.executor.params.items():
+        g_ref = ref_params[n].grad
+        clear = g_ref.abs() > 1e-2 * g_ref.abs().max()
+        got, want = rec["param"].detach().cpu(), ref_params[n].detach()
+        assert rel_err(got[clear], want[clear]) < 1e-3, n
+
+
+def test_unsupported_nodes_raise(cuda):
+    model = make_lm()
+    model.dropout_p = 0.1
+    gm = hap_amd.build_program(copy.deepcopy(model), hap_amd.ShardingPlan([RATIOS4], 0), 8)
+    with pytest.raises(ValueError):
+        hap_amd.compile_program(gm, [(8, 16), (8, 16)])

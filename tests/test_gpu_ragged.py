@@ -1,0 +1,122 @@
+"""Device-local halves of the uneven collectives through the C ABI, bit-exact against the reference's own
+torch.cat / torch.split / slicing on the CPU (/root/reference/collectives.py:9-29, 88-103, 146-166)."""
+import pytest
+import torch
+
+from hap_amd import ops
+from oracle.ops import _accumulate
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.bfloat16, torch.float32, torch.int64, torch.int16]
+
+
+def rnd(shape, dtype, g):
+    if dtype.is_floating_point:
+        return torch.randn(shape, generator=g).to(dtype)
+    return torch.randint(-1000, 1000, shape, generator=g).to(dtype)
+
+
+CASES = [  # (shape of the full tensor, dim, lengths)
+    ((10, 6), 0, [1, 2, 3, 4]),
+    ((5, 10), 1, [1, 2, 3, 4]),
+    ((4, 10, 24), 1, [3, 3, 1, 3]),
+    ((8, 16, 40), 0, [3, 3, 1, 1]),
+    ((3, 5, 48), 2, [18, 18, 6, 6]),
+    ((7, 9), 1, [4, 0, 5, 0]),               # zero-length shards
+    ((6, 7, 3), 1, [2, 5]),                  # odd inner size: narrow vector path
+    ((2, 1, 4096), 1, [1]),
+]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape,dim,L", CASES)
+def test_pad_split_concat_slice_layouts(cuda, dtype, shape, dim, L):
+    g = torch.Generator().manual_seed(11)
+    full = rnd(shape, dtype, g)
+    m = max(L)
+    shards = list(torch.split(full, L, dim=dim))
+    dfull = full.to(cuda)
+    # pad: head equals the shard, tail keeps what the buffer held before (the reference leaves it uninitialised)
+    for sh in shards:
+        out = torch.full(ops._with_dim(sh.shape, dim, m), 7, dtype=dtype, device=cuda)
+        ops.pad_rows(sh.contiguous().to(cuda), dim, m, out)
+        head, tail = out.cpu().split([sh.shape[dim], m - sh.shape[dim]], dim=dim)
+        assert torch.equal(head, sh) and (tail == 7).all()
+    # split + pad
+    outs = [torch.full(ops._with_dim(shape, dim, m), 7, dtype=dtype, device=cuda) for _ in L]
+    ops.split_pad(dfull, L, dim, m, outs)
+    for o, sh in zip(outs, shards):
+        head, tail = o.cpu().split([sh.shape[dim], m - sh.shape[dim]], dim=dim)
+        assert torch.equal(head, sh) and (tail == 7).all()
+    # unpad + concat of those padded slices gives the full tensor back
+    assert torch.equal(ops.unpad_concat(outs, L, dim).cpu(), full)
+    # unpadded split / concat
+    pieces = ops.split_rows(dfull, L, dim)
+    for p, sh in zip(pieces, shards):
+        assert torch.equal(p.cpu(), sh)
+    assert torch.equal(ops.concat_rows(pieces, dim).cpu(), full)
+    # dynamic_slice and its inverse
+    for r in range(len(L)):
+        off = sum(L[:r])
+        s = ops.slice_rows(dfull, dim, off, L[r])
+        assert torch.equal(s.cpu(), shards[r])
+        back = torch.zeros(shape, dtype=dtype, device=cuda)
+        ops.place_rows(s, back, dim, off)
+        want = torch.zeros(shape, dtype=dtype)
+        want.narrow(dim, off, L[r]).copy_(shards[r])
+        assert torch.equal(back.cpu(), want)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_concat_with_fused_relu(cuda, dtype):
+    g = torch.Generator().manual_seed(3)
+    pieces = [torch.randn(3, 8, n, generator=g).to(dtype) for n in (48, 48, 16, 16)]
+    out = ops.concat_rows([p.to(cuda) for p in pieces], 2, act="relu")
+    assert torch.equal(out.cpu(), torch.relu(torch.cat(pieces, dim=2)))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("W", [1, 2, 3, 4, 8])
+@pytest.mark.parametrize("shape,dim,off,length", [((40, 64), 0, 7, 20), ((4, 10, 24), 1, 3, 4), ((5, 9, 7), 1, 0, 9),
+                                                  ((3, 64), 1, 8, 48)])
+def test_ragged_reduce_bit_exact(cuda, dtype, W, shape, dim, off, length):
+    g = torch.Generator().manual_seed(W)
+    parts = [torch.randn(shape, generator=g).to(dtype) for _ in range(W)]
+    got = ops.ragged_reduce([p.to(cuda) for p in parts], dim, off, length)
+    want = _accumulate([p.narrow(dim, off, length) for p in parts])
+    assert torch.equal(got.cpu(), want)
+
+
+def test_config5_shapes_round_trip_and_reduce(cuda):
+    """8 ragged bf16 shards [S_i, 4096], S_i in [1000, 3000] from the seed: pad to max, split, concat, reduce."""
+    g = torch.Generator().manual_seed(39)
+    S = torch.randint(1000, 3001, (8,), generator=g).tolist()
+    m, total = max(S), sum(S)
+    shards = [torch.randn(s, 4096, generator=g).bfloat16().to(cuda) for s in S]
+    padded = [ops.pad_rows(x, 0, m) for x in shards]
+    full = ops.unpad_concat(padded, S, 0)
+    assert full.shape == (total, 4096)
+    assert torch.equal(full, torch.cat(shards, dim=0))                        # layout, checked on the GPU side
+    again = ops.split_pad(full, S, 0, m)
+    for a, x, s in zip(again, shards, S):
+        assert torch.equal(a[:s], x)
+    # reduce-scatter layout: 8 virtual ranks each hold a full [total, 4096] tensor
+    fulls = [torch.randn(total, 4096, generator=g).bfloat16().to(cuda) for _ in range(8)]
+    off = 0
+    acc = torch.zeros(total, 4096, dtype=torch.float32, device=cuda)
+    for f in fulls:
+        acc += f.float()                                                        # same rank order, float32
+    for r, s in enumerate(S):
+        out = ops.ragged_reduce(fulls, 0, off, s)
+        assert torch.equal(out, acc[off:off + s].bfloat16())
+        off += s
+
+
+def test_bad_arguments_are_refused(cuda):
+    from hap_amd._lib import HapmiError
+    x = torch.zeros(4, 8, device=cuda)
+    with pytest.raises(HapmiError):
+        ops.slice_rows(x, 0, 3, 2)
+    with pytest.raises(HapmiError):
+        ops.pad_rows(x, 0, 3)
