@@ -58,7 +58,23 @@ def _compare(model, ratios, B, x, y, dtype, ranks, opt, **kw):
                 torch.testing.assert_close(g, ref, rtol=tol, atol=tol * ref.abs().max().item())
         ref_params = dict(run.programs[r].named_parameters())
         for n, p in params.items():
-            assert rel_err(p, ref_params[n].detach()) < tol, (r, n)
+            new_ref = ref_params[n].detach()
+            if opt["kind"] == "sgd":
+                assert rel_err(p, new_ref) < tol, (r, n)
+                continue
+            # Adam's first step is -lr * sign(g): where the true gradient is zero up to rounding (the key bias
+            # of softmax attention, dropped experts) its sign is noise on both sides.  So (a) the update must be
+            # torch.optim.Adam's on the GPU's own gradients, and (b) it must agree with the oracle's wherever
+            # the oracle's gradient is clearly non-zero.
+            old = dict(ex_initial[r])[n]
+            twin = old.clone().requires_grad_(True)
+            twin.grad = grads[n].clone()
+            torch.optim.Adam([twin], lr=opt["lr"]).step()
+            torch.testing.assert_close(p, twin.detach(), rtol=1e-5, atol=1e-8)
+            g_ref = ref_grads[r][n].float()
+            clear = g_ref.abs() > 1e-2 * g_ref.abs().max()
+            if clear.any():
+                assert rel_err((p - old)[clear], (new_ref - old)[clear]) < max(tol, 1e-3), (r, n)
     return run
 
 
