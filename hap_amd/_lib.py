@@ -31,6 +31,7 @@ class GemmArgs(ctypes.Structure):
         ("strideA1", ctypes.c_int64), ("strideA2", ctypes.c_int64),
         ("strideB1", ctypes.c_int64), ("strideB2", ctypes.c_int64),
         ("strideC1", ctypes.c_int64), ("strideC2", ctypes.c_int64),
+        ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_int64),
     ]
 
 

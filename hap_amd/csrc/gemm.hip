@@ -1,16 +1,18 @@
 // MFMA GEMM for gfx950: C = alpha * op(A) * op(B) (+ bias) (act) (+ C), float32 accumulation.
 //
-// One kernel template serves bf16 (v_mfma_f32_32x32x16_bf16) and float32
-// (v_mfma_f32_32x32x2_f32) inputs.  Both operands are staged in LDS as
-// [row][k] with k contiguous, so the register fragment of either type is one
-// 16-byte LDS read; an operand whose reduction dimension is the slow one in
-// memory (dgrad's weight, both operands of wgrad) is transposed in registers on
-// its way into LDS.  Ragged M / N / K are handled by guarded edge loads and
-// stores; the interior of every tile runs unguarded 16-byte accesses.
+// One kernel template serves bf16 (v_mfma_f32_32x32x16_bf16) and float32 (v_mfma_f32_32x32x2_f32) inputs.
+// Both operands are staged in LDS as [row][k] with 128 bytes of k per row, so the register fragment of
+// either type is one 16-byte LDS read.  Rows are not padded; the eight 16-byte chunks of a row are
+// XOR-swizzled with (row ^ row >> 3) & 7, which makes the fragment reads, the row-wise tile stores and the
+// transposing tile stores spread over all banks.  An operand whose reduction dimension is the slow one in
+// memory (dgrad's weight, both operands of wgrad) is transposed in registers on its way into LDS.
+// Ragged M / N / K are handled by guarded edge loads and stores; the interior of every tile runs unguarded
+// 16-byte accesses.  Small outputs with a long reduction (wgrad) are split along K over blockIdx.y into
+// a caller-provided float32 workspace and summed in split order by a second kernel (deterministic).
 //
-// The MFMA "A" operand is fed from op(B) rows (n) and the "B" operand from op(A)
-// rows (m): each lane then holds 4 consecutive n of one m in its accumulators
-// and the epilogue issues 8/16-byte stores along the contiguous dimension of C.
+// The MFMA "A" operand is fed from op(B) rows (n) and the "B" operand from op(A) rows (m): each lane then
+// holds 4 consecutive n of one m in its accumulators and the epilogue issues 8/16-byte stores along the
+// contiguous dimension of C.
 #include "common.h"
 #include <vector>
 #include <mutex>
@@ -19,13 +21,11 @@ namespace {
 
 template <typename TI> struct Mma;
 template <> struct Mma<bf16_t> {
-    static constexpr int EPV = 8;
     __device__ __forceinline__ static void run(f32x16 &acc, const Vec16<bf16_t> &a, const Vec16<bf16_t> &b) {
         acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, b.v, acc, 0, 0, 0);
     }
 };
 template <> struct Mma<float> {
-    static constexpr int EPV = 4;
     __device__ __forceinline__ static void run(f32x16 &acc, const Vec16<float> &a, const Vec16<float> &b) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.v[i], b.v[i], acc, 0, 0, 0);
@@ -43,6 +43,9 @@ struct GemmParams {
     float alpha;
     int accumulate, act;
     int tiles_m, tiles_n;
+    int splits, ktiles_per_split;
+    float *ws;                 // split-K workspace [splits][M][ws_ld] (float32)
+    int64_t ws_ld;
 };
 
 __device__ __forceinline__ float apply_act(float v, int act) {
@@ -51,21 +54,23 @@ __device__ __forceinline__ float apply_act(float v, int act) {
     return v;
 }
 
+constexpr int ROW_BYTES = 128;                       // k bytes per LDS row
+__device__ __forceinline__ int swz(int row) { return (row ^ (row >> 3)) & 7; }
+
 // Loads one operand tile [ROWS][BK] (row = m or n index, k = reduction index) from global memory into
-// registers.  KMAJOR: memory is [row][k] (k contiguous); otherwise memory is [k][row] (row contiguous).
-template <typename TI, int ROWS, int BK, int THREADS, bool KMAJOR> struct TileLoader {
+// registers and stores it into the swizzled LDS tile.  KMAJOR: memory is [row][k] (k contiguous);
+// otherwise memory is [k][row] (row contiguous) and 4(k) x EPV(row) register blocks are transposed.
+template <typename TI, int ROWS, int THREADS, bool KMAJOR> struct TileLoader {
     static constexpr int EPV = 16 / sizeof(TI);
-    // KMAJOR: vectors along k; thread -> (row, kvec)
-    static constexpr int KV = BK / EPV;                         // vectors per row
+    static constexpr int BK = ROW_BYTES / sizeof(TI);
+    static constexpr int KV = 8;                                  // 16-byte chunks per row
     static constexpr int ROWS_PER_PASS = THREADS / KV;
     static constexpr int PASSES_K = ROWS / ROWS_PER_PASS;
-    // !KMAJOR: 4(k) x EPV(row) blocks; thread -> (kgroup, rowvec)
-    static constexpr int RV = ROWS / EPV;                       // row-vectors per k line
+    static constexpr int RV = ROWS / EPV;                         // row-vectors per k line
     static constexpr int BLOCKS = (BK / 4) * RV;
-    static constexpr int PASSES_T = BLOCKS / THREADS;
+    static constexpr int PASSES_T = (BLOCKS + THREADS - 1) / THREADS;
     static constexpr int NV = KMAJOR ? PASSES_K : PASSES_T * 4;
-    static_assert(KMAJOR ? (ROWS % ROWS_PER_PASS == 0 && PASSES_K >= 1) : (BLOCKS % THREADS == 0 && PASSES_T >= 1),
-                  "tile does not divide over the block");
+    static_assert(!KMAJOR || (ROWS % ROWS_PER_PASS == 0 && PASSES_K >= 1), "tile does not divide over the block");
 
     Vec16<TI> v[NV];
 
@@ -94,6 +99,7 @@ template <typename TI, int ROWS, int BK, int THREADS, bool KMAJOR> struct TileLo
 #pragma unroll
             for (int p = 0; p < PASSES_T; ++p) {
                 const int blk = t + p * THREADS;
+                if (BLOCKS % THREADS != 0 && blk >= BLOCKS) break;
                 const int rv = blk % RV, kg = blk / RV;
                 const int64_t rr = (int64_t)rv * EPV;
 #pragma unroll
@@ -108,26 +114,32 @@ template <typename TI, int ROWS, int BK, int THREADS, bool KMAJOR> struct TileLo
         }
     }
 
-    // LDS tile is [ROWS][LDK] elements, k contiguous
-    template <int LDK> __device__ __forceinline__ void store(TI *lds) const {
+    __device__ __forceinline__ void store(char *lds) const {
         const int t = threadIdx.x;
         if (KMAJOR) {
             const int kv = t % KV, r0 = t / KV;
 #pragma unroll
-            for (int p = 0; p < PASSES_K; ++p)
-                *(Vec16<TI> *)(lds + (r0 + p * ROWS_PER_PASS) * LDK + kv * EPV) = v[p];
+            for (int p = 0; p < PASSES_K; ++p) {
+                const int row = r0 + p * ROWS_PER_PASS;
+                *(Vec16<TI> *)(lds + row * ROW_BYTES + ((kv ^ swz(row)) << 4)) = v[p];
+            }
         } else {
             typedef TI quad_t __attribute__((ext_vector_type(4)));
+            constexpr int QB = 4 * sizeof(TI);                    // bytes of 4 consecutive k: 8 (bf16) or 16 (f32)
 #pragma unroll
             for (int p = 0; p < PASSES_T; ++p) {
                 const int blk = t + p * THREADS;
+                if (BLOCKS % THREADS != 0 && blk >= BLOCKS) break;
                 const int rv = blk % RV, kg = blk / RV;
+                const int kbyte = kg * QB;                        // logical byte offset inside the row
+                const int chunk = kbyte >> 4, within = kbyte & 15;
 #pragma unroll
                 for (int e = 0; e < EPV; ++e) {
                     quad_t q4;
 #pragma unroll
                     for (int q = 0; q < 4; ++q) q4[q] = v[p * 4 + q].v[e];
-                    *(quad_t *)(lds + (rv * EPV + e) * LDK + kg * 4) = q4;
+                    const int row = rv * EPV + e;
+                    *(quad_t *)(lds + row * ROW_BYTES + ((chunk ^ swz(row)) << 4) + within) = q4;
                 }
             }
         }
@@ -138,15 +150,15 @@ template <typename TI, typename TO, int BM, int BN, int WAVES_M, int WAVES_N, bo
 __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_kernel(GemmParams p) {
     constexpr int THREADS = WAVES_M * WAVES_N * 64;
     constexpr int EPV = 16 / sizeof(TI);
-    constexpr int BK = 128 / sizeof(TI);              // 128 bytes of k per LDS row
-    constexpr int LDK = BK + EPV;                     // +16 bytes: conflict-free 16-byte fragment reads
+    constexpr int BK = ROW_BYTES / sizeof(TI);
     constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
     constexpr int TM = WTM / 32, TN = WTN / 32;
-    constexpr int KSTEPS = BK / (2 * EPV);            // fragment pairs (one per lane half) per tile
+    constexpr int KSTEPS = 4;                                     // 32 bytes of k per lane-half pair
+    constexpr int A_BYTES = BM * ROW_BYTES, B_BYTES = BN * ROW_BYTES;
 
     extern __shared__ __attribute__((aligned(16))) char smem[];
-    TI *As = (TI *)smem;                              // [2][BM][LDK]
-    TI *Bs = As + 2 * BM * LDK;                       // [2][BN][LDK]
+    char *As = smem;                                              // [2][BM][128 B]
+    char *Bs = smem + 2 * A_BYTES;                                // [2][BN][128 B]
 
     // tile mapping: blocks go round-robin over the 8 XCDs; give each XCD a contiguous range of tiles and
     // walk it in columns of 8 m-tiles so that concurrently running tiles share A rows / B columns in L2
@@ -169,17 +181,35 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_kernel(GemmParams 
     const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
     const int64_t m_left = p.M - m0, n_left = p.N - n0;
 
+    const int nk_total = (int)((p.K + BK - 1) / BK);
+    const int kt0 = (int)blockIdx.y * p.ktiles_per_split;
+    const int kt1 = (kt0 + p.ktiles_per_split) < nk_total ? (kt0 + p.ktiles_per_split) : nk_total;
+    if (kt0 >= kt1) return;                                       // uniform for the whole block
+
     const TI *a_base = A_KMAJOR ? A + m0 * p.lda : A + m0;     // element (m0, k=0)
     const TI *b_base = B_KMAJOR ? B + n0 * p.ldb : B + n0;
     const int64_t a_kstep = A_KMAJOR ? (int64_t)BK : (int64_t)BK * p.lda;
     const int64_t b_kstep = B_KMAJOR ? (int64_t)BK : (int64_t)BK * p.ldb;
 
-    TileLoader<TI, BM, BK, THREADS, A_KMAJOR> la;
-    TileLoader<TI, BN, BK, THREADS, B_KMAJOR> lb;
+    TileLoader<TI, BM, THREADS, A_KMAJOR> la;
+    TileLoader<TI, BN, THREADS, B_KMAJOR> lb;
 
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int wm = (wave % WAVES_M) * WTM, wn = (wave / WAVES_M) * WTN;
-    const int frow = lane & 31, fk = (lane >> 5) * EPV;
+    const int frow = lane & 31, fh = lane >> 5;
+
+    // byte offset of this lane's fragment for k-step 0 inside a tile; k-step s is at offset ^ (s << 5)
+    int a_off[TM], b_off[TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+        const int row = wm + i * 32 + frow;
+        a_off[i] = row * ROW_BYTES + ((fh ^ swz(row)) << 4);
+    }
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        const int row = wn + j * 32 + frow;
+        b_off[j] = row * ROW_BYTES + ((fh ^ swz(row)) << 4);
+    }
 
     f32x16 acc[TM][TN];
 #pragma unroll
@@ -189,42 +219,43 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_kernel(GemmParams 
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    const int nk = (int)((p.K + BK - 1) / BK);
-    la.load(a_base, p.lda, m_left, p.K);
-    lb.load(b_base, p.ldb, n_left, p.K);
-    la.template store<LDK>(As);
-    lb.template store<LDK>(Bs);
+    la.load(a_base + (int64_t)kt0 * a_kstep, p.lda, m_left, p.K - (int64_t)kt0 * BK);
+    lb.load(b_base + (int64_t)kt0 * b_kstep, p.ldb, n_left, p.K - (int64_t)kt0 * BK);
+    la.store(As);
+    lb.store(Bs);
     __syncthreads();
 
-    for (int kt = 0; kt < nk; ++kt) {
-        const int cur = kt & 1;
-        if (kt + 1 < nk) {
+    for (int kt = kt0; kt < kt1; ++kt) {
+        const int cur = (kt - kt0) & 1;
+        if (kt + 1 < kt1) {
             const int64_t k_left = p.K - (int64_t)(kt + 1) * BK;
             la.load(a_base + (int64_t)(kt + 1) * a_kstep, p.lda, m_left, k_left);
             lb.load(b_base + (int64_t)(kt + 1) * b_kstep, p.ldb, n_left, k_left);
         }
-        const TI *as = As + cur * BM * LDK + wm * LDK;
-        const TI *bs = Bs + cur * BN * LDK + wn * LDK;
+        const char *as = As + cur * A_BYTES;
+        const char *bs = Bs + cur * B_BYTES;
 #pragma unroll
         for (int ks = 0; ks < KSTEPS; ++ks) {
             Vec16<TI> fa[TM], fb[TN];
 #pragma unroll
-            for (int i = 0; i < TM; ++i) fa[i] = *(const Vec16<TI> *)(as + (i * 32 + frow) * LDK + ks * 2 * EPV + fk);
+            for (int i = 0; i < TM; ++i) fa[i] = *(const Vec16<TI> *)(as + (a_off[i] ^ (ks << 5)));
 #pragma unroll
-            for (int j = 0; j < TN; ++j) fb[j] = *(const Vec16<TI> *)(bs + (j * 32 + frow) * LDK + ks * 2 * EPV + fk);
+            for (int j = 0; j < TN; ++j) fb[j] = *(const Vec16<TI> *)(bs + (b_off[j] ^ (ks << 5)));
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
                 for (int j = 0; j < TN; ++j) Mma<TI>::run(acc[i][j], fb[j], fa[i]);
         }
-        if (kt + 1 < nk) {
-            la.template store<LDK>(As + (cur ^ 1) * BM * LDK);
-            lb.template store<LDK>(Bs + (cur ^ 1) * BN * LDK);
+        if (kt + 1 < kt1) {
+            la.store(As + (cur ^ 1) * A_BYTES);
+            lb.store(Bs + (cur ^ 1) * B_BYTES);
         }
         __syncthreads();
     }
 
     // epilogue: acc[i][j][r] is C[m, n] with m = wm + i*32 + lane%32, n = wn + j*32 + (r/4)*8 + (lane/32)*4 + r%4
+    const bool split = p.splits > 1;
+    const bool lead = blockIdx.y == 0;                            // the split that adds the bias
     const int64_t mrow_base = m0 + wm + (lane & 31);
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
@@ -241,10 +272,18 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_kernel(GemmParams 
                 for (int e = 0; e < 4; ++e) v[e] = acc[i][j][q * 4 + e] * p.alpha;
                 TO *dst = C + m * p.ldc + n;
                 const bool full = (n + 4 <= p.N);
-                if (p.bias) {
+                if (p.bias && lead) {
 #pragma unroll
                     for (int e = 0; e < 4; ++e)
                         if (full || n + e < p.N) v[e] += p.bias[n + e];
+                }
+                if (split) {
+                    // partial sums of this k-range go to the workspace [split][M][Npad]; a second kernel
+                    // adds them up in split order and applies bias / activation / accumulation
+                    float *w = p.ws + ((int64_t)blockIdx.y * p.M + m) * p.ws_ld + n;
+                    f32x4 o = {v[0], v[1], v[2], v[3]};
+                    *(f32x4 *)w = o;                              // ws_ld is a multiple of 4 and >= N rounded up
+                    continue;
                 }
                 if (p.act != HAPMI_ACT_NONE) {
 #pragma unroll
@@ -276,17 +315,21 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_kernel(GemmParams 
     }
 }
 
-template <typename TI, int BM, int BN> constexpr size_t gemm_smem() {
-    constexpr int EPV = 16 / sizeof(TI);
-    constexpr int BK = 128 / sizeof(TI);
-    return (size_t)2 * (BM + BN) * (BK + EPV) * sizeof(TI);
-}
+// ---- tile configurations ------------------------------------------------------------------------
+struct TileCfg {
+    int bm, bn, wm, wn;
+};
+constexpr TileCfg kCfg[] = {{128, 128, 2, 2}, {256, 256, 2, 4}};
+constexpr int kNumCfg = 2;
+constexpr int kNumCU = 256;
+int g_force_cfg = -1;
+int g_force_splits = 0;
 
 // ---- instrumentation: HIP events around every launch --------------------------------------------
 struct ProfState {
     std::mutex mu;
     bool on = false;
-    std::vector<hipEvent_t> pool;          // events not in use
+    std::vector<hipEvent_t> pool;
     std::vector<std::pair<hipEvent_t, hipEvent_t>> pending;
     double flops = 0.0;
     int64_t launches = 0;
@@ -309,8 +352,8 @@ int launch_cfg(const GemmParams &p, int transA, int transB, int64_t batch, hipSt
     GemmParams q = p;
     q.tiles_m = (int)hapmi_cdiv(p.M, BM);
     q.tiles_n = (int)hapmi_cdiv(p.N, BN);
-    dim3 grid((unsigned)(q.tiles_m * q.tiles_n), 1, (unsigned)batch), block(WM * WN * 64);
-    const size_t smem = gemm_smem<TI, BM, BN>();
+    dim3 grid((unsigned)(q.tiles_m * q.tiles_n), (unsigned)q.splits, (unsigned)batch), block(WM * WN * 64);
+    const size_t smem = (size_t)2 * (BM + BN) * ROW_BYTES;
 #define HAPMI_GEMM_LAUNCH(AK, BK_)                                                                        \
     do {                                                                                                  \
         auto kern = gemm_kernel<TI, TO, BM, BN, WM, WN, AK, BK_>;                                         \
@@ -333,12 +376,83 @@ int launch_cfg(const GemmParams &p, int transA, int transB, int64_t batch, hipSt
     return HAPMI_OK;
 }
 
+int choose_cfg(int64_t M, int64_t N, int64_t batch, bool wide) {
+    if (g_force_cfg >= 0 && g_force_cfg < kNumCfg) return (g_force_cfg == 1 && !wide) ? 0 : g_force_cfg;
+    if (!wide) return 0;
+    // 256x256 tiles run one per CU: take them only when the tile count fills whole rounds of the 256 CUs
+    const int64_t t = hapmi_cdiv(M, 256) * hapmi_cdiv(N, 256) * batch;
+    const int64_t rounds = hapmi_cdiv(t, kNumCU);
+    const double fill = (double)t / (double)(rounds * kNumCU);
+    const double edge = ((double)M * (double)N) / ((double)hapmi_cdiv(M, 256) * 256.0 * (double)hapmi_cdiv(N, 256) * 256.0);
+    return (fill * edge >= 0.88) ? 1 : 0;
+}
+
+// Small outputs with a long reduction do not fill the chip: split K over blockIdx.y.
+int choose_splits(const TileCfg &c, int64_t M, int64_t N, int64_t K, int64_t batch, int bk, int64_t max_splits) {
+    if (max_splits < 2 || batch != 1) return 1;
+    const int64_t nk = hapmi_cdiv(K, bk);
+    int64_t s;
+    if (g_force_splits > 0) {
+        s = g_force_splits;
+    } else {
+        const int64_t tiles = hapmi_cdiv(M, c.bm) * hapmi_cdiv(N, c.bn);
+        const int64_t slots = (c.bm == 128) ? 2 * kNumCU : kNumCU;      // co-resident blocks
+        if (tiles * 4 > slots * 3 || nk < 16) return 1;
+        s = slots / tiles;
+        if (s > nk / 8) s = nk / 8;
+    }
+    if (s > max_splits) s = max_splits;
+    if (s > nk) s = nk;
+    return (int)(s < 1 ? 1 : s);
+}
+
+template <typename TO>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *ws, TO *C, int64_t M, int64_t N, int64_t ws_ld,
+                                                          int64_t ldc, int splits, int accumulate, int act) {
+    const int64_t groups = ws_ld / 4, total = M * groups;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+        const int64_t m = i / groups, n = (i - m * groups) * 4;
+        if (n >= N) continue;
+        f32x4 acc = *(const f32x4 *)(ws + m * ws_ld + n);
+        for (int s = 1; s < splits; ++s) {
+            const f32x4 v = *(const f32x4 *)(ws + ((int64_t)s * M + m) * ws_ld + n);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[e] += v[e];
+        }
+        TO *dst = C + m * ldc + n;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            if (n + e < N) {
+                float x = apply_act(acc[e], act);
+                if (accumulate) x += (float)dst[e];
+                dst[e] = (TO)x;
+            }
+        }
+    }
+}
+
 template <typename TI, typename TO>
-int launch_typed(const GemmParams &p, int transA, int transB, int64_t batch, hipStream_t st) {
-    // big tiles when they still give every CU at least ~2 tiles of work, else smaller ones
-    const int64_t t256 = hapmi_cdiv(p.M, 256) * hapmi_cdiv(p.N, 128) * batch;
-    if (t256 >= 256 * 2 && p.M >= 256 && p.N >= 128) return launch_cfg<TI, TO, 256, 128, 2, 2>(p, transA, transB, batch, st);
-    return launch_cfg<TI, TO, 128, 128, 2, 2>(p, transA, transB, batch, st);
+int launch_typed(GemmParams &p, int transA, int transB, int64_t batch, hipStream_t st, bool wide, void *workspace,
+                 int64_t workspace_bytes) {
+    const int bk = ROW_BYTES / (int)sizeof(TI);
+    const int c = choose_cfg(p.M, p.N, batch, wide && sizeof(TI) == 2);
+    const int64_t nk = hapmi_cdiv(p.K, bk);
+    p.ws_ld = (p.N + 3) / 4 * 4;
+    const int64_t per_split = p.M * p.ws_ld * 4;
+    const int64_t max_splits = (workspace && ((uintptr_t)workspace % 16) == 0 && per_split > 0) ? workspace_bytes / per_split : 0;
+    p.splits = choose_splits(kCfg[c], p.M, p.N, p.K, batch, bk, max_splits);
+    p.ktiles_per_split = (int)hapmi_cdiv(nk, p.splits);
+    p.splits = (int)hapmi_cdiv(nk, p.ktiles_per_split);
+    p.ws = (float *)workspace;
+    int rc;
+    if (c == 1) rc = launch_cfg<bf16_t, TO, 256, 256, 2, 4>(p, transA, transB, batch, st);
+    else rc = launch_cfg<TI, TO, 128, 128, 2, 2>(p, transA, transB, batch, st);
+    if (rc || p.splits <= 1) return rc;
+    int64_t gx = hapmi_cdiv(p.M * (p.ws_ld / 4), 256);
+    if (gx > 256 * 16) gx = 256 * 16;
+    hipLaunchKernelGGL((splitk_reduce_kernel<TO>), dim3((unsigned)gx), dim3(256), 0, st, (const float *)p.ws, (TO *)p.C,
+                       p.M, p.N, p.ws_ld, p.ldc, p.splits, p.accumulate, p.act);
+    return HAPMI_OK;
 }
 
 }  // namespace
@@ -377,6 +491,10 @@ extern "C" int hapmi_gemm(const hapmi_gemm_args *a, hapmi_stream_t stream) {
     p.sC1 = a->strideC1; p.sC2 = a->strideC2;
     p.alpha = a->alpha; p.accumulate = a->accumulate; p.act = a->act;
     p.tiles_m = p.tiles_n = 0;
+    p.splits = 1;
+    p.ktiles_per_split = 1;
+    p.ws = nullptr;
+    p.ws_ld = 0;
 
     hipStream_t st = (hipStream_t)stream;
     hipEvent_t e0 = nullptr, e1 = nullptr;
@@ -390,14 +508,14 @@ extern "C" int hapmi_gemm(const hapmi_gemm_args *a, hapmi_stream_t stream) {
             prof = e0 && e1;
         }
     }
-    if (prof) hipEventRecord(e0, st);
+    if (prof) (void)hipEventRecord(e0, st);
     int rc;
-    if (a->in_dtype == HAPMI_BF16 && a->out_dtype == HAPMI_BF16) rc = launch_typed<bf16_t, bf16_t>(p, a->transA, a->transB, batch, st);
-    else if (a->in_dtype == HAPMI_BF16) rc = launch_typed<bf16_t, float>(p, a->transA, a->transB, batch, st);
-    else if (a->out_dtype == HAPMI_F32) rc = launch_typed<float, float>(p, a->transA, a->transB, batch, st);
-    else rc = launch_typed<float, bf16_t>(p, a->transA, a->transB, batch, st);
+    if (a->in_dtype == HAPMI_BF16 && a->out_dtype == HAPMI_BF16) rc = launch_typed<bf16_t, bf16_t>(p, a->transA, a->transB, batch, st, true, a->workspace, a->workspace_bytes);
+    else if (a->in_dtype == HAPMI_BF16) rc = launch_typed<bf16_t, float>(p, a->transA, a->transB, batch, st, true, a->workspace, a->workspace_bytes);
+    else if (a->out_dtype == HAPMI_F32) rc = launch_typed<float, float>(p, a->transA, a->transB, batch, st, false, a->workspace, a->workspace_bytes);
+    else rc = launch_typed<float, bf16_t>(p, a->transA, a->transB, batch, st, false, a->workspace, a->workspace_bytes);
     if (prof) {
-        hipEventRecord(e1, st);
+        (void)hipEventRecord(e1, st);
         std::lock_guard<std::mutex> lk(g_prof.mu);
         g_prof.pending.emplace_back(e0, e1);
         g_prof.flops += 2.0 * (double)a->M * (double)a->N * (double)a->K * (double)batch;
@@ -405,6 +523,12 @@ extern "C" int hapmi_gemm(const hapmi_gemm_args *a, hapmi_stream_t stream) {
     }
     if (rc) return rc;
     HAPMI_CHECK_LAUNCH("gemm");
+    return HAPMI_OK;
+}
+
+extern "C" int hapmi_gemm_tuning(int tile_config, int k_splits) {
+    g_force_cfg = tile_config;
+    g_force_splits = k_splits;
     return HAPMI_OK;
 }
 

@@ -86,6 +86,8 @@ class ShardExecutor:
                                 for a in example_inputs]
         self.rank_hint, self.world_hint = rank, world_size
         self._param_reduce: List[Callable[[], None]] = []
+        self.gemm_workspace = torch.empty(64 << 20, dtype=torch.float32, device=self.dev)   # 256 MiB of split-K scratch
+        ops.set_gemm_workspace(self.gemm_workspace)
         self._prepare_params()
         self._compile()
         self._finish_param_reduce()

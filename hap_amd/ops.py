@@ -228,11 +228,21 @@ def ragged_reduce(contribs: Sequence[torch.Tensor], dim: int, offset: int, lengt
 # GEMM
 # ---------------------------------------------------------------------------
 
+_gemm_ws: Optional[torch.Tensor] = None
+
+
+def set_gemm_workspace(t: Optional[torch.Tensor]) -> None:
+    """Scratch buffer for split-K partial sums, shared by all GEMM calls that follow (one stream)."""
+    global _gemm_ws
+    _gemm_ws = t
+
+
 def gemm(A: torch.Tensor, B: torch.Tensor, C: torch.Tensor, M: int, N: int, K: int, *, transA=False, transB=False,
          lda=None, ldb=None, ldc=None, bias: Optional[torch.Tensor] = None, accumulate=False, act=None, alpha=1.0,
          batch1=1, batch2=1, strideA=(0, 0), strideB=(0, 0), strideC=(0, 0),
-         offA=0, offB=0, offC=0):
-    """C = alpha * op(A) @ op(B) (+bias)(act)(+C).  Offsets and strides are in elements."""
+         offA=0, offB=0, offC=0, workspace: Optional[torch.Tensor] = None):
+    """C = alpha * op(A) @ op(B) (+bias)(act)(+C).  Offsets and strides are in elements.  ``workspace`` (or
+    the buffer installed with ``set_gemm_workspace``) lets the library split a long reduction over K."""
     _dev(A, B, C, bias)
     if A.dtype != B.dtype:
         raise TypeError("gemm operands must share a dtype")
@@ -254,6 +264,11 @@ def gemm(A: torch.Tensor, B: torch.Tensor, C: torch.Tensor, M: int, N: int, K: i
     a.strideA1, a.strideA2 = strideA
     a.strideB1, a.strideB2 = strideB
     a.strideC1, a.strideC2 = strideC
+    ws = workspace if workspace is not None else _gemm_ws
+    if ws is not None and ws.is_cuda and ws.device == A.device:
+        a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel() * ws.element_size()
+    else:
+        a.workspace, a.workspace_bytes = 0, 0
     zb = lambda st: (batch1 - 1) * st[0] + (batch2 - 1) * st[1]
     _need(A, _span(K if transA else M, M if transA else K, a.lda) + zb(strideA), "gemm A", offA)
     _need(B, _span(N if transB else K, K if transB else N, a.ldb) + zb(strideB), "gemm B", offB)

@@ -115,8 +115,14 @@ typedef struct {
     float alpha;                 /* result scaled before bias */
     int64_t batch1, batch2;      /* >= 1 */
     int64_t strideA1, strideA2, strideB1, strideB2, strideC1, strideC2;
+    void *workspace;             /* optional float32 scratch for split-K (16-byte aligned) or NULL;   */
+    int64_t workspace_bytes;     /* a split needs M * roundup(N, 4) * 4 bytes; unused when batch > 1 */
 } hapmi_gemm_args;
 int hapmi_gemm(const hapmi_gemm_args *args_host, hapmi_stream_t stream);
+
+/* Tuning hook for measurements: force tile configuration `tile_config` (0: 128x128, 1: 256x128,
+ * 2: 256x256 / 4 waves, 3: 256x256 / 8 waves; -1 = automatic) and `k_splits` (0 = automatic). */
+int hapmi_gemm_tuning(int tile_config, int k_splits);
 
 /* ---- row-wise kernels ------------------------------------------------- */
 /* operator.add + F.layer_norm(x, (width,)) without affine, eps (hap.rs:1515, 1653):

@@ -244,3 +244,29 @@ def test_optimizers_match_torch(cuda):
     ops.clip_coef(ss, 0.5, coef)
     want = min(1.0, 0.5 / (grads[0].norm().item() + 1e-6))
     assert abs(coef.item() - want) < 1e-6 * want
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("cfg", [0, 1])
+def test_gemm_split_k_and_tile_configs(cuda, dtype, cfg):
+    """Forced tile configuration and K splits (workspace partial sums + ordered reduction) give the same product."""
+    from hap_amd._lib import lib
+    g = torch.Generator().manual_seed(5)
+    M, N, K = 200, 136, 2048
+    A = torch.randn(K, M, generator=g).to(dtype)
+    B = torch.randn(K, N, generator=g).to(dtype)
+    bias = torch.randn(N, generator=g)
+    C0 = torch.randn(M, N, generator=g)
+    ws = torch.empty(8 * M * N, dtype=torch.float32, device=cuda)
+    want = A.double().t() @ B.double() + bias.double()
+    try:
+        for splits in (1, 3, 8):
+            lib().hapmi_gemm_tuning(cfg, splits)
+            C = C0.clone().to(cuda)
+            ops.gemm(A.to(cuda), B.to(cuda), C, M, N, K, transA=True, bias=bias.to(cuda), accumulate=True, workspace=ws)
+            close(C, want + C0.double(), dtype, scale=2.0)
+            out = torch.empty(M, N, dtype=dtype, device=cuda)
+            ops.gemm(A.to(cuda), B.to(cuda), out, M, N, K, transA=True, bias=bias.to(cuda), act="relu", workspace=ws)
+            close(out, torch.relu(want), dtype, scale=2.0)
+    finally:
+        lib().hapmi_gemm_tuning(-1, 0)
