@@ -1,0 +1,436 @@
+// Fused scaled-dot-product attention for bf16, head_dim 64, on the packed projection qkv[b, S, 3*H*64].
+//
+// Everything is computed "transposed" so that the softmax dimension lives inside a lane:
+//   forward / dQ : S^T[kv][q] = K Q^T   -> each lane owns one query column (lane % 32) and 32 kv rows per tile,
+//                  so row max / row sum are per-lane loops plus one exchange with lane ^ 32;
+//   dK / dV      : S[q][kv]   = Q K^T   -> each lane owns one kv column.
+// The probability tile leaves the MFMA in accumulator layout (lane = column, registers = rows); it is fed to
+// the next MFMA as its B operand straight from registers by choosing the k-order (slot (h, j) of step s is row
+// 16 s + 8 (j / 4) + 4 h + j % 4), and the matching A operand is read from LDS in that same order.
+// K / V / Q / dO tiles sit in LDS in the swizzled [row][128 B] layout of tile.h; the transposed copies
+// (V^T, K^T, Q^T, dO^T) are produced by the transposing loader.
+#include "common.h"
+#include "tile.h"
+
+namespace {
+
+constexpr int HD = 64;                 // head dimension (bf16: one 128-byte LDS row)
+constexpr int TILE = 64;               // rows of the streamed operand per iteration
+constexpr int AT_THREADS = 256;        // 4 waves, 32 rows of the stationary operand each
+constexpr int TILE_BYTES = TILE * ROW_BYTES;
+
+typedef Vec16<bf16_t> frag_t;
+
+// standard operand fragment of k-step s: k = 16 s + 8 h .. + 8 of `row`
+__device__ __forceinline__ frag_t frag_rowk(const char *tile, int row, int s, int h) {
+    return *(const frag_t *)(tile + row * ROW_BYTES + ((((s << 1) | h) ^ swz(row)) << 4));
+}
+// fragment in accumulator order: slots j < 4 -> k = 16 s + 4 h + j, slots j >= 4 -> k = 16 s + 8 + 4 h + (j - 4)
+__device__ __forceinline__ frag_t frag_perm(const char *tile, int row, int s, int h) {
+    const int sw = swz(row);
+    const char *base = tile + row * ROW_BYTES + (h << 3);
+    const bf16x4 lo = *(const bf16x4 *)(base + (((s << 1) ^ sw) << 4));
+    const bf16x4 hi = *(const bf16x4 *)(base + ((((s << 1) | 1) ^ sw) << 4));
+    frag_t f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        f.v[j] = lo[j];
+        f.v[4 + j] = hi[j];
+    }
+    return f;
+}
+// 8 rows (one k-step) of an accumulator tile as a B operand
+__device__ __forceinline__ frag_t acc_to_b(const f32x16 &a, int sp) {
+    frag_t f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) f.v[j] = (bf16_t)a[sp * 8 + j];
+    return f;
+}
+__device__ __forceinline__ f32x16 zero16() {
+    f32x16 z;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) z[r] = 0.f;
+    return z;
+}
+__device__ __forceinline__ f32x16 mma(const frag_t &a, const frag_t &b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, b.v, c, 0, 0, 0);
+}
+// row index inside a 32-row accumulator tile held in register r by a lane of half h
+__device__ __forceinline__ int acc_row(int r, int h) { return ((r >> 2) << 3) + (h << 2) + (r & 3); }
+
+__device__ __forceinline__ frag_t load_row_frag(const bf16_t *row_ptr, bool valid, int s, int h) {
+    frag_t f;
+    if (valid) f = *(const frag_t *)(row_ptr + 16 * s + 8 * h);
+    else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) f.v[j] = (bf16_t)0.f;
+    }
+    return f;
+}
+
+// ---------------------------------------------------------------------------------------------
+// forward
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(AT_THREADS) void attn_fwd_kernel(const bf16_t *qkv, const float *mask, bf16_t *out,
+                                                            float *lse, int S, int H, float scale) {
+    __shared__ __attribute__((aligned(16))) char Ks[TILE_BYTES];
+    __shared__ __attribute__((aligned(16))) char Vts[TILE_BYTES];
+    const int E = H * HD, ld = 3 * E;
+    const int b = blockIdx.y / H, hh = blockIdx.y % H;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, c = lane & 31, h = lane >> 5;
+    const int q = blockIdx.x * 128 + wave * 32 + c;
+    const bool qok = q < S;
+    const bf16_t *Q = qkv + (int64_t)b * S * ld + hh * HD;
+    const bf16_t *K = Q + E, *V = Q + 2 * E;
+
+    frag_t qf[4];
+#pragma unroll
+    for (int s = 0; s < 4; ++s) qf[s] = load_row_frag(Q + (int64_t)q * ld, qok, s, h);
+
+    f32x16 ot[2] = {zero16(), zero16()};
+    float m = -INFINITY, lsum = 0.f;
+    TileLoader<bf16_t, TILE, AT_THREADS, true> lk;
+    TileLoader<bf16_t, HD, AT_THREADS, false> lv;
+    const bool vec_mask = mask && ((S & 3) == 0);
+
+    for (int kv0 = 0; kv0 < S; kv0 += TILE) {
+        lk.load(K + (int64_t)kv0 * ld, ld, S - kv0, HD);
+        lv.load(V + (int64_t)kv0 * ld, ld, HD, S - kv0);
+        __syncthreads();                                   // every wave is done with the previous tiles
+        lk.store(Ks);
+        lv.store(Vts);
+        __syncthreads();
+
+        f32x16 st[2] = {zero16(), zero16()};
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int s = 0; s < 4; ++s) st[t] = mma(frag_rowk(Ks, t * 32 + c, s, h), qf[s], st[t]);
+
+        float mx = -INFINITY;
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int kv = kv0 + t * 32 + g * 8 + h * 4;
+                float mk[4] = {0.f, 0.f, 0.f, 0.f};
+                if (mask && qok) {
+                    if (vec_mask && kv + 4 <= S) {
+                        const f32x4 mv = *(const f32x4 *)(mask + (int64_t)q * S + kv);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) mk[e] = mv[e];
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            if (kv + e < S) mk[e] = mask[(int64_t)q * S + kv + e];
+                    }
+                }
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    float v = st[t][g * 4 + e] * scale + mk[e];
+                    if (kv + e >= S) v = -INFINITY;
+                    st[t][g * 4 + e] = v;
+                    mx = fmaxf(mx, v);
+                }
+            }
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float m_new = fmaxf(m, mx);
+        const float msub = (m_new == -INFINITY) ? 0.f : m_new;
+        const float alpha = (m_new == -INFINITY) ? 1.f : __expf(m - m_new);
+        float psum = 0.f;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float p = __expf(st[t][r] - msub);
+                st[t][r] = p;
+                psum += p;
+            }
+        lsum = lsum * alpha + psum;
+        m = m_new;
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) ot[u][r] *= alpha;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            const frag_t pb = acc_to_b(st[s >> 1], s & 1);
+#pragma unroll
+            for (int u = 0; u < 2; ++u) ot[u] = mma(frag_perm(Vts, u * 32 + c, s, h), pb, ot[u]);
+        }
+    }
+    const float l = lsum + __shfl_xor(lsum, 32, 64);
+    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    if (qok) {
+        bf16_t *orow = out + ((int64_t)b * S + q) * E + hh * HD;
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                bf16x4 o;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) o[e] = (bf16_t)(ot[u][g * 4 + e] * inv);
+                *(bf16x4 *)(orow + u * 32 + g * 8 + h * 4) = o;
+            }
+        if (h == 0) lse[((int64_t)b * H + hh) * S + q] = m + __logf(l);
+    }
+}
+
+// delta[b, h, q] = sum_d dO[b, q, h, d] * O[b, q, h, d]
+__global__ __launch_bounds__(256) void attn_delta_kernel(const bf16_t *out, const bf16_t *dout, float *delta, int64_t rows,
+                                                       int S, int H) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;        // (b, q, h)
+    if (i >= rows * H) return;
+    const int64_t row = i / H;
+    const int hh = (int)(i % H);
+    const frag_t *o = (const frag_t *)(out + row * H * HD + hh * HD);
+    const frag_t *d = (const frag_t *)(dout + row * H * HD + hh * HD);
+    float acc = 0.f;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        const frag_t a = o[k], g = d[k];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc += (float)a.v[e] * (float)g.v[e];
+    }
+    const int64_t bidx = row / S, q = row % S;
+    delta[(bidx * H + hh) * S + q] = acc;
+}
+
+// ---------------------------------------------------------------------------------------------
+// dQ: lanes own query columns, kv tiles are streamed
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(AT_THREADS) void attn_bwd_dq_kernel(const bf16_t *qkv, const bf16_t *dout, const float *lse,
+                                                               const float *delta, const float *mask, bf16_t *dqkv,
+                                                               int S, int H, float scale) {
+    __shared__ __attribute__((aligned(16))) char Ks[TILE_BYTES];
+    __shared__ __attribute__((aligned(16))) char Vs[TILE_BYTES];
+    __shared__ __attribute__((aligned(16))) char Kts[TILE_BYTES];
+    const int E = H * HD, ld = 3 * E;
+    const int b = blockIdx.y / H, hh = blockIdx.y % H;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, c = lane & 31, h = lane >> 5;
+    const int q = blockIdx.x * 128 + wave * 32 + c;
+    const bool qok = q < S;
+    const bf16_t *Q = qkv + (int64_t)b * S * ld + hh * HD;
+    const bf16_t *K = Q + E, *V = Q + 2 * E;
+    const bf16_t *dO = dout + (int64_t)b * S * E + hh * HD;
+
+    frag_t qf[4], dof[4];
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+        qf[s] = load_row_frag(Q + (int64_t)q * ld, qok, s, h);
+        dof[s] = load_row_frag(dO + (int64_t)q * E, qok, s, h);
+    }
+    const float lse_q = qok ? lse[((int64_t)b * H + hh) * S + q] : 0.f;
+    const float delta_q = qok ? delta[((int64_t)b * H + hh) * S + q] : 0.f;
+    f32x16 dqt[2] = {zero16(), zero16()};
+    TileLoader<bf16_t, TILE, AT_THREADS, true> lk, lv;
+    TileLoader<bf16_t, HD, AT_THREADS, false> lkt;
+    const bool vec_mask = mask && ((S & 3) == 0);
+
+    for (int kv0 = 0; kv0 < S; kv0 += TILE) {
+        lk.load(K + (int64_t)kv0 * ld, ld, S - kv0, HD);
+        lv.load(V + (int64_t)kv0 * ld, ld, S - kv0, HD);
+        lkt.load(K + (int64_t)kv0 * ld, ld, HD, S - kv0);
+        __syncthreads();
+        lk.store(Ks);
+        lv.store(Vs);
+        lkt.store(Kts);
+        __syncthreads();
+
+        f32x16 st[2] = {zero16(), zero16()}, dp[2] = {zero16(), zero16()};
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                st[t] = mma(frag_rowk(Ks, t * 32 + c, s, h), qf[s], st[t]);
+                dp[t] = mma(frag_rowk(Vs, t * 32 + c, s, h), dof[s], dp[t]);
+            }
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int kv = kv0 + t * 32 + g * 8 + h * 4;
+                float mk[4] = {0.f, 0.f, 0.f, 0.f};
+                if (mask && qok) {
+                    if (vec_mask && kv + 4 <= S) {
+                        const f32x4 mv = *(const f32x4 *)(mask + (int64_t)q * S + kv);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) mk[e] = mv[e];
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            if (kv + e < S) mk[e] = mask[(int64_t)q * S + kv + e];
+                    }
+                }
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int r = g * 4 + e;
+                    float p = (qok && kv + e < S) ? __expf(st[t][r] * scale + mk[e] - lse_q) : 0.f;
+                    dp[t][r] = p * (dp[t][r] - delta_q) * scale;
+                }
+            }
+        }
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            const frag_t db = acc_to_b(dp[s >> 1], s & 1);
+#pragma unroll
+            for (int u = 0; u < 2; ++u) dqt[u] = mma(frag_perm(Kts, u * 32 + c, s, h), db, dqt[u]);
+        }
+    }
+    if (qok) {
+        bf16_t *drow = dqkv + ((int64_t)b * S + q) * ld + hh * HD;
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                bf16x4 o;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) o[e] = (bf16_t)dqt[u][g * 4 + e];
+                *(bf16x4 *)(drow + u * 32 + g * 8 + h * 4) = o;
+            }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// dK, dV: lanes own kv columns, query tiles are streamed
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(AT_THREADS) void attn_bwd_dkv_kernel(const bf16_t *qkv, const bf16_t *dout, const float *lse,
+                                                                const float *delta, const float *mask, bf16_t *dqkv,
+                                                                int S, int H, float scale) {
+    __shared__ __attribute__((aligned(16))) char Qs[TILE_BYTES];
+    __shared__ __attribute__((aligned(16))) char dOs[TILE_BYTES];
+    __shared__ __attribute__((aligned(16))) char Qts[TILE_BYTES];
+    __shared__ __attribute__((aligned(16))) char dOts[TILE_BYTES];
+    __shared__ float lse_s[TILE], delta_s[TILE];
+    const int E = H * HD, ld = 3 * E;
+    const int b = blockIdx.y / H, hh = blockIdx.y % H;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, c = lane & 31, h = lane >> 5;
+    const int kv = blockIdx.x * 128 + wave * 32 + c;
+    const bool kok = kv < S;
+    const bf16_t *Q = qkv + (int64_t)b * S * ld + hh * HD;
+    const bf16_t *K = Q + E, *V = Q + 2 * E;
+    const bf16_t *dO = dout + (int64_t)b * S * E + hh * HD;
+    const float *lse_b = lse + ((int64_t)b * H + hh) * S, *delta_b = delta + ((int64_t)b * H + hh) * S;
+
+    frag_t kf[4], vf[4];
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+        kf[s] = load_row_frag(K + (int64_t)kv * ld, kok, s, h);
+        vf[s] = load_row_frag(V + (int64_t)kv * ld, kok, s, h);
+    }
+    f32x16 dvt[2] = {zero16(), zero16()}, dkt[2] = {zero16(), zero16()};
+    TileLoader<bf16_t, TILE, AT_THREADS, true> lq, ldo;
+    TileLoader<bf16_t, HD, AT_THREADS, false> lqt, ldot;
+
+    for (int q0 = 0; q0 < S; q0 += TILE) {
+        lq.load(Q + (int64_t)q0 * ld, ld, S - q0, HD);
+        ldo.load(dO + (int64_t)q0 * E, E, S - q0, HD);
+        lqt.load(Q + (int64_t)q0 * ld, ld, HD, S - q0);
+        ldot.load(dO + (int64_t)q0 * E, E, HD, S - q0);
+        __syncthreads();
+        lq.store(Qs);
+        ldo.store(dOs);
+        lqt.store(Qts);
+        ldot.store(dOts);
+        if (threadIdx.x < TILE) {
+            const int qq = q0 + threadIdx.x;
+            lse_s[threadIdx.x] = qq < S ? lse_b[qq] : 0.f;
+            delta_s[threadIdx.x] = qq < S ? delta_b[qq] : 0.f;
+        }
+        __syncthreads();
+
+        f32x16 sc[2] = {zero16(), zero16()}, dp[2] = {zero16(), zero16()};
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                sc[t] = mma(frag_rowk(Qs, t * 32 + c, s, h), kf[s], sc[t]);
+                dp[t] = mma(frag_rowk(dOs, t * 32 + c, s, h), vf[s], dp[t]);
+            }
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int ql = t * 32 + acc_row(r, h), qq = q0 + ql;
+                float p = 0.f;
+                if (kok && qq < S) {
+                    const float mk = mask ? mask[(int64_t)qq * S + kv] : 0.f;
+                    p = __expf(sc[t][r] * scale + mk - lse_s[ql]);
+                }
+                sc[t][r] = p;
+                dp[t][r] = p * (dp[t][r] - delta_s[ql]) * scale;
+            }
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            const frag_t pb = acc_to_b(sc[s >> 1], s & 1), db = acc_to_b(dp[s >> 1], s & 1);
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                dvt[u] = mma(frag_perm(dOts, u * 32 + c, s, h), pb, dvt[u]);
+                dkt[u] = mma(frag_perm(Qts, u * 32 + c, s, h), db, dkt[u]);
+            }
+        }
+    }
+    if (kok) {
+        bf16_t *drow = dqkv + ((int64_t)b * S + kv) * ld + hh * HD;
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                bf16x4 ok_, ov;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    ok_[e] = (bf16_t)dkt[u][g * 4 + e];
+                    ov[e] = (bf16_t)dvt[u][g * 4 + e];
+                }
+                *(bf16x4 *)(drow + E + u * 32 + g * 8 + h * 4) = ok_;
+                *(bf16x4 *)(drow + 2 * E + u * 32 + g * 8 + h * 4) = ov;
+            }
+    }
+}
+
+int check_attn(const char *name, int64_t b, int64_t S, int64_t H) {
+    HAPMI_REQUIRE(b >= 0 && S >= 1 && H >= 1, HAPMI_EINVAL, "%s: bad shape", name);
+    HAPMI_REQUIRE(S < (1ll << 24) && b * H <= 65535, HAPMI_ELIMIT, "%s: b*H %lld above 65535 or S too long", name,
+                  (long long)(b * H));
+    return HAPMI_OK;
+}
+
+}  // namespace
+
+extern "C" int hapmi_attention_fwd(const void *qkv, const float *mask, void *out, float *lse, int64_t b, int64_t S,
+                                   int64_t H, float scale, hapmi_stream_t stream) {
+    int rc = check_attn("attention_fwd", b, S, H);
+    if (rc) return rc;
+    if (b == 0) return HAPMI_OK;
+    HAPMI_REQUIRE(qkv && out && lse, HAPMI_EINVAL, "attention_fwd: null pointer");
+    HAPMI_REQUIRE(((uintptr_t)qkv % 16) == 0 && ((uintptr_t)out % 16) == 0 && (!mask || ((uintptr_t)mask % 16) == 0),
+                  HAPMI_EALIGN, "attention_fwd: pointers must be 16-byte aligned");
+    dim3 grid((unsigned)hapmi_cdiv(S, 128), (unsigned)(b * H));
+    hipLaunchKernelGGL(attn_fwd_kernel, grid, dim3(AT_THREADS), 0, (hipStream_t)stream, (const bf16_t *)qkv, mask,
+                       (bf16_t *)out, lse, (int)S, (int)H, scale);
+    HAPMI_CHECK_LAUNCH("attention_fwd");
+    return HAPMI_OK;
+}
+
+extern "C" int hapmi_attention_bwd(const void *qkv, const void *out, const void *dout, const float *lse,
+                                   const float *mask, void *dqkv, float *delta_ws, int64_t b, int64_t S, int64_t H,
+                                   float scale, hapmi_stream_t stream) {
+    int rc = check_attn("attention_bwd", b, S, H);
+    if (rc) return rc;
+    if (b == 0) return HAPMI_OK;
+    HAPMI_REQUIRE(qkv && out && dout && lse && dqkv && delta_ws, HAPMI_EINVAL, "attention_bwd: null pointer");
+    HAPMI_REQUIRE(((uintptr_t)qkv % 16) == 0 && ((uintptr_t)out % 16) == 0 && ((uintptr_t)dout % 16) == 0 &&
+                      ((uintptr_t)dqkv % 16) == 0 && (!mask || ((uintptr_t)mask % 16) == 0),
+                  HAPMI_EALIGN, "attention_bwd: pointers must be 16-byte aligned");
+    hipStream_t st = (hipStream_t)stream;
+    hipLaunchKernelGGL(attn_delta_kernel, dim3((unsigned)hapmi_cdiv(b * S * H, 256)), dim3(256), 0, st,
+                       (const bf16_t *)out, (const bf16_t *)dout, delta_ws, b * S, (int)S, (int)H);
+    dim3 grid((unsigned)hapmi_cdiv(S, 128), (unsigned)(b * H));
+    hipLaunchKernelGGL(attn_bwd_dq_kernel, grid, dim3(AT_THREADS), 0, st, (const bf16_t *)qkv, (const bf16_t *)dout, lse,
+                       (const float *)delta_ws, mask, (bf16_t *)dqkv, (int)S, (int)H, scale);
+    hipLaunchKernelGGL(attn_bwd_dkv_kernel, grid, dim3(AT_THREADS), 0, st, (const bf16_t *)qkv, (const bf16_t *)dout, lse,
+                       (const float *)delta_ws, mask, (bf16_t *)dqkv, (int)S, (int)H, scale);
+    HAPMI_CHECK_LAUNCH("attention_bwd");
+    return HAPMI_OK;
+}

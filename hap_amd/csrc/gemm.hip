@@ -14,6 +14,7 @@
 // holds 4 consecutive n of one m in its accumulators and the epilogue issues 8/16-byte stores along the
 // contiguous dimension of C.
 #include "common.h"
+#include "tile.h"
 #include <vector>
 #include <mutex>
 
@@ -53,98 +54,6 @@ __device__ __forceinline__ float apply_act(float v, int act) {
     if (act == HAPMI_ACT_GELU) return 0.5f * v * (1.0f + erff(v * 0.70710678118654752f));
     return v;
 }
-
-constexpr int ROW_BYTES = 128;                       // k bytes per LDS row
-__device__ __forceinline__ int swz(int row) { return (row ^ (row >> 3)) & 7; }
-
-// Loads one operand tile [ROWS][BK] (row = m or n index, k = reduction index) from global memory into
-// registers and stores it into the swizzled LDS tile.  KMAJOR: memory is [row][k] (k contiguous);
-// otherwise memory is [k][row] (row contiguous) and 4(k) x EPV(row) register blocks are transposed.
-template <typename TI, int ROWS, int THREADS, bool KMAJOR> struct TileLoader {
-    static constexpr int EPV = 16 / sizeof(TI);
-    static constexpr int BK = ROW_BYTES / sizeof(TI);
-    static constexpr int KV = 8;                                  // 16-byte chunks per row
-    static constexpr int ROWS_PER_PASS = THREADS / KV;
-    static constexpr int PASSES_K = ROWS / ROWS_PER_PASS;
-    static constexpr int RV = ROWS / EPV;                         // row-vectors per k line
-    static constexpr int BLOCKS = (BK / 4) * RV;
-    static constexpr int PASSES_T = (BLOCKS + THREADS - 1) / THREADS;
-    static constexpr int NV = KMAJOR ? PASSES_K : PASSES_T * 4;
-    static_assert(!KMAJOR || (ROWS % ROWS_PER_PASS == 0 && PASSES_K >= 1), "tile does not divide over the block");
-
-    Vec16<TI> v[NV];
-
-    __device__ __forceinline__ static Vec16<TI> guarded(const TI *p, int64_t n_valid) {
-        Vec16<TI> r;
-#pragma unroll
-        for (int e = 0; e < EPV; ++e) r.set(e, (e < n_valid) ? ld_f(p, e) : 0.f);
-        return r;
-    }
-
-    // base: pointer to element (row0, k0) of the operand; rows_left / k_left: valid extent from there
-    __device__ __forceinline__ void load(const TI *base, int64_t ld, int64_t rows_left, int64_t k_left) {
-        const int t = threadIdx.x;
-        if (KMAJOR) {
-            const int kv = t % KV, r0 = t / KV;
-#pragma unroll
-            for (int p = 0; p < PASSES_K; ++p) {
-                const int row = r0 + p * ROWS_PER_PASS;
-                const int64_t kk = (int64_t)kv * EPV;
-                const TI *src = base + (int64_t)row * ld + kk;
-                if (row < rows_left && kk + EPV <= k_left) v[p] = *(const Vec16<TI> *)src;
-                else if (row < rows_left && kk < k_left) v[p] = guarded(src, k_left - kk);
-                else v[p] = guarded(src, 0);
-            }
-        } else {
-#pragma unroll
-            for (int p = 0; p < PASSES_T; ++p) {
-                const int blk = t + p * THREADS;
-                if (BLOCKS % THREADS != 0 && blk >= BLOCKS) break;
-                const int rv = blk % RV, kg = blk / RV;
-                const int64_t rr = (int64_t)rv * EPV;
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const int64_t kk = (int64_t)kg * 4 + q;
-                    const TI *src = base + kk * ld + rr;
-                    if (kk < k_left && rr + EPV <= rows_left) v[p * 4 + q] = *(const Vec16<TI> *)src;
-                    else if (kk < k_left && rr < rows_left) v[p * 4 + q] = guarded(src, rows_left - rr);
-                    else v[p * 4 + q] = guarded(src, 0);
-                }
-            }
-        }
-    }
-
-    __device__ __forceinline__ void store(char *lds) const {
-        const int t = threadIdx.x;
-        if (KMAJOR) {
-            const int kv = t % KV, r0 = t / KV;
-#pragma unroll
-            for (int p = 0; p < PASSES_K; ++p) {
-                const int row = r0 + p * ROWS_PER_PASS;
-                *(Vec16<TI> *)(lds + row * ROW_BYTES + ((kv ^ swz(row)) << 4)) = v[p];
-            }
-        } else {
-            typedef TI quad_t __attribute__((ext_vector_type(4)));
-            constexpr int QB = 4 * sizeof(TI);                    // bytes of 4 consecutive k: 8 (bf16) or 16 (f32)
-#pragma unroll
-            for (int p = 0; p < PASSES_T; ++p) {
-                const int blk = t + p * THREADS;
-                if (BLOCKS % THREADS != 0 && blk >= BLOCKS) break;
-                const int rv = blk % RV, kg = blk / RV;
-                const int kbyte = kg * QB;                        // logical byte offset inside the row
-                const int chunk = kbyte >> 4, within = kbyte & 15;
-#pragma unroll
-                for (int e = 0; e < EPV; ++e) {
-                    quad_t q4;
-#pragma unroll
-                    for (int q = 0; q < 4; ++q) q4[q] = v[p * 4 + q].v[e];
-                    const int row = rv * EPV + e;
-                    *(quad_t *)(lds + row * ROW_BYTES + ((chunk ^ swz(row)) << 4) + within) = q4;
-                }
-            }
-        }
-    }
-};
 
 template <typename TI, typename TO, int BM, int BN, int WAVES_M, int WAVES_N, bool A_KMAJOR, bool B_KMAJOR>
 __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_kernel(GemmParams p) {

@@ -58,7 +58,7 @@ def _round_up(n, m):
 
 class ShardExecutor:
     def __init__(self, gm: torch.fx.GraphModule, example_inputs, dtype: str = "fp32", wire: Optional[Wire] = None,
-                 rank: int = 0, world_size: int = 1, device: str = "cuda:0"):
+                 rank: int = 0, world_size: int = 1, device: str = "cuda:0", fused_attention: bool = True):
         """``example_inputs``: the program's inputs (global batch) as tensors or shapes; activations are
         sized from them.  ``rank`` / ``world_size`` are only needed by all_reduce / replicate, whose node
         forms do not carry them (collectives.py:86, 182)."""
@@ -86,6 +86,8 @@ class ShardExecutor:
                                 for a in example_inputs]
         self.rank_hint, self.world_hint = rank, world_size
         self._param_reduce: List[Callable[[], None]] = []
+        self._scratch_pool: Dict[tuple, torch.Tensor] = {}
+        self.fused_attention = fused_attention
         self.gemm_workspace = torch.empty(64 << 20, dtype=torch.float32, device=self.dev)   # 256 MiB of split-K scratch
         ops.set_gemm_workspace(self.gemm_workspace)
         self._prepare_params()
@@ -140,6 +142,14 @@ class ShardExecutor:
 
     def _val(self, x):
         return self.env[x] if isinstance(x, torch.fx.Node) else x
+
+    def _scratch(self, key, shape, dtype=None):
+        """Backward-only temporaries that live inside one node's backward closure are shared between
+        nodes of the same shape (the launches of a step are serialised on one stream)."""
+        k = (key, tuple(shape), dtype or self.cdt)
+        if k not in self._scratch_pool:
+            self._scratch_pool[k] = self._new(shape, dtype)
+        return self._scratch_pool[k]
 
     def _grad_slot(self, v: Val):
         """Buffer that the next contribution to d(v) goes into and whether it must accumulate."""
@@ -490,11 +500,16 @@ class ShardExecutor:
                 self._unsupported(node, "attn_mask must be a float32 [L, S] additive mask")
             mask_t = mask.t
         scale = 1.0 / math.sqrt(hd)
+        fused = self.fused_attention and self.dtype == "bf16" and hd == 64
         Sp = _round_up(S, self.epv)
         qkv = self._new((b, S, 3 * E))
-        P = self._new((b, H, S, Sp))
         ctx = self._new((b, S, E))
         o = self._new((b, S, E))
+        if fused:
+            lse = self._new((b, H, S), torch.float32)
+            P = None
+        else:
+            P = self._new((b, H, S, Sp))
         out_bsd = Val("tensor", o, needs_grad=True)
         out = Val("transposed", None, src=out_bsd, dims=(0, 1), needs_grad=True)
         M = b * S
@@ -502,11 +517,14 @@ class ShardExecutor:
 
         def forward():
             ops.gemm(x.t, w_in.t, qkv, M, 3 * E, E, transB=True, bias=b_in.meta["master"])
-            ops.gemm(qkv, qkv, P, S, S, hd, transB=True, lda=3 * E, ldb=3 * E, ldc=Sp, alpha=scale, batch1=b, batch2=H,
-                     strideA=sQ, strideB=sQ, strideC=sP, offB=E)
-            ops.softmax_fwd(P, mask_t, P, b * H * S, S, Sp, S)
-            ops.gemm(P, qkv, ctx, S, hd, S, lda=Sp, ldb=3 * E, ldc=E, batch1=b, batch2=H, strideA=sP, strideB=sQ,
-                     strideC=(S * E, hd), offB=2 * E)
+            if fused:
+                ops.attention_fwd(qkv, mask_t, ctx, lse, b, S, H, scale)
+            else:
+                ops.gemm(qkv, qkv, P, S, S, hd, transB=True, lda=3 * E, ldb=3 * E, ldc=Sp, alpha=scale, batch1=b,
+                         batch2=H, strideA=sQ, strideB=sQ, strideC=sP, offB=E)
+                ops.softmax_fwd(P, mask_t, P, b * H * S, S, Sp, S)
+                ops.gemm(P, qkv, ctx, S, hd, S, lda=Sp, ldb=3 * E, ldc=E, batch1=b, batch2=H, strideA=sP, strideB=sQ,
+                         strideC=(S * E, hd), offB=2 * E)
             ops.gemm(ctx, w_out.t, o, M, E, E, transB=True, bias=b_out.meta["master"])
         self.fwd.append(forward)
 
@@ -514,9 +532,12 @@ class ShardExecutor:
             if out_bsd.grad is None:
                 return
             do = out_bsd.grad
-            dctx = self._new((b, S, E))
-            dP = self._new((b, H, S, Sp))
-            dqkv = self._new((b, S, 3 * E))
+            dctx = self._scratch("attn_dctx", (b, S, E))
+            dqkv = self._scratch("attn_dqkv", (b, S, 3 * E))
+            if fused:
+                delta = self._scratch("attn_delta", (b, H, S), torch.float32)
+            else:
+                dP = self._scratch("attn_dP", (b, H, S, Sp))
             gwo, acc_wo = self._param_grad_slot(w_out)
             gbo, acc_bo = self._param_grad_slot(b_out)
             gwi, acc_wi = self._param_grad_slot(w_in)
@@ -527,17 +548,20 @@ class ShardExecutor:
                 ops.gemm(do, ctx, gwo, E, E, M, transA=True, accumulate=acc_wo)
                 ops.colsum(do, gbo, M, E, E, acc_bo)
                 ops.gemm(do, w_out.t, dctx, M, E, E)
-                # dP = dctx V^T ; dV = P^T dctx
-                ops.gemm(dctx, qkv, dP, S, S, hd, transB=True, lda=E, ldb=3 * E, ldc=Sp, batch1=b, batch2=H,
-                         strideA=(S * E, hd), strideB=sQ, strideC=sP, offB=2 * E)
-                ops.gemm(P, dctx, dqkv, S, hd, S, transA=True, lda=Sp, ldb=E, ldc=3 * E, batch1=b, batch2=H,
-                         strideA=sP, strideB=(S * E, hd), strideC=sQ, offC=2 * E)
-                ops.softmax_bwd(dP, P, dP, b * H * S, S, Sp)
-                # dQ = scale dS K ; dK = scale dS^T Q
-                ops.gemm(dP, qkv, dqkv, S, hd, S, lda=Sp, ldb=3 * E, ldc=3 * E, alpha=scale, batch1=b, batch2=H,
-                         strideA=sP, strideB=sQ, strideC=sQ, offB=E)
-                ops.gemm(dP, qkv, dqkv, S, hd, S, transA=True, lda=Sp, ldb=3 * E, ldc=3 * E, alpha=scale, batch1=b,
-                         batch2=H, strideA=sP, strideB=sQ, strideC=sQ, offC=E)
+                if fused:
+                    ops.attention_bwd(qkv, ctx, dctx, lse, mask_t, dqkv, delta, b, S, H, scale)
+                else:
+                    # dP = dctx V^T ; dV = P^T dctx
+                    ops.gemm(dctx, qkv, dP, S, S, hd, transB=True, lda=E, ldb=3 * E, ldc=Sp, batch1=b, batch2=H,
+                             strideA=(S * E, hd), strideB=sQ, strideC=sP, offB=2 * E)
+                    ops.gemm(P, dctx, dqkv, S, hd, S, transA=True, lda=Sp, ldb=E, ldc=3 * E, batch1=b, batch2=H,
+                             strideA=sP, strideB=(S * E, hd), strideC=sQ, offC=2 * E)
+                    ops.softmax_bwd(dP, P, dP, b * H * S, S, Sp)
+                    # dQ = scale dS K ; dK = scale dS^T Q
+                    ops.gemm(dP, qkv, dqkv, S, hd, S, lda=Sp, ldb=3 * E, ldc=3 * E, alpha=scale, batch1=b, batch2=H,
+                             strideA=sP, strideB=sQ, strideC=sQ, offB=E)
+                    ops.gemm(dP, qkv, dqkv, S, hd, S, transA=True, lda=Sp, ldb=3 * E, ldc=3 * E, alpha=scale, batch1=b,
+                             batch2=H, strideA=sP, strideB=sQ, strideC=sQ, offC=E)
                 ops.gemm(dqkv, x.t, gwi, 3 * E, E, M, transA=True, accumulate=acc_wi)
                 ops.colsum(dqkv, gbi, M, 3 * E, 3 * E, acc_bi)
                 if gx is not None:
@@ -1002,9 +1026,10 @@ class ShardExecutor:
 
 
 def compile_program(gm: torch.fx.GraphModule, example_inputs, dtype: str = "fp32", wire: Optional[Wire] = None,
-                    rank: int = 0, world_size: int = 1, device: str = "cuda:0") -> ShardExecutor:
+                    rank: int = 0, world_size: int = 1, device: str = "cuda:0", **kw) -> ShardExecutor:
     """Compile the emitted program for the global-batch shapes of ``example_inputs`` (tensors or shapes)."""
-    return ShardExecutor(gm, example_inputs, dtype=dtype, wire=wire, rank=rank, world_size=world_size, device=device)
+    return ShardExecutor(gm, example_inputs, dtype=dtype, wire=wire, rank=rank, world_size=world_size, device=device,
+                         **kw)
 
 
 def _finish_param_reduce(self: ShardExecutor):

@@ -339,6 +339,36 @@ def softmax_bwd(dp, p, ds, rows, width, ld):
     check(lib().hapmi_softmax_bwd(_ptr(dp), _ptr(p), _ptr(ds), rows, width, ld, dtype_code(p), _stream()))
 
 
+def _check_attn(qkv, out, lse, mask, b, S, H):
+    E = H * 64
+    _need(qkv, b * S * 3 * E, "attention qkv")
+    _need(out, b * S * E, "attention out")
+    _need(lse, b * H * S, "attention lse")
+    _need(mask, S * S, "attention mask")
+    if qkv.dtype != torch.bfloat16 or out.dtype != torch.bfloat16 or lse.dtype != torch.float32:
+        raise TypeError("attention: bf16 qkv / out and float32 lse expected")
+    if mask is not None and mask.dtype != torch.float32:
+        raise TypeError("attention: float32 mask expected")
+
+
+def attention_fwd(qkv, mask, out, lse, b, S, H, scale):
+    _dev(qkv, mask, out, lse)
+    _check_attn(qkv, out, lse, mask, b, S, H)
+    check(lib().hapmi_attention_fwd(_ptr(qkv), _ptr(mask), _ptr(out), _ptr(lse), b, S, H, ctypes.c_float(scale), _stream()))
+
+
+def attention_bwd(qkv, out, dout, lse, mask, dqkv, delta_ws, b, S, H, scale):
+    _dev(qkv, out, dout, lse, mask, dqkv, delta_ws)
+    _check_attn(qkv, out, lse, mask, b, S, H)
+    _need(dout, b * S * H * 64, "attention dout")
+    _need(dqkv, b * S * 3 * H * 64, "attention dqkv")
+    _need(delta_ws, b * H * S, "attention delta")
+    if dout.dtype != torch.bfloat16 or dqkv.dtype != torch.bfloat16 or delta_ws.dtype != torch.float32:
+        raise TypeError("attention_bwd: dtype mismatch")
+    check(lib().hapmi_attention_bwd(_ptr(qkv), _ptr(out), _ptr(dout), _ptr(lse), _ptr(mask), _ptr(dqkv), _ptr(delta_ws),
+                                    b, S, H, ctypes.c_float(scale), _stream()))
+
+
 def logsoftmax_nll(logits, targets, row_loss, dlogits, rows, width, ld, ignore_index=-100, grad_scale=1.0):
     _dev(logits, targets, row_loss, dlogits)
     if targets.dtype != torch.int64:

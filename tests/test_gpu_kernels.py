@@ -270,3 +270,35 @@ def test_gemm_split_k_and_tile_configs(cuda, dtype, cfg):
             close(out, torch.relu(want), dtype, scale=2.0)
     finally:
         lib().hapmi_gemm_tuning(-1, 0)
+
+
+@pytest.mark.parametrize("S,causal", [(16, True), (128, True), (197, False), (512, False), (200, True), (64, False)])
+def test_fused_attention_forward_backward(cuda, S, causal):
+    """Fused bf16 attention against the explicit softmax(QK^T * scale + mask) V of
+    F.multi_head_attention_forward, computed in float64 from the same bf16 inputs."""
+    g = torch.Generator().manual_seed(S)
+    b, H, hd = 2, 3, 64
+    E = H * hd
+    qkv = torch.randn(b, S, 3 * E, generator=g).bfloat16()
+    dout = torch.randn(b, S, E, generator=g).bfloat16()
+    mask = torch.triu(torch.full((S, S), float("-inf")), diagonal=1) if causal else None
+    scale = 1.0 / math.sqrt(hd)
+    out = torch.empty(b, S, E, dtype=torch.bfloat16, device=cuda)
+    lse = torch.empty(b, H, S, dtype=torch.float32, device=cuda)
+    dq = qkv.to(cuda)
+    dmask = mask.to(cuda) if causal else None
+    ops.attention_fwd(dq, dmask, out, lse, b, S, H, scale)
+    x = qkv.double().requires_grad_(True)
+    q, k, v = [t.view(b, S, H, hd).transpose(1, 2) for t in x.split(E, dim=2)]
+    sc = q @ k.transpose(-1, -2) * scale
+    if causal:
+        sc = sc + mask.double()
+    want = (torch.softmax(sc, -1) @ v).transpose(1, 2).reshape(b, S, E)
+    close(out, want.detach(), torch.bfloat16)
+    torch.testing.assert_close(lse.cpu(), torch.logsumexp(sc, -1).float().detach(), rtol=1e-3, atol=1e-3)
+    want.backward(dout.double())
+    dqkv = torch.full((b, S, 3 * E), float("nan"), dtype=torch.bfloat16, device=cuda)
+    delta = torch.empty(b, H, S, dtype=torch.float32, device=cuda)
+    ops.attention_bwd(dq, out, dout.to(cuda), lse, dmask, dqkv, delta, b, S, H, scale)
+    for name, got, ref in zip("qkv", dqkv.float().cpu().split(E, dim=2), x.grad.split(E, dim=2)):
+        assert rel_err(got, ref) < 2e-2, (name, rel_err(got, ref))
