@@ -128,21 +128,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_kernel(GemmParams 
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    la.load(a_base + (int64_t)kt0 * a_kstep, p.lda, m_left, p.K - (int64_t)kt0 * BK);
-    lb.load(b_base + (int64_t)kt0 * b_kstep, p.ldb, n_left, p.K - (int64_t)kt0 * BK);
-    la.store(As);
-    lb.store(Bs);
-    __syncthreads();
-
-    for (int kt = kt0; kt < kt1; ++kt) {
-        const int cur = (kt - kt0) & 1;
-        if (kt + 1 < kt1) {
-            const int64_t k_left = p.K - (int64_t)(kt + 1) * BK;
-            la.load(a_base + (int64_t)(kt + 1) * a_kstep, p.lda, m_left, k_left);
-            lb.load(b_base + (int64_t)(kt + 1) * b_kstep, p.ldb, n_left, k_left);
-        }
-        const char *as = As + cur * A_BYTES;
-        const char *bs = Bs + cur * B_BYTES;
+    auto compute_tile = [&](const char *as, const char *bs) {
 #pragma unroll
         for (int ks = 0; ks < KSTEPS; ++ks) {
             Vec16<TI> fa[TM], fb[TN];
@@ -155,11 +141,51 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_kernel(GemmParams 
 #pragma unroll
                 for (int j = 0; j < TN; ++j) Mma<TI>::run(acc[i][j], fb[j], fa[i]);
         }
-        if (kt + 1 < kt1) {
-            la.store(As + (cur ^ 1) * A_BYTES);
-            lb.store(Bs + (cur ^ 1) * B_BYTES);
-        }
+    };
+
+    // A ragged last k-tile (K not a multiple of the tile depth) is done first, alone, with guarded loads, so
+    // that the main loop below only ever sees complete k-tiles and stays free of branches.
+    int kt_end = kt1;
+    if ((p.K % BK) != 0 && kt1 == nk_total) {
+        kt_end = kt1 - 1;
+        const int64_t k_left = p.K - (int64_t)kt_end * BK;
+        la.load(a_base + (int64_t)kt_end * a_kstep, p.lda, m_left, k_left);
+        lb.load(b_base + (int64_t)kt_end * b_kstep, p.ldb, n_left, k_left);
+        la.store(As);
+        lb.store(Bs);
         __syncthreads();
+        compute_tile(As, Bs);
+        __syncthreads();
+    }
+
+    if (kt0 < kt_end) {
+        // complete k-tiles: row-major operands go global -> LDS directly, k-major operands through registers
+        // (transposed on the LDS store)
+        if (A_KMAJOR) la.init_direct(p.lda, m_left);
+        else la.init_offsets(p.lda, m_left);
+        if (B_KMAJOR) lb.init_direct(p.ldb, n_left);
+        else lb.init_offsets(p.ldb, n_left);
+        auto issue_tile = [&](int kt, int buf) {
+            if (A_KMAJOR) la.load_direct(a_base + (int64_t)kt * a_kstep, As + buf * A_BYTES);
+            else la.load_fast(a_base + (int64_t)kt * a_kstep, p.lda);
+            if (B_KMAJOR) lb.load_direct(b_base + (int64_t)kt * b_kstep, Bs + buf * B_BYTES);
+            else lb.load_fast(b_base + (int64_t)kt * b_kstep, p.ldb);
+        };
+        auto commit_tile = [&](int buf) {
+            if (!A_KMAJOR) la.store(As + buf * A_BYTES);
+            if (!B_KMAJOR) lb.store(Bs + buf * B_BYTES);
+            __builtin_amdgcn_s_waitcnt(0x0F70);                   // vmcnt(0): this wave's direct loads have landed
+        };
+        issue_tile(kt0, 0);
+        commit_tile(0);
+        __syncthreads();
+        for (int kt = kt0; kt < kt_end; ++kt) {
+            const int cur = (kt - kt0) & 1;
+            if (kt + 1 < kt_end) issue_tile(kt + 1, cur ^ 1);
+            compute_tile(As + cur * A_BYTES, Bs + cur * B_BYTES);
+            if (kt + 1 < kt_end) commit_tile(cur ^ 1);
+            __syncthreads();
+        }
     }
 
     // epilogue: acc[i][j][r] is C[m, n] with m = wm + i*32 + lane%32, n = wn + j*32 + (r/4)*8 + (lane/32)*4 + r%4
@@ -228,8 +254,8 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_kernel(GemmParams 
 struct TileCfg {
     int bm, bn, wm, wn;
 };
-constexpr TileCfg kCfg[] = {{128, 128, 2, 2}, {256, 256, 2, 4}};
-constexpr int kNumCfg = 2;
+constexpr TileCfg kCfg[] = {{128, 128, 2, 2}, {256, 256, 2, 4}, {384, 192, 4, 2}, {192, 256, 2, 4}, {256, 192, 4, 2}};
+constexpr int kNumCfg = 5;
 constexpr int kNumCU = 256;
 int g_force_cfg = -1;
 int g_force_splits = 0;
@@ -285,34 +311,40 @@ int launch_cfg(const GemmParams &p, int transA, int transB, int64_t batch, hipSt
     return HAPMI_OK;
 }
 
-int choose_cfg(int64_t M, int64_t N, int64_t batch, bool wide) {
-    if (g_force_cfg >= 0 && g_force_cfg < kNumCfg) return (g_force_cfg == 1 && !wide) ? 0 : g_force_cfg;
-    if (!wide) return 0;
-    // 256x256 tiles run one per CU: take them only when the tile count fills whole rounds of the 256 CUs
-    const int64_t t = hapmi_cdiv(M, 256) * hapmi_cdiv(N, 256) * batch;
-    const int64_t rounds = hapmi_cdiv(t, kNumCU);
-    const double fill = (double)t / (double)(rounds * kNumCU);
-    const double edge = ((double)M * (double)N) / ((double)hapmi_cdiv(M, 256) * 256.0 * (double)hapmi_cdiv(N, 256) * 256.0);
-    return (fill * edge >= 0.88) ? 1 : 0;
-}
+// Tile shape and K split are chosen together from a small cost model (units: microseconds):
+//   rounds of tiles over the co-resident block slots x (tile FLOPs / per-slot rate + fixed prologue/epilogue)
+//   + the split-K reduction traffic.  128x128 tiles run two blocks per CU (512 slots), the 8-wave tiles one.
+struct Choice {
+    int cfg, splits;
+};
 
-// Small outputs with a long reduction do not fill the chip: split K over blockIdx.y.
-int choose_splits(const TileCfg &c, int64_t M, int64_t N, int64_t K, int64_t batch, int bk, int64_t max_splits) {
-    if (max_splits < 2 || batch != 1) return 1;
+Choice choose(int64_t M, int64_t N, int64_t K, int64_t batch, int bk, bool wide, int64_t max_splits, bool row_major_operands) {
+    static const int kSplitMenu[] = {1, 2, 3, 4, 6, 8, 12, 16, 24, 32};
     const int64_t nk = hapmi_cdiv(K, bk);
-    int64_t s;
-    if (g_force_splits > 0) {
-        s = g_force_splits;
-    } else {
-        const int64_t tiles = hapmi_cdiv(M, c.bm) * hapmi_cdiv(N, c.bn);
-        const int64_t slots = (c.bm == 128) ? 2 * kNumCU : kNumCU;      // co-resident blocks
-        if (tiles * 4 > slots * 3 || nk < 16) return 1;
-        s = slots / tiles;
-        if (s > nk / 8) s = nk / 8;
+    Choice best{0, 1};
+    double best_t = 1e30;
+    for (int c = 0; c < kNumCfg; ++c) {
+        if (g_force_cfg >= 0 && g_force_cfg < kNumCfg && c != g_force_cfg && (wide || g_force_cfg == 0)) continue;
+        if (c > 0 && !wide) continue;
+        if (c == 2 && !row_major_operands && g_force_cfg != 2) continue;   // 384x192 with a transposing loader spills registers
+        const int64_t tiles = hapmi_cdiv(M, kCfg[c].bm) * hapmi_cdiv(N, kCfg[c].bn) * batch;
+        const double slots = c == 0 ? 2.0 * kNumCU : 1.0 * kNumCU;
+        const double rate = c == 0 ? 1.75 : 4.1;                         // TFLOP/s per slot in steady state
+        const double fixed = c == 0 ? 2.0 : 3.5;                         // us per tile: first loads + epilogue
+        for (int s : kSplitMenu) {
+            if (g_force_splits > 0 && s != g_force_splits && !(s == 1 && (max_splits < g_force_splits || batch != 1))) continue;
+            if (s > 1 && (s > max_splits || batch != 1 || nk / s < 4)) continue;
+            const double tile_us = 2.0 * kCfg[c].bm * kCfg[c].bn * (double)bk * (double)hapmi_cdiv(nk, s) / (rate * 1e6);
+            const double rounds = (double)hapmi_cdiv(tiles * s, (int64_t)slots);
+            double t = rounds * (tile_us + fixed);
+            if (s > 1) t += 2.0 + (double)s * (double)M * (double)N * 8.0 / 3.0e6;   // launch + write/read at ~3 TB/s
+            if (t < best_t) {
+                best_t = t;
+                best = Choice{c, s};
+            }
+        }
     }
-    if (s > max_splits) s = max_splits;
-    if (s > nk) s = nk;
-    return (int)(s < 1 ? 1 : s);
+    return best;
 }
 
 template <typename TO>
@@ -344,18 +376,24 @@ template <typename TI, typename TO>
 int launch_typed(GemmParams &p, int transA, int transB, int64_t batch, hipStream_t st, bool wide, void *workspace,
                  int64_t workspace_bytes) {
     const int bk = ROW_BYTES / (int)sizeof(TI);
-    const int c = choose_cfg(p.M, p.N, batch, wide && sizeof(TI) == 2);
     const int64_t nk = hapmi_cdiv(p.K, bk);
     p.ws_ld = (p.N + 3) / 4 * 4;
     const int64_t per_split = p.M * p.ws_ld * 4;
     const int64_t max_splits = (workspace && ((uintptr_t)workspace % 16) == 0 && per_split > 0) ? workspace_bytes / per_split : 0;
-    p.splits = choose_splits(kCfg[c], p.M, p.N, p.K, batch, bk, max_splits);
+    const Choice ch = choose(p.M, p.N, p.K, batch, bk, wide && sizeof(TI) == 2, max_splits, !transA && transB);
+    const int c = ch.cfg;
+    p.splits = ch.splits;
     p.ktiles_per_split = (int)hapmi_cdiv(nk, p.splits);
     p.splits = (int)hapmi_cdiv(nk, p.ktiles_per_split);
     p.ws = (float *)workspace;
     int rc;
-    if (c == 1) rc = launch_cfg<bf16_t, TO, 256, 256, 2, 4>(p, transA, transB, batch, st);
-    else rc = launch_cfg<TI, TO, 128, 128, 2, 2>(p, transA, transB, batch, st);
+    switch (c) {
+        case 1: rc = launch_cfg<bf16_t, TO, 256, 256, 2, 4>(p, transA, transB, batch, st); break;
+        case 2: rc = launch_cfg<bf16_t, TO, 384, 192, 4, 2>(p, transA, transB, batch, st); break;
+        case 3: rc = launch_cfg<bf16_t, TO, 192, 256, 2, 4>(p, transA, transB, batch, st); break;
+        case 4: rc = launch_cfg<bf16_t, TO, 256, 192, 4, 2>(p, transA, transB, batch, st); break;
+        default: rc = launch_cfg<TI, TO, 128, 128, 2, 2>(p, transA, transB, batch, st);
+    }
     if (rc || p.splits <= 1) return rc;
     int64_t gx = hapmi_cdiv(p.M * (p.ws_ld / 4), 256);
     if (gx > 256 * 16) gx = 256 * 16;

@@ -24,6 +24,86 @@ template <typename TI, int ROWS, int THREADS, bool KMAJOR> struct TileLoader {
 
     Vec16<TI> v[NV];
 
+    // ---- branch-free path for k-tiles that lie completely inside K -------------------------------------
+    // Rows beyond rows_left are clamped to the last valid row / row-vector: they are loaded (in bounds) and
+    // multiplied, but the epilogue never stores them.  A row-vector that straddles rows_left stays inside
+    // the operand's leading dimension, which is a multiple of the vector width.
+    static constexpr int NOFF = KMAJOR ? PASSES_K : PASSES_T;
+    int off[NOFF];                                                // element offsets from the tile's base
+
+    __device__ __forceinline__ void init_offsets(int64_t ld, int64_t rows_left) {
+        const int t = threadIdx.x;
+        const int last = (int)(rows_left < ROWS ? rows_left : ROWS) - 1;
+        if (KMAJOR) {
+            const int kv = t % KV, r0 = t / KV;
+#pragma unroll
+            for (int p = 0; p < PASSES_K; ++p) {
+                int row = r0 + p * ROWS_PER_PASS;
+                row = row < last ? row : last;
+                off[p] = row * (int)ld + kv * EPV;
+            }
+        } else {
+            const int last_rr = (last / EPV) * EPV;
+#pragma unroll
+            for (int p = 0; p < PASSES_T; ++p) {
+                int blk = t + p * THREADS;
+                blk = blk < BLOCKS ? blk : BLOCKS - 1;            // idle threads repeat the last block (never stored)
+                const int rv = blk % RV, kg = blk / RV;
+                int rr = rv * EPV;
+                rr = rr < last_rr ? rr : last_rr;
+                off[p] = kg * 4 * (int)ld + rr;
+            }
+        }
+    }
+
+    // ---- direct global -> LDS path (row-major operands only) ---------------------------------------------
+    // One global_load_lds_dwordx4 per wave fills 1024 contiguous LDS bytes = 8 tile rows; lane l lands in row
+    // l / 8, physical chunk l % 8, so it fetches the logical chunk (l % 8) ^ swz(row) of that row.
+    static constexpr int NWAVES = THREADS / 64;
+    static constexpr int PASSES_D = ROWS / (8 * NWAVES);
+    int doff[KMAJOR ? (PASSES_D > 0 ? PASSES_D : 1) : 1];
+
+    __device__ __forceinline__ void init_direct(int64_t ld, int64_t rows_left) {
+        static_assert(!KMAJOR || ROWS % (8 * NWAVES) == 0, "direct loads need ROWS to be a multiple of 8 * waves");
+        const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+        const int last = (int)(rows_left < ROWS ? rows_left : ROWS) - 1;
+#pragma unroll
+        for (int p = 0; p < PASSES_D; ++p) {
+            const int row = (p * NWAVES + wave) * 8 + (lane >> 3);
+            const int chunk = (lane & 7) ^ swz(row);
+            doff[p] = (row < last ? row : last) * (int)ld + chunk * EPV;
+        }
+    }
+
+    __device__ __forceinline__ void load_direct(const TI *base, char *lds) const {
+        // Issued as inline assembly on purpose: for the builtin the compiler cannot tell which LDS reads alias
+        // the in-flight transfer and waits for vmcnt(0) before every ds_read, which serialises the prefetch
+        // with the MFMA loop.  The caller waits for vmcnt(0) itself before the barrier that publishes the tile.
+        typedef __attribute__((address_space(3))) char lds_char;
+        const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+#pragma unroll
+        for (int p = 0; p < PASSES_D; ++p) {
+            const uint32_t lds_addr = (uint32_t)(uintptr_t)(lds_char *)(lds + (p * NWAVES + wave) * 8 * ROW_BYTES);
+            const TI *src = base + doff[p];
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                         :
+                         : "s"(lds_addr), "v"(src)
+                         : "memory");
+        }
+    }
+
+    __device__ __forceinline__ void load_fast(const TI *base, int64_t ld) {
+        if (KMAJOR) {
+#pragma unroll
+            for (int p = 0; p < PASSES_K; ++p) v[p] = *(const Vec16<TI> *)(base + off[p]);
+        } else {
+#pragma unroll
+            for (int p = 0; p < PASSES_T; ++p)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) v[p * 4 + q] = *(const Vec16<TI> *)(base + off[p] + q * (int)ld);
+        }
+    }
+
     __device__ __forceinline__ static Vec16<TI> guarded(const TI *p, int64_t n_valid) {
         Vec16<TI> r;
 #pragma unroll

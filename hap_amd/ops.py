@@ -270,8 +270,10 @@ def gemm(A: torch.Tensor, B: torch.Tensor, C: torch.Tensor, M: int, N: int, K: i
     else:
         a.workspace, a.workspace_bytes = 0, 0
     zb = lambda st: (batch1 - 1) * st[0] + (batch2 - 1) * st[1]
-    _need(A, _span(K if transA else M, M if transA else K, a.lda) + zb(strideA), "gemm A", offA)
-    _need(B, _span(N if transB else K, K if transB else N, a.ldb) + zb(strideB), "gemm B", offB)
+    epv = 16 // A.element_size()
+    up = lambda n: (n + epv - 1) // epv * epv          # the kernel reads whole 16-byte vectors along a row
+    _need(A, _span(K if transA else M, up(M) if transA else K, a.lda) + zb(strideA), "gemm A", offA)
+    _need(B, _span(N if transB else K, K if transB else up(N), a.ldb) + zb(strideB), "gemm B", offB)
     _need(C, _span(M, N, a.ldc) + zb(strideC), "gemm C", offC)
     _need(bias, N, "gemm bias")
     if min(strideA + strideB + strideC) < 0:
