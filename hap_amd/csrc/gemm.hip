@@ -188,61 +188,76 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void gemm_kernel(GemmParams 
         }
     }
 
-    // epilogue: acc[i][j][r] is C[m, n] with m = wm + i*32 + lane%32, n = wn + j*32 + (r/4)*8 + (lane/32)*4 + r%4
+    // epilogue: acc[i][j][r] is C[m, n] with m = wm + i*32 + lane%32, n = wn + j*32 + (r/4)*8 + (lane/32)*4 + r%4.
+    // Each wave stages one 32-row band of its tile at a time as float32 in a private slice of the (now idle)
+    // operand LDS and reads it back row-wise, so that global stores (and the reads of an accumulating C)
+    // are whole 128/256-byte row segments instead of 8-byte pieces scattered over 32 rows.
     const bool split = p.splits > 1;
     const bool lead = blockIdx.y == 0;                            // the split that adds the bias
-    const int64_t mrow_base = m0 + wm + (lane & 31);
+    constexpr int SROW = WTN * 4 + 16;                            // staged row: WTN floats + 16 B (bank spread)
+    constexpr int NWAVES = WAVES_M * WAVES_N;
+    static_assert(32 * SROW * NWAVES <= 2 * (A_BYTES + B_BYTES), "epilogue staging does not fit the operand LDS");
+    char *stage = smem + wave * (32 * SROW);
+    constexpr int QPR = WTN / 4;                                  // float4 groups per staged row
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
-        const int64_t m = mrow_base + i * 32;
-        if (m >= p.M) continue;
 #pragma unroll
-        for (int j = 0; j < TN; ++j) {
+        for (int j = 0; j < TN; ++j)
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-                const int64_t n = n0 + wn + j * 32 + q * 8 + (lane >> 5) * 4;
-                if (n >= p.N) continue;
-                float v[4];
+                f32x4 o;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) v[e] = acc[i][j][q * 4 + e] * p.alpha;
-                TO *dst = C + m * p.ldc + n;
-                const bool full = (n + 4 <= p.N);
-                if (p.bias && lead) {
+                for (int e = 0; e < 4; ++e) o[e] = acc[i][j][q * 4 + e] * p.alpha;
+                *(f32x4 *)(stage + (lane & 31) * SROW + (j * 32 + q * 8 + (lane >> 5) * 4) * 4) = o;
+            }
+        // read back: 32 rows x QPR groups, 64 groups per pass, consecutive lanes along a row
 #pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        if (full || n + e < p.N) v[e] += p.bias[n + e];
+        for (int g0 = 0; g0 < 32 * QPR; g0 += 64) {
+            const int gidx = g0 + lane;
+            if ((32 * QPR) % 64 != 0 && gidx >= 32 * QPR) break;
+            const int row = gidx / QPR, qc = gidx % QPR;
+            const int64_t m = m0 + wm + i * 32 + row;
+            const int64_t n = n0 + wn + qc * 4;
+            if (m >= p.M || n >= p.N) continue;
+            const f32x4 sv = *(const f32x4 *)(stage + row * SROW + qc * 16);
+            float v[4] = {sv[0], sv[1], sv[2], sv[3]};
+            const bool full = (n + 4 <= p.N);
+            if (p.bias && lead) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (full || n + e < p.N) v[e] += p.bias[n + e];
+            }
+            if (split) {
+                // partial sums of this k-range go to the workspace [split][M][Npad]; a second kernel adds them
+                // up in split order and applies activation / accumulation
+                float *w = p.ws + ((int64_t)blockIdx.y * p.M + m) * p.ws_ld + n;
+                f32x4 o = {v[0], v[1], v[2], v[3]};
+                *(f32x4 *)w = o;                                  // ws_ld is a multiple of 4 and >= N rounded up
+                continue;
+            }
+            if (p.act != HAPMI_ACT_NONE) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = apply_act(v[e], p.act);
+            }
+            TO *dst = C + m * p.ldc + n;
+            if (full && ((p.ldc & 3) == 0)) {
+                typedef TO out4_t __attribute__((ext_vector_type(4)));
+                if (p.accumulate) {
+                    const out4_t old = *(const out4_t *)dst;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] += (float)old[e];
                 }
-                if (split) {
-                    // partial sums of this k-range go to the workspace [split][M][Npad]; a second kernel
-                    // adds them up in split order and applies bias / activation / accumulation
-                    float *w = p.ws + ((int64_t)blockIdx.y * p.M + m) * p.ws_ld + n;
-                    f32x4 o = {v[0], v[1], v[2], v[3]};
-                    *(f32x4 *)w = o;                              // ws_ld is a multiple of 4 and >= N rounded up
-                    continue;
-                }
-                if (p.act != HAPMI_ACT_NONE) {
+                out4_t o;
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) v[e] = apply_act(v[e], p.act);
-                }
-                if (full && ((p.ldc & 3) == 0)) {
-                    typedef TO out4_t __attribute__((ext_vector_type(4)));
-                    if (p.accumulate) {
-                        const out4_t old = *(const out4_t *)dst;
+                for (int e = 0; e < 4; ++e) o[e] = (TO)v[e];
+                *(out4_t *)dst = o;
+            } else {
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) v[e] += (float)old[e];
-                    }
-                    out4_t o;
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) o[e] = (TO)v[e];
-                    *(out4_t *)dst = o;
-                } else {
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        if (n + e < p.N) {
-                            float x = v[e];
-                            if (p.accumulate) x += (float)dst[e];
-                            dst[e] = (TO)x;
-                        }
+                for (int e = 0; e < 4; ++e) {
+                    if (n + e < p.N) {
+                        float x = v[e];
+                        if (p.accumulate) x += (float)dst[e];
+                        dst[e] = (TO)x;
                     }
                 }
             }
