@@ -135,6 +135,39 @@ __global__ __launch_bounds__(256) void colsum_kernel(const T *x, float *out, int
     if (rg == 0 && col < N) atomicAdd(out + col, part[0][c] + part[1][c] + part[2][c] + part[3][c]);
 }
 
+// vectorised form: 32 column groups of one 16-byte vector x 8 row groups per block
+constexpr int CSV_ROWS_PER_BLOCK = 128;
+template <typename T>
+__global__ __launch_bounds__(256) void colsum_vec_kernel(const T *x, float *out, int64_t M, int64_t N, int64_t ldx) {
+    constexpr int EPV = Vec16<T>::N;
+    __shared__ float part[8][32 * EPV + 1];
+    const int cg = threadIdx.x & 31, rg = threadIdx.x >> 5;
+    const int64_t col = ((int64_t)blockIdx.x * 32 + cg) * EPV;
+    const int64_t r0 = (int64_t)blockIdx.y * CSV_ROWS_PER_BLOCK;
+    const int64_t r1 = r0 + CSV_ROWS_PER_BLOCK < M ? r0 + CSV_ROWS_PER_BLOCK : M;
+    float s[EPV];
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) s[e] = 0.f;
+    if (col < N)                                              // N is a multiple of EPV on this path
+        for (int64_t r = r0 + rg; r < r1; r += 8) {
+            const Vec16<T> v = *(const Vec16<T> *)(x + r * ldx + col);
+#pragma unroll
+            for (int e = 0; e < EPV; ++e) s[e] += v.get(e);
+        }
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) part[rg][cg * EPV + e] = s[e];
+    __syncthreads();
+    for (int c = threadIdx.x; c < 32 * EPV; c += 256) {
+        const int64_t gc = (int64_t)blockIdx.x * 32 * EPV + c;
+        if (gc < N) {
+            float t = 0.f;
+#pragma unroll
+            for (int g = 0; g < 8; ++g) t += part[g][c];
+            atomicAdd(out + gc, t);
+        }
+    }
+}
+
 template <typename TS, typename TD>
 __global__ __launch_bounds__(EW_THREADS) void cast_kernel(const TS *s, TD *d, int64_t n) {
     const int64_t step = (int64_t)gridDim.x * EW_THREADS * 4;
@@ -194,6 +227,14 @@ extern "C" int hapmi_colsum(const void *x, float *out, int64_t M, int64_t N, int
         hipLaunchKernelGGL(zero_f32_kernel, dim3(ew_grid(N)), dim3(EW_THREADS), 0, (hipStream_t)stream, out, N);
     }
     if (M == 0) return HAPMI_OK;
+    const int64_t epv = dtype == HAPMI_F32 ? 4 : 8;
+    if (aligned16(x) && ldx % epv == 0 && N % epv == 0) {
+        dim3 vgrid((unsigned)hapmi_cdiv(N, 32 * epv), (unsigned)hapmi_cdiv(M, CSV_ROWS_PER_BLOCK));
+        if (dtype == HAPMI_F32) hipLaunchKernelGGL((colsum_vec_kernel<float>), vgrid, dim3(256), 0, (hipStream_t)stream, (const float *)x, out, M, N, ldx);
+        else hipLaunchKernelGGL((colsum_vec_kernel<bf16_t>), vgrid, dim3(256), 0, (hipStream_t)stream, (const bf16_t *)x, out, M, N, ldx);
+        HAPMI_CHECK_LAUNCH("colsum");
+        return HAPMI_OK;
+    }
     dim3 grid((unsigned)hapmi_cdiv(N, 64), (unsigned)hapmi_cdiv(M, CS_ROWS_PER_BLOCK));
     if (dtype == HAPMI_F32) hipLaunchKernelGGL((colsum_kernel<float>), grid, dim3(256), 0, (hipStream_t)stream, (const float *)x, out, M, N, ldx);
     else hipLaunchKernelGGL((colsum_kernel<bf16_t>), grid, dim3(256), 0, (hipStream_t)stream, (const bf16_t *)x, out, M, N, ldx);
@@ -387,8 +428,22 @@ __device__ __forceinline__ float adam_one(float p, float g, float &m, float &v, 
     return p - (h.lr / h.bc1) * (m / denom);
 }
 
+// state = {step count, 1 - beta1^step, 1 - beta2^step}: advanced on the device so that a captured HIP graph,
+// whose kernel arguments are frozen, still sees the right bias corrections on every replay
+__global__ void adam_advance_kernel(float *state, float beta1, float beta2) {
+    const double step = (double)state[0] + 1.0;
+    state[0] = (float)step;
+    state[1] = (float)(1.0 - pow((double)beta1, step));
+    state[2] = (float)(1.0 - pow((double)beta2, step));
+}
+
 __global__ __launch_bounds__(EW_THREADS) void adam_kernel(float *p, const float *g, float *m, float *v, bf16_t *shadow,
-                                                        int64_t n, AdamHyper h, const float *gscale) {
+                                                        int64_t n, AdamHyper h, const float *gscale,
+                                                        const float *state) {
+    if (state) {
+        h.bc1 = state[1];
+        h.bc2 = state[2];
+    }
     const float gs = gscale ? gscale[0] : 1.0f;
     const int64_t nv = n / 4, step = (int64_t)gridDim.x * EW_THREADS;
     for (int64_t i = (int64_t)blockIdx.x * EW_THREADS + threadIdx.x; i < nv; i += step) {
@@ -458,8 +513,25 @@ extern "C" int hapmi_adam_step(float *param, const float *grad, float *exp_avg, 
                       (!shadow || ((uintptr_t)shadow % 8) == 0),
                   HAPMI_EALIGN, "adam_step: misaligned buffer");
     AdamHyper h{lr, beta1, beta2, eps, bias_corr1, bias_corr2};
-    hipLaunchKernelGGL(adam_kernel, dim3(ew_grid(hapmi_cdiv(n, 4))), dim3(EW_THREADS), 0, (hipStream_t)stream, param, grad, exp_avg, exp_avg_sq, (bf16_t *)shadow, n, h, grad_scale_dev);
+    hipLaunchKernelGGL(adam_kernel, dim3(ew_grid(hapmi_cdiv(n, 4))), dim3(EW_THREADS), 0, (hipStream_t)stream, param, grad, exp_avg, exp_avg_sq, (bf16_t *)shadow, n, h, grad_scale_dev, (const float *)nullptr);
     HAPMI_CHECK_LAUNCH("adam_step");
+    return HAPMI_OK;
+}
+
+extern "C" int hapmi_adam_step_dev(float *param, const float *grad, float *exp_avg, float *exp_avg_sq, void *shadow,
+                                   int64_t n, float lr, float beta1, float beta2, float eps, float *state_dev,
+                                   const float *grad_scale_dev, hapmi_stream_t stream) {
+    HAPMI_REQUIRE(n >= 0, HAPMI_EINVAL, "adam_step_dev: negative size");
+    HAPMI_REQUIRE(state_dev, HAPMI_EINVAL, "adam_step_dev: null state");
+    hipLaunchKernelGGL(adam_advance_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream, state_dev, beta1, beta2);
+    if (n == 0) return HAPMI_OK;
+    HAPMI_REQUIRE(param && grad && exp_avg && exp_avg_sq, HAPMI_EINVAL, "adam_step_dev: null pointer");
+    HAPMI_REQUIRE(aligned16(param) && aligned16(grad) && aligned16(exp_avg) && aligned16(exp_avg_sq) &&
+                      (!shadow || ((uintptr_t)shadow % 8) == 0),
+                  HAPMI_EALIGN, "adam_step_dev: misaligned buffer");
+    AdamHyper h{lr, beta1, beta2, eps, 1.f, 1.f};
+    hipLaunchKernelGGL(adam_kernel, dim3(ew_grid(hapmi_cdiv(n, 4))), dim3(EW_THREADS), 0, (hipStream_t)stream, param, grad, exp_avg, exp_avg_sq, (bf16_t *)shadow, n, h, grad_scale_dev, (const float *)state_dev);
+    HAPMI_CHECK_LAUNCH("adam_step_dev");
     return HAPMI_OK;
 }
 

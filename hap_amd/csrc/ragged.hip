@@ -5,6 +5,8 @@
 
 namespace {
 
+int g_grid_shift = 2;      // grid cap = 4096 << shift blocks (hapmi_ragged_tuning changes it for measurements)
+
 struct Segment {
     const char *src;
     char *dst;
@@ -102,7 +104,7 @@ int launch_segments(const SegmentList &list, int act, int dtype, hipStream_t str
     }
     if (max_chunks == 0) return HAPMI_OK;
     int64_t gx = hapmi_cdiv(max_chunks, (int64_t)COPY_THREADS * COPY_UNROLL);
-    const int64_t cap = hapmi_cdiv(256 * 16, list.n);   // ~16 blocks per CU over all segments
+    const int64_t cap = hapmi_cdiv((int64_t)(256 * 16) << g_grid_shift, list.n);   // blocks over all segments
     if (gx > cap) gx = cap;
     if (gx < 1) gx = 1;
     dim3 grid((unsigned)gx, (unsigned)list.n), block(COPY_THREADS);
@@ -283,47 +285,99 @@ struct ReduceArgs {
 
 constexpr int RED_THREADS = 256;
 
-template <typename T, int NW>
-__global__ __launch_bounds__(RED_THREADS) void ragged_reduce_kernel(ReduceArgs a, T *dst, int64_t outer,
-                                                                   int64_t src_len, int64_t offset, int64_t len,
-                                                                   int64_t inner, int n_dyn) {
+int g_red_variant = 0;      // measurement hook: bit0 nontemporal loads, bit1 nontemporal store, bit2 two vectors per thread
+
+struct ReduceOut {
+    void *dst;
+    int64_t offset, len;       // rows [offset, offset + len) of the sharded dimension
+};
+struct ReduceOuts {
+    int n;
+    ReduceOut out[HAPMI_MAX_RANKS];
+};
+
+template <typename T> __device__ __forceinline__ Vec16<T> ldv(const T *p, bool nt) {
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    union { u32x4 u; Vec16<T> v; } x;
+    x.u = nt ? __builtin_nontemporal_load((const u32x4 *)p) : *(const u32x4 *)p;
+    return x.v;
+}
+template <typename T> __device__ __forceinline__ void stv(T *p, const Vec16<T> &v, bool nt) {
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    union { u32x4 u; Vec16<T> v; } x;
+    x.v = v;
+    if (nt) __builtin_nontemporal_store(x.u, (u32x4 *)p);
+    else *(u32x4 *)p = x.u;
+}
+
+// blockIdx.y selects the output shard; every output is outs.out[y].len rows of the rank-ordered float32 sum
+template <typename T, int NW, int VAR>
+__global__ __launch_bounds__(RED_THREADS) void ragged_reduce_kernel(ReduceArgs a, ReduceOuts outs, int64_t outer,
+                                                                   int64_t src_len, int64_t inner, int n_dyn) {
     constexpr int EPV = Vec16<T>::N;
+    constexpr int U = (VAR & 4) ? 2 : 1;
+    constexpr bool NTL = VAR & 1, NTS = VAR & 2;
+    const ReduceOut od = outs.out[blockIdx.y];
+    T *dst = (T *)od.dst;
+    const int64_t offset = od.offset, len = od.len;
     const uint64_t vec_per_row = (uint64_t)(len * inner) / EPV;     // contiguous run per outer index
     const uint64_t total = vec_per_row * (uint64_t)outer;
-    const uint64_t step = (uint64_t)gridDim.x * RED_THREADS;
+    const uint64_t step = (uint64_t)gridDim.x * RED_THREADS * U;
     const int nw = NW > 0 ? NW : n_dyn;
-    for (uint64_t c = (uint64_t)blockIdx.x * RED_THREADS + threadIdx.x; c < total; c += step) {
-        uint64_t o = 0, col = c;
-        if (outer > 1) {
-            o = c / vec_per_row;
-            col = c - o * vec_per_row;
+    for (uint64_t c0 = (uint64_t)blockIdx.x * RED_THREADS * U + threadIdx.x; c0 < total; c0 += step) {
+        uint64_t soff[U], doff[U];
+        bool ok[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const uint64_t c = c0 + (uint64_t)u * RED_THREADS;
+            ok[u] = c < total;
+            uint64_t o = 0, col = c;
+            if (outer > 1) {
+                o = c / vec_per_row;
+                col = c - o * vec_per_row;
+            }
+            soff[u] = (o * (uint64_t)src_len + (uint64_t)offset) * (uint64_t)inner + col * EPV;
+            doff[u] = (o * (uint64_t)len) * (uint64_t)inner + col * EPV;
         }
-        const uint64_t soff = (o * (uint64_t)src_len + (uint64_t)offset) * (uint64_t)inner + col * EPV;
-        float acc[EPV];
+        float acc[U][EPV];
         if (NW > 0) {
-            Vec16<T> v[NW > 0 ? NW : 1];
+            Vec16<T> v[U][NW > 0 ? NW : 1];
 #pragma unroll
-            for (int w = 0; w < NW; ++w) v[w] = *(const Vec16<T> *)((const T *)a.src[w] + soff);
+            for (int u = 0; u < U; ++u)
 #pragma unroll
-            for (int e = 0; e < EPV; ++e) acc[e] = v[0].get(e);
+                for (int w = 0; w < NW; ++w)
+                    if (ok[u]) v[u][w] = ldv((const T *)a.src[w] + soff[u], NTL);
 #pragma unroll
-            for (int w = 1; w < NW; ++w)
+            for (int u = 0; u < U; ++u) {
 #pragma unroll
-                for (int e = 0; e < EPV; ++e) acc[e] += v[w].get(e);
+                for (int e = 0; e < EPV; ++e) acc[u][e] = v[u][0].get(e);
+#pragma unroll
+                for (int w = 1; w < NW; ++w)
+#pragma unroll
+                    for (int e = 0; e < EPV; ++e) acc[u][e] += v[u][w].get(e);
+            }
         } else {
-            Vec16<T> v = *(const Vec16<T> *)((const T *)a.src[0] + soff);
 #pragma unroll
-            for (int e = 0; e < EPV; ++e) acc[e] = v.get(e);
-            for (int w = 1; w < nw; ++w) {
-                v = *(const Vec16<T> *)((const T *)a.src[w] + soff);
+            for (int u = 0; u < U; ++u) {
+                if (!ok[u]) continue;
+                Vec16<T> v = ldv((const T *)a.src[0] + soff[u], NTL);
 #pragma unroll
-                for (int e = 0; e < EPV; ++e) acc[e] += v.get(e);
+                for (int e = 0; e < EPV; ++e) acc[u][e] = v.get(e);
+                for (int w = 1; w < nw; ++w) {
+                    v = ldv((const T *)a.src[w] + soff[u], NTL);
+#pragma unroll
+                    for (int e = 0; e < EPV; ++e) acc[u][e] += v.get(e);
+                }
             }
         }
-        Vec16<T> r;
 #pragma unroll
-        for (int e = 0; e < EPV; ++e) r.set(e, acc[e]);
-        *(Vec16<T> *)(dst + (o * (uint64_t)len) * (uint64_t)inner + col * EPV) = r;
+        for (int u = 0; u < U; ++u) {
+            if (!ok[u]) continue;
+            Vec16<T> r;
+#pragma unroll
+            for (int e = 0; e < EPV; ++e) r.set(e, acc[u][e]);
+            stv(dst + doff[u], r, NTS);
+        }
     }
 }
 
@@ -343,41 +397,67 @@ __global__ __launch_bounds__(RED_THREADS) void ragged_reduce_scalar_kernel(Reduc
     }
 }
 
-template <typename T>
-int launch_reduce(const ReduceArgs &a, void *dst, int64_t outer, int64_t src_len, int64_t offset, int64_t len,
-                  int64_t inner, hipStream_t stream) {
-    constexpr int EPV = Vec16<T>::N;
-    const int64_t esz = sizeof(T);
-    bool vec_ok = ((len * inner) % EPV == 0) && ((src_len * inner) % EPV == 0) && ((offset * inner) % EPV == 0) &&
-                  ((uintptr_t)dst % 16 == 0);
-    for (int w = 0; w < a.n; ++w) vec_ok = vec_ok && ((uintptr_t)a.src[w] % 16 == 0);
-    (void)esz;
-    if (vec_ok) {
-        const int64_t total = outer * (len * inner / EPV);
-        int64_t gx = hapmi_cdiv(total, RED_THREADS);
-        if (gx > 256 * 16) gx = 256 * 16;
-        dim3 grid((unsigned)gx), block(RED_THREADS);
-        switch (a.n) {
-#define HAPMI_RED_CASE(NW)                                                                                   \
-    case NW:                                                                                                 \
-        hipLaunchKernelGGL((ragged_reduce_kernel<T, NW>), grid, block, 0, stream, a, (T *)dst, outer, src_len, \
-                           offset, len, inner, a.n);                                                         \
+template <typename T, int VAR>
+void launch_reduce_var(const ReduceArgs &a, const ReduceOuts &outs, int64_t outer, int64_t src_len, int64_t inner,
+                       dim3 grid, hipStream_t stream) {
+    dim3 block(RED_THREADS);
+    switch (a.n) {
+#define HAPMI_RED_CASE(NW)                                                                                        \
+    case NW:                                                                                                      \
+        hipLaunchKernelGGL((ragged_reduce_kernel<T, NW, VAR>), grid, block, 0, stream, a, outs, outer, src_len, inner, \
+                           a.n);                                                                                  \
         break;
-            HAPMI_RED_CASE(1)
-            HAPMI_RED_CASE(2)
-            HAPMI_RED_CASE(4)
-            HAPMI_RED_CASE(8)
+        HAPMI_RED_CASE(1)
+        HAPMI_RED_CASE(2)
+        HAPMI_RED_CASE(4)
+        HAPMI_RED_CASE(8)
 #undef HAPMI_RED_CASE
-            default:
-                hipLaunchKernelGGL((ragged_reduce_kernel<T, 0>), grid, block, 0, stream, a, (T *)dst, outer, src_len,
-                                   offset, len, inner, a.n);
+        default:
+            hipLaunchKernelGGL((ragged_reduce_kernel<T, 0, VAR>), grid, block, 0, stream, a, outs, outer, src_len, inner,
+                               a.n);
+    }
+}
+
+template <typename T>
+int launch_reduce(const ReduceArgs &a, const ReduceOuts &outs, int64_t outer, int64_t src_len, int64_t inner,
+                  hipStream_t stream) {
+    constexpr int EPV = Vec16<T>::N;
+    bool vec_ok = ((src_len * inner) % EPV == 0);
+    int64_t max_len = 0;
+    for (int r = 0; r < outs.n; ++r) {
+        const ReduceOut &o = outs.out[r];
+        vec_ok = vec_ok && ((o.len * inner) % EPV == 0) && ((o.offset * inner) % EPV == 0) && ((uintptr_t)o.dst % 16 == 0);
+        if (o.len > max_len) max_len = o.len;
+    }
+    for (int w = 0; w < a.n; ++w) vec_ok = vec_ok && ((uintptr_t)a.src[w] % 16 == 0);
+    if (vec_ok) {
+        const int u = (g_red_variant & 4) ? 2 : 1;
+        const int64_t total = outer * (max_len * inner / EPV);
+        int64_t gx = hapmi_cdiv(total, (int64_t)RED_THREADS * u);
+        const int64_t cap = hapmi_cdiv((int64_t)(256 * 16) << g_grid_shift, outs.n);
+        if (gx > cap) gx = cap;
+        if (gx < 1) gx = 1;
+        dim3 grid((unsigned)gx, (unsigned)outs.n);
+        switch (g_red_variant & 7) {
+            case 1: launch_reduce_var<T, 1>(a, outs, outer, src_len, inner, grid, stream); break;
+            case 2: launch_reduce_var<T, 2>(a, outs, outer, src_len, inner, grid, stream); break;
+            case 3: launch_reduce_var<T, 3>(a, outs, outer, src_len, inner, grid, stream); break;
+            case 4: launch_reduce_var<T, 4>(a, outs, outer, src_len, inner, grid, stream); break;
+            case 5: launch_reduce_var<T, 5>(a, outs, outer, src_len, inner, grid, stream); break;
+            case 6: launch_reduce_var<T, 6>(a, outs, outer, src_len, inner, grid, stream); break;
+            case 7: launch_reduce_var<T, 7>(a, outs, outer, src_len, inner, grid, stream); break;
+            default: launch_reduce_var<T, 0>(a, outs, outer, src_len, inner, grid, stream);
         }
     } else {
-        const int64_t total = outer * len * inner;
-        int64_t gx = hapmi_cdiv(total, RED_THREADS);
-        if (gx > 256 * 16) gx = 256 * 16;
-        hipLaunchKernelGGL((ragged_reduce_scalar_kernel<T>), dim3((unsigned)gx), dim3(RED_THREADS), 0, stream, a,
-                           (T *)dst, outer, src_len, offset, len, inner);
+        for (int r = 0; r < outs.n; ++r) {
+            const ReduceOut &o = outs.out[r];
+            const int64_t total = outer * o.len * inner;
+            if (total == 0) continue;
+            int64_t gx = hapmi_cdiv(total, RED_THREADS);
+            if (gx > 256 * 16) gx = 256 * 16;
+            hipLaunchKernelGGL((ragged_reduce_scalar_kernel<T>), dim3((unsigned)gx), dim3(RED_THREADS), 0, stream, a,
+                               (T *)o.dst, outer, src_len, o.offset, o.len, inner);
+        }
     }
     HAPMI_CHECK_LAUNCH("ragged_reduce");
     return HAPMI_OK;
@@ -388,20 +468,64 @@ int launch_reduce(const ReduceArgs &a, void *dst, int64_t outer, int64_t src_len
 extern "C" int hapmi_ragged_reduce(const void *const *contribs, int n_ranks, void *dst, int64_t outer,
                                    int64_t src_len, int64_t offset, int64_t len, int64_t inner, int dtype,
                                    hapmi_stream_t stream) {
+    void *dsts[1] = {dst};
+    const int64_t offs[1] = {offset}, lens[1] = {len};
+    return hapmi_ragged_reduce_multi(contribs, n_ranks, dsts, offs, lens, 1, outer, src_len, inner, dtype, stream);
+}
+
+extern "C" int hapmi_ragged_reduce_multi(const void *const *contribs, int n_ranks, void *const *dsts,
+                                         const int64_t *offsets, const int64_t *lengths, int n_outputs,
+                                         int64_t outer, int64_t src_len, int64_t inner, int dtype,
+                                         hapmi_stream_t stream) {
     HAPMI_REQUIRE(n_ranks >= 1 && n_ranks <= HAPMI_MAX_RANKS && contribs, HAPMI_EINVAL,
                   "ragged_reduce: n_ranks %d outside 1..%d", n_ranks, HAPMI_MAX_RANKS);
+    HAPMI_REQUIRE(n_outputs >= 1 && n_outputs <= HAPMI_MAX_RANKS && dsts && offsets && lengths, HAPMI_EINVAL,
+                  "ragged_reduce: n_outputs %d outside 1..%d", n_outputs, HAPMI_MAX_RANKS);
     HAPMI_REQUIRE(hapmi_dtype_ok(dtype), HAPMI_EINVAL, "ragged_reduce: bad dtype %d", dtype);
-    HAPMI_REQUIRE(outer >= 0 && len >= 0 && inner > 0 && offset >= 0 && offset + len <= src_len, HAPMI_EINVAL,
-                  "ragged_reduce: [%lld, %lld) outside 0..%lld", (long long)offset, (long long)(offset + len),
-                  (long long)src_len);
-    if (outer == 0 || len == 0) return HAPMI_OK;
+    HAPMI_REQUIRE(outer >= 0 && inner > 0 && src_len >= 0, HAPMI_EINVAL, "ragged_reduce: bad shape");
+    ReduceOuts outs;
+    outs.n = 0;
+    for (int r = 0; r < n_outputs; ++r) {
+        HAPMI_REQUIRE(lengths[r] >= 0 && offsets[r] >= 0 && offsets[r] + lengths[r] <= src_len, HAPMI_EINVAL,
+                      "ragged_reduce: [%lld, %lld) outside 0..%lld", (long long)offsets[r],
+                      (long long)(offsets[r] + lengths[r]), (long long)src_len);
+        if (lengths[r] == 0 || outer == 0) continue;
+        HAPMI_REQUIRE(dsts[r], HAPMI_EINVAL, "ragged_reduce: null destination");
+        outs.out[outs.n++] = ReduceOut{dsts[r], offsets[r], lengths[r]};
+    }
+    if (outs.n == 0) return HAPMI_OK;
     ReduceArgs a;
     a.n = n_ranks;
     for (int w = 0; w < n_ranks; ++w) {
         HAPMI_REQUIRE(contribs[w], HAPMI_EINVAL, "ragged_reduce: contribution %d is NULL", w);
         a.src[w] = contribs[w];
     }
-    HAPMI_REQUIRE(dst, HAPMI_EINVAL, "ragged_reduce: null destination");
-    if (dtype == HAPMI_F32) return launch_reduce<float>(a, dst, outer, src_len, offset, len, inner, (hipStream_t)stream);
-    return launch_reduce<bf16_t>(a, dst, outer, src_len, offset, len, inner, (hipStream_t)stream);
+    if (dtype == HAPMI_F32) return launch_reduce<float>(a, outs, outer, src_len, inner, (hipStream_t)stream);
+    return launch_reduce<bf16_t>(a, outs, outer, src_len, inner, (hipStream_t)stream);
+}
+
+extern "C" int hapmi_pad_rows_multi(const void *const *srcs, void *const *dsts, const int64_t *lengths, int n_shards,
+                                    int64_t outer, int64_t padded_len, int64_t inner_bytes, hapmi_stream_t stream) {
+    int64_t total;
+    int rc = check_lengths(lengths, n_shards, &total, "pad_rows_multi");
+    if (rc) return rc;
+    HAPMI_REQUIRE(outer >= 0 && inner_bytes > 0 && srcs && dsts, HAPMI_EINVAL, "pad_rows_multi: bad argument");
+    SegmentList list;
+    list.n = 0;
+    for (int i = 0; i < n_shards; ++i) {
+        HAPMI_REQUIRE(lengths[i] <= padded_len, HAPMI_EINVAL, "pad_rows_multi: length %lld above padded length %lld",
+                      (long long)lengths[i], (long long)padded_len);
+        if (lengths[i] > 0 && outer > 0) {
+            HAPMI_REQUIRE(srcs[i] && dsts[i], HAPMI_EINVAL, "pad_rows_multi: null pointer");
+            list.seg[list.n++] = {(const char *)srcs[i], (char *)dsts[i], outer, lengths[i] * inner_bytes,
+                                  lengths[i] * inner_bytes, padded_len * inner_bytes};
+        }
+    }
+    return launch_segments(list, HAPMI_ACT_NONE, 0, (hipStream_t)stream, "pad_rows_multi");
+}
+
+extern "C" int hapmi_ragged_tuning(int reduce_variant, int grid_shift) {
+    g_red_variant = reduce_variant < 0 ? 0 : (reduce_variant & 7);
+    g_grid_shift = grid_shift < 0 ? 2 : (grid_shift & 7);
+    return HAPMI_OK;
 }

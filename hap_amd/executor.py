@@ -105,15 +105,24 @@ class ShardExecutor:
         self.param_names, self.buffers = [], {}
         metas = []
         off = 0
+        found = []
         for name in used:
             obj = self._fetch(name)
             if isinstance(obj, torch.nn.Parameter):
-                n = obj.numel()
-                metas.append((name, obj, off, n))
-                off += _round_up(n, 64)        # keep every view 256-byte aligned
-                self.param_names.append(name)
+                found.append((name, obj))
             else:
                 self.buffers[name] = obj
+        # vectors (biases) first and contiguous: their gradients are column sums accumulated with atomics, so
+        # one fill per step clears all of them
+        found.sort(key=lambda kv: 0 if kv[1].dim() == 1 else 1)
+        self.n_vector_region = 0
+        for name, obj in found:
+            n = obj.numel()
+            metas.append((name, obj, off, n))
+            off += _round_up(n, 64)            # keep every view 256-byte aligned
+            if obj.dim() == 1:
+                self.n_vector_region = off
+            self.param_names.append(name)
         self.n_flat = off
         self.master = torch.zeros(max(off, 4), dtype=torch.float32, device=self.dev)
         self.flat_grad = torch.zeros_like(self.master)
@@ -161,6 +170,8 @@ class ShardExecutor:
     def _param_grad_slot(self, v: Val):
         first = not v.meta.get("grad_written", False)
         v.meta["grad_written"] = True
+        if v.meta["grad"].dim() == 1:
+            return v.meta["grad"], True       # the vector region is cleared once at the start of backward
         return v.meta["grad"], not first
 
     def _unsupported(self, node, why):
@@ -975,6 +986,8 @@ class ShardExecutor:
         return self.loss[0]
 
     def backward(self):
+        if self.n_vector_region:
+            ops.fill_zero(self.flat_grad[:self.n_vector_region])
         for f in self.bwd:
             f()
         self._reduce_replicated_grads()
@@ -992,6 +1005,7 @@ class ShardExecutor:
         if kind == "adam":
             self.exp_avg = torch.zeros_like(self.master)
             self.exp_avg_sq = torch.zeros_like(self.master)
+            self._adam_state = torch.zeros(4, dtype=torch.float32, device=self.dev)   # step, 1-b1^t, 1-b2^t
         if clip_grad_norm is not None:
             self._sumsq = torch.zeros(1, dtype=torch.float32, device=self.dev)
             self._coef = torch.ones(1, dtype=torch.float32, device=self.dev)
@@ -1011,8 +1025,8 @@ class ShardExecutor:
         if o["kind"] == "sgd":
             ops.sgd_step(self.master, self.flat_grad, self.shadow, o["lr"], coef)
         else:
-            ops.adam_step(self.master, self.flat_grad, self.exp_avg, self.exp_avg_sq, self.shadow, o["lr"],
-                          o["betas"][0], o["betas"][1], o["eps"], self._step_count, coef)
+            ops.adam_step_dev(self.master, self.flat_grad, self.exp_avg, self.exp_avg_sq, self.shadow, o["lr"],
+                              o["betas"][0], o["betas"][1], o["eps"], self._adam_state, coef)
 
     def train_step(self, *args) -> torch.Tensor:
         loss = self.forward(*args)

@@ -224,6 +224,48 @@ def ragged_reduce(contribs: Sequence[torch.Tensor], dim: int, offset: int, lengt
     return out
 
 
+def ragged_reduce_multi(contribs: Sequence[torch.Tensor], dim: int, offsets: Sequence[int], lengths: Sequence[int],
+                        outs: Optional[Sequence[torch.Tensor]] = None) -> List[torch.Tensor]:
+    """One launch for several output shards: outs[r] = sum_w contribs[w].narrow(dim, offsets[r], lengths[r])."""
+    _dev(*contribs)
+    ref = contribs[0]
+    outer, src_len, inner = _oli(ref.shape, dim)
+    if outs is None:
+        outs = [torch.empty(_with_dim(ref.shape, dim, l), dtype=ref.dtype, device=ref.device) for l in lengths]
+    for c in contribs:
+        _need(c, outer * src_len * inner, "ragged_reduce contribution")
+        if c.dtype != ref.dtype:
+            raise TypeError("ragged_reduce: dtype mismatch")
+    for o, off, l in zip(outs, offsets, lengths):
+        _dev(o)
+        _need(o, outer * l * inner, "ragged_reduce dst")
+        if o.dtype != ref.dtype or off < 0 or off + l > src_len:
+            raise _lib.HapmiError("ragged_reduce_multi: bad output shard")
+    check(lib().hapmi_ragged_reduce_multi(_ptrs(contribs), len(contribs), _ptrs(outs), _i64(offsets), _i64(lengths),
+                                          len(lengths), outer, src_len, inner, dtype_code(ref), _stream()))
+    return list(outs)
+
+
+def pad_rows_multi(srcs: Sequence[torch.Tensor], dim: int, padded_len: int,
+                   outs: Optional[Sequence[torch.Tensor]] = None) -> List[torch.Tensor]:
+    """collectives.padded for several shards in one launch."""
+    _dev(*srcs)
+    ref = srcs[0]
+    outer, _, inner = _oli(ref.shape, dim)
+    lengths = [s.shape[dim] for s in srcs]
+    if outs is None:
+        outs = [torch.empty(_with_dim(ref.shape, dim, padded_len), dtype=ref.dtype, device=ref.device) for _ in srcs]
+    for s, o, l in zip(srcs, outs, lengths):
+        _dev(o)
+        _need(s, outer * l * inner, "pad_rows_multi src")
+        _need(o, outer * padded_len * inner, "pad_rows_multi dst")
+        if o.dtype != ref.dtype or s.dtype != ref.dtype:
+            raise TypeError("pad_rows_multi: dtype mismatch")
+    check(lib().hapmi_pad_rows_multi(_ptrs(srcs), _ptrs(outs), _i64(lengths), len(srcs), outer, padded_len,
+                                     inner * ref.element_size(), _stream()))
+    return list(outs)
+
+
 # ---------------------------------------------------------------------------
 # GEMM
 # ---------------------------------------------------------------------------
@@ -528,6 +570,22 @@ def adam_step(param, grad, exp_avg, exp_avg_sq, shadow, lr, beta1, beta2, eps, s
     check(lib().hapmi_adam_step(_ptr(param), _ptr(grad), _ptr(exp_avg), _ptr(exp_avg_sq), _ptr(shadow), param.numel(),
                                 ctypes.c_float(lr), ctypes.c_float(beta1), ctypes.c_float(beta2), ctypes.c_float(eps),
                                 ctypes.c_float(bc1), ctypes.c_float(bc2), _ptr(grad_scale), _stream()))
+
+
+def adam_step_dev(param, grad, exp_avg, exp_avg_sq, shadow, lr, beta1, beta2, eps, state, grad_scale=None):
+    """Adam with the step count / bias corrections in ``state`` (float32[4] on the device, zero at start)."""
+    _dev(param, grad, exp_avg, exp_avg_sq, shadow, grad_scale, state)
+    for t_ in (grad, exp_avg, exp_avg_sq):
+        _need(t_, param.numel(), "adam_step_dev")
+        if t_.dtype != torch.float32:
+            raise TypeError("adam_step_dev: float32 state expected")
+    _need(shadow, param.numel(), "adam_step_dev shadow")
+    _need(state, 3, "adam_step_dev state")
+    if param.dtype != torch.float32 or state.dtype != torch.float32 or (shadow is not None and shadow.dtype != torch.bfloat16):
+        raise TypeError("adam_step_dev: dtype mismatch")
+    check(lib().hapmi_adam_step_dev(_ptr(param), _ptr(grad), _ptr(exp_avg), _ptr(exp_avg_sq), _ptr(shadow), param.numel(),
+                                    ctypes.c_float(lr), ctypes.c_float(beta1), ctypes.c_float(beta2), ctypes.c_float(eps),
+                                    _ptr(state), _ptr(grad_scale), _stream()))
 
 
 def sumsq(g, out):

@@ -2,10 +2,10 @@
 [S_i, 4096] bf16, S_i uniform in [1000, 3000] from the seed, packed in one GPU's HBM.
 
 Algorithmic bytes (payload read + payload written; pad tails are not credited):
-  pad            2 * sum(S) * 4096 * 2 B   (8 launches, one per shard)
+  pad            2 * sum(S) * 4096 * 2 B   (1 launch for the 8 shards)
   unpad+concat   2 * sum(S) * 4096 * 2 B   (1 launch)
   split+pad      2 * sum(S) * 4096 * 2 B   (1 launch)
-  ragged reduce  9 * sum(S) * 4096 * 2 B   (8 launches, one output shard each: 8 reads + 1 write)
+  ragged reduce  9 * sum(S) * 4096 * 2 B   (1 launch for the 8 output shards: 8 reads + 1 write)
 """
 from __future__ import annotations
 
@@ -49,12 +49,10 @@ def run(steps: int = 50, warmup: int = 10, cpu_baseline: bool = True) -> dict:
     payload = total * WIDTH * 2
 
     def pad_all():
-        for x, p in zip(shards, padded):
-            ops.pad_rows(x, 0, m, p)
+        ops.pad_rows_multi(shards, 0, m, padded)
 
     def reduce_all():
-        for r in range(8):
-            ops.ragged_reduce(fulls, 0, offs[r], S[r], outs[r])
+        ops.ragged_reduce_multi(fulls, 0, offs, S, outs)
 
     t_pad = _time(pad_all, steps, warmup)
     t_cat = _time(lambda: ops.unpad_concat(padded, S, 0, full), steps, warmup)

@@ -96,6 +96,20 @@ int hapmi_concat_rows(const void *const *pieces_host, const int64_t *lengths_hos
 int hapmi_ragged_reduce(const void *const *contribs_host, int n_ranks, void *dst, int64_t outer, int64_t src_len,
                         int64_t offset, int64_t len, int64_t inner, int dtype, hapmi_stream_t stream);
 
+/* The same sum for several output shards in ONE launch (every rank's piece of a reduce_scatter when the
+ * ranks' tensors share one device): dsts[r][outer, lengths[r], inner] = sum_w contribs[w][:, offsets[r]:offsets[r]+lengths[r], :]. */
+int hapmi_ragged_reduce_multi(const void *const *contribs_host, int n_ranks, void *const *dsts_host,
+                              const int64_t *offsets_host, const int64_t *lengths_host, int n_outputs, int64_t outer,
+                              int64_t src_len, int64_t inner, int dtype, hapmi_stream_t stream);
+
+/* collectives.py:9-12 padded() for several shards in ONE launch: dsts[i][outer, padded_len, inner] <- srcs[i][outer, lengths[i], inner]. */
+int hapmi_pad_rows_multi(const void *const *srcs_host, void *const *dsts_host, const int64_t *lengths_host, int n_shards,
+                         int64_t outer, int64_t padded_len, int64_t inner_bytes, hapmi_stream_t stream);
+
+/* Tuning hook for measurements of the kernels above: reduce_variant bit 0 / 1 = non-temporal loads / stores,
+ * bit 2 = two vectors per thread; grid_shift caps the grid at 4096 << shift blocks; -1 = defaults (0, 2). */
+int hapmi_ragged_tuning(int reduce_variant, int grid_shift);
+
 /* ---- GEMM: F.linear (hap.rs:1032) and the expert einsums (hap.rs:2273) --
  * C[z] = op(A[z]) * op(B[z]) (+ bias[N]) (act) (+ C[z] if accumulate)
  * op(A) is [M,K]: transA=0 -> A stored [M,K] (lda), transA=1 -> A stored [K,M];
@@ -242,6 +256,12 @@ int hapmi_sgd_step(float *param, const float *grad, void *shadow, int64_t n, flo
 int hapmi_adam_step(float *param, const float *grad, float *exp_avg, float *exp_avg_sq, void *shadow, int64_t n,
                     float lr, float beta1, float beta2, float eps, float bias_corr1, float bias_corr2,
                     const float *grad_scale_dev, hapmi_stream_t stream);
+/* The same update with the step count and bias corrections held on the device: state_dev[0..2] = {step,
+ * 1 - beta1^step, 1 - beta2^step} (zero-initialised by the caller) is advanced by one and then used, so the
+ * call can be captured in a HIP graph and replayed. */
+int hapmi_adam_step_dev(float *param, const float *grad, float *exp_avg, float *exp_avg_sq, void *shadow, int64_t n,
+                        float lr, float beta1, float beta2, float eps, float *state_dev,
+                        const float *grad_scale_dev, hapmi_stream_t stream);
 /* out[0] += sum g^2 (float32 atomics over block partials; out zeroed by the caller) */
 int hapmi_sumsq(const float *g, int64_t n, float *out, hapmi_stream_t stream);
 /* torch.nn.utils.clip_grad_norm_ coefficient (worker.py:74): coef = min(1, max_norm / (sqrt(sumsq) + 1e-6)) */

@@ -302,3 +302,21 @@ def test_fused_attention_forward_backward(cuda, S, causal):
     ops.attention_bwd(dq, out, dout.to(cuda), lse, dmask, dqkv, delta, b, S, H, scale)
     for name, got, ref in zip("qkv", dqkv.float().cpu().split(E, dim=2), x.grad.split(E, dim=2)):
         assert rel_err(got, ref) < 2e-2, (name, rel_err(got, ref))
+
+
+def test_adam_with_device_step_state_matches_torch(cuda):
+    """The graph-capturable Adam (step count and bias corrections advanced on the device)."""
+    g = torch.Generator().manual_seed(21)
+    n = 777
+    p0 = torch.randn(n, generator=g)
+    ref = p0.clone().requires_grad_(True)
+    opt = torch.optim.Adam([ref], lr=5e-4)
+    p, m, v = p0.clone().to(cuda), torch.zeros(n, device=cuda), torch.zeros(n, device=cuda)
+    state = torch.zeros(4, device=cuda)
+    for i in range(5):
+        gr = torch.randn(n, generator=g)
+        ref.grad = gr.clone()
+        opt.step()
+        ops.adam_step_dev(p, gr.to(cuda), m, v, None, 5e-4, 0.9, 0.999, 1e-8, state)
+    torch.testing.assert_close(p.cpu(), ref.detach(), rtol=1e-5, atol=1e-7)
+    assert state[0].item() == 5.0

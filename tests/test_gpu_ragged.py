@@ -120,3 +120,18 @@ def test_bad_arguments_are_refused(cuda):
         ops.slice_rows(x, 0, 3, 2)
     with pytest.raises(HapmiError):
         ops.pad_rows(x, 0, 3)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_multi_shard_launches_match_single_ones(cuda, dtype):
+    g = torch.Generator().manual_seed(17)
+    L = [5, 0, 9, 2]
+    shards = [torch.randn(3, l, 24, generator=g).to(dtype).to(cuda) for l in L]
+    padded = ops.pad_rows_multi(shards, 1, 9, [torch.full((3, 9, 24), 7, dtype=dtype, device=cuda) for _ in L])
+    for p, s, l in zip(padded, shards, L):
+        assert torch.equal(p[:, :l], s) and (p[:, l:] == 7).all()
+    fulls = [torch.randn(3, 16, 24, generator=g).to(dtype).to(cuda) for _ in range(4)]
+    offs = [0, 5, 5, 14]
+    outs = ops.ragged_reduce_multi(fulls, 1, offs, L)
+    for o, off, l in zip(outs, offs, L):
+        assert torch.equal(o, ops.ragged_reduce(fulls, 1, off, l))
