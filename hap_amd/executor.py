@@ -1034,6 +1034,30 @@ class ShardExecutor:
         self.step()
         return loss
 
+    def capture_train_step(self):
+        """Capture forward + backward + optimizer step (on the inputs loaded last) into a HIP graph and return a
+        ``replay()`` callable.  Everything a step launches is a kernel on static buffers (no memset nodes, no
+        allocation, Adam's step count lives on the device), so replays equal eager steps."""
+        if self._opt is None:
+            raise RuntimeError("configure_optimizer() first")
+        if self._shadow_stale:
+            self.refresh_shadow()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        side = torch.cuda.Stream()
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(graph, stream=side):
+                self.forward()
+                self.backward()
+                self.step()
+        torch.cuda.synchronize()
+        self._graph = graph
+
+        def replay() -> torch.Tensor:
+            graph.replay()
+            return self.loss[0]
+        return replay
+
     def mark_params_dirty(self):
         """Call after parameters were changed from outside (e.g. by a torch.optim optimizer)."""
         self._shadow_stale = True
