@@ -127,6 +127,8 @@ def main():
     ap.add_argument("--workload", default="bert", choices=list(WORKLOADS) + ["ragged"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--graph", action="store_true", help="replay the step from a captured HIP graph")
+    ap.add_argument("--overlap", action="store_true",
+                    help="launch the weight-gradient GEMMs on a second stream (per-kernel event times then overlap)")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py: this build executes ONE device's shard; no collective crosses the device, "
@@ -144,7 +146,8 @@ def main():
     desc, dtype = WORKLOADS[args.workload]
     gm, x, y, meta = build_workload(args.workload)
     wire = hap_amd.SyntheticWire(seed=39, scale=1.0, grad_scale=1e-3, share_shapes=True)
-    ex = hap_amd.compile_program(gm, [x, y], dtype=dtype, wire=wire, rank=0, world_size=len(meta["ratios"]))
+    ex = hap_amd.compile_program(gm, [x, y], dtype=dtype, wire=wire, rank=0, world_size=len(meta["ratios"]),
+                                 overlap_wgrad=args.overlap)
     ex.configure_optimizer(**meta["opt"])
     ex.load_inputs(x, y)                              # inputs resident in HBM before the timed region
     torch.cuda.synchronize()
@@ -207,6 +210,7 @@ def main():
         "dtype": dtype, "data": "synthetic",
         "config": {"workload": desc, "local_batch": meta["local_batch"], "global_batch": meta["global_batch"],
                    "seq_len": meta["seq_len"], "launch": "hip-graph" if graph is not None else "eager",
+                   "wgrad_stream": "side" if args.overlap else "main",
                    "final_loss": loss},
         "roofline": {"bound": "mfma", "kernel": "gemm_kernel (all GEMM launches of the step)",
                      "achieved": achieved, "peak": peak, "unit": "TFLOP/s", "frac": achieved / peak,

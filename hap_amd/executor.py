@@ -58,7 +58,8 @@ def _round_up(n, m):
 
 class ShardExecutor:
     def __init__(self, gm: torch.fx.GraphModule, example_inputs, dtype: str = "fp32", wire: Optional[Wire] = None,
-                 rank: int = 0, world_size: int = 1, device: str = "cuda:0", fused_attention: bool = True):
+                 rank: int = 0, world_size: int = 1, device: str = "cuda:0", fused_attention: bool = True,
+                 overlap_wgrad: bool = False):
         """``example_inputs``: the program's inputs (global batch) as tensors or shapes; activations are
         sized from them.  ``rank`` / ``world_size`` are only needed by all_reduce / replicate, whose node
         forms do not carry them (collectives.py:86, 182)."""
@@ -88,6 +89,18 @@ class ShardExecutor:
         self._param_reduce: List[Callable[[], None]] = []
         self._scratch_pool: Dict[tuple, torch.Tensor] = {}
         self.fused_attention = fused_attention
+        # Optional: weight-gradient GEMMs (and bias column sums) feed nothing but the optimizer, so they can be
+        # launched on a second stream of the same priority, next to the activation-gradient chain on the main
+        # stream; the side stream joins before the gradients of replicated parameters are reduced.  Measured on
+        # the BERT-large shard this hides host launch latency of eager steps (about 6 %), but adds nothing to a
+        # step replayed from a HIP graph, so it is off by default.
+        self.overlap_wgrad = overlap_wgrad
+        self._side_stream = torch.cuda.Stream(device=self.dev) if overlap_wgrad else None
+        self._side_join = torch.cuda.Event() if overlap_wgrad else None
+        self._side_used = False
+        self._side_readers: Dict[int, torch.cuda.Event] = {}   # storage -> event after its last side-stream reader
+        self.side_workspace = torch.empty(64 << 20, dtype=torch.float32, device=self.dev) if overlap_wgrad else None
+        self._single_use_params = self._find_single_use_params(gm)
         self.gemm_workspace = torch.empty(64 << 20, dtype=torch.float32, device=self.dev)   # 256 MiB of split-K scratch
         ops.set_gemm_workspace(self.gemm_workspace)
         self._prepare_params()
@@ -165,6 +178,7 @@ class ShardExecutor:
         if v.grad is None:
             v.grad = self._new(v.t.shape if v.t is not None else v.shape)
             return v.grad, False
+        self._guard_write(v.grad)
         return v.grad, True
 
     def _param_grad_slot(self, v: Val):
@@ -173,6 +187,67 @@ class ShardExecutor:
         if v.meta["grad"].dim() == 1:
             return v.meta["grad"], True       # the vector region is cleared once at the start of backward
         return v.meta["grad"], not first
+
+    @staticmethod
+    def _find_single_use_params(gm):
+        """Names of parameters with exactly one consumer in the program (through replicate / all_gather
+        wrappers): only their gradients can be produced off the main stream without ordering against another
+        contribution."""
+        names = set()
+        for node in gm.graph.nodes:
+            if node.op != "get_attr":
+                continue
+            n, ok = node, True
+            while ok:
+                users = list(n.users)
+                if len(users) != 1:
+                    ok = False
+                elif users[0].op == "call_function" and users[0].target in (collectives.replicate, collectives.all_gather,
+                                                                             models.new_segment):
+                    n = users[0]
+                else:
+                    break
+            if ok:
+                names.add(node.target)
+        return names
+
+    def _side_ok(self, *vals) -> bool:
+        return self.overlap_wgrad and all(v is None or v.meta.get("name") in self._single_use_params for v in vals)
+
+    def _emit_side(self, fn: Callable[[], None], reads):
+        """Append ``fn`` to the backward list so that its launches run on the side stream, ordered after
+        everything the main stream has enqueued so far.  ``reads`` are the buffers ``fn`` reads: gradient
+        buffers alias each other through residual adds and are accumulated into in place later in the
+        backward list, so a later main-stream writer of one of them first waits for ``fn``
+        (see _guard_write)."""
+        fork, done = torch.cuda.Event(), torch.cuda.Event()
+        side = self._side_stream
+        for t in reads:
+            self._side_readers[t.untyped_storage().data_ptr()] = done
+
+        def run():
+            fork.record(torch.cuda.current_stream())
+            side.wait_event(fork)
+            with torch.cuda.stream(side):
+                fn()
+            done.record(side)
+            self._side_used = True
+        self.bwd.append(run)
+
+    def _guard_write(self, t: Optional[torch.Tensor]):
+        """Called while the backward list is built, right before a launch that writes into ``t`` is appended:
+        when a side-stream launch appended earlier reads ``t``'s storage, the main stream waits for it first."""
+        if t is None or not self._side_readers:
+            return
+        done = self._side_readers.pop(t.untyped_storage().data_ptr(), None)
+        if done is not None:
+            self.bwd.append(lambda: torch.cuda.current_stream().wait_event(done))
+
+    def _join_side(self):
+        if self._side_used:
+            self._side_join.record(self._side_stream)
+            torch.cuda.current_stream().wait_event(self._side_join)
+            self._side_used = False
 
     def _unsupported(self, node, why):
         raise ValueError(f"node {node.name} ({node.target}): {why}")
@@ -355,6 +430,7 @@ class ShardExecutor:
             v.grad = src
         else:
             g = v.grad
+            self._guard_write(g)
             self.bwd.append(lambda: ops.add(g, src, g))
 
     def _transpose(self, node):
@@ -430,10 +506,18 @@ class ShardExecutor:
                 return
             dy = out.grad
             gw, accw = self._param_grad_slot(w)
-            self.bwd.append(lambda: ops.gemm(dy, xt, gw, N, K, M, transA=True, lda=ldc, ldb=lda, accumulate=accw))
-            if b is not None:
-                gb, accb = self._param_grad_slot(b)
-                self.bwd.append(lambda: ops.colsum(dy, gb, M, N, ldc, accb))
+            gb, accb = self._param_grad_slot(b) if b is not None else (None, False)
+            side = self._side_ok(w, b)
+
+            def wgrad():
+                ops.gemm(dy, xt, gw, N, K, M, transA=True, lda=ldc, ldb=lda, accumulate=accw,
+                         workspace=self.side_workspace if side else None)
+                if gb is not None:
+                    ops.colsum(dy, gb, M, N, ldc, accb)
+            if side:
+                self._emit_side(wgrad, (dy, xt))
+            else:
+                self.bwd.append(wgrad)
             if x.kind == "cls_view":
                 src = x.meta["src"]
                 if src.grad is None:
@@ -481,6 +565,7 @@ class ShardExecutor:
     def _relu_backward_through(self, out: Val):
         """For a producer that applied relu itself: d(pre-activation) = d(out) * (out > 0), in place."""
         g = out.grad
+        self._guard_write(g)
         self.bwd.append(lambda: ops.act_bwd(g, out.t, g, "relu"))
 
     # ---- attention ------------------------------------------------------------------------------
@@ -544,7 +629,9 @@ class ShardExecutor:
                 return
             do = out_bsd.grad
             dctx = self._scratch("attn_dctx", (b, S, E))
-            dqkv = self._scratch("attn_dqkv", (b, S, 3 * E))
+            side = self._side_ok(w_out, b_out, w_in, b_in)
+            # the in-projection's weight gradient reads dqkv from the side stream, so it cannot be shared scratch
+            dqkv = self._new((b, S, 3 * E)) if side else self._scratch("attn_dqkv", (b, S, 3 * E))
             if fused:
                 delta = self._scratch("attn_delta", (b, H, S), torch.float32)
             else:
@@ -555,9 +642,19 @@ class ShardExecutor:
             gbi, acc_bi = self._param_grad_slot(b_in)
             gx, acc_x = self._grad_slot(x) if x.needs_grad else (None, False)
 
-            def backward():
-                ops.gemm(do, ctx, gwo, E, E, M, transA=True, accumulate=acc_wo)
+            ws = self.side_workspace if side else None
+
+            def wgrad_out():
+                ops.gemm(do, ctx, gwo, E, E, M, transA=True, accumulate=acc_wo, workspace=ws)
                 ops.colsum(do, gbo, M, E, E, acc_bo)
+
+            def wgrad_in():
+                ops.gemm(dqkv, x.t, gwi, 3 * E, E, M, transA=True, accumulate=acc_wi, workspace=ws)
+                ops.colsum(dqkv, gbi, M, 3 * E, 3 * E, acc_bi)
+
+            def backward():
+                if not side:
+                    wgrad_out()
                 ops.gemm(do, w_out.t, dctx, M, E, E)
                 if fused:
                     ops.attention_bwd(qkv, ctx, dctx, lse, mask_t, dqkv, delta, b, S, H, scale)
@@ -573,11 +670,24 @@ class ShardExecutor:
                              strideA=sP, strideB=sQ, strideC=sQ, offB=E)
                     ops.gemm(dP, qkv, dqkv, S, hd, S, transA=True, lda=Sp, ldb=3 * E, ldc=3 * E, alpha=scale, batch1=b,
                              batch2=H, strideA=sP, strideB=sQ, strideC=sQ, offC=E)
-                ops.gemm(dqkv, x.t, gwi, 3 * E, E, M, transA=True, accumulate=acc_wi)
-                ops.colsum(dqkv, gbi, M, 3 * E, 3 * E, acc_bi)
-                if gx is not None:
-                    ops.gemm(dqkv, w_in.t, gx, M, E, 3 * E, accumulate=acc_x)
-            self.bwd.append(backward)
+                if not side:
+                    wgrad_in()
+
+            def dgrad_in():
+                ops.gemm(dqkv, w_in.t, gx, M, E, 3 * E, accumulate=acc_x)
+            if side:
+                # do is final here; dqkv is final once `backward` is enqueued.  d(x) usually aliases do (the
+                # residual add hands one buffer to both), so the in-projection's data gradient, which
+                # accumulates into it, is ordered after the out-projection's weight gradient.
+                self._emit_side(wgrad_out, (do, ctx))
+                self.bwd.append(backward)
+                self._emit_side(wgrad_in, (dqkv, x.t))
+            else:
+                self.bwd.append(backward)
+            if gx is not None:
+                if acc_x:
+                    self._guard_write(gx)
+                self.bwd.append(dgrad_in)
         self._tape.append(emit)
         return Val("mha", None, out=out)
 
@@ -990,6 +1100,7 @@ class ShardExecutor:
             ops.fill_zero(self.flat_grad[:self.n_vector_region])
         for f in self.bwd:
             f()
+        self._join_side()
         self._reduce_replicated_grads()
 
     def _reduce_replicated_grads(self):
