@@ -8,7 +8,7 @@
 // the next MFMA as its B operand straight from registers by choosing the k-order (slot (h, j) of step s is row
 // 16 s + 8 (j / 4) + 4 h + j % 4), and the matching A operand is read from LDS in that same order.
 // K / V / Q / dO tiles sit in LDS in the swizzled [row][128 B] layout of tile.h; the transposed copies
-// (V^T, K^T, Q^T, dO^T) are produced by the transposing loader.
+// (V^T, K^T, Q^T, dO^T) are written from the same registers as the row-major ones (PairLoader).
 #include "common.h"
 #include "tile.h"
 
@@ -68,10 +68,38 @@ __device__ __forceinline__ frag_t load_row_frag(const bf16_t *row_ptr, bool vali
     return f;
 }
 
+// One [64 rows][64 d] operand tile (memory [row][d], row stride ld) held as two 16-byte vectors per thread
+// (rows 2 * (t / 8) and + 1, d chunk t % 8).  The same registers fill the row-major LDS tile [row][d] and the
+// transposed one [d][row], so a tile that is needed both ways is fetched from global memory once.
+struct PairLoader {
+    frag_t v[2];
+    __device__ __forceinline__ void load(const bf16_t *base, int64_t ld, int64_t rows_left) {
+        const int c8 = threadIdx.x & 7, r0 = (threadIdx.x >> 3) * 2;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) v[i] = load_row_frag(base + (int64_t)(r0 + i) * ld + c8 * 8, r0 + i < rows_left, 0, 0);
+    }
+    __device__ __forceinline__ void store_rows(char *lds) const {
+        const int c8 = threadIdx.x & 7, r0 = (threadIdx.x >> 3) * 2;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) *(frag_t *)(lds + (r0 + i) * ROW_BYTES + ((c8 ^ swz(r0 + i)) << 4)) = v[i];
+    }
+    __device__ __forceinline__ void store_transposed(char *lds) const {
+        const int c8 = threadIdx.x & 7, r0 = (threadIdx.x >> 3) * 2;       // r0 is even: both rows share a 4-byte slot
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const int d = c8 * 8 + e;
+            bf16x2 pr;
+            pr[0] = v[0].v[e];
+            pr[1] = v[1].v[e];
+            *(bf16x2 *)(lds + d * ROW_BYTES + (((r0 >> 3) ^ swz(d)) << 4) + (r0 & 7) * 2) = pr;
+        }
+    }
+};
+
 // ---------------------------------------------------------------------------------------------
 // forward
 // ---------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(AT_THREADS) void attn_fwd_kernel(const bf16_t *qkv, const float *mask, bf16_t *out,
+__global__ __launch_bounds__(AT_THREADS, 2) void attn_fwd_kernel(const bf16_t *qkv, const float *mask, bf16_t *out,
                                                             float *lse, int S, int H, float scale) {
     __shared__ __attribute__((aligned(16))) char Ks[TILE_BYTES];
     __shared__ __attribute__((aligned(16))) char Vts[TILE_BYTES];
@@ -89,17 +117,22 @@ __global__ __launch_bounds__(AT_THREADS) void attn_fwd_kernel(const bf16_t *qkv,
 
     f32x16 ot[2] = {zero16(), zero16()};
     float m = -INFINITY, lsum = 0.f;
-    TileLoader<bf16_t, TILE, AT_THREADS, true> lk;
-    TileLoader<bf16_t, HD, AT_THREADS, false> lv;
+    PairLoader lk, lv;
     const bool vec_mask = mask && ((S & 3) == 0);
 
+    // The next tile's global loads are issued before the current tile is multiplied, so their latency is
+    // covered by the MFMA / softmax work; the registers are written to LDS at the top of the next iteration.
+    lk.load(K, ld, S);
+    lv.load(V, ld, S);
     for (int kv0 = 0; kv0 < S; kv0 += TILE) {
-        lk.load(K + (int64_t)kv0 * ld, ld, S - kv0, HD);
-        lv.load(V + (int64_t)kv0 * ld, ld, HD, S - kv0);
         __syncthreads();                                   // every wave is done with the previous tiles
-        lk.store(Ks);
-        lv.store(Vts);
+        lk.store_rows(Ks);
+        lv.store_transposed(Vts);
         __syncthreads();
+        if (kv0 + TILE < S) {
+            lk.load(K + (int64_t)(kv0 + TILE) * ld, ld, S - kv0 - TILE);
+            lv.load(V + (int64_t)(kv0 + TILE) * ld, ld, S - kv0 - TILE);
+        }
 
         f32x16 st[2] = {zero16(), zero16()};
 #pragma unroll
@@ -200,7 +233,7 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(const bf16_t *out, cons
 // ---------------------------------------------------------------------------------------------
 // dQ: lanes own query columns, kv tiles are streamed
 // ---------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(AT_THREADS) void attn_bwd_dq_kernel(const bf16_t *qkv, const bf16_t *dout, const float *lse,
+__global__ __launch_bounds__(AT_THREADS, 2) void attn_bwd_dq_kernel(const bf16_t *qkv, const bf16_t *dout, const float *lse,
                                                                const float *delta, const float *mask, bf16_t *dqkv,
                                                                int S, int H, float scale) {
     __shared__ __attribute__((aligned(16))) char Ks[TILE_BYTES];
@@ -224,30 +257,32 @@ __global__ __launch_bounds__(AT_THREADS) void attn_bwd_dq_kernel(const bf16_t *q
     const float lse_q = qok ? lse[((int64_t)b * H + hh) * S + q] : 0.f;
     const float delta_q = qok ? delta[((int64_t)b * H + hh) * S + q] : 0.f;
     f32x16 dqt[2] = {zero16(), zero16()};
-    TileLoader<bf16_t, TILE, AT_THREADS, true> lk, lv;
-    TileLoader<bf16_t, HD, AT_THREADS, false> lkt;
+    PairLoader lk, lv;
     const bool vec_mask = mask && ((S & 3) == 0);
 
+    lk.load(K, ld, S);
+    lv.load(V, ld, S);
     for (int kv0 = 0; kv0 < S; kv0 += TILE) {
-        lk.load(K + (int64_t)kv0 * ld, ld, S - kv0, HD);
-        lv.load(V + (int64_t)kv0 * ld, ld, S - kv0, HD);
-        lkt.load(K + (int64_t)kv0 * ld, ld, HD, S - kv0);
         __syncthreads();
-        lk.store(Ks);
-        lv.store(Vs);
-        lkt.store(Kts);
+        lk.store_rows(Ks);
+        lk.store_transposed(Kts);
+        lv.store_rows(Vs);
         __syncthreads();
+        if (kv0 + TILE < S) {
+            const int64_t nx = kv0 + TILE;
+            lk.load(K + nx * ld, ld, S - nx);
+            lv.load(V + nx * ld, ld, S - nx);
+        }
 
-        f32x16 st[2] = {zero16(), zero16()}, dp[2] = {zero16(), zero16()};
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-            for (int s = 0; s < 4; ++s) {
-                st[t] = mma(frag_rowk(Ks, t * 32 + c, s, h), qf[s], st[t]);
-                dp[t] = mma(frag_rowk(Vs, t * 32 + c, s, h), dof[s], dp[t]);
-            }
+        // one 32-row kv block at a time keeps only one score / dP accumulator pair live
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
+            f32x16 st = zero16(), dp = zero16();
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                st = mma(frag_rowk(Ks, t * 32 + c, s, h), qf[s], st);
+                dp = mma(frag_rowk(Vs, t * 32 + c, s, h), dof[s], dp);
+            }
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
                 const int kv = kv0 + t * 32 + g * 8 + h * 4;
@@ -266,16 +301,16 @@ __global__ __launch_bounds__(AT_THREADS) void attn_bwd_dq_kernel(const bf16_t *q
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     const int r = g * 4 + e;
-                    float p = (qok && kv + e < S) ? __expf(st[t][r] * scale + mk[e] - lse_q) : 0.f;
-                    dp[t][r] = p * (dp[t][r] - delta_q) * scale;
+                    float p = (qok && kv + e < S) ? __expf(st[r] * scale + mk[e] - lse_q) : 0.f;
+                    dp[r] = p * (dp[r] - delta_q) * scale;
                 }
             }
-        }
 #pragma unroll
-        for (int s = 0; s < 4; ++s) {
-            const frag_t db = acc_to_b(dp[s >> 1], s & 1);
+            for (int sp = 0; sp < 2; ++sp) {
+                const frag_t db = acc_to_b(dp, sp);
 #pragma unroll
-            for (int u = 0; u < 2; ++u) dqt[u] = mma(frag_perm(Kts, u * 32 + c, s, h), db, dqt[u]);
+                for (int u = 0; u < 2; ++u) dqt[u] = mma(frag_perm(Kts, u * 32 + c, t * 2 + sp, h), db, dqt[u]);
+            }
         }
     }
     if (qok) {
@@ -295,14 +330,14 @@ __global__ __launch_bounds__(AT_THREADS) void attn_bwd_dq_kernel(const bf16_t *q
 // ---------------------------------------------------------------------------------------------
 // dK, dV: lanes own kv columns, query tiles are streamed
 // ---------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(AT_THREADS) void attn_bwd_dkv_kernel(const bf16_t *qkv, const bf16_t *dout, const float *lse,
+__global__ __launch_bounds__(AT_THREADS, 2) void attn_bwd_dkv_kernel(const bf16_t *qkv, const bf16_t *dout, const float *lse,
                                                                 const float *delta, const float *mask, bf16_t *dqkv,
                                                                 int S, int H, float scale) {
     __shared__ __attribute__((aligned(16))) char Qs[TILE_BYTES];
     __shared__ __attribute__((aligned(16))) char dOs[TILE_BYTES];
     __shared__ __attribute__((aligned(16))) char Qts[TILE_BYTES];
     __shared__ __attribute__((aligned(16))) char dOts[TILE_BYTES];
-    __shared__ float lse_s[TILE], delta_s[TILE];
+    __shared__ __attribute__((aligned(16))) float lse_s[TILE], delta_s[TILE];
     const int E = H * HD, ld = 3 * E;
     const int b = blockIdx.y / H, hh = blockIdx.y % H;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, c = lane & 31, h = lane >> 5;
@@ -320,54 +355,61 @@ __global__ __launch_bounds__(AT_THREADS) void attn_bwd_dkv_kernel(const bf16_t *
         vf[s] = load_row_frag(V + (int64_t)kv * ld, kok, s, h);
     }
     f32x16 dvt[2] = {zero16(), zero16()}, dkt[2] = {zero16(), zero16()};
-    TileLoader<bf16_t, TILE, AT_THREADS, true> lq, ldo;
-    TileLoader<bf16_t, HD, AT_THREADS, false> lqt, ldot;
+    PairLoader lq, ldo;
 
+    lq.load(Q, ld, S);
+    ldo.load(dO, E, S);
     for (int q0 = 0; q0 < S; q0 += TILE) {
-        lq.load(Q + (int64_t)q0 * ld, ld, S - q0, HD);
-        ldo.load(dO + (int64_t)q0 * E, E, S - q0, HD);
-        lqt.load(Q + (int64_t)q0 * ld, ld, HD, S - q0);
-        ldot.load(dO + (int64_t)q0 * E, E, HD, S - q0);
         __syncthreads();
-        lq.store(Qs);
-        ldo.store(dOs);
-        lqt.store(Qts);
-        ldot.store(dOts);
+        lq.store_rows(Qs);
+        lq.store_transposed(Qts);
+        ldo.store_rows(dOs);
+        ldo.store_transposed(dOts);
         if (threadIdx.x < TILE) {
             const int qq = q0 + threadIdx.x;
-            lse_s[threadIdx.x] = qq < S ? lse_b[qq] : 0.f;
+            lse_s[threadIdx.x] = qq < S ? lse_b[qq] : INFINITY;
             delta_s[threadIdx.x] = qq < S ? delta_b[qq] : 0.f;
         }
         __syncthreads();
+        if (q0 + TILE < S) {
+            const int64_t nx = q0 + TILE;
+            lq.load(Q + nx * ld, ld, S - nx);
+            ldo.load(dO + nx * E, E, S - nx);
+        }
 
-        f32x16 sc[2] = {zero16(), zero16()}, dp[2] = {zero16(), zero16()};
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
+        // one 32-row query block at a time keeps only one score / dP accumulator pair live; the loop is kept
+        // rolled so that the scheduler cannot pull the second block's fragments ahead of the first one's math
+#pragma unroll 1
+        for (int t = 0; t < 2; ++t) {
+            f32x16 sc = zero16(), dp = zero16();
 #pragma unroll
             for (int s = 0; s < 4; ++s) {
-                sc[t] = mma(frag_rowk(Qs, t * 32 + c, s, h), kf[s], sc[t]);
-                dp[t] = mma(frag_rowk(dOs, t * 32 + c, s, h), vf[s], dp[t]);
+                sc = mma(frag_rowk(Qs, t * 32 + c, s, h), kf[s], sc);
+                dp = mma(frag_rowk(dOs, t * 32 + c, s, h), vf[s], dp);
             }
 #pragma unroll
-        for (int t = 0; t < 2; ++t)
+            for (int g = 0; g < 4; ++g) {
+                // accumulator registers 4 g .. 4 g + 3 are query rows ql .. ql + 3
+                const int ql = t * 32 + g * 8 + h * 4;
+                const f32x4 l4 = *(const f32x4 *)(lse_s + ql), d4 = *(const f32x4 *)(delta_s + ql);
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int ql = t * 32 + acc_row(r, h), qq = q0 + ql;
-                float p = 0.f;
-                if (kok && qq < S) {
-                    const float mk = mask ? mask[(int64_t)qq * S + kv] : 0.f;
-                    p = __expf(sc[t][r] * scale + mk - lse_s[ql]);
+                for (int e = 0; e < 4; ++e) {
+                    const int r = g * 4 + e;
+                    float x = sc[r] * scale - l4[e];                 // rows beyond S carry lse = +inf: p = 0
+                    if (mask) x += (kok && q0 + ql + e < S) ? mask[(int64_t)(q0 + ql + e) * S + kv] : 0.f;
+                    const float p = __expf(x);
+                    sc[r] = p;
+                    dp[r] = p * (dp[r] - d4[e]) * scale;
                 }
-                sc[t][r] = p;
-                dp[t][r] = p * (dp[t][r] - delta_s[ql]) * scale;
             }
 #pragma unroll
-        for (int s = 0; s < 4; ++s) {
-            const frag_t pb = acc_to_b(sc[s >> 1], s & 1), db = acc_to_b(dp[s >> 1], s & 1);
+            for (int sp = 0; sp < 2; ++sp) {
+                const frag_t pb = acc_to_b(sc, sp), db = acc_to_b(dp, sp);
 #pragma unroll
-            for (int u = 0; u < 2; ++u) {
-                dvt[u] = mma(frag_perm(dOts, u * 32 + c, s, h), pb, dvt[u]);
-                dkt[u] = mma(frag_perm(Qts, u * 32 + c, s, h), db, dkt[u]);
+                for (int u = 0; u < 2; ++u) {
+                    dvt[u] = mma(frag_perm(dOts, u * 32 + c, t * 2 + sp, h), pb, dvt[u]);
+                    dkt[u] = mma(frag_perm(Qts, u * 32 + c, t * 2 + sp, h), db, dkt[u]);
+                }
             }
         }
     }
