@@ -63,7 +63,57 @@ def _prototypes():
     return out
 
 
-def lib() -> ctypes.CDLL:
+class _Recorder:
+    """Stands in for the library while a launch list is being recorded: every entry point behaves as usual and
+    a successful call is appended to the list as (ctypes function, argument tuple).  The tuple keeps the
+    argument blocks and host arrays of the call alive, so the list can be replayed call by call."""
+
+    def __init__(self, handle, log):
+        self._handle, self._log, self._wrapped = handle, log, {}
+
+    def __getattr__(self, name):
+        w = self._wrapped.get(name)
+        if w is None:
+            fn, log = getattr(self._handle, name), self._log
+
+            def w(*args):
+                rc = fn(*args)
+                if rc == 0 and fn.restype is ctypes.c_int:
+                    log.append((fn, args))
+                return rc
+            self._wrapped[name] = w
+        return w
+
+
+_recorder = None
+
+
+def start_recording() -> None:
+    """Record every library call made through ``lib()`` until ``stop_recording``."""
+    global _recorder
+    if _recorder is not None:
+        raise HapmiError("a launch list is already being recorded")
+    _recorder = _Recorder(_load(), [])
+
+
+def stop_recording():
+    global _recorder
+    rec, _recorder = _recorder, None
+    return rec._log if rec is not None else []
+
+
+def replay(calls) -> None:
+    for fn, args in calls:
+        rc = fn(*args)
+        if rc != 0:
+            raise HapmiError(f"libhapmi error {rc} in {fn.__name__}: {_load().hapmi_last_error().decode()}")
+
+
+def lib():
+    return _recorder if _recorder is not None else _load()
+
+
+def _load() -> ctypes.CDLL:
     global _lib
     if _lib is None:
         if not os.path.exists(_PATH):
@@ -81,4 +131,4 @@ def lib() -> ctypes.CDLL:
 
 def check(rc: int) -> None:
     if rc != 0:
-        raise HapmiError(f"libhapmi error {rc}: {lib().hapmi_last_error().decode()}")
+        raise HapmiError(f"libhapmi error {rc}: {_load().hapmi_last_error().decode()}")

@@ -16,6 +16,8 @@
 #include "gemm_kernel.h"
 #include <vector>
 #include <mutex>
+#include <map>
+#include <tuple>
 
 HAPMI_GEMM_DECLARE_CFG(0);
 HAPMI_GEMM_DECLARE_CFG(1);
@@ -37,6 +39,11 @@ constexpr int kNumCfg = 7;
 constexpr int kNumCU = 256;
 int g_force_cfg = -1;
 int g_force_splits = 0;
+
+// ---- plan table: (M, N, K, batch, transA, transB, in, out) -> (configuration, splits) ------------
+typedef std::tuple<int64_t, int64_t, int64_t, int64_t, int, int, int, int> PlanKey;
+std::map<PlanKey, std::pair<int, int>> g_plans;
+std::mutex g_plans_mu;
 
 // ---- instrumentation: HIP events around every launch --------------------------------------------
 struct ProfState {
@@ -129,7 +136,18 @@ int launch_typed(GemmParams &p, int transA, int transB, int64_t batch, hipStream
     p.ws_ld = (p.N + 3) / 4 * 4;
     const int64_t per_split = p.M * p.ws_ld * 4;
     const int64_t max_splits = (workspace && ((uintptr_t)workspace % 16) == 0 && per_split > 0) ? workspace_bytes / per_split : 0;
-    const Choice ch = choose(p.M, p.N, p.K, batch, bk, wide && sizeof(TI) == 2, max_splits, !transA && transB);
+    Choice ch = choose(p.M, p.N, p.K, batch, bk, wide && sizeof(TI) == 2, max_splits, !transA && transB);
+    if (g_force_cfg < 0 && g_force_splits <= 0) {
+        std::lock_guard<std::mutex> lk(g_plans_mu);
+        auto it = g_plans.find(PlanKey(p.M, p.N, p.K, batch, (int)(transA != 0), (int)(transB != 0), sizeof(TI) == 2 ? HAPMI_BF16 : HAPMI_F32,
+                                       sizeof(TO) == 2 ? HAPMI_BF16 : HAPMI_F32));
+        if (it != g_plans.end()) {
+            const int pc = it->second.first, ps = it->second.second;
+            const bool cfg_ok = pc == 0 || (pc < kNumCfg && wide && sizeof(TI) == 2);
+            const bool split_ok = ps == 1 || (ps > 1 && ps <= max_splits && batch == 1 && nk / ps >= 1);
+            if (cfg_ok && split_ok) ch = Choice{pc, ps};
+        }
+    }
     const int c = ch.cfg;
     p.splits = ch.splits;
     p.ktiles_per_split = (int)hapmi_cdiv(nk, p.splits);
@@ -228,6 +246,24 @@ extern "C" int hapmi_gemm(const hapmi_gemm_args *a, hapmi_stream_t stream) {
 extern "C" int hapmi_gemm_tuning(int tile_config, int k_splits) {
     g_force_cfg = tile_config;
     g_force_splits = k_splits;
+    return HAPMI_OK;
+}
+
+extern "C" int hapmi_gemm_plan_set(int64_t M, int64_t N, int64_t K, int64_t batch, int transA, int transB, int in_dtype,
+                                   int out_dtype, int tile_config, int k_splits) {
+    HAPMI_REQUIRE(hapmi_dtype_ok(in_dtype) && hapmi_dtype_ok(out_dtype), HAPMI_EINVAL, "gemm_plan_set: bad dtype");
+    HAPMI_REQUIRE(tile_config < kNumCfg && k_splits >= 1 && k_splits <= 64, HAPMI_EINVAL,
+                  "gemm_plan_set: configuration %d / splits %d out of range", tile_config, k_splits);
+    const PlanKey key(M, N, K, batch, (int)(transA != 0), (int)(transB != 0), in_dtype, out_dtype);
+    std::lock_guard<std::mutex> lk(g_plans_mu);
+    if (tile_config < 0) g_plans.erase(key);
+    else g_plans[key] = std::make_pair(tile_config, k_splits);
+    return HAPMI_OK;
+}
+
+extern "C" int hapmi_gemm_plan_clear(void) {
+    std::lock_guard<std::mutex> lk(g_plans_mu);
+    g_plans.clear();
     return HAPMI_OK;
 }
 

@@ -59,7 +59,7 @@ def _round_up(n, m):
 class ShardExecutor:
     def __init__(self, gm: torch.fx.GraphModule, example_inputs, dtype: str = "fp32", wire: Optional[Wire] = None,
                  rank: int = 0, world_size: int = 1, device: str = "cuda:0", fused_attention: bool = True,
-                 overlap_wgrad: bool = False):
+                 overlap_wgrad: bool = False, launch_lists: bool = True):
         """``example_inputs``: the program's inputs (global batch) as tensors or shapes; activations are
         sized from them.  ``rank`` / ``world_size`` are only needed by all_reduce / replicate, whose node
         forms do not carry them (collectives.py:86, 182)."""
@@ -101,6 +101,12 @@ class ShardExecutor:
         self._side_readers: Dict[int, torch.cuda.Event] = {}   # storage -> event after its last side-stream reader
         self.side_workspace = torch.empty(64 << 20, dtype=torch.float32, device=self.dev) if overlap_wgrad else None
         self._single_use_params = self._find_single_use_params(gm)
+        # Every launch of a step is a library call on static buffers with constant arguments, so the calls of
+        # the first forward / backward / optimizer phase are recorded and later phases replay the recorded
+        # calls directly (no per-call argument marshalling or host-side checks: about 10 us of interpreter
+        # time per launch otherwise).  Keyed by stream; not used together with the side stream.
+        self.launch_lists = launch_lists and not overlap_wgrad
+        self._lists: Dict[tuple, list] = {}
         self.gemm_workspace = torch.empty(64 << 20, dtype=torch.float32, device=self.dev)   # 256 MiB of split-K scratch
         ops.set_gemm_workspace(self.gemm_workspace)
         self._prepare_params()
@@ -1091,11 +1097,32 @@ class ShardExecutor:
             self.load_inputs(*args)
         if self._shadow_stale:
             self.refresh_shadow()
-        for f in self.fwd:
-            f()
+        self._run_phase("fwd", self.fwd)
         return self.loss[0]
 
+    def _run_phase(self, name: str, closures):
+        if not self.launch_lists or torch.cuda.is_current_stream_capturing():
+            for f in closures:
+                f()
+            return
+        key = (name, torch.cuda.current_stream().cuda_stream)
+        calls = self._lists.get(key)
+        if calls is not None:
+            ops._lib.replay(calls)
+            return
+        ops._lib.start_recording()
+        try:
+            for f in closures:
+                f()
+        except BaseException:
+            ops._lib.stop_recording()
+            raise
+        self._lists[key] = ops._lib.stop_recording()
+
     def backward(self):
+        self._run_phase("bwd", [self._backward_launches])
+
+    def _backward_launches(self):
         if self.n_vector_region:
             ops.fill_zero(self.flat_grad[:self.n_vector_region])
         for f in self.bwd:
@@ -1113,6 +1140,7 @@ class ShardExecutor:
         if kind not in ("adam", "sgd"):
             raise ValueError("optimizer must be 'adam' or 'sgd'")
         self._opt = dict(kind=kind, lr=lr, betas=betas, eps=eps, clip=clip_grad_norm)
+        self._lists = {k: v for k, v in self._lists.items() if k[0] != "step"}
         if kind == "adam":
             self.exp_avg = torch.zeros_like(self.master)
             self.exp_avg_sq = torch.zeros_like(self.master)
@@ -1123,16 +1151,19 @@ class ShardExecutor:
         self._step_count = 0
 
     def step(self):
-        o = self._opt
-        if o is None:
+        if self._opt is None:
             raise RuntimeError("configure_optimizer() first")
+        self._step_count += 1
+        self._run_phase("step", [self._step_launches])
+
+    def _step_launches(self):
+        o = self._opt
         coef = None
         if o["clip"] is not None:
             ops.fill_zero(self._sumsq)
             ops.sumsq(self.flat_grad, self._sumsq)
             ops.clip_coef(self._sumsq, o["clip"], self._coef)
             coef = self._coef
-        self._step_count += 1
         if o["kind"] == "sgd":
             ops.sgd_step(self.master, self.flat_grad, self.shadow, o["lr"], coef)
         else:
@@ -1168,6 +1199,37 @@ class ShardExecutor:
             graph.replay()
             return self.loss[0]
         return replay
+
+    def autotune_gemms(self, verbose: bool = False):
+        """Run one forward + backward with the loaded inputs while recording every GEMM call, then time the
+        legal tile configurations / K splits of each distinct problem signature on the recorded operands and
+        pin the winners in the library's plan table (process-wide; other signatures keep the cost model).
+        Buffers that the timed launches overwrite or accumulate into are activations and gradients, which the
+        next step rewrites before reading; parameters and optimizer state are not touched."""
+        if any(rec["buf"] is None for rec in self.inputs):
+            raise RuntimeError("load_inputs() first")
+        ops.record_gemms(True)
+        try:
+            self.forward()
+            self.backward()
+        finally:
+            log = ops.record_gemms(False)
+        torch.cuda.synchronize()
+        flush = torch.zeros(512 << 20, dtype=torch.int8, device=self.dev)
+        seen, report = set(), []
+        for a, keep in log:
+            key = (a.M, a.N, a.K, a.batch1 * a.batch2, a.transA, a.transB, a.in_dtype, a.out_dtype)
+            if key in seen:
+                continue
+            seen.add(key)
+            cfg, splits, us = ops.autotune_gemm(a, flush)
+            report.append((key, cfg, splits, us))
+            if verbose:
+                print(f"gemm M{a.M} N{a.N} K{a.K} batch{key[3]} tA{a.transA} tB{a.transB}: config {cfg}, "
+                      f"{splits} split(s), {us:.1f} us", flush=True)
+        del flush
+        torch.cuda.synchronize()
+        return report
 
     def mark_params_dirty(self):
         """Call after parameters were changed from outside (e.g. by a torch.optim optimizer)."""

@@ -320,8 +320,69 @@ def gemm(A: torch.Tensor, B: torch.Tensor, C: torch.Tensor, M: int, N: int, K: i
     _need(bias, N, "gemm bias")
     if min(strideA + strideB + strideC) < 0:
         raise _lib.HapmiError("gemm: negative batch stride")
+    if _gemm_log is not None:
+        _gemm_log.append((a, (A, B, C, bias, ws)))          # the tensors keep the recorded pointers alive
     check(lib().hapmi_gemm(ctypes.byref(a), _stream()))
     return C
+
+
+_gemm_log = None
+_SPLIT_MENU = (1, 2, 3, 4, 6, 8, 12, 16)
+_N_TILE_CONFIGS = 7
+
+
+def record_gemms(on: bool):
+    """Start (True) or stop (False) recording the argument blocks of every ``gemm`` call; stopping returns
+    the list recorded so far."""
+    global _gemm_log
+    log, _gemm_log = _gemm_log, ([] if on else None)
+    return log or []
+
+
+def autotune_gemm(a: "GemmArgs", flush: Optional[torch.Tensor] = None, repeats: int = 3):
+    """Time every tile configuration / K split that is legal for the recorded call ``a`` on its own operands
+    and pin the fastest in the library's plan table (``hapmi_gemm_plan_set``).  Each sample is one launch
+    bracketed by events after ``flush`` (a buffer larger than the caches) has been overwritten, so operands
+    and output start as cold as they are inside a training step.  Returns (config, splits, microseconds)."""
+    L = lib()
+    batch = a.batch1 * a.batch2
+    bf16_in = a.in_dtype == 1
+    nk = -(-a.K // (64 if bf16_in else 32))
+    per_split = a.M * ((a.N + 3) // 4 * 4) * 4
+    max_splits = a.workspace_bytes // per_split if (a.workspace and per_split) else 0
+    cands = []
+    for cfg in range(_N_TILE_CONFIGS if bf16_in else 1):
+        for s in _SPLIT_MENU:
+            if s > 1 and (s > max_splits or batch != 1 or nk // s < 4):
+                continue
+            cands.append((cfg, s))
+    stream = _stream()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    best = None
+    try:
+        for cfg, s in cands:
+            check(L.hapmi_gemm_tuning(cfg, s))
+            check(L.hapmi_gemm(ctypes.byref(a), stream))            # warm-up: code objects, LDS limit
+            samples = []
+            for _ in range(repeats):
+                if flush is not None:
+                    flush.add_(1)
+                e0.record()
+                check(L.hapmi_gemm(ctypes.byref(a), stream))
+                e1.record()
+                e1.synchronize()
+                samples.append(e0.elapsed_time(e1) * 1e3)
+            t = sorted(samples)[len(samples) // 2]
+            if best is None or t < best[2]:
+                best = (cfg, s, t)
+    finally:
+        check(L.hapmi_gemm_tuning(-1, 0))
+    check(L.hapmi_gemm_plan_set(a.M, a.N, a.K, batch, a.transA, a.transB, a.in_dtype, a.out_dtype, best[0], best[1]))
+    return best
+
+
+def clear_gemm_plans():
+    check(lib().hapmi_gemm_plan_clear())
 
 
 def linear(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, out_dtype=None, act=None) -> torch.Tensor:

@@ -134,9 +134,19 @@ typedef struct {
 } hapmi_gemm_args;
 int hapmi_gemm(const hapmi_gemm_args *args_host, hapmi_stream_t stream);
 
-/* Tuning hook for measurements: force tile configuration `tile_config` (0: 128x128, 1: 256x128,
- * 2: 256x256 / 4 waves, 3: 256x256 / 8 waves; -1 = automatic) and `k_splits` (0 = automatic). */
+/* Tuning hook for measurements: force tile configuration `tile_config` (block tile / waves: 0: 128x128 / 2x2,
+ * 1: 256x256 / 2x4, 2: 384x192 / 4x2, 3: 192x256 / 2x4, 4: 256x192 / 4x2, 5: 256x128 / 4x2, 6: 128x256 / 2x4;
+ * 1..6 take bf16 operands only; -1 = automatic) and `k_splits` (0 = automatic). */
 int hapmi_gemm_tuning(int tile_config, int k_splits);
+
+/* Plan table: pin the tile configuration and K split that hapmi_gemm uses for one problem signature
+ * (shape, batch = batch1 * batch2, transposes, element types).  A caller that has timed the candidates on
+ * its own operands (hap_amd.ops.autotune_gemm does) stores the winner here; signatures without a plan fall
+ * back to the built-in cost model.  tile_config < 0 removes the entry; hapmi_gemm_plan_clear empties the
+ * table.  No counterpart in the reference (its GEMMs are cuBLAS calls behind F.linear, hap.rs:1032). */
+int hapmi_gemm_plan_set(int64_t M, int64_t N, int64_t K, int64_t batch, int transA, int transB, int in_dtype,
+                        int out_dtype, int tile_config, int k_splits);
+int hapmi_gemm_plan_clear(void);
 
 /* ---- row-wise kernels ------------------------------------------------- */
 /* operator.add + F.layer_norm(x, (width,)) without affine, eps (hap.rs:1515, 1653):

@@ -224,3 +224,47 @@ def test_side_stream_weight_gradients_equal_main_stream(cuda, dtype):
                 assert torch.equal(ga, gb), (n, (ga - gb).abs().max().item())
             else:
                 torch.testing.assert_close(ga, gb, rtol=1e-4, atol=1e-5 * gb.abs().max().item())
+
+
+@pytest.mark.parametrize("family", ["lm", "vit", "moe"])
+def test_recorded_launch_lists_equal_closure_execution(cuda, family):
+    """By default the library calls of the first forward / backward / optimizer phase are recorded and later
+    phases replay the recorded calls.  Against an executor that runs its closures every time: identical losses
+    and matrix gradients over repeated forward + backward passes (parameters held fixed), and matching
+    parameters after optimizer steps (vector gradients are summed with float atomics, hence a tolerance)."""
+    if family == "lm":
+        model, (x, y), ratios, B, kw = make_lm(vocab=211, S=32, d=64, H=1, F=128, layers=2), lm_batch(8, 32, 211), RATIOS4, 8, {}
+    elif family == "vit":
+        model, (x, y), ratios, B, kw = make_vit(img=32, patch=8, d=64, F=128), vit_batch(8, 32, 10), RATIOS4, 8, dict(ffn="batch")
+    else:
+        model, (x, y), ratios, B, kw = make_moe(), lm_batch(4, 16, 61), RATIOS_E, 4, dict(ffn="batch", batch_sharded=False)
+
+    def build(lists):
+        plan = hap_amd.ShardingPlan([list(ratios)], 0, ffn=kw.get("ffn", "column"))
+        gm = hap_amd.build_program(copy.deepcopy(model), plan, B, batch_sharded=kw.get("batch_sharded", True))
+        ex = hap_amd.compile_program(gm, [x, y], dtype="bf16", wire=hap_amd.SyntheticWire(seed=3, grad_scale=1e-2),
+                                     rank=0, world_size=len(ratios), launch_lists=lists)
+        ex.configure_optimizer(kind="adam", lr=5e-4, clip_grad_norm=0.5)
+        return ex
+
+    a, b = build(True), build(False)
+    assert a.launch_lists and not b.launch_lists
+    for it in range(3):
+        la = a.forward(x, y).item()
+        a.backward()
+        lb = b.forward(x, y).item()
+        b.backward()
+        torch.cuda.synchronize()
+        assert la == lb, it
+        for n, rec in a.params.items():
+            ga, gb = rec["grad"], b.params[n]["grad"]
+            torch.testing.assert_close(ga, gb, rtol=1e-4, atol=1e-5 * max(gb.abs().max().item(), 1e-30))
+    assert ("fwd", torch.cuda.current_stream().cuda_stream) in a._lists and not b._lists
+    for it in range(3):
+        la, lb = a.train_step(x, y).item(), b.train_step(x, y).item()
+        assert la == pytest.approx(lb, rel=1e-4), it
+    torch.cuda.synchronize()
+    for n, rec in a.params.items():
+        g = b.params[n]["grad"]
+        clear = g.abs() > 1e-3 * g.abs().max()
+        torch.testing.assert_close(rec["master"][clear], b.params[n]["master"][clear], rtol=1e-3, atol=1e-5)
