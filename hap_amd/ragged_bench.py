@@ -33,6 +33,13 @@ def _time(fn, steps, warmup):
     return start.elapsed_time(stop) / steps * 1e-3
 
 
+# HBM bytes of one ragged_reduce launch on the seeded workload below, from rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE (KiB per dispatch: 501861.1 and 125456.0), the fetch counter scaled by 2.0: the factor at which
+# the plain unpad+concat copy of the same 125456 KiB payload reads its known size (it counts 62774.0 KiB).
+PROFILED_S = [2201, 1374, 2567, 2270, 1333, 2391, 1194, 2352]
+PROFILED_REDUCE_TRAFFIC = int((501861.1 * 2.0 + 125456.0) * 1024)
+
+
 def run(steps: int = 50, warmup: int = 10, cpu_baseline: bool = True) -> dict:
     ops.init()
     dev = torch.device("cuda:0")
@@ -70,7 +77,9 @@ def run(steps: int = 50, warmup: int = 10, cpu_baseline: bool = True) -> dict:
         "config": {"workload": "8 ragged shards [S_i, 4096] bf16, S_i in [1000, 3000] (seed 39)", "S": S,
                    "per_kernel_GBps": gbs},
         "roofline": {"bound": "hbm", "kernel": "ragged_reduce_kernel<bf16, 8>", "achieved": gbs["ragged_reduce"],
-                     "peak": HBM_PEAK, "unit": "GB/s", "frac": gbs["ragged_reduce"] / HBM_PEAK, "traffic": None},
+                     "peak": HBM_PEAK, "unit": "GB/s", "frac": gbs["ragged_reduce"] / HBM_PEAK,
+                     "algorithmic_bytes": 9 * payload,
+                     "traffic": PROFILED_REDUCE_TRAFFIC if S == PROFILED_S else None},
     }
     if cpu_baseline:
         cores = min(os.cpu_count() or 1, 16)
