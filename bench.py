@@ -126,7 +126,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="bert", choices=list(WORKLOADS) + ["ragged"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--graph", action="store_true", help="replay the step from a captured HIP graph")
+    ap.add_argument("--eager", action="store_true",
+                    help="launch every kernel of the timed steps from the host instead of replaying a captured HIP graph")
     ap.add_argument("--no-autotune", action="store_true",
                     help="keep the built-in cost model instead of timing tile configurations per GEMM shape first")
     ap.add_argument("--overlap", action="store_true",
@@ -166,7 +167,7 @@ def main():
     for _ in range(args.warmup):
         one_step()
     torch.cuda.synchronize()
-    if args.graph:
+    if not args.eager:
         graph = torch.cuda.CUDAGraph()
         side = torch.cuda.Stream()
         with torch.cuda.stream(side):
@@ -196,7 +197,8 @@ def main():
         lib().hapmi_prof_gemm_collect(ctypes.byref(ms), ctypes.byref(n_launch), ctypes.byref(flops))
         lib().hapmi_prof_gemm_enable(0)
     else:
-        # kernel durations cannot be bracketed inside a replayed graph: profile the same launches eagerly
+        # HIP events cannot bracket a kernel inside a replayed graph: the same launches are issued eagerly for
+        # three more steps right after the timed region and their per-launch durations are what `roofline` reports
         lib().hapmi_prof_gemm_enable(1)
         for _ in range(3):
             one_step()
@@ -220,6 +222,7 @@ def main():
                    "final_loss": loss},
         "roofline": {"bound": "mfma", "kernel": "gemm_kernel (all GEMM launches of the step)",
                      "achieved": achieved, "peak": peak, "unit": "TFLOP/s", "frac": achieved / peak,
+                     "measured_over": "the timed steps" if graph is None else "3 eager steps after the timed graph replays",
                      "launches_per_step": n_launch.value / max(1, args.steps if graph is None else 3),
                      "gemm_ms_per_step": ms.value / max(1, args.steps if graph is None else 3), "traffic": None},
     }

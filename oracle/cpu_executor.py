@@ -123,9 +123,9 @@ class JointCPURun:
                 raise ValueError(node0.op)
         return result
 
-    def step(self, x, y, optimizers: Optional[list] = None) -> List[torch.Tensor]:
-        """zero_grad -> forward -> backward of the summed loss -> optimizer step
-        (worker.py:59-76 without the gradient clipping)."""
+    def step(self, x, y, optimizers: Optional[list] = None, clip_grad_norm: Optional[float] = None) -> List[torch.Tensor]:
+        """zero_grad -> forward -> backward of the summed loss -> [clip_grad_norm_ over each rank's own
+        gradients, worker.py:74] -> optimizer step (worker.py:59-76)."""
         for p in self.programs:
             p.zero_grad(set_to_none=True)
         losses = self.forward(x, y)
@@ -133,6 +133,9 @@ class JointCPURun:
         for l in losses[1:]:
             total = total + l.float()
         total.backward()
+        if clip_grad_norm is not None:
+            for p in self.programs:
+                torch.nn.utils.clip_grad_norm_(p.parameters(), clip_grad_norm)
         if optimizers is not None:
             for opt in optimizers:
                 opt.step()
