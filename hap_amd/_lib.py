@@ -32,6 +32,7 @@ class GemmArgs(ctypes.Structure):
         ("strideB1", ctypes.c_int64), ("strideB2", ctypes.c_int64),
         ("strideC1", ctypes.c_int64), ("strideC2", ctypes.c_int64),
         ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_int64),
+        ("a_rowsum", ctypes.c_void_p),
     ]
 
 

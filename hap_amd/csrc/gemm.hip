@@ -212,6 +212,9 @@ extern "C" int hapmi_gemm(const hapmi_gemm_args *a, hapmi_stream_t stream) {
     p.ktiles_per_split = 1;
     p.ws = nullptr;
     p.ws_ld = 0;
+    p.rowsum = a->a_rowsum;
+    HAPMI_REQUIRE(!a->a_rowsum || (a->transA && a->batch1 * a->batch2 == 1), HAPMI_EINVAL,
+                  "gemm: a_rowsum needs transA = 1 (A stored [K, M]) and a single problem");
 
     hipStream_t st = (hipStream_t)stream;
     hipEvent_t e0 = nullptr, e1 = nullptr;

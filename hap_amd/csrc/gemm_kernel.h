@@ -30,6 +30,7 @@ struct GemmParams {
     int tiles_m, tiles_n;
     int splits, ktiles_per_split;
     float *ws;                 // split-K workspace [splits][M][ws_ld] (float32)
+    float *rowsum;             // optional: rowsum[m] += sum_k op(A)[m, k] (float32 atomics; A stored [K, M] only)
     int64_t ws_ld;
 };
 
@@ -150,6 +151,27 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, (WAVES_M * WAVES_N <= 4 ? 2 
         }
     };
 
+    // Optional row sums of op(A) (the bias gradient when A is dY of a weight-gradient GEMM): A tiles of a
+    // k-major operand pass through registers on their way to LDS, where they are summed along k.  Every block
+    // of a tile row sees the same A tiles, so the k-tiles are dealt round-robin over the tiles_n blocks of
+    // the row: each block adds 1/tiles_n of the work instead of one block in tiles_n doing all of it.
+    const bool do_rs = !A_KMAJOR && p.rowsum != nullptr;
+    constexpr int RS_N = A_KMAJOR ? 1 : decltype(la)::PASSES_T * decltype(la)::EPV;
+    float rs[RS_N];
+#pragma unroll
+    for (int e = 0; e < RS_N; ++e) rs[e] = 0.f;
+    auto rs_add = [&]() {
+        if (!A_KMAJOR) {
+            constexpr int EPV_ = decltype(la)::EPV;
+#pragma unroll
+            for (int pp = 0; pp < decltype(la)::PASSES_T; ++pp)
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+#pragma unroll
+                    for (int e = 0; e < EPV_; ++e) rs[pp * EPV_ + e] += la.v[pp * 4 + q].get(e);
+        }
+    };
+
     // A ragged last k-tile (K not a multiple of the tile depth) is done first, alone, with guarded loads, so
     // that the main loop below only ever sees complete k-tiles and stays free of branches.
     int kt_end = kt1;
@@ -158,6 +180,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, (WAVES_M * WAVES_N <= 4 ? 2 
         const int64_t k_left = p.K - (int64_t)kt_end * BK;
         la.load(a_base + (int64_t)kt_end * a_kstep, p.lda, m_left, k_left);
         lb.load(b_base + (int64_t)kt_end * b_kstep, p.ldb, n_left, k_left);
+        if (do_rs && kt_end % p.tiles_n == tn) rs_add();
         la.store(As);
         lb.store(Bs);
         __syncthreads();
@@ -178,21 +201,46 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, (WAVES_M * WAVES_N <= 4 ? 2 
             if (B_KMAJOR) lb.load_direct(b_base + (int64_t)kt * b_kstep, Bs + buf * B_BYTES);
             else lb.load_fast(b_base + (int64_t)kt * b_kstep, p.ldb);
         };
-        auto commit_tile = [&](int buf) {
+        auto commit_tile = [&](int buf, int kt) {
+            if (do_rs && kt % p.tiles_n == tn) rs_add();
             if (!A_KMAJOR) la.store(As + buf * A_BYTES);
             if (!B_KMAJOR) lb.store(Bs + buf * B_BYTES);
             __builtin_amdgcn_s_waitcnt(0x0F70);                   // vmcnt(0): this wave's direct loads have landed
         };
         issue_tile(kt0, 0);
-        commit_tile(0);
+        commit_tile(0, kt0);
         __syncthreads();
         for (int kt = kt0; kt < kt_end; ++kt) {
             const int cur = (kt - kt0) & 1;
             if (kt + 1 < kt_end) issue_tile(kt + 1, cur ^ 1);
             compute_tile(As + cur * A_BYTES, Bs + cur * B_BYTES);
-            if (kt + 1 < kt_end) commit_tile(cur ^ 1);
+            if (kt + 1 < kt_end) commit_tile(cur ^ 1, kt + 1);
             __syncthreads();
         }
+    }
+
+    if (do_rs) {
+        // reduce the per-thread sums over the threads that share a row-vector (LDS float atomics), then one
+        // global atomic per row; the operand LDS is idle here (the main loop ended with a barrier)
+        constexpr int EPV_ = decltype(la)::EPV, RV_ = decltype(la)::RV, BLOCKS_ = decltype(la)::BLOCKS;
+        float *red = (float *)smem;
+        for (int t = threadIdx.x; t < BM; t += THREADS) red[t] = 0.f;
+        __syncthreads();
+        if (!A_KMAJOR) {
+#pragma unroll
+            for (int pp = 0; pp < decltype(la)::PASSES_T; ++pp) {
+                const int blk = threadIdx.x + pp * THREADS;
+                if (blk < BLOCKS_) {
+                    const int rv = blk % RV_;
+#pragma unroll
+                    for (int e = 0; e < EPV_; ++e) atomicAdd(red + rv * EPV_ + e, rs[pp * EPV_ + e]);
+                }
+            }
+        }
+        __syncthreads();
+        for (int t = threadIdx.x; t < BM; t += THREADS)
+            if (t < m_left) atomicAdd(p.rowsum + m0 + t, red[t]);
+        __syncthreads();
     }
 
     // epilogue: acc[i][j][r] is C[m, n] with m = wm + i*32 + lane%32, n = wn + j*32 + (r/4)*8 + (lane/32)*4 + r%4.

@@ -516,10 +516,9 @@ class ShardExecutor:
             side = self._side_ok(w, b)
 
             def wgrad():
+                # the bias gradient (column sums of dy) is taken by the same kernel as dy passes through it
                 ops.gemm(dy, xt, gw, N, K, M, transA=True, lda=ldc, ldb=lda, accumulate=accw,
-                         workspace=self.side_workspace if side else None)
-                if gb is not None:
-                    ops.colsum(dy, gb, M, N, ldc, accb)
+                         workspace=self.side_workspace if side else None, a_rowsum=gb)
             if side:
                 self._emit_side(wgrad, (dy, xt))
             else:
@@ -651,12 +650,10 @@ class ShardExecutor:
             ws = self.side_workspace if side else None
 
             def wgrad_out():
-                ops.gemm(do, ctx, gwo, E, E, M, transA=True, accumulate=acc_wo, workspace=ws)
-                ops.colsum(do, gbo, M, E, E, acc_bo)
+                ops.gemm(do, ctx, gwo, E, E, M, transA=True, accumulate=acc_wo, workspace=ws, a_rowsum=gbo)
 
             def wgrad_in():
-                ops.gemm(dqkv, x.t, gwi, 3 * E, E, M, transA=True, accumulate=acc_wi, workspace=ws)
-                ops.colsum(dqkv, gbi, M, 3 * E, 3 * E, acc_bi)
+                ops.gemm(dqkv, x.t, gwi, 3 * E, E, M, transA=True, accumulate=acc_wi, workspace=ws, a_rowsum=gbi)
 
             def backward():
                 if not side:

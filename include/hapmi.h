@@ -131,6 +131,10 @@ typedef struct {
     int64_t strideA1, strideA2, strideB1, strideB2, strideC1, strideC2;
     void *workspace;             /* optional float32 scratch for split-K (16-byte aligned) or NULL;   */
     int64_t workspace_bytes;     /* a split needs M * roundup(N, 4) * 4 bytes; unused when batch > 1 */
+    float *a_rowsum;             /* optional: a_rowsum[m] += sum over k of op(A)[m, k] (float32 atomics, so the
+                                  * caller clears it): the bias gradient of F.linear when the call is the weight
+                                  * gradient dW = dY^T X, i.e. the column sum that autograd takes of dY
+                                  * (hap.rs:1032 F.linear with bias).  Needs transA = 1 and batch 1; NULL = off */
 } hapmi_gemm_args;
 int hapmi_gemm(const hapmi_gemm_args *args_host, hapmi_stream_t stream);
 

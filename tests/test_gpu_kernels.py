@@ -272,6 +272,37 @@ def test_gemm_split_k_and_tile_configs(cuda, dtype, cfg):
         lib().hapmi_gemm_tuning(-1, 0)
 
 
+@pytest.mark.parametrize("dtype,cfg", [(torch.float32, 0), (torch.bfloat16, 0), (torch.bfloat16, 1), (torch.bfloat16, 2),
+                                       (torch.bfloat16, 3), (torch.bfloat16, 4), (torch.bfloat16, 5), (torch.bfloat16, 6)])
+@pytest.mark.parametrize("tB", [False, True])
+def test_gemm_row_sums_of_a_transposed_operand(cuda, dtype, cfg, tB):
+    """a_rowsum: the weight-gradient call dW = dY^T X also returns the column sums of dY (the bias gradient),
+    added into a caller-cleared float32 vector -- for every tile configuration, with and without K splits,
+    ragged M / N / K, on top of earlier contents."""
+    from hap_amd._lib import lib
+    g = torch.Generator().manual_seed(11 + cfg)
+    M, N, K = 328, 520, 1000                                   # not multiples of any tile; K not a multiple of 64
+    A = torch.randn(K, M, generator=g).to(dtype)
+    B = (torch.randn(N, K, generator=g) if tB else torch.randn(K, N, generator=g)).to(dtype)
+    start = torch.randn(M, generator=g)
+    want_c = A.double().t() @ (B.double().t() if tB else B.double())
+    want_rs = start.double() + A.double().sum(0)
+    ws = torch.empty(8 * M * 520, dtype=torch.float32, device=cuda)
+    try:
+        for splits in (1, 4):
+            lib().hapmi_gemm_tuning(cfg, splits)
+            C = torch.empty(M, N, dtype=torch.float32, device=cuda)
+            rs = start.clone().to(cuda)
+            ops.gemm(A.to(cuda), B.to(cuda), C, M, N, K, transA=True, transB=tB, workspace=ws, a_rowsum=rs)
+            close(C, want_c, dtype, scale=2.0)
+            tol = 1e-5 if dtype == torch.float32 else 1e-4       # float32 sums of exactly represented inputs
+            torch.testing.assert_close(rs.cpu().double(), want_rs, rtol=tol, atol=tol * K ** 0.5)
+    finally:
+        lib().hapmi_gemm_tuning(-1, 0)
+    with pytest.raises(Exception):
+        ops.gemm(A.t().contiguous().to(cuda), B.to(cuda), C, M, N, K, transA=False, transB=tB, a_rowsum=rs)
+
+
 @pytest.mark.parametrize("S,causal", [(16, True), (128, True), (197, False), (512, False), (200, True), (64, False)])
 def test_fused_attention_forward_backward(cuda, S, causal):
     """Fused bf16 attention against the explicit softmax(QK^T * scale + mask) V of
