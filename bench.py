@@ -13,6 +13,7 @@ from __future__ import annotations
 
 import argparse
 import json
+import math
 import os
 import sys
 import time
@@ -143,7 +144,7 @@ def main():
 
     import torch
     import hap_amd
-    from hap_amd import ops
+    from hap_amd import ops, planner
     from hap_amd._lib import lib
 
     desc, dtype = WORKLOADS[args.workload]
@@ -226,6 +227,10 @@ def main():
                      "launches_per_step": n_launch.value / max(1, args.steps if graph is None else 3),
                      "gemm_ms_per_step": ms.value / max(1, args.steps if graph is None else 3), "traffic": None},
     }
+    # the reference calibrates its planner with hap.stat / (seconds of one training step) (profiler.py:33-39)
+    shard_stat = planner.stat(gm, {"input_shape": {"x": tuple(x.shape), "y": tuple(y.shape)}})
+    result["config"]["hap_stat_flops_of_shard"] = shard_stat
+    result["config"]["device_flops"] = math.floor(shard_stat / (ms_per_step * 1e-3))
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(args.workload, meta)
     print(json.dumps(result))

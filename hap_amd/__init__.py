@@ -10,12 +10,14 @@ Public surface (mirrors what /root/reference exposes for this path):
 * ``compile(gm, example_inputs, ...)``    -- ``ShardModule``: call it like the
   reference's ``dmodel`` (worker.py:59-76): ``loss = m(x, y); loss.backward();
   optimizer.step()``, or drive ``m.executor`` directly (``train_step``).
+* ``planner.stat(gm, {"input_shape": ...})`` -- hap.stat (hap.rs:190-209), plus
+  the device_flops calibration and the cost of the fixed plan forms.
 """
 from __future__ import annotations
 
 import torch
 
-from . import collectives, models  # noqa: F401
+from . import collectives, models, planner  # noqa: F401
 from .sharding import ShardingPlan, shard_inplace, sharding_lengths, sharding_round  # noqa: F401
 from .program import build_program  # noqa: F401
 from .executor import ShardExecutor, compile_program  # noqa: F401
