@@ -157,6 +157,27 @@ class ShardExecutor:
             self.params[name] = dict(param=p, master=view, grad=g, shadow=sh, offset=o, numel=n)
         if self.shadow is not None:
             ops.cast(self.master, self.shadow)
+        # whole-shape float32 gradients of parameters that are stored as shards and gathered at use; vectors
+        # first, as in the flat gradient buffer, so that one fill clears them
+        gathered = []
+        for node in self.gm.graph.nodes:
+            if (node.op == "call_function" and node.target is collectives.all_gather
+                    and node.args[0].op == "get_attr" and node.args[0].target in self.params):
+                shape = (sum(node.args[2]),) + tuple(self.params[node.args[0].target]["param"].shape[1:])
+                gathered.append((node.args[0].target, shape))
+        gathered.sort(key=lambda kv: 0 if len(kv[1]) == 1 else 1)
+        off, spans = 0, []
+        self.n_gathered_vector_region = 0
+        for name, shape in gathered:
+            n = 1
+            for v in shape:
+                n *= v
+            spans.append((name, shape, off, n))
+            off += _round_up(n, 64)
+            if len(shape) == 1:
+                self.n_gathered_vector_region = off
+        self.gathered_grad = torch.zeros(max(off, 4), dtype=torch.float32, device=self.dev) if gathered else None
+        self._gathered_grads = {name: self.gathered_grad[o:o + n].view(shape) for name, shape, o, n in spans}
 
     def _fetch(self, target: str):
         obj = self.gm
@@ -823,10 +844,10 @@ class ShardExecutor:
         """pad own shard -> [wire] -> cut pads and concatenate.  Returns the full tensor."""
         m, W = max(L), len(L)
         pshape = ops._with_dim(x_t.shape, dim, m)
-        own = self._new(pshape)
-        peers = self._peers(tag, direction, rank, W, pshape, False)
+        own = self._new(pshape, x_t.dtype)
+        peers = self._peers(tag, direction, rank, W, pshape, False, x_t.dtype)
         slices = [own if s == rank else peers[s] for s in range(W)]
-        full = self._new(ops._with_dim(x_t.shape, dim, sum(L)))
+        full = self._new(ops._with_dim(x_t.shape, dim, sum(L)), x_t.dtype)
         sink.append(lambda: (ops.pad_rows(x_t, dim, m, own), ops.unpad_concat(slices, L, dim, full)))
         return full
 
@@ -834,16 +855,18 @@ class ShardExecutor:
         """split + pad -> [wire] -> rank-ordered float32 sum of the pieces for this rank, pad cut off."""
         m, W = max(L), len(L)
         pshape = ops._with_dim(full_t.shape, dim, m)
-        sent = [self._new(pshape) for _ in range(W)]
-        peers = self._peers(tag, direction, rank, W, pshape, True)
+        sent = [self._new(pshape, full_t.dtype) for _ in range(W)]
+        peers = self._peers(tag, direction, rank, W, pshape, True, full_t.dtype)
         contribs = [sent[rank] if s == rank else peers[s] for s in range(W)]
         contribs = [c for c in contribs if c is not None]
-        out = out_t if out_t is not None else self._new(ops._with_dim(full_t.shape, dim, L[rank]))
+        out = out_t if out_t is not None else self._new(ops._with_dim(full_t.shape, dim, L[rank]), full_t.dtype)
         sink.append(lambda: (ops.split_pad(full_t, L, dim, m, sent), ops.ragged_reduce(contribs, dim, 0, L[rank], out)))
         return out
 
     def _all_gather(self, node):
         x, dim, L, rank = self._val(node.args[0]), node.args[1], list(node.args[2]), node.args[3]
+        if x.kind == "param":
+            return self._gathered_param(node, x, dim, L, rank)
         if x.t is None or x.ld is not None:
             self._unsupported(node, f"all_gather of a {x.kind} value")
         full = self._emit_gather(node.name, "fwd", x.t, dim, L, rank, self.fwd)
@@ -858,6 +881,28 @@ class ShardExecutor:
                 part = self._emit_scatter(node.name, "bwd", out.grad, dim, L, rank, self.bwd)
                 g = x.grad
                 self.bwd.append(lambda: ops.add(g, part, g))
+        self._tape.append(emit)
+        return out
+
+    def _gathered_param(self, node, x: Val, dim, L, rank):
+        """A parameter stored as its dim-0 shard and gathered at use (get_attr_zero, hap.rs:2527-2547).  Forward:
+        the shard (bf16 shadow for matrices, float32 master for vectors, which consumers add in float32) is
+        gathered every step.  The consumers see a whole parameter whose float32 gradient is a buffer of the
+        whole shape; once they have all written it, that gradient is reduce-scattered into the shard's slot
+        of the flat gradient buffer (all_gather's backward, collectives.py:63-68)."""
+        if dim != 0 or x.t.shape[0] != L[rank]:
+            self._unsupported(node, "a gathered parameter must be a dim-0 shard of the plan's length")
+        vector = x.t.dim() == 1
+        src = x.meta["master"] if vector else x.t
+        full = self._emit_gather(node.name, "fwd", src, 0, L, rank, self.fwd)
+        full_grad = self._gathered_grads[x.meta["name"]]
+        out = Val("param", full, master=full if vector else None, grad=full_grad, needs_grad=True, shard_of=x.meta["name"])
+
+        def emit():
+            if not out.meta.get("grad_written"):
+                return
+            x.meta["grad_written"] = True
+            self._emit_scatter(node.name, "bwd", full_grad, 0, L, rank, self.bwd, out_t=x.meta["grad"])
         self._tape.append(emit)
         return out
 
@@ -1122,6 +1167,8 @@ class ShardExecutor:
     def _backward_launches(self):
         if self.n_vector_region:
             ops.fill_zero(self.flat_grad[:self.n_vector_region])
+        if self.n_gathered_vector_region:
+            ops.fill_zero(self.gathered_grad[:self.n_gathered_vector_region])
         for f in self.bwd:
             f()
         self._join_side()

@@ -8,6 +8,8 @@ these graphs is an executor for the synthesizer's output:
 
 * inputs       placeholder -> ``.split(lengths, dim)`` -> ``getitem(rank)``  (hap.rs:2504-2520)
 * parameters   replicated: ``get_attr`` -> ``collectives.replicate``          (hap.rs:2561-2568)
+               ZeRO: ``get_attr`` of the dim-0 shard -> ``collectives.all_gather(p, 0, L, rank)``
+                                                                             (hap.rs:2527-2547)
                sharded: ``get_attr`` of a tensor sliced in place             (hap.rs:2588-2596, 36-47)
 * ops          ``F.linear(x, w, b)`` (1032), ``torch.transpose(x, a, b)`` (1213),
                ``F.multi_head_attention_forward(**kw)`` + 2 getitems (1301-1327),
@@ -30,6 +32,9 @@ Plans (each step is a legal Hoare triple of hap.rs:2786-3419):
 ``ffn="batch"``   pure uneven data parallelism;
 MoE layers        gating on replicated tokens, experts sharded over the
                   expert dimension, combine -> reduce_scatter / all_reduce.
+``zero=True``     on top of any of them: every parameter that would be
+                  replicated is stored as a dim-0 shard (the reference's
+                  ``extra_ps`` / force_zero mode).
 """
 from __future__ import annotations
 
@@ -65,10 +70,25 @@ class _Emitter:
 
     # parameters ---------------------------------------------------------
     def replicated(self, target: str):
+        """A parameter or buffer every device needs whole: kept whole and ``replicate``d (hap.rs:2561-2568), or,
+        under ``plan.zero``, stored as its dim-0 shard and ``all_gather``ed at use (get_attr_zero,
+        hap.rs:2527-2547; a leading dimension of 1 keeps the replicated form, as there)."""
         if target not in self._attr_cache:
-            attr = self.g.get_attr(target)
-            self._attr_cache[target] = self.g.call_function(collectives.replicate, (attr,))
+            if self.plan.zero and self._shape(target)[0] != 1:
+                lengths = self.plan.lengths(self._shape(target)[0])
+                shard_inplace(self.module, target, lengths, 0, self.rank)
+                attr = self.g.get_attr(target)
+                self._attr_cache[target] = self.g.call_function(collectives.all_gather, (attr, 0, lengths, self.rank))
+            else:
+                attr = self.g.get_attr(target)
+                self._attr_cache[target] = self.g.call_function(collectives.replicate, (attr,))
         return self._attr_cache[target]
+
+    def _shape(self, target: str):
+        obj = self.module
+        for atom in target.split("."):
+            obj = getattr(obj, atom)
+        return tuple(obj.shape)
 
     def sharded(self, target: str, full_length: int, dim: int):
         if target not in self._attr_cache:

@@ -55,6 +55,7 @@ class ShardingPlan:
     rank: int
     ffn: str = "column"          # "column": FFN1 column-sharded (plan P1); "batch": pure DP (plan P2)
     segment: int = 0
+    zero: bool = False           # parameters stored as dim-0 shards and all_gather-ed at use (hap.rs:2527-2547)
 
     @property
     def world_size(self) -> int:

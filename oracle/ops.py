@@ -167,6 +167,14 @@ def _accumulate(parts: Sequence[torch.Tensor]) -> torch.Tensor:
     return acc.to(parts[0].dtype)
 
 
+def _snapshot(messages):
+    """Detached copies for the wire log: a message that needed no padding or splitting is the sender's own tensor
+    (a parameter, when parameters are gathered), which a later optimizer step would change under the log."""
+    if isinstance(messages, torch.Tensor):
+        return messages.detach().clone()
+    return [_snapshot(m) for m in messages]
+
+
 class JointWorld:
     """All W ranks of the SPMD program live in one process; each collective is
     one autograd node over the W per-rank tensors, so one backward pass yields
@@ -186,7 +194,7 @@ class JointWorld:
             def forward(ctx, *xs):
                 m = max(L)
                 sent = [_padded(x, dim, m).contiguous() for x in xs]                    # :19
-                world.log[(tag, "fwd")] = [[sent[src] for _ in range(world.W)] for src in range(world.W)]
+                world.log[(tag, "fwd")] = _snapshot([[sent[src] for _ in range(world.W)] for src in range(world.W)])
                 out = torch.cat([s.split([l, m - l], dim=dim)[0] for s, l in zip(sent, L)], dim=dim)  # :20
                 return tuple(out.clone() for _ in range(world.W))
 
@@ -195,7 +203,7 @@ class JointWorld:
                 m = max(L)
                 sent = [[_padded(p, dim, m).contiguous() for p in torch.split(g.contiguous(), L, dim=dim)]
                         for g in gs]                                                       # :24-25
-                world.log[(tag, "bwd")] = sent
+                world.log[(tag, "bwd")] = _snapshot(sent)
                 outs = []
                 for r in range(world.W):
                     red = _accumulate([sent[src][r] for src in range(world.W)])            # :27
@@ -214,7 +222,7 @@ class JointWorld:
                 m = max(L)
                 sent = [[_padded(p, dim, m).contiguous() for p in torch.split(x.contiguous(), L, dim=dim)]
                         for x in xs]                                                       # :92-93
-                world.log[(tag, "fwd")] = sent
+                world.log[(tag, "fwd")] = _snapshot(sent)
                 outs = []
                 for r in range(world.W):
                     red = _accumulate([sent[src][r] for src in range(world.W)])            # :95
@@ -225,7 +233,7 @@ class JointWorld:
             def backward(ctx, *gs):
                 m = max(L)
                 sent = [_padded(g.contiguous(), dim, m).contiguous() for g in gs]          # :101
-                world.log[(tag, "bwd")] = [[sent[src] for _ in range(world.W)] for src in range(world.W)]
+                world.log[(tag, "bwd")] = _snapshot([[sent[src] for _ in range(world.W)] for src in range(world.W)])
                 grad = torch.cat([s.split([l, m - l], dim=dim)[0] for s, l in zip(sent, L)], dim=dim)  # :102
                 return tuple(grad.clone() for _ in range(world.W))
 
@@ -240,7 +248,7 @@ class JointWorld:
             def forward(ctx, *xs):
                 sent = [[p.contiguous() for p in torch.split(x.contiguous(), split_L, dim=split_dim)]
                         for x in xs]                                                       # :156-158
-                world.log[(tag, "fwd")] = sent
+                world.log[(tag, "fwd")] = _snapshot(sent)
                 return tuple(torch.cat([sent[src][r] for src in range(world.W)], dim=cat_dim)  # :159
                              for r in range(world.W))
 
@@ -248,7 +256,7 @@ class JointWorld:
             def backward(ctx, *gs):
                 sent = [[p.contiguous() for p in torch.split(g.contiguous(), cat_L, dim=cat_dim)]
                         for g in gs]                                                       # :163-165
-                world.log[(tag, "bwd")] = sent
+                world.log[(tag, "bwd")] = _snapshot(sent)
                 return tuple(torch.cat([sent[src][r] for src in range(world.W)], dim=split_dim)  # :166
                              for r in range(world.W))
 
@@ -262,14 +270,14 @@ class JointWorld:
             @staticmethod
             def forward(ctx, *xs):
                 sent = [x.contiguous() for x in xs]
-                world.log[(tag, "fwd")] = [[sent[src] for _ in range(world.W)] for src in range(world.W)]
+                world.log[(tag, "fwd")] = _snapshot([[sent[src] for _ in range(world.W)] for src in range(world.W)])
                 total = _accumulate(sent)
                 return tuple(total.clone() for _ in range(world.W))
 
             @staticmethod
             def backward(ctx, *gs):
                 sent = [g.clone() for g in gs]
-                world.log[(tag, "bwd")] = [[sent[src] for _ in range(world.W)] for src in range(world.W)]
+                world.log[(tag, "bwd")] = _snapshot([[sent[src] for _ in range(world.W)] for src in range(world.W)])
                 total = _accumulate(sent)
                 return tuple(total.clone() for _ in range(world.W))
 
@@ -287,7 +295,7 @@ class JointWorld:
             @staticmethod
             def backward(ctx, *gs):
                 sent = [g.contiguous() for g in gs]
-                world.log[(tag, "bwd")] = [[sent[src] for _ in range(world.W)] for src in range(world.W)]
+                world.log[(tag, "bwd")] = _snapshot([[sent[src] for _ in range(world.W)] for src in range(world.W)])
                 total = _accumulate(sent)
                 return tuple(total.clone() for _ in range(world.W))
 

@@ -16,7 +16,7 @@ pytestmark = pytest.mark.gpu
 
 def _gpu_rank(model, ratios, rank, B, x, y, log, dtype, opt, **kw):
     m = copy.deepcopy(model)
-    plan = hap_amd.ShardingPlan([list(ratios)], rank, ffn=kw.get("ffn", "column"))
+    plan = hap_amd.ShardingPlan([list(ratios)], rank, ffn=kw.get("ffn", "column"), zero=kw.get("zero", False))
     gm = hap_amd.build_program(m, plan, B, activation=kw.get("activation", "relu"),
                                batch_sharded=kw.get("batch_sharded", True))
     ex = hap_amd.compile_program(gm, [x, y], dtype=dtype, wire=hap_amd.ReplayWire(log, rank), rank=rank,
@@ -127,6 +127,29 @@ def test_moe_bf16_routing_matches(cuda):
     model = make_moe(d=64, F=96, std=0.3)
     x, y = lm_batch(4, 16, 61)
     run = _compare(model, RATIOS_E, 4, x, y, "bf16", [0], ADAM, ffn="batch", batch_sharded=False)
+
+
+@pytest.mark.parametrize("ffn", ["column", "batch"])
+def test_zero_sharded_parameters_lm_fp32(cuda, ffn):
+    """Parameters stored as dim-0 shards, all_gather-ed forward and reduce-scattered backward (hap.rs:2527-2547)."""
+    model = make_lm()
+    x, y = lm_batch(8, 16, 97)
+    _compare(model, RATIOS4, 8, x, y, "fp32", [0, 3], SGD, ffn=ffn, zero=True)
+
+
+def test_zero_sharded_parameters_bf16_adam(cuda):
+    model = make_lm(vocab=1003, S=32, d=64, H=4, F=128, layers=2, causal=False)
+    x, y = lm_batch(8, 32, 1003, mlm=True)
+    _compare(model, RATIOS4, 8, x, y, "bf16", [0, 2], ADAM, zero=True)
+
+
+def test_zero_sharded_parameters_vit_and_moe(cuda):
+    model = make_vit(img=32, patch=8, d=64, F=128)
+    x, y = vit_batch(8, 32, 10)
+    _compare(model, RATIOS4, 8, x, y, "fp32", [0, 3], ADAM, ffn="batch", zero=True)
+    model = make_moe()
+    x, y = lm_batch(16, 16, 61)
+    _compare(model, RATIOS_E, 16, x, y, "fp32", [0, 2], ADAM, ffn="batch", zero=True)
 
 
 def test_module_facade_is_a_drop_in(cuda):

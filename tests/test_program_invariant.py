@@ -19,7 +19,7 @@ def _single(model, x, y):
     return loss.detach(), dict(m.named_parameters())
 
 
-def _check(model, run, x, y, sharded):
+def _check(model, run, x, y, sharded, whole_norm=False):
     loss1, p1 = _single(model, x, y)
     losses = run.step(x, y)
     torch.testing.assert_close(sum(l.double() for l in losses).float(), loss1, rtol=1e-5, atol=1e-5)
@@ -36,7 +36,12 @@ def _check(model, run, x, y, sharded):
             dim, L = sharded[name]
             want = torch.split(ref_p.grad, L, dim)
             for r in range(W):
-                assert rel_err(grads[r], want[r]) < 2e-5, (name, r)
+                if whole_norm:
+                    # a shard may hold only rows whose true gradient is zero (the key bias of softmax attention):
+                    # its error is measured against the whole parameter's gradient
+                    assert (grads[r] - want[r]).norm() < 2e-5 * ref_p.grad.norm(), (name, r)
+                else:
+                    assert rel_err(grads[r], want[r]) < 2e-5, (name, r)
         else:
             for r in range(W):                 # replicate.backward all-reduces: every rank holds the full gradient
                 assert rel_err(grads[r], ref_p.grad) < 2e-5, (name, r)
@@ -86,3 +91,39 @@ def test_moe_spmd_equals_single_device(batch_sharded):
             torch.testing.assert_close(l, loss1, rtol=1e-5, atol=1e-5)
         return
     _check(model, run, x, y, sharded)
+
+
+def _zero_sharded(model, ratios, already=()):
+    """Under the ZeRO form every parameter with a leading dimension other than 1 is a dim-0 shard (hap.rs:2527-2547)."""
+    out = {}
+    for name, p in model.named_parameters():
+        if name not in already and p.shape[0] != 1:
+            out[name] = (0, hap_amd.sharding_lengths(p.shape[0], ratios))
+    return out
+
+
+@pytest.mark.parametrize("ffn", ["column", "batch"])
+def test_zero_lm_spmd_equals_single_device(ffn):
+    model = make_lm()
+    B = 8
+    x, y = lm_batch(B, 16, 97)
+    run = joint_cpu(model, RATIOS4, B, ffn=ffn, zero=True)
+    # the shards are what the program's modules hold: 97 vocabulary rows over 4 ranks, 96 in_proj rows, ...
+    held = dict(run.programs[2].named_parameters())
+    assert held["encoder.weight"].shape[0] == hap_amd.sharding_lengths(97, RATIOS4)[2]
+    assert held["layers.0.self_attn.in_proj_weight"].shape == (12, 32)
+    assert run.programs[2].src_mask.shape == (2, 16)
+    _check(model, run, x, y, _zero_sharded(model, RATIOS4), whole_norm=True)
+
+
+def test_zero_vit_and_moe_spmd_equal_single_device():
+    model = make_vit()
+    x, y = vit_batch(8, 16, 10)
+    run = joint_cpu(model, RATIOS4, 8, ffn="batch", zero=True)
+    assert dict(run.programs[0].named_parameters())["pos_embed"].shape == (1, 17, 32)      # leading 1: left whole
+    _check(model, run, x, y, _zero_sharded(model, RATIOS4), whole_norm=True)
+
+    model = make_moe()
+    x, y = lm_batch(16, 16, 61)
+    run = joint_cpu(model, RATIOS_E, 16, ffn="batch", zero=True)
+    _check(model, run, x, y, _zero_sharded(model, RATIOS_E), whole_norm=True)
