@@ -5,7 +5,9 @@
 // either type is one 16-byte LDS read.  Rows are not padded; the eight 16-byte chunks of a row are
 // XOR-swizzled with (row ^ row >> 3) & 7, which makes the fragment reads, the row-wise tile stores and the
 // transposing tile stores spread over all banks.  An operand whose reduction dimension is the slow one in
-// memory (dgrad's weight, both operands of wgrad) is transposed in registers on its way into LDS.
+// memory (dgrad's weight, both operands of wgrad) is, for bf16, kept in LDS as it lies in memory and
+// transposed by the LDS reads that assemble its fragments (TrTile); for float32 it is transposed in
+// registers on its way into LDS.
 // Ragged M / N / K are handled by guarded edge loads and stores; the interior of every tile runs unguarded
 // 16-byte accesses.  Small outputs with a long reduction (wgrad) are split along K over blockIdx.y into
 // a caller-provided float32 workspace and summed in split order by a second kernel (deterministic).
@@ -16,6 +18,7 @@
 #pragma once
 #include "common.h"
 #include "tile.h"
+#include <type_traits>
 
 struct GemmParams {
     const void *A, *B;
@@ -108,24 +111,31 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, (WAVES_M * WAVES_N <= 4 ? 2 
     const int64_t a_kstep = A_KMAJOR ? (int64_t)BK : (int64_t)BK * p.lda;
     const int64_t b_kstep = B_KMAJOR ? (int64_t)BK : (int64_t)BK * p.ldb;
 
-    TileLoader<TI, BM, THREADS, A_KMAJOR> la;
-    TileLoader<TI, BN, THREADS, B_KMAJOR> lb;
+    // bf16 operands stored [k][row] stay that way in LDS and are transposed by the fragment reads
+    constexpr bool A_TR = !A_KMAJOR && sizeof(TI) == 2, B_TR = !B_KMAJOR && sizeof(TI) == 2;
+    typedef TrTile<BM, THREADS> TrA;
+    typedef TrTile<BN, THREADS> TrB;
+    typename std::conditional<A_TR, TrA, TileLoader<TI, BM, THREADS, A_KMAJOR>>::type la;
+    typename std::conditional<B_TR, TrB, TileLoader<TI, BN, THREADS, B_KMAJOR>>::type lb;
 
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int wm = (wave % WAVES_M) * WTM, wn = (wave / WAVES_M) * WTN;
     const int frow = lane & 31, fh = lane >> 5;
 
     // byte offset of this lane's fragment for k-step 0 inside a tile; k-step s is at offset ^ (s << 5)
+    // ([row][k] tiles) or 16 k lines further ([k][row] tiles)
     int a_off[TM], b_off[TN];
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
         const int row = wm + i * 32 + frow;
-        a_off[i] = row * ROW_BYTES + ((fh ^ swz(row)) << 4);
+        if constexpr (A_TR) a_off[i] = TrA::frag_offset(wm + i * 32);
+        else a_off[i] = row * ROW_BYTES + ((fh ^ swz(row)) << 4);
     }
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
         const int row = wn + j * 32 + frow;
-        b_off[j] = row * ROW_BYTES + ((fh ^ swz(row)) << 4);
+        if constexpr (B_TR) b_off[j] = TrB::frag_offset(wn + j * 32);
+        else b_off[j] = row * ROW_BYTES + ((fh ^ swz(row)) << 4);
     }
 
     f32x16 acc[TM][TN];
@@ -141,9 +151,15 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, (WAVES_M * WAVES_N <= 4 ? 2 
         for (int ks = 0; ks < KSTEPS; ++ks) {
             Vec16<TI> fa[TM], fb[TN];
 #pragma unroll
-            for (int i = 0; i < TM; ++i) fa[i] = *(const Vec16<TI> *)(as + (a_off[i] ^ (ks << 5)));
+            for (int i = 0; i < TM; ++i) {
+                if constexpr (A_TR) fa[i].v = TrA::read_frag(as, a_off[i], ks);
+                else fa[i] = *(const Vec16<TI> *)(as + (a_off[i] ^ (ks << 5)));
+            }
 #pragma unroll
-            for (int j = 0; j < TN; ++j) fb[j] = *(const Vec16<TI> *)(bs + (b_off[j] ^ (ks << 5)));
+            for (int j = 0; j < TN; ++j) {
+                if constexpr (B_TR) fb[j].v = TrB::read_frag(bs, b_off[j], ks);
+                else fb[j] = *(const Vec16<TI> *)(bs + (b_off[j] ^ (ks << 5)));
+            }
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -151,25 +167,28 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, (WAVES_M * WAVES_N <= 4 ? 2 
         }
     };
 
-    // Optional row sums of op(A) (the bias gradient when A is dY of a weight-gradient GEMM): A tiles of a
-    // k-major operand pass through registers on their way to LDS, where they are summed along k.  Every block
-    // of a tile row sees the same A tiles, so the k-tiles are dealt round-robin over the tiles_n blocks of
-    // the row: each block adds 1/tiles_n of the work instead of one block in tiles_n doing all of it.
+    // Optional row sums of op(A) (the bias gradient when A is dY of a weight-gradient GEMM), taken from the A
+    // tiles as they pass: float32 tiles in registers on their way to LDS (rs_add), bf16 tiles from LDS once
+    // they are complete (rs_add_lds).  Every block of a tile row sees the same A tiles, so the k-tiles are
+    // dealt round-robin over the tiles_n blocks of the row: each block adds 1/tiles_n of the work instead of
+    // one block in tiles_n doing all of it.
     const bool do_rs = !A_KMAJOR && p.rowsum != nullptr;
-    constexpr int RS_N = A_KMAJOR ? 1 : decltype(la)::PASSES_T * decltype(la)::EPV;
+    constexpr int RS_N = A_KMAJOR ? 1 : (A_TR ? 8 : TileLoader<TI, BM, THREADS, false>::PASSES_T * EPV);
     float rs[RS_N];
 #pragma unroll
     for (int e = 0; e < RS_N; ++e) rs[e] = 0.f;
     auto rs_add = [&]() {
-        if (!A_KMAJOR) {
-            constexpr int EPV_ = decltype(la)::EPV;
+        if constexpr (!A_KMAJOR && !A_TR) {
 #pragma unroll
             for (int pp = 0; pp < decltype(la)::PASSES_T; ++pp)
 #pragma unroll
                 for (int q = 0; q < 4; ++q)
 #pragma unroll
-                    for (int e = 0; e < EPV_; ++e) rs[pp * EPV_ + e] += la.v[pp * 4 + q].get(e);
+                    for (int e = 0; e < EPV; ++e) rs[pp * EPV + e] += la.v[pp * 4 + q].get(e);
         }
+    };
+    auto rs_add_lds = [&](const char *as) {
+        if constexpr (A_TR) TrA::add_row_sums(as, rs);
     };
 
     // A ragged last k-tile (K not a multiple of the tile depth) is done first, alone, with guarded loads, so
@@ -184,6 +203,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, (WAVES_M * WAVES_N <= 4 ? 2 
         la.store(As);
         lb.store(Bs);
         __syncthreads();
+        if (do_rs && kt_end % p.tiles_n == tn) rs_add_lds(As);
         compute_tile(As, Bs);
         __syncthreads();
     }
@@ -191,20 +211,21 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, (WAVES_M * WAVES_N <= 4 ? 2 
     if (kt0 < kt_end) {
         // complete k-tiles: row-major operands go global -> LDS directly, k-major operands through registers
         // (transposed on the LDS store)
-        if (A_KMAJOR) la.init_direct(p.lda, m_left);
+        constexpr bool A_DIRECT = A_KMAJOR || A_TR, B_DIRECT = B_KMAJOR || B_TR;
+        if constexpr (A_DIRECT) la.init_direct(p.lda, m_left);
         else la.init_offsets(p.lda, m_left);
-        if (B_KMAJOR) lb.init_direct(p.ldb, n_left);
+        if constexpr (B_DIRECT) lb.init_direct(p.ldb, n_left);
         else lb.init_offsets(p.ldb, n_left);
         auto issue_tile = [&](int kt, int buf) {
-            if (A_KMAJOR) la.load_direct(a_base + (int64_t)kt * a_kstep, As + buf * A_BYTES);
+            if constexpr (A_DIRECT) la.load_direct(a_base + (int64_t)kt * a_kstep, As + buf * A_BYTES);
             else la.load_fast(a_base + (int64_t)kt * a_kstep, p.lda);
-            if (B_KMAJOR) lb.load_direct(b_base + (int64_t)kt * b_kstep, Bs + buf * B_BYTES);
+            if constexpr (B_DIRECT) lb.load_direct(b_base + (int64_t)kt * b_kstep, Bs + buf * B_BYTES);
             else lb.load_fast(b_base + (int64_t)kt * b_kstep, p.ldb);
         };
         auto commit_tile = [&](int buf, int kt) {
             if (do_rs && kt % p.tiles_n == tn) rs_add();
-            if (!A_KMAJOR) la.store(As + buf * A_BYTES);
-            if (!B_KMAJOR) lb.store(Bs + buf * B_BYTES);
+            if constexpr (!A_DIRECT) la.store(As + buf * A_BYTES);
+            if constexpr (!B_DIRECT) lb.store(Bs + buf * B_BYTES);
             __builtin_amdgcn_s_waitcnt(0x0F70);                   // vmcnt(0): this wave's direct loads have landed
         };
         issue_tile(kt0, 0);
@@ -213,6 +234,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, (WAVES_M * WAVES_N <= 4 ? 2 
         for (int kt = kt0; kt < kt_end; ++kt) {
             const int cur = (kt - kt0) & 1;
             if (kt + 1 < kt_end) issue_tile(kt + 1, cur ^ 1);
+            if (do_rs && kt % p.tiles_n == tn) rs_add_lds(As + cur * A_BYTES);
             compute_tile(As + cur * A_BYTES, Bs + cur * B_BYTES);
             if (kt + 1 < kt_end) commit_tile(cur ^ 1, kt + 1);
             __syncthreads();
@@ -222,18 +244,23 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, (WAVES_M * WAVES_N <= 4 ? 2 
     if (do_rs) {
         // reduce the per-thread sums over the threads that share a row-vector (LDS float atomics), then one
         // global atomic per row; the operand LDS is idle here (the main loop ended with a barrier)
-        constexpr int EPV_ = decltype(la)::EPV, RV_ = decltype(la)::RV, BLOCKS_ = decltype(la)::BLOCKS;
         float *red = (float *)smem;
         for (int t = threadIdx.x; t < BM; t += THREADS) red[t] = 0.f;
         __syncthreads();
-        if (!A_KMAJOR) {
+        if constexpr (A_TR) {
+            if ((int)threadIdx.x < TrA::KP * TrA::CPR) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) atomicAdd(red + ((int)threadIdx.x % TrA::CPR) * 8 + e, rs[e]);
+            }
+        } else if constexpr (!A_KMAJOR) {
+            constexpr int RV_ = decltype(la)::RV, BLOCKS_ = decltype(la)::BLOCKS;
 #pragma unroll
             for (int pp = 0; pp < decltype(la)::PASSES_T; ++pp) {
                 const int blk = threadIdx.x + pp * THREADS;
                 if (blk < BLOCKS_) {
                     const int rv = blk % RV_;
 #pragma unroll
-                    for (int e = 0; e < EPV_; ++e) atomicAdd(red + rv * EPV_ + e, rs[pp * EPV_ + e]);
+                    for (int e = 0; e < EPV; ++e) atomicAdd(red + rv * EPV + e, rs[pp * EPV + e]);
                 }
             }
         }

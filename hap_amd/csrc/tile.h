@@ -176,3 +176,106 @@ template <typename TI, int ROWS, int THREADS, bool KMAJOR> struct TileLoader {
     }
 };
 
+// A bf16 operand whose reduction dimension is the slow one in memory ([k][row], rows contiguous) kept in LDS
+// the way it lies in memory: [64 k][ROWS] with the 16-byte chunks (8 rows) of a k line XOR-swizzled.  It goes
+// global -> LDS directly (no registers, no transposing stores); the MFMA fragment (8 consecutive k of one row
+// per lane) is assembled by two transposing LDS reads (ds_read_b64_tr_b16).  Within each group of 16 lanes
+// that instruction hands lane j the elements D[4e + j/4][j%4], e = 0..3, of the 16 x 4 matrix D whose row i
+// is the 8 bytes at lane i's address: with lane i pointing at k line i/4, rows 4*(i%4).., lane j receives 4
+// consecutive k of row j.  The swizzle makes the 4 k lines x 64 bytes that a half wave touches in one read
+// fall into different banks: a line is a multiple of 256 bytes -> chunk ^= 4*(k%4); 384-byte lines (ROWS
+// 192) already alternate between bank halves -> chunk ^= 4*((k/2)%2).
+template <int ROWS, int THREADS> struct TrTile {
+    static constexpr int BK = 64;
+    static constexpr int CPR = ROWS / 8;                          // 16-byte chunks per k line
+    static constexpr int LINE = ROWS * 2;                         // bytes per k line
+    static constexpr int CHUNKS = BK * CPR;
+    static constexpr int PASSES = CHUNKS / THREADS;
+    static_assert(ROWS % 64 == 0 && CHUNKS % THREADS == 0, "tile does not divide over the block");
+    static_assert(CPR % 16 == 0 || CPR % 16 == 8, "no bank swizzle for this line length");
+    typedef short v4s __attribute__((ext_vector_type(4)));
+    typedef __attribute__((address_space(3))) v4s lds_v4s;
+
+    __device__ __forceinline__ static int sw(int k) { return CPR % 16 == 0 ? ((k & 3) << 2) : (((k >> 1) & 1) << 2); }
+
+    int doff[PASSES];
+    bf16x8 v[PASSES];                                             // ragged last k-tile only
+
+    // rows beyond rows_left are clamped to the last valid chunk (loaded in bounds, never stored by the epilogue)
+    __device__ __forceinline__ void init_direct(int64_t ld, int64_t rows_left) {
+        const int last_c = ((int)(rows_left < ROWS ? rows_left : ROWS) - 1) >> 3;
+#pragma unroll
+        for (int p = 0; p < PASSES; ++p) {
+            const int q = p * THREADS + threadIdx.x, k = q / CPR;
+            int c = (q % CPR) ^ sw(k);
+            c = c < last_c ? c : last_c;
+            doff[p] = k * (int)ld + c * 8;
+        }
+    }
+
+    __device__ __forceinline__ void load_direct(const bf16_t *base, char *lds) const {
+        typedef __attribute__((address_space(3))) char lds_char;
+        const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+#pragma unroll
+        for (int p = 0; p < PASSES; ++p) {
+            const uint32_t lds_addr = (uint32_t)(uintptr_t)(lds_char *)(lds + (p * (THREADS / 64) + wave) * 1024);
+            const bf16_t *src = base + doff[p];
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                         :
+                         : "s"(lds_addr), "v"(src)
+                         : "memory");
+        }
+    }
+
+    // guarded path for a k-tile that ends inside K
+    __device__ __forceinline__ void load(const bf16_t *base, int64_t ld, int64_t rows_left, int64_t k_left) {
+#pragma unroll
+        for (int p = 0; p < PASSES; ++p) {
+            const int q = p * THREADS + threadIdx.x, k = q / CPR;
+            const int r0 = ((q % CPR) ^ sw(k)) * 8;
+            const bf16_t *src = base + (int64_t)k * ld + r0;
+            if (k < k_left && r0 + 8 <= rows_left) {
+                v[p] = *(const bf16x8 *)src;
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) v[p][e] = (k < k_left && r0 + e < rows_left) ? src[e] : (bf16_t)0.f;
+            }
+        }
+    }
+    __device__ __forceinline__ void store(char *lds) const {
+#pragma unroll
+        for (int p = 0; p < PASSES; ++p) *(bf16x8 *)(lds + (p * THREADS + threadIdx.x) * 16) = v[p];
+    }
+
+    // byte offset of this lane's first transposing read for the 32-row fragment starting at row r0 (k-step 0)
+    __device__ __forceinline__ static int frag_offset(int r0) {
+        const int lane = threadIdx.x & 63, i16 = lane & 15;
+        const int k = 8 * (lane >> 5) + (i16 >> 2);
+        const int row = r0 + 16 * ((lane >> 4) & 1) + 4 * (i16 & 3);
+        return k * LINE + (((row >> 3) ^ sw(k)) << 4) + ((row & 7) << 1);
+    }
+    __device__ __forceinline__ static bf16x8 read_frag(const char *tile, int off, int ks) {
+        union { v4s h[2]; bf16x8 v; } u;
+        u.h[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s *)(tile + off + ks * 16 * LINE));
+        u.h[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s *)(tile + off + ks * 16 * LINE + 4 * LINE));
+        return u.v;
+    }
+
+    // sums over k of the tile's rows: thread t < KP * CPR owns the 8 rows of chunk t % CPR on k lines t / CPR + i * KP
+    static constexpr int KP = THREADS / CPR;
+    static constexpr int RS_PASSES = (BK + KP - 1) / KP;
+    __device__ __forceinline__ static void add_row_sums(const char *tile, float (&rs)[8]) {
+        const int t = threadIdx.x;
+        if (t >= KP * CPR) return;
+        const int c = t % CPR;
+#pragma unroll
+        for (int i = 0; i < RS_PASSES; ++i) {
+            const int k = t / CPR + i * KP;
+            if (k < BK) {
+                const bf16x8 x = *(const bf16x8 *)(tile + k * LINE + ((c ^ sw(k)) << 4));
+#pragma unroll
+                for (int e = 0; e < 8; ++e) rs[e] += (float)x[e];
+            }
+        }
+    }
+};
