@@ -1,4 +1,4 @@
-// Top-2 gating in index form and the dispatch / combine row gathers of the MoE layer.
+// Top-2 and switch (top-1) gating in index form and the dispatch / combine row gathers of the MoE layer.
 // Integer routing (expert index, slot, token_of_slot) is exact; gate values are float32.
 #include "common.h"
 
@@ -12,6 +12,9 @@ constexpr int GATE_MAX_E = 64;
 // first choice among the earlier first choices of the same expert.  Pass B: positions of the second choices,
 // offset per expert by the SUM of its first-choice positions (n(n+1)/2), as the reference adds
 // sum(position_in_expert[:, :, 0, :]) rather than the count.  A position >= C drops the choice (slot 0).
+// TOP_K = 1 is switch gating: pass A only; the second entry of every record is written as a dropped choice
+// (gate 0, slot 0), so the dispatch / combine kernels and the gate backward serve both kinds of record.
+template <int TOP_K>
 __global__ __launch_bounds__(GATE_THREADS) void top2_gate_kernel(const float *logits, float *probs, int32_t *index,
                                                                int32_t *slot, float *gate, int32_t *token_of_slot,
                                                                int S, int E, int C) {
@@ -25,7 +28,7 @@ __global__ __launch_bounds__(GATE_THREADS) void top2_gate_kernel(const float *lo
     for (int e = tid; e < E; e += GATE_THREADS) run[e] = 0;
     __syncthreads();
 
-    for (int pass = 0; pass < 2; ++pass) {
+    for (int pass = 0; pass < TOP_K; ++pass) {
         for (int s0 = 0; s0 < S; s0 += GATE_THREADS) {
             const int s = s0 + tid;
             const bool valid = s < S;
@@ -55,7 +58,8 @@ __global__ __launch_bounds__(GATE_THREADS) void top2_gate_kernel(const float *lo
                     index[tok * 2 + 0] = i0;
                     index[tok * 2 + 1] = i1;
                     gate[tok * 2 + 0] = p0;
-                    gate[tok * 2 + 1] = p1;
+                    gate[tok * 2 + 1] = TOP_K == 2 ? p1 : 0.f;
+                    if (TOP_K == 1) slot[tok * 2 + 1] = 0;
                     my = i0;
                 } else {
                     my = index[tok * 2 + 1];
@@ -281,9 +285,23 @@ extern "C" int hapmi_top2_gate(const float *logits, float *probs, int32_t *index
     HAPMI_REQUIRE(S < (1ll << 30) && B < (1ll << 31) && E * C < (1ll << 31), HAPMI_ELIMIT, "top2_gate: shape too large");
     if (B == 0) return HAPMI_OK;
     HAPMI_REQUIRE(logits && probs && index && slot && gate && token_of_slot, HAPMI_EINVAL, "top2_gate: null pointer");
-    hipLaunchKernelGGL(top2_gate_kernel, dim3((unsigned)B), dim3(GATE_THREADS), 0, (hipStream_t)stream, logits, probs,
+    hipLaunchKernelGGL(top2_gate_kernel<2>, dim3((unsigned)B), dim3(GATE_THREADS), 0, (hipStream_t)stream, logits, probs,
                        index, slot, gate, token_of_slot, (int)S, (int)E, (int)C);
     HAPMI_CHECK_LAUNCH("top2_gate");
+    return HAPMI_OK;
+}
+
+extern "C" int hapmi_switch_gate(const float *logits, float *probs, int32_t *index, int32_t *slot, float *gate,
+                                 int32_t *token_of_slot, int64_t B, int64_t S, int64_t E, int64_t C,
+                                 hapmi_stream_t stream) {
+    HAPMI_REQUIRE(B >= 0 && S >= 1 && C >= 1, HAPMI_EINVAL, "switch_gate: bad shape");
+    HAPMI_REQUIRE(E >= 2 && E <= GATE_MAX_E, HAPMI_ELIMIT, "switch_gate: n_expert %lld outside 2..%d", (long long)E, GATE_MAX_E);
+    HAPMI_REQUIRE(S < (1ll << 30) && B < (1ll << 31) && E * C < (1ll << 31), HAPMI_ELIMIT, "switch_gate: shape too large");
+    if (B == 0) return HAPMI_OK;
+    HAPMI_REQUIRE(logits && probs && index && slot && gate && token_of_slot, HAPMI_EINVAL, "switch_gate: null pointer");
+    hipLaunchKernelGGL(top2_gate_kernel<1>, dim3((unsigned)B), dim3(GATE_THREADS), 0, (hipStream_t)stream, logits, probs,
+                       index, slot, gate, token_of_slot, (int)S, (int)E, (int)C);
+    HAPMI_CHECK_LAUNCH("switch_gate");
     return HAPMI_OK;
 }
 

@@ -289,7 +289,8 @@ class ShardExecutor:
             torch.log_softmax: self._log_softmax, F.nll_loss: self._nll_loss,
             F.conv2d: self._conv2d, torch.flatten: self._flatten,
             models.append_cls_token: self._append_cls, models.get_cls_token: self._get_cls,
-            models.new_segment: self._alias, models.top_2_gating: self._gating, torch.einsum: self._einsum,
+            models.new_segment: self._alias, models.top_2_gating: self._gating, models.switch_gating: self._gating,
+            torch.einsum: self._einsum,
             collectives.replicate: self._replicate, collectives.all_gather: self._all_gather,
             collectives.reduce_scatter: self._reduce_scatter, collectives.all_to_all: self._all_to_all,
             collectives.all_reduce: self._all_reduce, collectives.dynamic_slice: self._dynamic_slice,
@@ -1014,7 +1015,8 @@ class ShardExecutor:
                  slot=self._new((B, S, 2), torch.int32), gate=self._new((B, S, 2), torch.float32),
                  token_of_slot=self._new((B, E, C), torch.int32))
         dgate = self._new((B, S, 2), torch.float32)
-        self.fwd.append(lambda: (ops.gemm(x.t, wg.t, logits, B * S, E, d), ops.top2_gate_into(logits, C, r)))
+        route = ops.switch_gate_into if node.target is models.switch_gating else ops.top2_gate_into
+        self.fwd.append(lambda: (ops.gemm(x.t, wg.t, logits, B * S, E, d), route(logits, C, r)))
         v = Val("gating", None, x=x, E=E, C=C, r=r, dgate=dgate, dgate_used=False)
 
         def emit():

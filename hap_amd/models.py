@@ -3,9 +3,10 @@
 Mirrors the interface of /root/reference/models.py for the three families on
 the hot path: ``RTransformer`` (models.py:65-88), ``VTransformer``
 (models.py:147-177), ``RMoE`` (models.py:90-118) with
-``Top2TransformerEncoderLayer`` (models.py:301-366), and the leaf functions
+``Top2TransformerEncoderLayer`` (models.py:301-366), ``RSwitch`` (models.py:120-145) with
+``SwitchTransformerEncoderLayer`` (models.py:368-434), and the leaf functions
 the emitted program calls by name: ``top_2_gating`` (models.py:440-441,
-477-502), ``append_cls_token`` (443-445), ``get_cls_token`` (447-449),
+477-502), ``switch_gating`` (436-437, 452-475), ``append_cls_token`` (443-445), ``get_cls_token`` (447-449),
 ``new_segment`` (531-533), ``positional_encoding`` (504-509).
 
 The classes here are parameter containers with the reference's parameter
@@ -66,6 +67,14 @@ def top_2_gating(gate_input, n_expert, capacity, gate_weight, train: bool = True
     return ops.top_2_gating_dense(gate_input, n_expert, capacity, gate_weight)
 
 
+@torch.fx.wrap
+def switch_gating(gate_input, n_expert, capacity, gate_weight, train: bool = True):
+    """Switch (top-1) softmax gating with per-expert capacity (models.py:436-437, 452-475).
+    Returns dense ``(dispatch, combine)``, each [B, S, E, C]; dispatch is float32."""
+    from . import ops
+    return ops.switch_gating_dense(gate_input, n_expert, capacity, gate_weight)
+
+
 # ---------------------------------------------------------------------------
 # parameter containers
 # ---------------------------------------------------------------------------
@@ -90,6 +99,11 @@ class Top2TransformerEncoderLayer(nn.Module):
         self.dropout_p = dropout
         self.n_expert = n_expert
         self.capacity = capacity
+
+
+class SwitchTransformerEncoderLayer(Top2TransformerEncoderLayer):
+    """Self-attention + switch (top-1) mixture-of-experts FFN (models.py:368-434): the parameters of the top-2
+    layer, routed by ``switch_gating``."""
 
 
 def _encoder_layer(emsize, nheads, nhid, dropout):
@@ -138,6 +152,18 @@ class RMoE(nn.Module):
             for i in range(nlayers)])
         self.decoder = nn.Linear(emsize, ntokens)
         self.segmentation = segmentation
+
+
+class RSwitch(RMoE):
+    """Transformer LM whose odd layers are switch MoE layers (models.py:120-145)."""
+
+    def __init__(self, ntokens, seqlen, emsize, nheads, nhid, dropout, n_expert, capacity, nlayers,
+                 segmentation=True, causal=True):
+        super().__init__(ntokens, seqlen, emsize, nheads, nhid, dropout, n_expert, capacity, nlayers, segmentation,
+                         causal)
+        for i in range(1, nlayers, 2):
+            self.layers[i] = SwitchTransformerEncoderLayer(emsize, nheads, nhid, dropout, n_expert=n_expert,
+                                                           capacity=capacity)
 
 
 class PatchEmbed(nn.Module):

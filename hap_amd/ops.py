@@ -709,6 +709,31 @@ def top2_gate_into(logits, capacity, r):
                                 _ptr(r["token_of_slot"]), B, S, E, capacity, _stream()))
 
 
+def switch_gate_into(logits, capacity, r):
+    """Switch (top-1) gating into top-2-shaped routing records: the second choice of every token is dropped."""
+    B, S, E = logits.shape
+    _dev(logits)
+    if logits.dtype != torch.float32 or not logits.is_contiguous():
+        raise TypeError("switch_gate: contiguous float32 logits expected")
+    _check_routing(r, B, S, E, capacity)
+    check(lib().hapmi_switch_gate(_ptr(logits), _ptr(r["probs"]), _ptr(r["index"]), _ptr(r["slot"]), _ptr(r["gate"]),
+                                  _ptr(r["token_of_slot"]), B, S, E, capacity, _stream()))
+
+
+def switch_gate(logits, capacity):
+    """logits [B,S,E] float32 -> dict(probs, index, slot, gate, token_of_slot), one kept choice per token at most."""
+    _dev(logits)
+    B, S, E = logits.shape
+    dev = logits.device
+    r = dict(probs=torch.empty(B, S, E, dtype=torch.float32, device=dev),
+             index=torch.empty(B, S, 2, dtype=torch.int32, device=dev),
+             slot=torch.empty(B, S, 2, dtype=torch.int32, device=dev),
+             gate=torch.empty(B, S, 2, dtype=torch.float32, device=dev),
+             token_of_slot=torch.empty(B, E, capacity, dtype=torch.int32, device=dev))
+    switch_gate_into(logits, capacity, r)
+    return r
+
+
 def top2_gate_bwd(r, dgate, dlogits):
     B, S, E = r["probs"].shape
     _check_routing(r, B, S, E)
@@ -840,3 +865,16 @@ def top_2_gating_dense(gate_input, n_expert, capacity, gate_weight):
     gemm(x, w, logits, B * S, n_expert, d)
     r = top2_gate(logits, capacity)
     return top2_densify(r, n_expert, capacity)
+
+
+def switch_gating_dense(gate_input, n_expert, capacity, gate_weight):
+    """Dense (dispatch, combine) [B,S,E,C] of switch gating from the index-form kernel (forward only)."""
+    _dev(gate_input, gate_weight)
+    B, S, d = gate_input.shape
+    x = gate_input.contiguous()
+    w = gate_weight.contiguous().to(x.dtype)
+    if n_expert % 4 != 0:
+        raise _lib.HapmiError("switch_gating: n_expert must be a multiple of 4")
+    logits = torch.empty(B, S, n_expert, dtype=torch.float32, device=x.device)
+    gemm(x, w, logits, B * S, n_expert, d)
+    return top2_densify(switch_gate(logits, capacity), n_expert, capacity)

@@ -170,7 +170,7 @@ def _call_shape(node, sh):
     if t is models.get_cls_token:
         b, _s, d = sh(a[0])
         return (b, d)
-    if t is models.top_2_gating:
+    if t in (models.top_2_gating, models.switch_gating):
         b, s, _d = sh(a[0])
         return [(b, s, a[1], a[2]), (b, s, a[1], a[2])]
     if t is torch.einsum:
@@ -206,7 +206,7 @@ def _node_flops(node, sh) -> int:
     if t in (models.append_cls_token, models.get_cls_token):     # hap.rs:2096, 2144
         s = sh(a[0])
         return s[0] * s[2]
-    if t is models.top_2_gating:                                 # hap.rs:2206
+    if t in (models.top_2_gating, models.switch_gating):         # hap.rs:2206 (switch: no handler there, same price)
         return 10 * _prod(sh(a[0]))
     if t is torch.einsum:                                        # hap.rs:2283-2286
         return _EINSUM_FLOPS[a[0]](sh(a[1]), sh(a[2]))

@@ -148,16 +148,16 @@ def _dense_ffn(e: _Emitter, h1, prefix: str, emsize: int, nhid: int, B: int, p: 
 
 
 def _moe_ffn(e: _Emitter, h1, prefix: str, emsize: int, n_expert: int, capacity: int, B: int,
-             batch_sharded: bool):
+             batch_sharded: bool, gating=models.top_2_gating):
     L_E = e.plan.lengths(n_expert)
     if batch_sharded:
         L_B = e.plan.lengths(B)
         tokens = e.call(collectives.all_gather, h1, 0, L_B, e.rank)
     else:
         tokens = h1
-    gating = e.call(models.top_2_gating, tokens, n_expert, capacity, e.replicated(prefix + "gate_weight"))
-    dispatch = e.call(operator.getitem, gating, 0)
-    combine = e.call(operator.getitem, gating, 1)
+    routed = e.call(gating, tokens, n_expert, capacity, e.replicated(prefix + "gate_weight"))
+    dispatch = e.call(operator.getitem, routed, 0)
+    combine = e.call(operator.getitem, routed, 1)
     dispatch = e.call(collectives.dynamic_slice, dispatch, 2, L_E, e.rank)
     combine = e.call(collectives.dynamic_slice, combine, 2, L_E, e.rank)
     w1 = e.sharded(prefix + "w1", n_expert, 0)
@@ -213,7 +213,11 @@ def build_program(model: nn.Module, plan: ShardingPlan, global_batch: int,
         prefix = f"layers.{i}."
         h1 = _attention(e, h, prefix, d, model.nheads, p, mask)
         if isinstance(layer, models.Top2TransformerEncoderLayer):
-            h = _moe_ffn(e, h1, prefix, d, layer.n_expert, layer.capacity, B, batch_sharded)
+            # the switch layer takes the top-2 layer's node forms with its own gating leaf (the reference's
+            # synthesizer has no handler for models.switch_gating; its models call it at models.py:421)
+            gating = (models.switch_gating if isinstance(layer, models.SwitchTransformerEncoderLayer)
+                      else models.top_2_gating)
+            h = _moe_ffn(e, h1, prefix, d, layer.n_expert, layer.capacity, B, batch_sharded, gating)
         else:
             h = _dense_ffn(e, h1, prefix, d, model.nhid, B, p, activation, batch_sharded)
 

@@ -234,6 +234,13 @@ int hapmi_append_cls_pos(const void *patches, const void *cls, const void *pos, 
  * token_of_slot[B, E, C] int32 (-1 = empty). */
 int hapmi_top2_gate(const float *logits, float *probs, int32_t *index, int32_t *slot, float *gate,
                     int32_t *token_of_slot, int64_t B, int64_t S, int64_t E, int64_t C, hapmi_stream_t stream);
+/* models.switch_gating (models.py:436-437, 452-475; the reference's synthesizer has no handler for it, its
+ * single-device models RSwitch / VSwitch call it): the same records with one choice per token -- position
+ * = 1-based rank among the earlier tokens of the same expert, kept while < C, combine weight = the softmax
+ * probability of the chosen expert.  The second entry of every record is a dropped choice (gate 0, slot 0),
+ * so every entry point below takes these records unchanged. */
+int hapmi_switch_gate(const float *logits, float *probs, int32_t *index, int32_t *slot, float *gate,
+                      int32_t *token_of_slot, int64_t B, int64_t S, int64_t E, int64_t C, hapmi_stream_t stream);
 /* dlogits = softmax backward of the two kept gate gradients */
 int hapmi_top2_gate_bwd(const float *probs, const int32_t *index, const int32_t *slot, const float *dgate,
                         float *dlogits, int64_t B, int64_t S, int64_t E, hapmi_stream_t stream);

@@ -55,9 +55,10 @@ class JointCPURun:
         args = self._lookup(r, node.args)
         kwargs = self._lookup(r, node.kwargs)
         t = node.target
-        if t is product_models.top_2_gating:
+        if t in (product_models.top_2_gating, product_models.switch_gating):
             x, n_expert, capacity, wg = args[:4]
-            dispatch, combine = ref.top_2_gating(x.float(), n_expert, capacity, wg.float())
+            gating = ref.top_2_gating if t is product_models.top_2_gating else ref.switch_gating
+            dispatch, combine = gating(x.float(), n_expert, capacity, wg.float())
             return dispatch, combine
         if t is product_models.append_cls_token:
             x, cls = args

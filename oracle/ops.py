@@ -9,6 +9,7 @@ Functions and the reference lines they follow:
   oracle/sharding_round.c, loaded through ctypes).
 * ``positional_encoding``  -- /root/reference/models.py:504-509.
 * ``top_2_gating``         -- /root/reference/models.py:477-502.
+* ``switch_gating``        -- /root/reference/models.py:452-475.
 * ``JointWorld`` collectives -- /root/reference/collectives.py:6-29 (padded,
   AllGather), 73-84 (AllReduce), 88-103 (ReduceScatter), 146-148
   (dynamic_slice), 152-166 (AllToAll), 171-180 (Replicate).
@@ -19,7 +20,8 @@ oracle calls the same public PyTorch routines on the CPU.
 Pins (see tests/test_oracle_*.py): sharding_round -- hand-derived known
 answers + invariants; positional_encoding -- closed form at chosen points;
 top_2_gating -- hand-worked routing vector, per-token brute force, slot
-invariants; collectives -- the ones-tensor expectations the reference keeps in
+invariants; switch_gating -- hand-worked routing vector, per-token brute force,
+slot invariants, agreement with the first choices of top_2_gating; collectives -- the ones-tensor expectations the reference keeps in
 collectives.py:195-323, round-trip identities.  Tie order of equal gate
 probabilities inside torch.topk is unspecified by PyTorch: parity unpinned for
 exact ties (they do not occur for the seeded continuous inputs used).
@@ -100,6 +102,47 @@ def top_2_gating(gate_input, n_expert: int, capacity: int, gate_weight, train: b
                * F.one_hot(pos, capacity)).sum(dim=2)                  # :498
     dispatch = (combine > 0).to(torch.float32)                         # :500
     return dispatch, combine
+
+
+def switch_gating(gate_input, n_expert: int, capacity: int, gate_weight, train: bool = True):
+    """models.py:452-475, dense form: returns (dispatch, combine), each
+    [B, S, E, C]; one expert per token, kept while its 1-based position among
+    the earlier tokens of that expert is below the capacity."""
+    logits = gate_input @ gate_weight                                  # :453
+    probs = torch.softmax(logits, dim=2)                               # :454
+    gate, index = probs.topk(1, dim=2)                                 # :456
+    gate, index = gate.squeeze(2), index.squeeze(2)                    # :457-458  [B,S]
+    chosen = F.one_hot(index, n_expert)                                # :460  [B,S,E] int64
+    pos = chosen.cumsum(dim=1) * chosen                                # :462  1-based
+    fits = pos < capacity                                              # :463-464
+    kept = chosen * fits
+    pos = pos * fits
+    kept_flag = kept.sum(dim=2)                                        # :466  [B,S]
+    combine = ((gate * kept_flag)[:, :, None, None]                    # :469
+               * F.one_hot(index, n_expert)[..., None]                 # :470
+               * F.one_hot(pos, capacity))                             # :471  one_hot over [B,S,E] -> [B,S,E,C]
+    dispatch = (combine > 0).to(torch.float32)                         # :473
+    return dispatch, combine
+
+
+def switch_gating_sparse(logits: torch.Tensor, capacity: int):
+    """Per-token brute force over fp32 logits [B,S,E] (pure Python loops; small
+    inputs only).  Returns (index[B,S] int64, slot[B,S] int64 with 0 =
+    dropped, gate[B,S] float)."""
+    B, S, E = logits.shape
+    probs = torch.softmax(logits, dim=2)
+    index = torch.zeros(B, S, dtype=torch.int64)
+    slot = torch.zeros(B, S, dtype=torch.int64)
+    gate = torch.zeros(B, S, dtype=probs.dtype)
+    for b in range(B):
+        seen = [0] * E
+        for s in range(S):
+            row = probs[b, s].tolist()
+            e = min(range(E), key=lambda i: (-row[i], i))
+            index[b, s], gate[b, s] = e, probs[b, s, e]
+            seen[e] += 1
+            slot[b, s] = seen[e] if seen[e] < capacity else 0
+    return index, slot, gate
 
 
 def top_2_gating_sparse(logits: torch.Tensor, capacity: int):

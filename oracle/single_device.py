@@ -4,7 +4,8 @@ modules.  TEST INFRASTRUCTURE ONLY.
 Used for the invariant that pins the program generator: the sum over ranks of
 the per-rank partial losses of the SPMD program equals the loss of the
 unsharded model (/root/reference/models.py:78-88 RTransformer.forward,
-108-118 RMoE.forward, 163-177 VTransformer.forward, 340-366 the top-2 layer).
+108-118 RMoE.forward, 137-145 RSwitch.forward, 163-177 VTransformer.forward, 340-366 the top-2 layer,
+405-434 the switch layer).
 """
 from __future__ import annotations
 
@@ -20,7 +21,9 @@ from . import ops as ref
 def _top2_layer(layer, x, mask):
     a = layer.self_attn(x, x, x, attn_mask=mask, need_weights=False)[0]            # models.py:346-351
     x = layer.norm1(x + a)                                                         # :341
-    dispatch, combine = ref.top_2_gating(x, layer.n_expert, layer.capacity, layer.gate_weight)  # :354
+    # the switch layer (models.py:405-434) differs from the top-2 layer in the gating call only (:421 / :354)
+    gating = ref.switch_gating if isinstance(layer, product_models.SwitchTransformerEncoderLayer) else ref.top_2_gating
+    dispatch, combine = gating(x, layer.n_expert, layer.capacity, layer.gate_weight)
     t = torch.einsum("bsd,bsec->becd", x, dispatch)                                # :356
     t = torch.relu(torch.einsum("edh,becd->bech", layer.w1, t))                    # :358-360
     t = torch.einsum("ehd,bech->becd", layer.w2, t)                                # :362

@@ -23,6 +23,12 @@ def make_moe(vocab=61, S=16, d=32, H=4, F=48, E=8, C=6, layers=2, seed=0, std=0.
     return models.init_normal_(m, std, seed)
 
 
+def make_switch(vocab=61, S=16, d=32, H=4, F=48, E=8, C=6, layers=2, seed=0, std=0.5):
+    torch.manual_seed(seed)
+    m = models.RSwitch(vocab, S, d, H, F, 0.0, E, C, layers)
+    return models.init_normal_(m, std, seed)
+
+
 def make_vit(classes=10, img=16, patch=4, d=32, H=4, F=64, layers=2, seed=0):
     torch.manual_seed(seed)
     n = (img // patch) ** 2

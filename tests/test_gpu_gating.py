@@ -1,6 +1,6 @@
-"""Top-2 gating and the dispatch / combine gathers on the GPU: routing (expert index, slot, dropped flags,
+"""Top-2 and switch gating and the dispatch / combine gathers on the GPU: routing (expert index, slot, dropped flags,
 dense layouts) is bit-exact against the oracle on the same float32 logits; gate values and the float paths
-within tolerance.  Reference: /root/reference/models.py:477-502, 356-364."""
+within tolerance.  Reference: /root/reference/models.py:477-502, 452-475, 356-364."""
 import pytest
 import torch
 
@@ -122,3 +122,52 @@ def test_gate_backward_matches_autograd(cuda):
     want_dw = x.reshape(-1, d).t() @ dlogits.cpu().reshape(-1, E)
     assert rel_err(want_dw, w.grad) < 1e-4
     assert rel_err(dlogits.cpu().reshape(-1, E) @ w.detach().t(), xr.grad.reshape(-1, d)) < 1e-4
+
+
+# ---- switch (top-1) gating, /root/reference/models.py:452-475 ---------------------------------------------------
+
+def test_switch_hand_worked_vector(cuda):
+    lg = torch.full((1, 6, 3), -4.0)
+    for s, e in enumerate([0, 0, 2, 0, 2, 1]):
+        lg[0, s, e] = 2.0
+    lg = torch.cat([lg, torch.full((1, 6, 1), -9.0)], 2)          # the kernel's GEMM path wants E % 4 == 0; expert 3 unused
+    r = ops.switch_gate(lg.to(cuda), 3)
+    assert r["index"].cpu()[0, :, 0].tolist() == [0, 0, 2, 0, 2, 1]
+    assert r["slot"].cpu()[0].tolist() == [[1, 0], [2, 0], [1, 0], [0, 0], [2, 0], [1, 0]]
+    assert r["gate"].cpu()[0, :, 1].tolist() == [0.0] * 6
+    assert r["token_of_slot"].cpu()[0].tolist() == [[-1, 0, 1], [-1, 5, -1], [-1, 2, 4], [-1, -1, -1]]
+
+
+@pytest.mark.parametrize("B,S,E,C", SHAPES)
+def test_switch_routing_is_bit_exact(cuda, B, S, E, C):
+    lg = _logits(B, S, E, 3 * S + E)
+    r = ops.switch_gate(lg.to(cuda), C)
+    idx, slot, gate = ref.switch_gating_sparse(lg, C)
+    assert torch.equal(r["index"].cpu().long()[:, :, 0], idx)
+    assert torch.equal(r["slot"].cpu().long()[:, :, 0], slot)
+    assert (r["slot"].cpu()[:, :, 1] == 0).all() and (r["gate"].cpu()[:, :, 1] == 0).all()
+    torch.testing.assert_close(r["gate"].cpu()[:, :, 0], gate, rtol=1e-5, atol=1e-7)
+    d_ref, c_ref = ref.switch_gating(lg, E, C, torch.eye(E))
+    d, c = ops.top2_densify(r, E, C)
+    assert torch.equal(d.cpu(), d_ref)
+    torch.testing.assert_close(c.cpu(), c_ref, rtol=1e-5, atol=1e-7)
+    tos = r["token_of_slot"].cpu()
+    assert (tos >= 0).sum().item() == int(d_ref.sum().item())
+    for b, s, e, k in d_ref.nonzero().tolist()[:200]:
+        assert tos[b, e, k] == s
+
+
+def test_switch_gate_backward_is_the_softmax_backward_of_the_kept_choice(cuda):
+    B, S, E, C = 2, 40, 8, 6
+    lg = _logits(B, S, E, 77)
+    r = ops.switch_gate(lg.to(cuda), C)
+    g = torch.Generator().manual_seed(78)
+    dgate = torch.randn(B, S, 2, generator=g)
+    dlogits = torch.empty(B, S, E, device=cuda)
+    ops.top2_gate_bwd(r, dgate.to(cuda), dlogits)
+    x = lg.clone().requires_grad_(True)
+    p = torch.softmax(x, 2)
+    idx, slot, _ = ref.switch_gating_sparse(lg, C)
+    chosen = p.gather(2, idx[:, :, None]).squeeze(2)
+    (chosen * dgate[:, :, 0] * (slot > 0)).sum().backward()
+    torch.testing.assert_close(dlogits.cpu(), x.grad, rtol=1e-5, atol=1e-7)

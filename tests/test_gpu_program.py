@@ -9,7 +9,8 @@ import pytest
 import torch
 
 import hap_amd
-from helpers import (RATIOS4, RATIOS_E, joint_cpu, lm_batch, make_lm, make_moe, make_vit, rel_err, vit_batch)
+from helpers import (RATIOS4, RATIOS_E, joint_cpu, lm_batch, make_lm, make_moe, make_switch, make_vit, rel_err,
+                     vit_batch)
 
 pytestmark = pytest.mark.gpu
 
@@ -121,6 +122,15 @@ def test_moe_fp32(cuda, batch_sharded):
     B = 16 if batch_sharded else 4
     x, y = lm_batch(B, 16, 61)
     _compare(model, RATIOS_E, B, x, y, "fp32", [0, 2], ADAM, ffn="batch", batch_sharded=batch_sharded)
+
+
+@pytest.mark.parametrize("dtype,batch_sharded", [("fp32", True), ("fp32", False), ("bf16", False)])
+def test_switch_moe(cuda, dtype, batch_sharded):
+    """RSwitch (models.py:120-145): switch-gated experts, expert-sharded, batch sharded or replicated."""
+    model = make_switch() if dtype == "fp32" else make_switch(d=64, F=96, std=0.3)
+    B = 16 if batch_sharded else 4
+    x, y = lm_batch(B, 16, 61)
+    _compare(model, RATIOS_E, B, x, y, dtype, [0, 2], ADAM, ffn="batch", batch_sharded=batch_sharded)
 
 
 def test_moe_bf16_routing_matches(cuda):

@@ -1,5 +1,6 @@
-"""Pins oracle.ops.top_2_gating (restatement of /root/reference/models.py:477-502) with a hand-worked
-routing vector, a per-token brute force and the slot invariants the algorithm implies."""
+"""Pins oracle.ops.top_2_gating (restatement of /root/reference/models.py:477-502) and oracle.ops.switch_gating
+(models.py:452-475), each with a hand-worked routing vector, a per-token brute force and the slot invariants the
+algorithm implies."""
 import torch
 
 from oracle import ops as ref
@@ -71,3 +72,49 @@ def test_gradient_flows_through_gates_only():
     assert not d.requires_grad and c.requires_grad
     c.sum().backward()
     assert w.grad.abs().sum() > 0
+
+
+# ---- switch (top-1) gating: oracle.ops.switch_gating restates /root/reference/models.py:452-475 ----------------
+
+def test_switch_hand_worked_vector():
+    # B=1, S=6, E=3, C=3; first choices t0:0 t1:0 t2:2 t3:0 t4:2 t5:1
+    # positions (1-based, per expert, in token order): e0 {t0:1, t1:2, t3:3 -> dropped (>= C)}, e2 {t2:1, t4:2}, e1 {t5:1}
+    lg = torch.full((1, 6, 3), -4.0)
+    for s, e in enumerate([0, 0, 2, 0, 2, 1]):
+        lg[0, s, e] = 2.0
+    d, c = ref.switch_gating(lg, 3, 3, torch.eye(3))
+    kept = sorted((s, e, k) for _, s, e, k in d.nonzero().tolist())
+    assert kept == [(0, 0, 1), (1, 0, 2), (2, 2, 1), (4, 2, 2), (5, 1, 1)]
+    probs = torch.softmax(lg, dim=2)
+    assert torch.equal(c[0, 1, 0, 2], probs[0, 1, 0]) and torch.equal(c[0, 5, 1, 1], probs[0, 5, 1])
+    assert c[0, 3].sum() == 0                                            # the dropped token reaches no expert
+    assert d.dtype == torch.float32 and d.shape == (1, 6, 3, 3)
+
+
+def test_switch_dense_restatement_equals_per_token_brute_force():
+    g = torch.Generator().manual_seed(15)
+    for (B, S, E, C) in [(2, 16, 4, 5), (3, 33, 8, 6), (1, 64, 16, 12), (2, 20, 4, 40)]:
+        x = torch.randn(B, S, 12, generator=g)
+        w = torch.randn(12, E, generator=g)
+        d, c = ref.switch_gating(x, E, C, w)
+        idx, slot, gate = ref.switch_gating_sparse(x @ w, C)
+        zeros = torch.zeros_like(idx)
+        d2, c2 = ref.densify(torch.stack([idx, zeros], 2), torch.stack([slot, zeros], 2),
+                             torch.stack([gate, torch.zeros_like(gate)], 2), E, C)
+        assert torch.equal(d, d2)
+        torch.testing.assert_close(c, c2, rtol=0, atol=0)
+
+
+def test_switch_invariants_and_agreement_with_the_first_choices_of_top_2():
+    g = torch.Generator().manual_seed(17)
+    B, S, E, C = 4, 48, 8, 10
+    x, w = torch.randn(B, S, 16, generator=g), torch.randn(16, E, generator=g)
+    d, c = ref.switch_gating(x, E, C, w)
+    assert torch.equal(d, (c > 0).float())
+    assert d[:, :, :, 0].sum() == 0                      # slot 0 never holds a token
+    assert (d.sum(dim=1) <= 1).all()                     # a slot holds at most one token
+    assert (d.sum(dim=(2, 3)) <= 1).all()                # a token has at most one destination
+    # the first choice of top-2 gating is routed by the same rule (models.py:485 vs :462)
+    idx2, slot2, gate2 = ref.top_2_gating_sparse(x @ w, C)
+    idx1, slot1, gate1 = ref.switch_gating_sparse(x @ w, C)
+    assert torch.equal(idx1, idx2[:, :, 0]) and torch.equal(slot1, slot2[:, :, 0]) and torch.equal(gate1, gate2[:, :, 0])

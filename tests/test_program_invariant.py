@@ -6,7 +6,8 @@ import copy
 import pytest
 import torch
 
-from helpers import (RATIOS4, RATIOS_E, joint_cpu, lm_batch, make_lm, make_moe, make_vit, rel_err, vit_batch)
+from helpers import (RATIOS4, RATIOS_E, joint_cpu, lm_batch, make_lm, make_moe, make_switch, make_vit, rel_err,
+                     vit_batch)
 from oracle import single_device
 import hap_amd
 
@@ -127,3 +128,15 @@ def test_zero_vit_and_moe_spmd_equal_single_device():
     x, y = lm_batch(16, 16, 61)
     run = joint_cpu(model, RATIOS_E, 16, ffn="batch", zero=True)
     _check(model, run, x, y, _zero_sharded(model, RATIOS_E), whole_norm=True)
+
+
+@pytest.mark.parametrize("zero", [False, True])
+def test_switch_moe_spmd_equals_single_device(zero):
+    """RSwitch (models.py:120-145): the top-2 plan forms with switch gating."""
+    model = make_switch()
+    x, y = lm_batch(16, 16, 61)
+    L_E = hap_amd.sharding_lengths(8, RATIOS_E)
+    run = joint_cpu(model, RATIOS_E, 16, ffn="batch", zero=zero)
+    assert sum(n.target is hap_amd.models.switch_gating for n in run.programs[0].graph.nodes) == 1
+    sharded = _zero_sharded(model, RATIOS_E) if zero else {"layers.1.w1": (0, L_E), "layers.1.w2": (0, L_E)}
+    _check(model, run, x, y, sharded, whole_norm=zero)
