@@ -290,6 +290,7 @@ class ShardExecutor:
             F.conv2d: self._conv2d, torch.flatten: self._flatten,
             models.append_cls_token: self._append_cls, models.get_cls_token: self._get_cls,
             models.new_segment: self._alias, models.top_2_gating: self._gating, models.switch_gating: self._gating,
+            models.head_parallel_attention: self._head_parallel_attention,
             torch.einsum: self._einsum,
             collectives.replicate: self._replicate, collectives.all_gather: self._all_gather,
             collectives.reduce_scatter: self._reduce_scatter, collectives.all_to_all: self._all_to_all,
@@ -427,9 +428,10 @@ class ShardExecutor:
                         self._accumulate_into(v, out.grad)
             self._tape.append(emit)
             return out
-        # broadcast over the leading dimension: [b, S, d] + [1, S, d]
+        # broadcast over the leading dimension(s): [b, S, d] + [1, S, d], or [b, S, d] + [d] (a bias)
         big, small = (a, b) if a.t.numel() >= b.t.numel() else (b, a)
-        if small.t.shape[0] != 1 or tuple(small.t.shape[1:]) != tuple(big.t.shape[1:]):
+        vector = small.t.dim() == 1 and small.t.shape[0] == big.t.shape[-1]
+        if not vector and (small.t.shape[0] != 1 or tuple(small.t.shape[1:]) != tuple(big.t.shape[1:])):
             self._unsupported(node, f"broadcast of {tuple(small.t.shape)} onto {tuple(big.t.shape)} is not supported")
         width = big.t.shape[-1]
         b_rows = small.t.numel() // width
@@ -445,7 +447,7 @@ class ShardExecutor:
             if small.kind == "param":
                 g, acc = self._param_grad_slot(small)
                 n = small.t.numel()
-                self.bwd.append(lambda: ops.colsum(out.grad, g, big.t.shape[0], n, n, acc))
+                self.bwd.append(lambda: ops.colsum(out.grad, g, rows // b_rows, n, n, acc))
         self._tape.append(emit)
         return out
 
@@ -608,15 +610,40 @@ class ShardExecutor:
         if float(kw.get("dropout_p", 0.0)) != 0.0:
             self._unsupported(node, "attention dropout with p > 0 is not implemented")
         x = q.meta["src"]
-        b, S, E = x.t.shape
-        H = kw["num_heads"]
-        if kw["embed_dim_to_check"] != E or E % H:
+        E = x.t.shape[2]
+        if kw["embed_dim_to_check"] != E or E % kw["num_heads"]:
             self._unsupported(node, "embed_dim mismatch")
-        hd = E // H
+        out_bsd = self._attention_core(node, x, kw["in_proj_weight"], kw["in_proj_bias"], kw["out_proj_weight"],
+                                       kw["out_proj_bias"], kw["num_heads"], kw.get("attn_mask"))
+        out = Val("transposed", None, src=out_bsd, dims=(0, 1), needs_grad=True)
+        return Val("mha", None, out=out)
+
+    def _head_parallel_attention(self, node):
+        """models.head_parallel_attention(x, in_proj_weight, in_proj_bias, out_proj_weight, num_heads, attn_mask):
+        the heads of this device on the whole batch; the output is the device's partial sum of the output
+        projection (no bias), which the program reduce-scatters."""
+        args = [self._val(a) for a in node.args]
+        x, w_in, b_in, w_out, H = args[:5]
+        mask = args[5] if len(args) > 5 else self._val(node.kwargs.get("attn_mask"))
+        if x.t is None or x.ld is not None or x.t.dim() != 3:
+            self._unsupported(node, "expects a materialised [batch, seq, d] tensor")
+        return self._attention_core(node, x, w_in, b_in, w_out, None, H, mask)
+
+    def _attention_core(self, node, x: Val, w_in: Val, b_in: Val, w_out: Val, b_out: Optional[Val], H: int, mask):
+        """qkv = x W_in^T + b_in over Ea = H * head_dim attention columns (all heads, or this device's heads),
+        softmax attention per head, out = ctx W_out^T (+ b_out).  x is [b, S, d]; W_in [3 Ea, d]; W_out [d_out, Ea]."""
+        for v in (w_in, b_in, w_out) + ((b_out,) if b_out is not None else ()):
+            if v.kind != "param":
+                self._unsupported(node, "attention weights must be parameters")
+        b, S, d = x.t.shape
+        Ea = w_in.t.shape[0] // 3
+        d_out = w_out.t.shape[0]
+        if tuple(w_in.t.shape) != (3 * Ea, d) or tuple(w_out.t.shape) != (d_out, Ea) or H < 1 or Ea % H:
+            self._unsupported(node, f"projection shapes {tuple(w_in.t.shape)} / {tuple(w_out.t.shape)} do not fit "
+                                    f"{H} heads on a width-{d} input")
+        hd = Ea // H
         if hd % self.epv:
             self._unsupported(node, f"head_dim {hd} must be a multiple of {self.epv}")
-        w_in, b_in, w_out, b_out = kw["in_proj_weight"], kw["in_proj_bias"], kw["out_proj_weight"], kw["out_proj_bias"]
-        mask = kw.get("attn_mask")
         mask_t = None
         if mask is not None:
             if tuple(mask.t.shape) != (S, S) or mask.t.dtype != torch.float32:
@@ -625,46 +652,46 @@ class ShardExecutor:
         scale = 1.0 / math.sqrt(hd)
         fused = self.fused_attention and self.dtype == "bf16" and hd == 64
         Sp = _round_up(S, self.epv)
-        qkv = self._new((b, S, 3 * E))
-        ctx = self._new((b, S, E))
-        o = self._new((b, S, E))
+        qkv = self._new((b, S, 3 * Ea))
+        ctx = self._new((b, S, Ea))
+        o = self._new((b, S, d_out))
         if fused:
             lse = self._new((b, H, S), torch.float32)
             P = None
         else:
             P = self._new((b, H, S, Sp))
         out_bsd = Val("tensor", o, needs_grad=True)
-        out = Val("transposed", None, src=out_bsd, dims=(0, 1), needs_grad=True)
         M = b * S
-        sQ, sP = (S * 3 * E, hd), (H * S * Sp, S * Sp)
+        sQ, sP = (S * 3 * Ea, hd), (H * S * Sp, S * Sp)
+        bias_out = b_out.meta["master"] if b_out is not None else None
 
         def forward():
-            ops.gemm(x.t, w_in.t, qkv, M, 3 * E, E, transB=True, bias=b_in.meta["master"])
+            ops.gemm(x.t, w_in.t, qkv, M, 3 * Ea, d, transB=True, bias=b_in.meta["master"])
             if fused:
                 ops.attention_fwd(qkv, mask_t, ctx, lse, b, S, H, scale)
             else:
-                ops.gemm(qkv, qkv, P, S, S, hd, transB=True, lda=3 * E, ldb=3 * E, ldc=Sp, alpha=scale, batch1=b,
-                         batch2=H, strideA=sQ, strideB=sQ, strideC=sP, offB=E)
+                ops.gemm(qkv, qkv, P, S, S, hd, transB=True, lda=3 * Ea, ldb=3 * Ea, ldc=Sp, alpha=scale, batch1=b,
+                         batch2=H, strideA=sQ, strideB=sQ, strideC=sP, offB=Ea)
                 ops.softmax_fwd(P, mask_t, P, b * H * S, S, Sp, S)
-                ops.gemm(P, qkv, ctx, S, hd, S, lda=Sp, ldb=3 * E, ldc=E, batch1=b, batch2=H, strideA=sP, strideB=sQ,
-                         strideC=(S * E, hd), offB=2 * E)
-            ops.gemm(ctx, w_out.t, o, M, E, E, transB=True, bias=b_out.meta["master"])
+                ops.gemm(P, qkv, ctx, S, hd, S, lda=Sp, ldb=3 * Ea, ldc=Ea, batch1=b, batch2=H, strideA=sP, strideB=sQ,
+                         strideC=(S * Ea, hd), offB=2 * Ea)
+            ops.gemm(ctx, w_out.t, o, M, d_out, Ea, transB=True, bias=bias_out)
         self.fwd.append(forward)
 
         def emit():
             if out_bsd.grad is None:
                 return
             do = out_bsd.grad
-            dctx = self._scratch("attn_dctx", (b, S, E))
+            dctx = self._scratch("attn_dctx", (b, S, Ea))
             side = self._side_ok(w_out, b_out, w_in, b_in)
             # the in-projection's weight gradient reads dqkv from the side stream, so it cannot be shared scratch
-            dqkv = self._new((b, S, 3 * E)) if side else self._scratch("attn_dqkv", (b, S, 3 * E))
+            dqkv = self._new((b, S, 3 * Ea)) if side else self._scratch("attn_dqkv", (b, S, 3 * Ea))
             if fused:
                 delta = self._scratch("attn_delta", (b, H, S), torch.float32)
             else:
                 dP = self._scratch("attn_dP", (b, H, S, Sp))
             gwo, acc_wo = self._param_grad_slot(w_out)
-            gbo, acc_bo = self._param_grad_slot(b_out)
+            gbo, acc_bo = self._param_grad_slot(b_out) if b_out is not None else (None, False)
             gwi, acc_wi = self._param_grad_slot(w_in)
             gbi, acc_bi = self._param_grad_slot(b_in)
             gx, acc_x = self._grad_slot(x) if x.needs_grad else (None, False)
@@ -672,34 +699,34 @@ class ShardExecutor:
             ws = self.side_workspace if side else None
 
             def wgrad_out():
-                ops.gemm(do, ctx, gwo, E, E, M, transA=True, accumulate=acc_wo, workspace=ws, a_rowsum=gbo)
+                ops.gemm(do, ctx, gwo, d_out, Ea, M, transA=True, accumulate=acc_wo, workspace=ws, a_rowsum=gbo)
 
             def wgrad_in():
-                ops.gemm(dqkv, x.t, gwi, 3 * E, E, M, transA=True, accumulate=acc_wi, workspace=ws, a_rowsum=gbi)
+                ops.gemm(dqkv, x.t, gwi, 3 * Ea, d, M, transA=True, accumulate=acc_wi, workspace=ws, a_rowsum=gbi)
 
             def backward():
                 if not side:
                     wgrad_out()
-                ops.gemm(do, w_out.t, dctx, M, E, E)
+                ops.gemm(do, w_out.t, dctx, M, Ea, d_out)
                 if fused:
                     ops.attention_bwd(qkv, ctx, dctx, lse, mask_t, dqkv, delta, b, S, H, scale)
                 else:
                     # dP = dctx V^T ; dV = P^T dctx
-                    ops.gemm(dctx, qkv, dP, S, S, hd, transB=True, lda=E, ldb=3 * E, ldc=Sp, batch1=b, batch2=H,
-                             strideA=(S * E, hd), strideB=sQ, strideC=sP, offB=2 * E)
-                    ops.gemm(P, dctx, dqkv, S, hd, S, transA=True, lda=Sp, ldb=E, ldc=3 * E, batch1=b, batch2=H,
-                             strideA=sP, strideB=(S * E, hd), strideC=sQ, offC=2 * E)
+                    ops.gemm(dctx, qkv, dP, S, S, hd, transB=True, lda=Ea, ldb=3 * Ea, ldc=Sp, batch1=b, batch2=H,
+                             strideA=(S * Ea, hd), strideB=sQ, strideC=sP, offB=2 * Ea)
+                    ops.gemm(P, dctx, dqkv, S, hd, S, transA=True, lda=Sp, ldb=Ea, ldc=3 * Ea, batch1=b, batch2=H,
+                             strideA=sP, strideB=(S * Ea, hd), strideC=sQ, offC=2 * Ea)
                     ops.softmax_bwd(dP, P, dP, b * H * S, S, Sp)
                     # dQ = scale dS K ; dK = scale dS^T Q
-                    ops.gemm(dP, qkv, dqkv, S, hd, S, lda=Sp, ldb=3 * E, ldc=3 * E, alpha=scale, batch1=b, batch2=H,
-                             strideA=sP, strideB=sQ, strideC=sQ, offB=E)
-                    ops.gemm(dP, qkv, dqkv, S, hd, S, transA=True, lda=Sp, ldb=3 * E, ldc=3 * E, alpha=scale, batch1=b,
-                             batch2=H, strideA=sP, strideB=sQ, strideC=sQ, offC=E)
+                    ops.gemm(dP, qkv, dqkv, S, hd, S, lda=Sp, ldb=3 * Ea, ldc=3 * Ea, alpha=scale, batch1=b, batch2=H,
+                             strideA=sP, strideB=sQ, strideC=sQ, offB=Ea)
+                    ops.gemm(dP, qkv, dqkv, S, hd, S, transA=True, lda=Sp, ldb=3 * Ea, ldc=3 * Ea, alpha=scale, batch1=b,
+                             batch2=H, strideA=sP, strideB=sQ, strideC=sQ, offC=Ea)
                 if not side:
                     wgrad_in()
 
             def dgrad_in():
-                ops.gemm(dqkv, w_in.t, gx, M, E, 3 * E, accumulate=acc_x)
+                ops.gemm(dqkv, w_in.t, gx, M, d, 3 * Ea, accumulate=acc_x)
             if side:
                 # do is final here; dqkv is final once `backward` is enqueued.  d(x) usually aliases do (the
                 # residual add hands one buffer to both), so the in-projection's data gradient, which
@@ -714,7 +741,7 @@ class ShardExecutor:
                     self._guard_write(gx)
                 self.bwd.append(dgrad_in)
         self._tape.append(emit)
-        return Val("mha", None, out=out)
+        return out_bsd
 
     # ---- loss -----------------------------------------------------------------------------------
     def _log_softmax(self, node):

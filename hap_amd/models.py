@@ -75,6 +75,17 @@ def switch_gating(gate_input, n_expert, capacity, gate_weight, train: bool = Tru
     return ops.switch_gating_dense(gate_input, n_expert, capacity, gate_weight)
 
 
+@torch.fx.wrap
+def head_parallel_attention(x, in_proj_weight, in_proj_bias, out_proj_weight, num_heads, attn_mask=None):
+    """Self-attention over ``num_heads`` of a layer's heads: ``in_proj_weight`` [3 * num_heads * hd, d] holds the
+    q, k and v rows of those heads, ``out_proj_weight`` [d, num_heads * hd] the matching columns of the output
+    projection.  Returns the [B, S, d] partial output (no output bias): the sum of the partial outputs of a
+    partition of the heads, plus the bias, is ``F.multi_head_attention_forward`` of the whole layer.  The
+    reference has no head-sharded form (its attention handler shards the batch only, hap.rs:1243-1386)."""
+    from . import ops
+    return ops.head_parallel_attention(x, in_proj_weight, in_proj_bias, out_proj_weight, num_heads, attn_mask)
+
+
 # ---------------------------------------------------------------------------
 # parameter containers
 # ---------------------------------------------------------------------------

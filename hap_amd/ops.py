@@ -7,6 +7,7 @@ are refused: there is no fallback path.
 from __future__ import annotations
 
 import ctypes
+import math
 from typing import List, Optional, Sequence
 
 import torch
@@ -479,6 +480,40 @@ def attention_bwd(qkv, out, dout, lse, mask, dqkv, delta_ws, b, S, H, scale):
         raise TypeError("attention_bwd: dtype mismatch")
     check(lib().hapmi_attention_bwd(_ptr(qkv), _ptr(out), _ptr(dout), _ptr(lse), _ptr(mask), _ptr(dqkv), _ptr(delta_ws),
                                     b, S, H, ctypes.c_float(scale), _stream()))
+
+
+def head_parallel_attention(x, w_in, b_in, w_out, num_heads, mask=None):
+    """Forward of models.head_parallel_attention on GPU tensors: qkv projection of the given heads, softmax
+    attention per head, partial output projection (no bias)."""
+    _dev(x, w_in, b_in, w_out, mask)
+    b, S, d = x.shape
+    Ea = w_in.shape[0] // 3
+    H = int(num_heads)
+    if tuple(w_in.shape) != (3 * Ea, d) or w_out.shape[1] != Ea or H < 1 or Ea % H:
+        raise ValueError("head_parallel_attention: projection shapes do not fit the heads")
+    hd = Ea // H
+    epv = 8 if x.dtype == torch.bfloat16 else 4
+    if hd % epv:
+        raise ValueError(f"head_parallel_attention: head_dim {hd} must be a multiple of {epv}")
+    if mask is not None and (tuple(mask.shape) != (S, S) or mask.dtype != torch.float32):
+        raise TypeError("head_parallel_attention: the mask must be a float32 [S, S] additive mask")
+    x = x.contiguous()
+    wi, wo = w_in.contiguous().to(x.dtype), w_out.contiguous().to(x.dtype)
+    Sp = (S + epv - 1) // epv * epv
+    M, scale = b * S, 1.0 / math.sqrt(hd)
+    qkv = torch.empty(b, S, 3 * Ea, dtype=x.dtype, device=x.device)
+    P = torch.empty(b, H, S, Sp, dtype=x.dtype, device=x.device)
+    ctx = torch.empty(b, S, Ea, dtype=x.dtype, device=x.device)
+    out = torch.empty(b, S, w_out.shape[0], dtype=x.dtype, device=x.device)
+    sQ, sP = (S * 3 * Ea, hd), (H * S * Sp, S * Sp)
+    gemm(x, wi, qkv, M, 3 * Ea, d, transB=True, bias=b_in.float().contiguous())
+    gemm(qkv, qkv, P, S, S, hd, transB=True, lda=3 * Ea, ldb=3 * Ea, ldc=Sp, alpha=scale, batch1=b, batch2=H,
+         strideA=sQ, strideB=sQ, strideC=sP, offB=Ea)
+    softmax_fwd(P, mask, P, b * H * S, S, Sp, S)
+    gemm(P, qkv, ctx, S, hd, S, lda=Sp, ldb=3 * Ea, ldc=Ea, batch1=b, batch2=H, strideA=sP, strideB=sQ,
+         strideC=(S * Ea, hd), offB=2 * Ea)
+    gemm(ctx, wo, out, M, w_out.shape[0], Ea, transB=True)
+    return out
 
 
 def logsoftmax_nll(logits, targets, row_loss, dlogits, rows, width, ld, ignore_index=-100, grad_scale=1.0):

@@ -151,6 +151,8 @@ def _call_shape(node, sh):
         L, N, E = sh(kw["query"])
         S = sh(kw["key"])[0]
         return [(L, N, E), (N, L, S)]
+    if t is models.head_parallel_attention:
+        return tuple(sh(a[0])[:2]) + (sh(a[3])[0],)
     if t is F.conv2d:
         n, _c, h, w = sh(a[0])
         o, _ci, kh, kw_ = sh(a[1])
@@ -195,6 +197,10 @@ def _node_flops(node, sh) -> int:
         L, N, E = sh(kw["query"])
         S = sh(kw["key"])[0]
         return 3 * L * N * E * S + 5 * L * S * N + 3 * L * N * E * S
+    if t is models.head_parallel_attention:                      # hap.rs:1330-1337 with E = the local heads' width
+        N, L, _d = sh(a[0])
+        Ea = sh(a[1])[0] // 3
+        return 3 * L * N * Ea * L + 5 * L * L * N + 3 * L * N * Ea * L
     if t is F.layer_norm:                                        # hap.rs:1656
         return 10 * _prod(sh(a[0]))
     if t is F.conv2d:                                            # hap.rs:1727

@@ -32,6 +32,10 @@ Plans (each step is a legal Hoare triple of hap.rs:2786-3419):
 ``ffn="batch"``   pure uneven data parallelism;
 MoE layers        gating on replicated tokens, experts sharded over the
                   expert dimension, combine -> reduce_scatter / all_reduce.
+``attn="heads"``  attention sharded over heads instead of samples (uneven head
+                  counts: rows of the in-projection, columns of the
+                  out-projection), all_gather before, reduce_scatter after;
+                  a form the reference's synthesizer cannot emit.
 ``zero=True``     on top of any of them: every parameter that would be
                   replicated is stored as a dim-0 shard (the reference's
                   ``extra_ps`` / force_zero mode).
@@ -48,7 +52,7 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from . import collectives, models
-from .sharding import ShardingPlan, shard_inplace
+from .sharding import ShardingPlan, shard_heads_inplace, shard_inplace
 
 
 class _Emitter:
@@ -96,8 +100,43 @@ class _Emitter:
             self._attr_cache[target] = self.g.get_attr(target)
         return self._attr_cache[target]
 
+    def sharded_as(self, target: str, lengths, dim: int):
+        """Like ``sharded`` with the lengths given (head counts scaled by the head width)."""
+        if target not in self._attr_cache:
+            shard_inplace(self.module, target, list(lengths), dim, self.rank)
+            self._attr_cache[target] = self.g.get_attr(target)
+        return self._attr_cache[target]
+
+    def head_sharded(self, target: str, head_lengths, head_dim: int):
+        if target not in self._attr_cache:
+            shard_heads_inplace(self.module, target, list(head_lengths), head_dim, self.rank)
+            self._attr_cache[target] = self.g.get_attr(target)
+        return self._attr_cache[target]
+
     def call(self, fn, *args, **kwargs):
         return self.g.call_function(fn, tuple(args), kwargs or None)
+
+
+def _head_parallel_attention(e: _Emitter, h, prefix: str, emsize: int, nheads: int, p: float, mask, B: int):
+    """Attention sharded over heads: the batch is gathered, every device runs its (uneven) share of the heads on
+    all samples with the matching rows of the in-projection and columns of the out-projection, and the partial
+    outputs are reduce-scattered back to the batch sharding; the output bias is added once, after the sum."""
+    plan = e.plan
+    hd = emsize // nheads
+    L_B, L_H = plan.lengths(B), plan.lengths(nheads)
+    if min(L_H) < 1:
+        raise ValueError(f"{nheads} heads over ratios {plan.ratios[0]} leave a device without a head")
+    full = e.call(collectives.all_gather, h, 0, L_B, e.rank)
+    partial = e.call(models.head_parallel_attention, full,
+                     e.head_sharded(prefix + "self_attn.in_proj_weight", L_H, hd),
+                     e.head_sharded(prefix + "self_attn.in_proj_bias", L_H, hd),
+                     e.sharded_as(prefix + "self_attn.out_proj.weight", [l * hd for l in L_H], 1),
+                     L_H[e.rank], mask)
+    out = e.call(collectives.reduce_scatter, partial, 0, L_B, e.rank)
+    out = e.call(operator.add, out, e.replicated(prefix + "self_attn.out_proj.bias"))
+    out = e.call(F.dropout, out, p)
+    s = e.call(operator.add, h, out)
+    return e.call(F.layer_norm, s, (emsize,))
 
 
 def _attention(e: _Emitter, h, prefix: str, emsize: int, nheads: int, p: float, mask):
@@ -211,7 +250,10 @@ def build_program(model: nn.Module, plan: ShardingPlan, global_batch: int,
 
     for i, layer in enumerate(model.layers):
         prefix = f"layers.{i}."
-        h1 = _attention(e, h, prefix, d, model.nheads, p, mask)
+        if plan.attn == "heads" and batch_sharded:
+            h1 = _head_parallel_attention(e, h, prefix, d, model.nheads, p, mask, B)
+        else:
+            h1 = _attention(e, h, prefix, d, model.nheads, p, mask)
         if isinstance(layer, models.Top2TransformerEncoderLayer):
             # the switch layer takes the top-2 layer's node forms with its own gating leaf (the reference's
             # synthesizer has no handler for models.switch_gating; its models call it at models.py:421)

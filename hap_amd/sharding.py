@@ -48,6 +48,22 @@ def shard_inplace(module: torch.nn.Module, target: str, lengths: Sequence[int], 
     p.data = torch.split(p.data, list(lengths), dim)[rank].contiguous()
 
 
+def shard_heads_inplace(module: torch.nn.Module, target: str, head_lengths: Sequence[int], head_dim: int,
+                        rank: int) -> None:
+    """Keep the q, k and v rows of this rank's heads of a packed in-projection ([3 * H * head_dim, ...] weight or
+    bias): rows [lo, hi) * head_dim of each of the three blocks, stacked in q, k, v order."""
+    try:
+        p = module.get_parameter(target)
+    except AttributeError:
+        p = module.get_buffer(target)
+    H = sum(head_lengths)
+    if p.data.shape[0] != 3 * H * head_dim:
+        raise ValueError(f"{target}: leading dimension {p.data.shape[0]} is not 3 * {H} heads * {head_dim}")
+    lo = sum(head_lengths[:rank])
+    blocks = p.data.view(3, H, head_dim, *p.data.shape[1:])[:, lo:lo + head_lengths[rank]]
+    p.data = blocks.reshape(3 * head_lengths[rank] * head_dim, *p.data.shape[1:]).contiguous()
+
+
 @dataclass
 class ShardingPlan:
     """Per-segment device ratios plus this device's rank (hap.rs:865, 178-180)."""
@@ -55,6 +71,7 @@ class ShardingPlan:
     rank: int
     ffn: str = "column"          # "column": FFN1 column-sharded (plan P1); "batch": pure DP (plan P2)
     segment: int = 0
+    attn: str = "batch"          # "batch": attention on the device's samples; "heads": on the device's heads of every sample
     zero: bool = False           # parameters stored as dim-0 shards and all_gather-ed at use (hap.rs:2527-2547)
 
     @property

@@ -60,6 +60,8 @@ class JointCPURun:
             gating = ref.top_2_gating if t is product_models.top_2_gating else ref.switch_gating
             dispatch, combine = gating(x.float(), n_expert, capacity, wg.float())
             return dispatch, combine
+        if t is product_models.head_parallel_attention:
+            return ref.head_parallel_attention(*args, **kwargs)
         if t is product_models.append_cls_token:
             x, cls = args
             return torch.cat((cls.expand(x.shape[0], -1, -1), x), dim=1)

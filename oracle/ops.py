@@ -10,6 +10,8 @@ Functions and the reference lines they follow:
 * ``positional_encoding``  -- /root/reference/models.py:504-509.
 * ``top_2_gating``         -- /root/reference/models.py:477-502.
 * ``switch_gating``        -- /root/reference/models.py:452-475.
+* ``head_parallel_attention`` -- no reference counterpart (the reference shards
+  attention over the batch only): softmax attention of a subset of heads.
 * ``JointWorld`` collectives -- /root/reference/collectives.py:6-29 (padded,
   AllGather), 73-84 (AllReduce), 88-103 (ReduceScatter), 146-148
   (dynamic_slice), 152-166 (AllToAll), 171-180 (Replicate).
@@ -102,6 +104,24 @@ def top_2_gating(gate_input, n_expert: int, capacity: int, gate_weight, train: b
                * F.one_hot(pos, capacity)).sum(dim=2)                  # :498
     dispatch = (combine > 0).to(torch.float32)                         # :500
     return dispatch, combine
+
+
+def head_parallel_attention(x, in_proj_weight, in_proj_bias, out_proj_weight, num_heads: int, attn_mask=None):
+    """Self-attention over a subset of a layer's heads, written out with plain tensor operations: the rows of
+    the packed in-projection are [q; k; v] of those heads, the out-projection holds their columns, and the
+    result is the partial output without the output bias.  (No reference counterpart; pinned by the identity
+    that the partial outputs of a partition of the heads plus the bias add up to
+    F.multi_head_attention_forward of the whole layer.)"""
+    b, S, _d = x.shape
+    Ea = in_proj_weight.shape[0] // 3
+    hd = Ea // num_heads
+    qkv = x @ in_proj_weight.t() + in_proj_bias
+    q, k, v = (t.reshape(b, S, num_heads, hd).transpose(1, 2) for t in qkv.split(Ea, dim=2))
+    scores = (q @ k.transpose(2, 3)) / math.sqrt(hd)
+    if attn_mask is not None:
+        scores = scores + attn_mask.to(scores.dtype)
+    ctx = (torch.softmax(scores.float(), dim=3).to(v.dtype) @ v).transpose(1, 2).reshape(b, S, Ea)
+    return ctx @ out_proj_weight.t()
 
 
 def switch_gating(gate_input, n_expert: int, capacity: int, gate_weight, train: bool = True):

@@ -57,7 +57,8 @@ def rank_programs(model, ratios, B, **kw):
     progs = []
     for r in range(len(ratios)):
         m = copy.deepcopy(model)
-        plan = hap_amd.ShardingPlan([list(ratios)], r, ffn=kw.get("ffn", "column"), zero=kw.get("zero", False))
+        plan = hap_amd.ShardingPlan([list(ratios)], r, ffn=kw.get("ffn", "column"), zero=kw.get("zero", False),
+                                     attn=kw.get("attn", "batch"))
         progs.append(hap_amd.build_program(m, plan, B, activation=kw.get("activation", "relu"),
                                            batch_sharded=kw.get("batch_sharded", True)))
     return progs

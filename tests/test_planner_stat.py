@@ -24,6 +24,7 @@ CASES = {
     "lm_column": dict(make=lambda: helpers.make_lm(), ratios=RATIOS4, B=16, kw=dict(ffn="column"), batch="lm"),
     "lm_batch": dict(make=lambda: helpers.make_lm(causal=False), ratios=RATIOS4, B=11, kw=dict(ffn="batch"), batch="lm"),
     "lm_zero": dict(make=lambda: helpers.make_lm(), ratios=RATIOS4, B=16, kw=dict(ffn="column", zero=True), batch="lm"),
+    "lm_heads": dict(make=lambda: helpers.make_lm(H=8), ratios=RATIOS4, B=16, kw=dict(ffn="batch", attn="heads"), batch="lm"),
     "vit": dict(make=lambda: helpers.make_vit(), ratios=RATIOS4, B=8, kw=dict(ffn="column"), batch="vit"),
     "moe": dict(make=lambda: helpers.make_moe(), ratios=RATIOS_E, B=8, kw=dict(ffn="batch"), batch="lm"),
     "moe_whole_batch": dict(make=lambda: helpers.make_moe(), ratios=RATIOS_E, B=4,

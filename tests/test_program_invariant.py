@@ -34,8 +34,13 @@ def _check(model, run, x, y, sharded, whole_norm=False):
             continue
         grads = [h.grad for h in held]
         if name in sharded:
-            dim, L = sharded[name]
-            want = torch.split(ref_p.grad, L, dim)
+            dim, L = sharded[name][:2]
+            if dim == "heads":                 # q, k, v rows of each rank's heads of a packed in-projection
+                hd = sharded[name][2]
+                blocks = ref_p.grad.view(3, sum(L), hd, *ref_p.grad.shape[1:])
+                want = [b.reshape(3 * l * hd, *ref_p.grad.shape[1:]) for b, l in zip(torch.split(blocks, L, 1), L)]
+            else:
+                want = torch.split(ref_p.grad, L, dim)
             for r in range(W):
                 if whole_norm:
                     # a shard may hold only rows whose true gradient is zero (the key bias of softmax attention):
@@ -140,3 +145,42 @@ def test_switch_moe_spmd_equals_single_device(zero):
     assert sum(n.target is hap_amd.models.switch_gating for n in run.programs[0].graph.nodes) == 1
     sharded = _zero_sharded(model, RATIOS_E) if zero else {"layers.1.w1": (0, L_E), "layers.1.w2": (0, L_E)}
     _check(model, run, x, y, sharded, whole_norm=zero)
+
+
+def _head_sharded(layers, L_H, hd):
+    out = {}
+    for i in range(layers):
+        out[f"layers.{i}.self_attn.in_proj_weight"] = ("heads", L_H, hd)
+        out[f"layers.{i}.self_attn.in_proj_bias"] = ("heads", L_H, hd)
+        out[f"layers.{i}.self_attn.out_proj.weight"] = (1, [l * hd for l in L_H])
+    return out
+
+
+@pytest.mark.parametrize("ffn", ["column", "batch"])
+def test_head_parallel_attention_lm_spmd_equals_single_device(ffn):
+    """8 heads over ratios .375/.375/.125/.125 -> 3, 3, 1, 1 heads per device."""
+    model = make_lm(H=8)
+    B = 8
+    x, y = lm_batch(B, 16, 97)
+    run = joint_cpu(model, RATIOS4, B, ffn=ffn, attn="heads")
+    L_H = hap_amd.sharding_lengths(8, RATIOS4)
+    assert L_H == [3, 3, 1, 1]
+    held = dict(run.programs[2].named_parameters())
+    assert held["layers.0.self_attn.in_proj_weight"].shape == (3 * 1 * 4, 32)
+    assert held["layers.0.self_attn.out_proj.weight"].shape == (32, 4)
+    sharded = _head_sharded(2, L_H, 4)
+    if ffn == "column":
+        L_F = hap_amd.sharding_lengths(64, RATIOS4)
+        for i in range(2):
+            sharded[f"layers.{i}.linear1.weight"] = (0, L_F)
+            sharded[f"layers.{i}.linear1.bias"] = (0, L_F)
+    _check(model, run, x, y, sharded, whole_norm=True)
+
+
+def test_head_parallel_attention_vit_with_zero_spmd_equals_single_device():
+    model = make_vit(H=4)
+    x, y = vit_batch(8, 16, 10)
+    run = joint_cpu(model, [.25, .25, .25, .25], 8, ffn="batch", attn="heads", zero=True)
+    sharded = _zero_sharded(model, [.25] * 4)
+    sharded.update(_head_sharded(2, [1, 1, 1, 1], 8))
+    _check(model, run, x, y, sharded, whole_norm=True)
