@@ -33,6 +33,7 @@ class GemmArgs(ctypes.Structure):
         ("strideC1", ctypes.c_int64), ("strideC2", ctypes.c_int64),
         ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_int64),
         ("a_rowsum", ctypes.c_void_p),
+        ("c_relu_mask", ctypes.c_void_p),
     ]
 
 

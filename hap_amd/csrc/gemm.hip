@@ -105,7 +105,8 @@ Choice choose(int64_t M, int64_t N, int64_t K, int64_t batch, int bk, bool wide,
 
 template <typename TO>
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *ws, TO *C, int64_t M, int64_t N, int64_t ws_ld,
-                                                          int64_t ldc, int splits, int accumulate, int act) {
+                                                          int64_t ldc, int splits, int accumulate, int act,
+                                                          const TO *relu_mask) {
     const int64_t groups = ws_ld / 4, total = M * groups;
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
         const int64_t m = i / groups, n = (i - m * groups) * 4;
@@ -121,6 +122,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *ws, TO 
         for (int e = 0; e < 4; ++e) {
             if (n + e < N) {
                 float x = apply_act(acc[e], act);
+                if (relu_mask && !((float)relu_mask[m * ldc + n + e] > 0.f)) x = 0.f;
                 if (accumulate) x += (float)dst[e];
                 dst[e] = (TO)x;
             }
@@ -168,7 +170,7 @@ int launch_typed(GemmParams &p, int transA, int transB, int64_t batch, hipStream
     int64_t gx = hapmi_cdiv(p.M * (p.ws_ld / 4), 256);
     if (gx > 256 * 16) gx = 256 * 16;
     hipLaunchKernelGGL((splitk_reduce_kernel<TO>), dim3((unsigned)gx), dim3(256), 0, st, (const float *)p.ws, (TO *)p.C,
-                       p.M, p.N, p.ws_ld, p.ldc, p.splits, p.accumulate, p.act);
+                       p.M, p.N, p.ws_ld, p.ldc, p.splits, p.accumulate, p.act, (const TO *)p.relu_mask);
     return HAPMI_OK;
 }
 
@@ -215,6 +217,9 @@ extern "C" int hapmi_gemm(const hapmi_gemm_args *a, hapmi_stream_t stream) {
     p.rowsum = a->a_rowsum;
     HAPMI_REQUIRE(!a->a_rowsum || (a->transA && a->batch1 * a->batch2 == 1), HAPMI_EINVAL,
                   "gemm: a_rowsum needs transA = 1 (A stored [K, M]) and a single problem");
+    p.relu_mask = a->c_relu_mask;
+    HAPMI_REQUIRE(!a->c_relu_mask || (a->batch1 * a->batch2 == 1 && ((uintptr_t)a->c_relu_mask % 16) == 0), HAPMI_EINVAL,
+                  "gemm: c_relu_mask needs a single problem and a 16-byte aligned pointer");
 
     hipStream_t st = (hipStream_t)stream;
     hipEvent_t e0 = nullptr, e1 = nullptr;

@@ -34,6 +34,7 @@ struct GemmParams {
     int splits, ktiles_per_split;
     float *ws;                 // split-K workspace [splits][M][ws_ld] (float32)
     float *rowsum;             // optional: rowsum[m] += sum_k op(A)[m, k] (float32 atomics; A stored [K, M] only)
+    const void *relu_mask;     // optional: [M][ldc] in C's element type; result elements whose mask is <= 0 become 0
     int64_t ws_ld;
 };
 
@@ -356,7 +357,18 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, (WAVES_M * WAVES_N <= 4 ? 2 
                     *(bf16x4 *)(stage + (lane & 31) * SROWH + (j * 32 + q * 8 + (lane >> 5) * 4) * 2) = o;
                 }
             bf16_t *band = (bf16_t *)C + (m0 + wm + i * 32) * p.ldc + n0 + wn;
-            if (interior) {
+            const bf16_t *mband = p.relu_mask ? (const bf16_t *)p.relu_mask + (m0 + wm + i * 32) * p.ldc + n0 + wn : nullptr;
+            if (interior && mband) {
+                // the producer of this operand's gradient applied relu itself: its output is the mask
+#pragma unroll
+                for (int g = 0; g < NG; ++g) {
+                    bf16x8 sv = *(const bf16x8 *)(stage + soff[g]);
+                    const bf16x8 mv = *(const bf16x8 *)(mband + goff[g]);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) sv[e] = (float)mv[e] > 0.f ? sv[e] : (bf16_t)0.f;
+                    *(bf16x8 *)(band + goff[g]) = sv;
+                }
+            } else if (interior) {
 #pragma unroll
                 for (int g = 0; g < NG; ++g) *(bf16x8 *)(band + goff[g]) = *(const bf16x8 *)(stage + soff[g]);
             } else {
@@ -366,8 +378,13 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, (WAVES_M * WAVES_N <= 4 ? 2 
                     const int64_t m = m0 + wm + i * 32 + row;
                     const int64_t n = n0 + wn + gc * 8;
                     if (m >= p.M || n >= p.N) continue;
-                    const bf16x8 sv = *(const bf16x8 *)(stage + soff[g]);
+                    bf16x8 sv = *(const bf16x8 *)(stage + soff[g]);
                     bf16_t *dst = band + goff[g];
+                    if (mband) {
+#pragma unroll
+                        for (int e = 0; e < 8; ++e)
+                            if (n + e < p.N && !((float)mband[goff[g] + e] > 0.f)) sv[e] = (bf16_t)0.f;
+                    }
                     if (n + 8 <= p.N) {
                         *(bf16x8 *)dst = sv;
                     } else {
@@ -416,6 +433,11 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, (WAVES_M * WAVES_N <= 4 ? 2 
                     continue;
                 }
                 TO *dst = band + row * (int)p.ldc + qc * 4;
+                if (p.relu_mask) {
+                    const out4_t mk = *(const out4_t *)((const TO *)p.relu_mask + (mb + row) * p.ldc + nb + qc * 4);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] = (float)mk[e] > 0.f ? v[e] : 0.f;
+                }
                 if (p.accumulate) {
                     const out4_t old = *(const out4_t *)dst;
 #pragma unroll
@@ -441,8 +463,15 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, (WAVES_M * WAVES_N <= 4 ? 2 
                 continue;
             }
             TO *dst = C + m * p.ldc + n;
+            f32x4 vm = v;
+            if (p.relu_mask) {
+                const TO *mk = (const TO *)p.relu_mask + m * p.ldc + n;
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (n + e < p.N && !((float)mk[e] > 0.f)) vm[e] = 0.f;
+            }
             if (n + 4 <= p.N && ((p.ldc & 3) == 0)) {
-                f32x4 x = v;
+                f32x4 x = vm;
                 if (p.accumulate) {
                     const out4_t old = *(const out4_t *)dst;
 #pragma unroll
@@ -456,7 +485,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, (WAVES_M * WAVES_N <= 4 ? 2 
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     if (n + e < p.N) {
-                        float x = v[e];
+                        float x = vm[e];
                         if (p.accumulate) x += (float)dst[e];
                         dst[e] = (TO)x;
                     }

@@ -59,7 +59,7 @@ def _round_up(n, m):
 class ShardExecutor:
     def __init__(self, gm: torch.fx.GraphModule, example_inputs, dtype: str = "fp32", wire: Optional[Wire] = None,
                  rank: int = 0, world_size: int = 1, device: str = "cuda:0", fused_attention: bool = True,
-                 overlap_wgrad: bool = False, launch_lists: bool = True):
+                 overlap_wgrad: bool = False, launch_lists: bool = True, relu_mask_in_dgrad: bool = False):
         """``example_inputs``: the program's inputs (global batch) as tensors or shapes; activations are
         sized from them.  ``rank`` / ``world_size`` are only needed by all_reduce / replicate, whose node
         forms do not carry them (collectives.py:86, 182)."""
@@ -95,6 +95,7 @@ class ShardExecutor:
         # the BERT-large shard this hides host launch latency of eager steps (about 6 %), but adds nothing to a
         # step replayed from a HIP graph, so it is off by default.
         self.overlap_wgrad = overlap_wgrad
+        self.relu_mask_in_dgrad = relu_mask_in_dgrad
         self._side_stream = torch.cuda.Stream(device=self.dev) if overlap_wgrad else None
         self._side_join = torch.cuda.Event() if overlap_wgrad else None
         self._side_used = False
@@ -557,7 +558,14 @@ class ShardExecutor:
                 self.bwd.append(lambda: ops.gemm(dy, w.t, g, M, K, N, lda=ldc, ldc=lda, accumulate=True))
             elif x.needs_grad:
                 g, acc = self._grad_slot(x)
-                self.bwd.append(lambda: ops.gemm(dy, w.t, g, M, K, N, lda=ldc, ldc=lda, accumulate=acc))
+                # x is the output of a producer that applied relu itself and this linear is its only reader:
+                # the data gradient leaves the GEMM already masked and the separate relu-backward pass is skipped
+                mask = None
+                if (self.relu_mask_in_dgrad and x.meta.get("fused_act") == "relu" and not acc and x.ld is None and self._only_reader(node, x)
+                        and not x.meta.get("relu_bwd_done")):
+                    mask = x.t
+                    x.meta["relu_bwd_done"] = True
+                self.bwd.append(lambda: ops.gemm(dy, w.t, g, M, K, N, lda=ldc, ldc=lda, accumulate=acc, relu_mask=mask))
         self._tape.append(emit)
         return out
 
@@ -587,12 +595,24 @@ class ShardExecutor:
         self._tape.append(emit)
         return out
 
+    def _only_reader(self, node, x: Val) -> bool:
+        """True when ``node`` is the only consumer of the value ``x``, followed back through the nodes that pass
+        it on unchanged (the relu a producer already applied, dropout with p = 0)."""
+        n = node.args[0]
+        while isinstance(n, torch.fx.Node) and self.env.get(n) is x:
+            if len(n.users) != 1:
+                return False
+            n = n.args[0] if n.args and isinstance(n.args[0], torch.fx.Node) else None
+        return True
+
     def _wants_fused_relu(self, node):
         users = list(node.users)
         return len(users) == 1 and users[0].target is F.relu
 
     def _relu_backward_through(self, out: Val):
         """For a producer that applied relu itself: d(pre-activation) = d(out) * (out > 0), in place."""
+        if out.meta.get("relu_bwd_done"):
+            return
         g = out.grad
         self._guard_write(g)
         self.bwd.append(lambda: ops.act_bwd(g, out.t, g, "relu"))
@@ -951,7 +971,13 @@ class ShardExecutor:
 
     def _emit_exchange(self, tag, direction, x_t, split_dim, cat_dim, split_L, cat_L, rank, sink, act=None):
         W = len(split_L)
-        pieces = [self._new(ops._with_dim(x_t.shape, split_dim, l)) for l in split_L]
+        # pieces along the slowest dimension are contiguous ranges of the input: views, as torch.split gives the
+        # reference (collectives.py:156); any other dimension needs the strided copy
+        views = split_dim == 0 and x_t.is_contiguous()
+        if views:
+            pieces = list(torch.split(x_t, list(split_L), 0))
+        else:
+            pieces = [self._new(ops._with_dim(x_t.shape, split_dim, l)) for l in split_L]
         own = pieces[rank]
         parts = []
         for src in range(W):
@@ -961,7 +987,10 @@ class ShardExecutor:
                 shape = ops._with_dim(own.shape, cat_dim, cat_L[src])
                 parts.append(self.wire.recv(tag, direction, src, shape, self.cdt, self.dev, reduction=False))
         out = self._new(ops._with_dim(own.shape, cat_dim, sum(cat_L)))
-        sink.append(lambda: (ops.split_rows(x_t, split_L, split_dim, pieces), ops.concat_rows(parts, cat_dim, out, act)))
+        if views:
+            sink.append(lambda: ops.concat_rows(parts, cat_dim, out, act))
+        else:
+            sink.append(lambda: (ops.split_rows(x_t, split_L, split_dim, pieces), ops.concat_rows(parts, cat_dim, out, act)))
         return out
 
     def _all_to_all(self, node):

@@ -284,11 +284,12 @@ def gemm(A: torch.Tensor, B: torch.Tensor, C: torch.Tensor, M: int, N: int, K: i
          lda=None, ldb=None, ldc=None, bias: Optional[torch.Tensor] = None, accumulate=False, act=None, alpha=1.0,
          batch1=1, batch2=1, strideA=(0, 0), strideB=(0, 0), strideC=(0, 0),
          offA=0, offB=0, offC=0, workspace: Optional[torch.Tensor] = None,
-         a_rowsum: Optional[torch.Tensor] = None):
+         a_rowsum: Optional[torch.Tensor] = None, relu_mask: Optional[torch.Tensor] = None):
     """C = alpha * op(A) @ op(B) (+bias)(act)(+C).  Offsets and strides are in elements.  ``workspace`` (or
     the buffer installed with ``set_gemm_workspace``) lets the library split a long reduction over K.
-    ``a_rowsum`` (float32[M], transA only): the sums over k of op(A)'s rows are added into it."""
-    _dev(A, B, C, bias, a_rowsum)
+    ``a_rowsum`` (float32[M], transA only): the sums over k of op(A)'s rows are added into it.
+    ``relu_mask`` ([M, ldc] like C): result elements whose mask is <= 0 are zero (relu backward)."""
+    _dev(A, B, C, bias, a_rowsum, relu_mask)
     if A.dtype != B.dtype:
         raise TypeError("gemm operands must share a dtype")
     a = GemmArgs()
@@ -326,10 +327,15 @@ def gemm(A: torch.Tensor, B: torch.Tensor, C: torch.Tensor, M: int, N: int, K: i
             raise TypeError("gemm a_rowsum: float32 vector, transA and a single problem expected")
         _need(a_rowsum, M, "gemm a_rowsum")
     a.a_rowsum = a_rowsum.data_ptr() if a_rowsum is not None else 0
+    if relu_mask is not None:
+        if relu_mask.dtype != C.dtype or batch1 * batch2 != 1:
+            raise TypeError("gemm relu_mask: C's element type and a single problem expected")
+        _need(relu_mask, _span(M, N, a.ldc), "gemm relu_mask")
+    a.c_relu_mask = relu_mask.data_ptr() if relu_mask is not None else 0
     if min(strideA + strideB + strideC) < 0:
         raise _lib.HapmiError("gemm: negative batch stride")
     if _gemm_log is not None:
-        _gemm_log.append((a, (A, B, C, bias, ws, a_rowsum)))          # the tensors keep the recorded pointers alive
+        _gemm_log.append((a, (A, B, C, bias, ws, a_rowsum, relu_mask)))          # the tensors keep the recorded pointers alive
     check(lib().hapmi_gemm(ctypes.byref(a), _stream()))
     return C
 

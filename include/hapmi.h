@@ -135,6 +135,10 @@ typedef struct {
                                   * caller clears it): the bias gradient of F.linear when the call is the weight
                                   * gradient dW = dY^T X, i.e. the column sum that autograd takes of dY
                                   * (hap.rs:1032 F.linear with bias).  Needs transA = 1 and batch 1; NULL = off */
+    const void *c_relu_mask;     /* optional: [M][ldc] in out_dtype; elements of the result (before accumulation)
+                                  * whose mask value is <= 0 are written as 0: the backward of F.relu
+                                  * (hap.rs:1417) when the call is the data gradient of the next F.linear and
+                                  * the mask is relu's output.  Needs batch 1; NULL = off */
 } hapmi_gemm_args;
 int hapmi_gemm(const hapmi_gemm_args *args_host, hapmi_stream_t stream);
 

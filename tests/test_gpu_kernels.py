@@ -303,6 +303,36 @@ def test_gemm_row_sums_of_a_transposed_operand(cuda, dtype, cfg, tB):
         ops.gemm(A.t().contiguous().to(cuda), B.to(cuda), C, M, N, K, transA=False, transB=tB, a_rowsum=rs)
 
 
+@pytest.mark.parametrize("dtype,out_dtype,cfg,splits,accumulate", [
+    (torch.bfloat16, torch.bfloat16, 0, 1, False), (torch.bfloat16, torch.bfloat16, 1, 1, False),
+    (torch.bfloat16, torch.bfloat16, 3, 1, False), (torch.bfloat16, torch.bfloat16, 0, 4, False),
+    (torch.bfloat16, torch.bfloat16, 0, 1, True), (torch.bfloat16, torch.float32, 5, 1, False),
+    (torch.float32, torch.float32, 0, 1, False), (torch.float32, torch.float32, 0, 4, True)])
+@pytest.mark.parametrize("shape", [(256, 512, 192), (328, 520, 1000)])
+def test_gemm_relu_mask_on_the_result(cuda, dtype, out_dtype, cfg, splits, accumulate, shape):
+    """c_relu_mask: C = (mask > 0) * (A B) (+ C): the relu backward of the tensor whose gradient the call computes,
+    in every store path (16-byte bf16 stores, float32 staging, split-K reduction, accumulation, ragged edges)."""
+    from hap_amd._lib import lib
+    M, N, K = shape
+    g = torch.Generator().manual_seed(M + cfg + splits)
+    A = torch.randn(M, K, generator=g).to(dtype)
+    B = torch.randn(K, N, generator=g).to(dtype)
+    mask = torch.relu(torch.randn(M, N, generator=g)).to(out_dtype)         # a relu output: zeros and positives
+    start = torch.randn(M, N, generator=g).to(out_dtype)
+    want = (A.double() @ B.double()) * (mask > 0)
+    if accumulate:
+        want = want + start.double()
+    ws = torch.empty(8 * M * 520, dtype=torch.float32, device=cuda)
+    try:
+        lib().hapmi_gemm_tuning(cfg, splits)
+        C = start.clone().to(cuda)
+        ops.gemm(A.to(cuda), B.to(cuda), C, M, N, K, workspace=ws, accumulate=accumulate, relu_mask=mask.to(cuda))
+        close(C, want, dtype if out_dtype == torch.float32 else out_dtype, scale=2.0)
+        assert (C.cpu()[mask == 0] == (start[mask == 0] if accumulate else 0)).all()
+    finally:
+        lib().hapmi_gemm_tuning(-1, 0)
+
+
 @pytest.mark.parametrize("S,causal", [(16, True), (128, True), (197, False), (512, False), (200, True), (64, False)])
 def test_fused_attention_forward_backward(cuda, S, causal):
     """Fused bf16 attention against the explicit softmax(QK^T * scale + mask) V of

@@ -290,6 +290,34 @@ def test_side_stream_weight_gradients_equal_main_stream(cuda, dtype):
                 torch.testing.assert_close(ga, gb, rtol=1e-4, atol=1e-5 * gb.abs().max().item())
 
 
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+def test_relu_mask_in_the_data_gradient_equals_the_separate_pass(cuda, dtype):
+    """relu_mask_in_dgrad=True folds relu's backward into the epilogue of the second FFN linear's data-gradient
+    GEMM (c_relu_mask): same loss, same gradients as the separate elementwise pass."""
+    model = make_lm(vocab=211, S=32, d=64, H=1, F=128, layers=2)
+    x, y = lm_batch(8, 32, 211)
+
+    def build(masked):
+        gm = hap_amd.build_program(copy.deepcopy(model), hap_amd.ShardingPlan([RATIOS4], 0), 8)
+        return hap_amd.compile_program(gm, [x, y], dtype=dtype, wire=hap_amd.SyntheticWire(seed=3, grad_scale=1e-2),
+                                       rank=0, world_size=4, relu_mask_in_dgrad=masked)
+
+    a, b = build(True), build(False)
+    la = a.forward(x, y).item()
+    a.backward()
+    lb = b.forward(x, y).item()
+    b.backward()
+    torch.cuda.synchronize()
+    assert la == lb
+    for n, rec in a.params.items():
+        ga, gb = rec["grad"], b.params[n]["grad"]
+        if ga.dim() >= 2 and n != "encoder.weight":
+            assert torch.equal(ga, gb), (n, (ga - gb).abs().max().item())
+        else:
+            torch.testing.assert_close(ga, gb, rtol=1e-4, atol=1e-5 * gb.abs().max().item())
+    assert len(a.bwd) == len(b.bwd) - 2                          # one relu-backward launch per layer gone
+
+
 @pytest.mark.parametrize("family", ["lm", "vit", "moe"])
 def test_recorded_launch_lists_equal_closure_execution(cuda, family):
     """By default the library calls of the first forward / backward / optimizer phase are recorded and later
