@@ -99,14 +99,32 @@ struct PairLoader {
 // ---------------------------------------------------------------------------------------------
 // forward
 // ---------------------------------------------------------------------------------------------
+// Which 128-row block and which (batch, head) a thread block works on.  Without a mask every block does the same
+// work and the grid is taken as it is.  With the causal mask the work grows with the query block (falls with
+// the key block): the blocks are renumbered so that the hardware, which starts blocks in the order of their
+// linear index, starts the longest ones first and the short ones fill the tail.
+template <bool CAUSAL> struct BlockOrder {
+    __device__ __forceinline__ static int linear() { return (int)(blockIdx.y * gridDim.x + blockIdx.x); }
+    __device__ __forceinline__ static int row_block(bool work_grows_with_index) {
+        if (!CAUSAL) return (int)blockIdx.x;
+        const int i = linear() / (int)gridDim.y;
+        return work_grows_with_index ? (int)gridDim.x - 1 - i : i;
+    }
+    __device__ __forceinline__ static int batch_head() { return CAUSAL ? linear() % (int)gridDim.y : (int)blockIdx.y; }
+};
+
+// CAUSAL: key j is visible to query i iff j <= i (the additive mask torch.triu(full(-inf), 1), models.py:76),
+// applied arithmetically; kv tiles that lie completely above the diagonal of the block's 128 queries are skipped.
+template <bool CAUSAL>
 __global__ __launch_bounds__(AT_THREADS, 2) void attn_fwd_kernel(const bf16_t *qkv, const float *mask, bf16_t *out,
                                                             float *lse, int S, int H, float scale) {
     __shared__ __attribute__((aligned(16))) char Ks[TILE_BYTES];
     __shared__ __attribute__((aligned(16))) char Vts[TILE_BYTES];
     const int E = H * HD, ld = 3 * E;
-    const int b = blockIdx.y / H, hh = blockIdx.y % H;
+    const int blk = BlockOrder<CAUSAL>::row_block(true), bh = BlockOrder<CAUSAL>::batch_head();
+    const int b = bh / H, hh = bh % H;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, c = lane & 31, h = lane >> 5;
-    const int q = blockIdx.x * 128 + wave * 32 + c;
+    const int q = blk * 128 + wave * 32 + c;
     const bool qok = q < S;
     const bf16_t *Q = qkv + (int64_t)b * S * ld + hh * HD;
     const bf16_t *K = Q + E, *V = Q + 2 * E;
@@ -122,14 +140,16 @@ __global__ __launch_bounds__(AT_THREADS, 2) void attn_fwd_kernel(const bf16_t *q
 
     // The next tile's global loads are issued before the current tile is multiplied, so their latency is
     // covered by the MFMA / softmax work; the registers are written to LDS at the top of the next iteration.
+    const int q_blk_end = blk * 128 + 128;
+    const int kv_end = (CAUSAL && q_blk_end < S) ? q_blk_end : S;
     lk.load(K, ld, S);
     lv.load(V, ld, S);
-    for (int kv0 = 0; kv0 < S; kv0 += TILE) {
+    for (int kv0 = 0; kv0 < kv_end; kv0 += TILE) {
         __syncthreads();                                   // every wave is done with the previous tiles
         lk.store_rows(Ks);
         lv.store_transposed(Vts);
         __syncthreads();
-        if (kv0 + TILE < S) {
+        if (kv0 + TILE < kv_end) {
             lk.load(K + (int64_t)(kv0 + TILE) * ld, ld, S - kv0 - TILE);
             lv.load(V + (int64_t)(kv0 + TILE) * ld, ld, S - kv0 - TILE);
         }
@@ -161,7 +181,7 @@ __global__ __launch_bounds__(AT_THREADS, 2) void attn_fwd_kernel(const bf16_t *q
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     float v = st[t][g * 4 + e] * scale + mk[e];
-                    if (kv + e >= S) v = -INFINITY;
+                    if (kv + e >= S || (CAUSAL && kv + e > q)) v = -INFINITY;
                     st[t][g * 4 + e] = v;
                     mx = fmaxf(mx, v);
                 }
@@ -233,6 +253,7 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(const bf16_t *out, cons
 // ---------------------------------------------------------------------------------------------
 // dQ: lanes own query columns, kv tiles are streamed
 // ---------------------------------------------------------------------------------------------
+template <bool CAUSAL>
 __global__ __launch_bounds__(AT_THREADS, 2) void attn_bwd_dq_kernel(const bf16_t *qkv, const bf16_t *dout, const float *lse,
                                                                const float *delta, const float *mask, bf16_t *dqkv,
                                                                int S, int H, float scale) {
@@ -240,9 +261,10 @@ __global__ __launch_bounds__(AT_THREADS, 2) void attn_bwd_dq_kernel(const bf16_t
     __shared__ __attribute__((aligned(16))) char Vs[TILE_BYTES];
     __shared__ __attribute__((aligned(16))) char Kts[TILE_BYTES];
     const int E = H * HD, ld = 3 * E;
-    const int b = blockIdx.y / H, hh = blockIdx.y % H;
+    const int blk = BlockOrder<CAUSAL>::row_block(true), bh = BlockOrder<CAUSAL>::batch_head();
+    const int b = bh / H, hh = bh % H;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, c = lane & 31, h = lane >> 5;
-    const int q = blockIdx.x * 128 + wave * 32 + c;
+    const int q = blk * 128 + wave * 32 + c;
     const bool qok = q < S;
     const bf16_t *Q = qkv + (int64_t)b * S * ld + hh * HD;
     const bf16_t *K = Q + E, *V = Q + 2 * E;
@@ -260,15 +282,17 @@ __global__ __launch_bounds__(AT_THREADS, 2) void attn_bwd_dq_kernel(const bf16_t
     PairLoader lk, lv;
     const bool vec_mask = mask && ((S & 3) == 0);
 
+    const int q_blk_end = blk * 128 + 128;
+    const int kv_end = (CAUSAL && q_blk_end < S) ? q_blk_end : S;
     lk.load(K, ld, S);
     lv.load(V, ld, S);
-    for (int kv0 = 0; kv0 < S; kv0 += TILE) {
+    for (int kv0 = 0; kv0 < kv_end; kv0 += TILE) {
         __syncthreads();
         lk.store_rows(Ks);
         lk.store_transposed(Kts);
         lv.store_rows(Vs);
         __syncthreads();
-        if (kv0 + TILE < S) {
+        if (kv0 + TILE < kv_end) {
             const int64_t nx = kv0 + TILE;
             lk.load(K + nx * ld, ld, S - nx);
             lv.load(V + nx * ld, ld, S - nx);
@@ -301,7 +325,7 @@ __global__ __launch_bounds__(AT_THREADS, 2) void attn_bwd_dq_kernel(const bf16_t
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     const int r = g * 4 + e;
-                    float p = (qok && kv + e < S) ? __expf(st[r] * scale + mk[e] - lse_q) : 0.f;
+                    float p = (qok && kv + e < S && !(CAUSAL && kv + e > q)) ? __expf(st[r] * scale + mk[e] - lse_q) : 0.f;
                     dp[r] = p * (dp[r] - delta_q) * scale;
                 }
             }
@@ -330,6 +354,7 @@ __global__ __launch_bounds__(AT_THREADS, 2) void attn_bwd_dq_kernel(const bf16_t
 // ---------------------------------------------------------------------------------------------
 // dK, dV: lanes own kv columns, query tiles are streamed
 // ---------------------------------------------------------------------------------------------
+template <bool CAUSAL>
 __global__ __launch_bounds__(AT_THREADS, 2) void attn_bwd_dkv_kernel(const bf16_t *qkv, const bf16_t *dout, const float *lse,
                                                                 const float *delta, const float *mask, bf16_t *dqkv,
                                                                 int S, int H, float scale) {
@@ -339,9 +364,10 @@ __global__ __launch_bounds__(AT_THREADS, 2) void attn_bwd_dkv_kernel(const bf16_
     __shared__ __attribute__((aligned(16))) char dOts[TILE_BYTES];
     __shared__ __attribute__((aligned(16))) float lse_s[TILE], delta_s[TILE];
     const int E = H * HD, ld = 3 * E;
-    const int b = blockIdx.y / H, hh = blockIdx.y % H;
+    const int blk = BlockOrder<CAUSAL>::row_block(false), bh = BlockOrder<CAUSAL>::batch_head();
+    const int b = bh / H, hh = bh % H;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, c = lane & 31, h = lane >> 5;
-    const int kv = blockIdx.x * 128 + wave * 32 + c;
+    const int kv = blk * 128 + wave * 32 + c;
     const bool kok = kv < S;
     const bf16_t *Q = qkv + (int64_t)b * S * ld + hh * HD;
     const bf16_t *K = Q + E, *V = Q + 2 * E;
@@ -357,9 +383,11 @@ __global__ __launch_bounds__(AT_THREADS, 2) void attn_bwd_dkv_kernel(const bf16_
     f32x16 dvt[2] = {zero16(), zero16()}, dkt[2] = {zero16(), zero16()};
     PairLoader lq, ldo;
 
-    lq.load(Q, ld, S);
-    ldo.load(dO, E, S);
-    for (int q0 = 0; q0 < S; q0 += TILE) {
+    // causal: queries before the block's first key see none of its keys
+    const int q_begin = CAUSAL ? blk * 128 : 0;
+    lq.load(Q + (int64_t)q_begin * ld, ld, S - q_begin);
+    ldo.load(dO + (int64_t)q_begin * E, E, S - q_begin);
+    for (int q0 = q_begin; q0 < S; q0 += TILE) {
         __syncthreads();
         lq.store_rows(Qs);
         lq.store_transposed(Qts);
@@ -397,7 +425,7 @@ __global__ __launch_bounds__(AT_THREADS, 2) void attn_bwd_dkv_kernel(const bf16_
                     const int r = g * 4 + e;
                     float x = sc[r] * scale - l4[e];                 // rows beyond S carry lse = +inf: p = 0
                     if (mask) x += (kok && q0 + ql + e < S) ? mask[(int64_t)(q0 + ql + e) * S + kv] : 0.f;
-                    const float p = __expf(x);
+                    const float p = (CAUSAL && kv > q0 + ql + e) ? 0.f : __expf(x);
                     sc[r] = p;
                     dp[r] = p * (dp[r] - d4[e]) * scale;
                 }
@@ -440,28 +468,34 @@ int check_attn(const char *name, int64_t b, int64_t S, int64_t H) {
 
 }  // namespace
 
-extern "C" int hapmi_attention_fwd(const void *qkv, const float *mask, void *out, float *lse, int64_t b, int64_t S,
-                                   int64_t H, float scale, hapmi_stream_t stream) {
+extern "C" int hapmi_attention_fwd(const void *qkv, const float *mask, int causal, void *out, float *lse, int64_t b,
+                                   int64_t S, int64_t H, float scale, hapmi_stream_t stream) {
     int rc = check_attn("attention_fwd", b, S, H);
     if (rc) return rc;
     if (b == 0) return HAPMI_OK;
     HAPMI_REQUIRE(qkv && out && lse, HAPMI_EINVAL, "attention_fwd: null pointer");
     HAPMI_REQUIRE(((uintptr_t)qkv % 16) == 0 && ((uintptr_t)out % 16) == 0 && (!mask || ((uintptr_t)mask % 16) == 0),
                   HAPMI_EALIGN, "attention_fwd: pointers must be 16-byte aligned");
+    HAPMI_REQUIRE(!(causal && mask), HAPMI_EINVAL, "attention_fwd: causal and an explicit mask exclude each other");
     dim3 grid((unsigned)hapmi_cdiv(S, 128), (unsigned)(b * H));
-    hipLaunchKernelGGL(attn_fwd_kernel, grid, dim3(AT_THREADS), 0, (hipStream_t)stream, (const bf16_t *)qkv, mask,
-                       (bf16_t *)out, lse, (int)S, (int)H, scale);
+    if (causal)
+        hipLaunchKernelGGL(attn_fwd_kernel<true>, grid, dim3(AT_THREADS), 0, (hipStream_t)stream, (const bf16_t *)qkv,
+                           (const float *)nullptr, (bf16_t *)out, lse, (int)S, (int)H, scale);
+    else
+        hipLaunchKernelGGL(attn_fwd_kernel<false>, grid, dim3(AT_THREADS), 0, (hipStream_t)stream, (const bf16_t *)qkv, mask,
+                           (bf16_t *)out, lse, (int)S, (int)H, scale);
     HAPMI_CHECK_LAUNCH("attention_fwd");
     return HAPMI_OK;
 }
 
 extern "C" int hapmi_attention_bwd(const void *qkv, const void *out, const void *dout, const float *lse,
-                                   const float *mask, void *dqkv, float *delta_ws, int64_t b, int64_t S, int64_t H,
-                                   float scale, hapmi_stream_t stream) {
+                                   const float *mask, int causal, void *dqkv, float *delta_ws, int64_t b, int64_t S,
+                                   int64_t H, float scale, hapmi_stream_t stream) {
     int rc = check_attn("attention_bwd", b, S, H);
     if (rc) return rc;
     if (b == 0) return HAPMI_OK;
     HAPMI_REQUIRE(qkv && out && dout && lse && dqkv && delta_ws, HAPMI_EINVAL, "attention_bwd: null pointer");
+    HAPMI_REQUIRE(!(causal && mask), HAPMI_EINVAL, "attention_bwd: causal and an explicit mask exclude each other");
     HAPMI_REQUIRE(((uintptr_t)qkv % 16) == 0 && ((uintptr_t)out % 16) == 0 && ((uintptr_t)dout % 16) == 0 &&
                       ((uintptr_t)dqkv % 16) == 0 && (!mask || ((uintptr_t)mask % 16) == 0),
                   HAPMI_EALIGN, "attention_bwd: pointers must be 16-byte aligned");
@@ -469,10 +503,17 @@ extern "C" int hapmi_attention_bwd(const void *qkv, const void *out, const void 
     hipLaunchKernelGGL(attn_delta_kernel, dim3((unsigned)hapmi_cdiv(b * S * H, 256)), dim3(256), 0, st,
                        (const bf16_t *)out, (const bf16_t *)dout, delta_ws, b * S, (int)S, (int)H);
     dim3 grid((unsigned)hapmi_cdiv(S, 128), (unsigned)(b * H));
-    hipLaunchKernelGGL(attn_bwd_dq_kernel, grid, dim3(AT_THREADS), 0, st, (const bf16_t *)qkv, (const bf16_t *)dout, lse,
-                       (const float *)delta_ws, mask, (bf16_t *)dqkv, (int)S, (int)H, scale);
-    hipLaunchKernelGGL(attn_bwd_dkv_kernel, grid, dim3(AT_THREADS), 0, st, (const bf16_t *)qkv, (const bf16_t *)dout, lse,
-                       (const float *)delta_ws, mask, (bf16_t *)dqkv, (int)S, (int)H, scale);
+    if (causal) {
+        hipLaunchKernelGGL(attn_bwd_dq_kernel<true>, grid, dim3(AT_THREADS), 0, st, (const bf16_t *)qkv, (const bf16_t *)dout,
+                           lse, (const float *)delta_ws, (const float *)nullptr, (bf16_t *)dqkv, (int)S, (int)H, scale);
+        hipLaunchKernelGGL(attn_bwd_dkv_kernel<true>, grid, dim3(AT_THREADS), 0, st, (const bf16_t *)qkv, (const bf16_t *)dout,
+                           lse, (const float *)delta_ws, (const float *)nullptr, (bf16_t *)dqkv, (int)S, (int)H, scale);
+    } else {
+        hipLaunchKernelGGL(attn_bwd_dq_kernel<false>, grid, dim3(AT_THREADS), 0, st, (const bf16_t *)qkv, (const bf16_t *)dout,
+                           lse, (const float *)delta_ws, mask, (bf16_t *)dqkv, (int)S, (int)H, scale);
+        hipLaunchKernelGGL(attn_bwd_dkv_kernel<false>, grid, dim3(AT_THREADS), 0, st, (const bf16_t *)qkv, (const bf16_t *)dout,
+                           lse, (const float *)delta_ws, mask, (bf16_t *)dqkv, (int)S, (int)H, scale);
+    }
     HAPMI_CHECK_LAUNCH("attention_bwd");
     return HAPMI_OK;
 }

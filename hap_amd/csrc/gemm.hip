@@ -75,7 +75,7 @@ struct Choice {
 };
 
 Choice choose(int64_t M, int64_t N, int64_t K, int64_t batch, int bk, bool wide, int64_t max_splits, bool row_major_operands) {
-    static const int kSplitMenu[] = {1, 2, 3, 4, 6, 8, 12, 16, 24, 32};
+    static const int kSplitMenu[] = {1, 2, 3, 4, 5, 6, 7, 8, 10, 12, 16, 24, 32};
     const int64_t nk = hapmi_cdiv(K, bk);
     Choice best{0, 1};
     double best_t = 1e30;
@@ -107,17 +107,43 @@ template <typename TO>
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *ws, TO *C, int64_t M, int64_t N, int64_t ws_ld,
                                                           int64_t ldc, int splits, int accumulate, int act,
                                                           const TO *relu_mask) {
+    // the partial sums of one output group are independent loads: they are issued eight at a time and added in
+    // split order afterwards (the order fixes the float32 result)
+    constexpr int U = 8;
     const int64_t groups = ws_ld / 4, total = M * groups;
+    const int64_t split_stride = M * ws_ld;
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
         const int64_t m = i / groups, n = (i - m * groups) * 4;
         if (n >= N) continue;
-        f32x4 acc = *(const f32x4 *)(ws + m * ws_ld + n);
-        for (int s = 1; s < splits; ++s) {
-            const f32x4 v = *(const f32x4 *)(ws + ((int64_t)s * M + m) * ws_ld + n);
+        const float *src = ws + m * ws_ld + n;
+        f32x4 acc = *(const f32x4 *)src;
+        for (int s0 = 1; s0 < splits; s0 += U) {
+            f32x4 v[U];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) acc[e] += v[e];
+            for (int j = 0; j < U; ++j)
+                if (s0 + j < splits) v[j] = *(const f32x4 *)(src + (int64_t)(s0 + j) * split_stride);
+#pragma unroll
+            for (int j = 0; j < U; ++j)
+                if (s0 + j < splits) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) acc[e] += v[j][e];
+                }
         }
         TO *dst = C + m * ldc + n;
+        if (n + 4 <= N && (ldc & 3) == 0 && !relu_mask) {
+            typedef TO out4_t __attribute__((ext_vector_type(4)));
+            out4_t o;
+            if (accumulate) {
+                const out4_t old = *(const out4_t *)dst;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) o[e] = (TO)(apply_act(acc[e], act) + (float)old[e]);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) o[e] = (TO)apply_act(acc[e], act);
+            }
+            *(out4_t *)dst = o;
+            continue;
+        }
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             if (n + e < N) {

@@ -671,6 +671,12 @@ class ShardExecutor:
             mask_t = mask.t
         scale = 1.0 / math.sqrt(hd)
         fused = self.fused_attention and self.dtype == "bf16" and hd == 64
+        # a constant mask (a buffer of the module, not a gathered shard) that is exactly the causal one is
+        # applied arithmetically by the fused kernels, which then also skip the key tiles above the diagonal
+        causal = False
+        if fused and mask is not None and mask.meta.get("name") is not None:
+            causal = bool(torch.equal(mask.t.cpu(), torch.triu(torch.full((S, S), float("-inf")), diagonal=1)))
+        fused_mask = None if causal else mask_t
         Sp = _round_up(S, self.epv)
         qkv = self._new((b, S, 3 * Ea))
         ctx = self._new((b, S, Ea))
@@ -688,7 +694,7 @@ class ShardExecutor:
         def forward():
             ops.gemm(x.t, w_in.t, qkv, M, 3 * Ea, d, transB=True, bias=b_in.meta["master"])
             if fused:
-                ops.attention_fwd(qkv, mask_t, ctx, lse, b, S, H, scale)
+                ops.attention_fwd(qkv, fused_mask, ctx, lse, b, S, H, scale, causal)
             else:
                 ops.gemm(qkv, qkv, P, S, S, hd, transB=True, lda=3 * Ea, ldb=3 * Ea, ldc=Sp, alpha=scale, batch1=b,
                          batch2=H, strideA=sQ, strideB=sQ, strideC=sP, offB=Ea)
@@ -729,7 +735,7 @@ class ShardExecutor:
                     wgrad_out()
                 ops.gemm(do, w_out.t, dctx, M, Ea, d_out)
                 if fused:
-                    ops.attention_bwd(qkv, ctx, dctx, lse, mask_t, dqkv, delta, b, S, H, scale)
+                    ops.attention_bwd(qkv, ctx, dctx, lse, fused_mask, dqkv, delta, b, S, H, scale, causal)
                 else:
                     # dP = dctx V^T ; dV = P^T dctx
                     ops.gemm(dctx, qkv, dP, S, S, hd, transB=True, lda=Ea, ldb=3 * Ea, ldc=Sp, batch1=b, batch2=H,

@@ -341,7 +341,7 @@ def gemm(A: torch.Tensor, B: torch.Tensor, C: torch.Tensor, M: int, N: int, K: i
 
 
 _gemm_log = None
-_SPLIT_MENU = (1, 2, 3, 4, 6, 8, 12, 16)
+_SPLIT_MENU = (1, 2, 3, 4, 5, 6, 7, 8, 10, 12, 16)
 _N_TILE_CONFIGS = 7
 
 
@@ -470,13 +470,15 @@ def _check_attn(qkv, out, lse, mask, b, S, H):
         raise TypeError("attention: float32 mask expected")
 
 
-def attention_fwd(qkv, mask, out, lse, b, S, H, scale):
+def attention_fwd(qkv, mask, out, lse, b, S, H, scale, causal=False):
+    """``causal``: the mask is torch.triu(full(-inf), 1); pass ``mask=None`` with it."""
     _dev(qkv, mask, out, lse)
     _check_attn(qkv, out, lse, mask, b, S, H)
-    check(lib().hapmi_attention_fwd(_ptr(qkv), _ptr(mask), _ptr(out), _ptr(lse), b, S, H, ctypes.c_float(scale), _stream()))
+    check(lib().hapmi_attention_fwd(_ptr(qkv), _ptr(mask), int(causal), _ptr(out), _ptr(lse), b, S, H,
+                                    ctypes.c_float(scale), _stream()))
 
 
-def attention_bwd(qkv, out, dout, lse, mask, dqkv, delta_ws, b, S, H, scale):
+def attention_bwd(qkv, out, dout, lse, mask, dqkv, delta_ws, b, S, H, scale, causal=False):
     _dev(qkv, out, dout, lse, mask, dqkv, delta_ws)
     _check_attn(qkv, out, lse, mask, b, S, H)
     _need(dout, b * S * H * 64, "attention dout")
@@ -484,8 +486,8 @@ def attention_bwd(qkv, out, dout, lse, mask, dqkv, delta_ws, b, S, H, scale):
     _need(delta_ws, b * H * S, "attention delta")
     if dout.dtype != torch.bfloat16 or dqkv.dtype != torch.bfloat16 or delta_ws.dtype != torch.float32:
         raise TypeError("attention_bwd: dtype mismatch")
-    check(lib().hapmi_attention_bwd(_ptr(qkv), _ptr(out), _ptr(dout), _ptr(lse), _ptr(mask), _ptr(dqkv), _ptr(delta_ws),
-                                    b, S, H, ctypes.c_float(scale), _stream()))
+    check(lib().hapmi_attention_bwd(_ptr(qkv), _ptr(out), _ptr(dout), _ptr(lse), _ptr(mask), int(causal), _ptr(dqkv),
+                                    _ptr(delta_ws), b, S, H, ctypes.c_float(scale), _stream()))
 
 
 def head_parallel_attention(x, w_in, b_in, w_out, num_heads, mask=None):

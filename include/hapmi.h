@@ -178,12 +178,14 @@ int hapmi_softmax_bwd(const void *dp, const void *p, void *ds, int64_t rows, int
 /* fused scaled-dot-product attention on packed projections (the explicit baddbmm / softmax / bmm path of
  * F.multi_head_attention_forward, hap.rs:1301-1327; bf16 only, head_dim 64):
  * qkv[b, S, 3*H*64] -> out[b, S, H*64]; lse[b, H, S] float32 (log-sum-exp of every score row) is kept for
- * backward; mask is NULL or an additive float32 [S, S].  Backward writes dqkv[b, S, 3*H*64] completely;
- * delta_ws is float32 scratch of b*H*S elements. */
-int hapmi_attention_fwd(const void *qkv, const float *mask, void *out, float *lse, int64_t b, int64_t S, int64_t H,
-                        float scale, hapmi_stream_t stream);
+ * backward; mask is NULL or an additive float32 [S, S].  causal != 0 (mask must then be NULL) stands for the
+ * mask torch.triu(full(-inf), diagonal=1) that the language models register as src_mask (models.py:76): the
+ * same result without reading a mask, and the key tiles above the diagonal are skipped.  Backward writes
+ * dqkv[b, S, 3*H*64] completely; delta_ws is float32 scratch of b*H*S elements. */
+int hapmi_attention_fwd(const void *qkv, const float *mask, int causal, void *out, float *lse, int64_t b, int64_t S,
+                        int64_t H, float scale, hapmi_stream_t stream);
 int hapmi_attention_bwd(const void *qkv, const void *out, const void *dout, const float *lse, const float *mask,
-                        void *dqkv, float *delta_ws, int64_t b, int64_t S, int64_t H, float scale,
+                        int causal, void *dqkv, float *delta_ws, int64_t b, int64_t S, int64_t H, float scale,
                         hapmi_stream_t stream);
 
 /* torch.log_softmax + F.nll_loss(reduction='sum', ignore_index) (hap.rs:1829, 1881) and their

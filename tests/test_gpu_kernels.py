@@ -333,10 +333,12 @@ def test_gemm_relu_mask_on_the_result(cuda, dtype, out_dtype, cfg, splits, accum
         lib().hapmi_gemm_tuning(-1, 0)
 
 
-@pytest.mark.parametrize("S,causal", [(16, True), (128, True), (197, False), (512, False), (200, True), (64, False)])
+@pytest.mark.parametrize("S,causal", [(16, True), (128, True), (197, False), (512, False), (200, True), (64, False),
+                                      (16, "flag"), (128, "flag"), (200, "flag"), (512, "flag"), (129, "flag")])
 def test_fused_attention_forward_backward(cuda, S, causal):
     """Fused bf16 attention against the explicit softmax(QK^T * scale + mask) V of
-    F.multi_head_attention_forward, computed in float64 from the same bf16 inputs."""
+    F.multi_head_attention_forward, computed in float64 from the same bf16 inputs.  causal = True hands the
+    kernels the additive mask, "flag" the causal flag instead (no mask read, key tiles above the diagonal skipped)."""
     g = torch.Generator().manual_seed(S)
     b, H, hd = 2, 3, 64
     E = H * hd
@@ -347,8 +349,9 @@ def test_fused_attention_forward_backward(cuda, S, causal):
     out = torch.empty(b, S, E, dtype=torch.bfloat16, device=cuda)
     lse = torch.empty(b, H, S, dtype=torch.float32, device=cuda)
     dq = qkv.to(cuda)
-    dmask = mask.to(cuda) if causal else None
-    ops.attention_fwd(dq, dmask, out, lse, b, S, H, scale)
+    flag = causal == "flag"
+    dmask = mask.to(cuda) if causal is True else None
+    ops.attention_fwd(dq, dmask, out, lse, b, S, H, scale, causal=flag)
     x = qkv.double().requires_grad_(True)
     q, k, v = [t.view(b, S, H, hd).transpose(1, 2) for t in x.split(E, dim=2)]
     sc = q @ k.transpose(-1, -2) * scale
@@ -360,7 +363,7 @@ def test_fused_attention_forward_backward(cuda, S, causal):
     want.backward(dout.double())
     dqkv = torch.full((b, S, 3 * E), float("nan"), dtype=torch.bfloat16, device=cuda)
     delta = torch.empty(b, H, S, dtype=torch.float32, device=cuda)
-    ops.attention_bwd(dq, out, dout.to(cuda), lse, dmask, dqkv, delta, b, S, H, scale)
+    ops.attention_bwd(dq, out, dout.to(cuda), lse, dmask, dqkv, delta, b, S, H, scale, causal=flag)
     for name, got, ref in zip("qkv", dqkv.float().cpu().split(E, dim=2), x.grad.split(E, dim=2)):
         assert rel_err(got, ref) < 2e-2, (name, rel_err(got, ref))
 
