@@ -134,6 +134,9 @@ def main():
     ap.add_argument("--relu-mask-in-dgrad", action="store_true",
                     help="mask the next linear's data gradient in the GEMM epilogue instead of running relu's backward "
                          "as its own pass (the step gains 0.1 ms, the GEMM brackets lose 0.5 ms)")
+    ap.add_argument("--gemm-plan-file", default=None,
+                    help="JSON file of pinned GEMM plans: loaded instead of autotuning when it exists, written after "
+                         "autotuning otherwise (a profiler run can then repeat the plan of an unprofiled run)")
     ap.add_argument("--overlap", action="store_true",
                     help="launch the weight-gradient GEMMs on a second stream (per-kernel event times then overlap)")
     args = ap.parse_args()
@@ -164,8 +167,15 @@ def main():
         ex.backward()
         ex.step()
 
-    if not args.no_autotune:
+    plan_source = "cost model"
+    if args.gemm_plan_file and os.path.exists(args.gemm_plan_file):
+        ops.load_gemm_plans(args.gemm_plan_file)      # untimed set-up: the plan of an earlier tuning run
+        plan_source = "autotuned (loaded)"
+    elif not args.no_autotune:
         ex.autotune_gemms()                           # untimed set-up: pins a tile configuration per GEMM shape
+        plan_source = "autotuned"
+        if args.gemm_plan_file:
+            ops.save_gemm_plans(args.gemm_plan_file)
 
     graph = None
     for _ in range(args.warmup):
@@ -222,7 +232,7 @@ def main():
         "config": {"workload": desc, "local_batch": meta["local_batch"], "global_batch": meta["global_batch"],
                    "seq_len": meta["seq_len"], "launch": "hip-graph" if graph is not None else "eager",
                    "wgrad_stream": "side" if args.overlap else "main",
-                   "gemm_plan": "cost model" if args.no_autotune else "autotuned",
+                   "gemm_plan": plan_source,
                    "final_loss": loss},
         "roofline": {"bound": "mfma", "kernel": "gemm_kernel (all GEMM launches of the step)",
                      "achieved": achieved, "peak": peak, "unit": "TFLOP/s", "frac": achieved / peak,

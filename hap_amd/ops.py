@@ -392,11 +392,37 @@ def autotune_gemm(a: "GemmArgs", flush: Optional[torch.Tensor] = None, repeats: 
     finally:
         check(L.hapmi_gemm_tuning(-1, 0))
     check(L.hapmi_gemm_plan_set(a.M, a.N, a.K, batch, a.transA, a.transB, a.in_dtype, a.out_dtype, best[0], best[1]))
+    _pinned_plans[(a.M, a.N, a.K, batch, a.transA, a.transB, a.in_dtype, a.out_dtype)] = (best[0], best[1])
     return best
+
+
+_pinned_plans = {}      # problem signature -> (tile configuration, K splits), as pinned in the library's plan table
 
 
 def clear_gemm_plans():
     check(lib().hapmi_gemm_plan_clear())
+    _pinned_plans.clear()
+
+
+def save_gemm_plans(path: str) -> int:
+    """Write the plans pinned by autotuning in this process as JSON; returns their number."""
+    import json
+    with open(path, "w") as f:
+        json.dump([list(k) + list(v) for k, v in sorted(_pinned_plans.items())], f)
+    return len(_pinned_plans)
+
+
+def load_gemm_plans(path: str) -> int:
+    """Pin the plans of a file written by ``save_gemm_plans`` (a tuning run on the same device)."""
+    import json
+    with open(path) as f:
+        rows = json.load(f)
+    for row in rows:
+        if len(row) != 10:
+            raise ValueError(f"{path}: a plan row has {len(row)} fields, 10 expected")
+        check(lib().hapmi_gemm_plan_set(*[int(v) for v in row]))
+        _pinned_plans[tuple(int(v) for v in row[:8])] = (int(row[8]), int(row[9]))
+    return len(rows)
 
 
 def linear(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, out_dtype=None, act=None) -> torch.Tensor:

@@ -384,3 +384,27 @@ def test_adam_with_device_step_state_matches_torch(cuda):
         ops.adam_step_dev(p, gr.to(cuda), m, v, None, 5e-4, 0.9, 0.999, 1e-8, state)
     torch.testing.assert_close(p.cpu(), ref.detach(), rtol=1e-5, atol=1e-7)
     assert state[0].item() == 5.0
+
+
+def test_gemm_plans_round_trip_through_a_file(cuda, tmp_path):
+    """Plans pinned by autotuning are written to and re-pinned from a JSON file."""
+    from hap_amd._lib import lib
+    M, N, K = 256, 384, 512
+    A0, B0 = torch.randn(M, K).bfloat16(), torch.randn(N, K).bfloat16()
+    A, B = A0.to(cuda), B0.to(cuda)
+    C = torch.empty(M, N, dtype=torch.bfloat16, device=cuda)
+    ops.clear_gemm_plans()
+    try:
+        ops.record_gemms(True)
+        ops.gemm(A, B, C, M, N, K, transB=True)
+        (args, _keep), = ops.record_gemms(False)
+        cfg, splits, _us = ops.autotune_gemm(args, None, repeats=1)
+        path = str(tmp_path / "plans.json")
+        assert ops.save_gemm_plans(path) == 1
+        ops.clear_gemm_plans()
+        assert ops.load_gemm_plans(path) == 1
+        assert ops._pinned_plans[(M, N, K, 1, 0, 1, 1, 1)] == (cfg, splits)
+        ops.gemm(A, B, C, M, N, K, transB=True)
+        close(C, A0.double() @ B0.double().t(), torch.bfloat16)
+    finally:
+        ops.clear_gemm_plans()
