@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload bert|lm|vit|moe|ragged]
 
-Default workload (N = 1): BASELINE config 2 -- BERT-large-style encoder, bf16 compute with float32 master
+Default workload (N = 1): the headline configuration -- BERT-large-style encoder, bf16 compute with float32 master
 weights, 24 layers, d 1024, 16 heads, FFN 4096 column-split to a local 1536 slice, seq 512, local batch 12
 of 32, vocab 30522, 15 % masked-LM targets, Adam.  Inputs are synthetic (seeded), resident in HBM before the
 timed region; the peers' halves of the collectives come from a seeded synthetic wire.

@@ -1,4 +1,4 @@
-"""Bandwidth of the device-local collective halves at BASELINE config 5: 8 virtual ragged shards
+"""Bandwidth of the device-local collective halves of the uneven-collective configuration: 8 virtual ragged shards
 [S_i, 4096] bf16, S_i uniform in [1000, 3000] from the seed, packed in one GPU's HBM.
 
 Algorithmic bytes (payload read + payload written; pad tails are not credited):

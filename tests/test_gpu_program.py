@@ -92,7 +92,7 @@ def test_lm_fp32_small(cuda, ffn):
 
 
 def test_config1_full_size_fp32(cuda):
-    """BASELINE config 1: 2-layer post-LN LM, d 512, 8 heads, FFN 2048 -> 768 local, seq 128, 3 of 8, vocab 33280."""
+    """The reference's CPU-runnable configuration at full size: 2-layer post-LN LM, d 512, 8 heads, FFN 2048 -> 768 local, seq 128, 3 of 8, vocab 33280."""
     model = make_lm(vocab=33280, S=128, d=512, H=8, F=2048, layers=2, seed=39)
     x, y = lm_batch(8, 128, 33280, seed=39)
     _compare(model, RATIOS4, 8, x, y, "fp32", [0], SGD)
