@@ -7,8 +7,13 @@
 // The probability tile leaves the MFMA in accumulator layout (lane = column, registers = rows); it is fed to
 // the next MFMA as its B operand straight from registers by choosing the k-order (slot (h, j) of step s is row
 // 16 s + 8 (j / 4) + 4 h + j % 4), and the matching A operand is read from LDS in that same order.
-// K / V / Q / dO tiles sit in LDS in the swizzled [row][128 B] layout of tile.h; the transposed copies
-// (V^T, K^T, Q^T, dO^T) are written from the same registers as the row-major ones (PairLoader).
+// K / V / Q / dO tiles sit in LDS row-major, [row][128 B of d], 16-byte chunks XOR-swizzled with aswz(row).
+// Fragments along d (k = d) are plain 16-byte reads; fragments of the TRANSPOSED tile (k = tile rows: V^T for
+// P V, K^T for dQ, Q^T and dO^T for dK / dV) are assembled from the same tile by transposing LDS reads
+// (ds_read_b64_tr_b16), so no transposed copy is ever written.  aswz keeps both kinds of read and the
+// row-wise tile stores free of bank conflicts: 16 lanes reading one chunk of 16 consecutive rows land in 16
+// different 16-byte slots (row & 3 picks the 64-byte quarter, row >> 2 the slot), and the four 64-byte pieces
+// of rows 4a .. 4a + 3 that a half wave touches in a transposing read fall into different quarters.
 #include "common.h"
 #include "tile.h"
 
@@ -21,24 +26,37 @@ constexpr int TILE_BYTES = TILE * ROW_BYTES;
 
 typedef Vec16<bf16_t> frag_t;
 
+__device__ __forceinline__ int aswz(int row) { return (((row >> 1) & 1) << 2) | ((row >> 2) & 3); }
+
 // standard operand fragment of k-step s: k = 16 s + 8 h .. + 8 of `row`
 __device__ __forceinline__ frag_t frag_rowk(const char *tile, int row, int s, int h) {
-    return *(const frag_t *)(tile + row * ROW_BYTES + ((((s << 1) | h) ^ swz(row)) << 4));
+    return *(const frag_t *)(tile + row * ROW_BYTES + ((((s << 1) | h) ^ aswz(row)) << 4));
 }
-// fragment in accumulator order: slots j < 4 -> k = 16 s + 4 h + j, slots j >= 4 -> k = 16 s + 8 + 4 h + (j - 4)
-__device__ __forceinline__ frag_t frag_perm(const char *tile, int row, int s, int h) {
-    const int sw = swz(row);
-    const char *base = tile + row * ROW_BYTES + (h << 3);
-    const bf16x4 lo = *(const bf16x4 *)(base + (((s << 1) ^ sw) << 4));
-    const bf16x4 hi = *(const bf16x4 *)(base + ((((s << 1) | 1) ^ sw) << 4));
-    frag_t f;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        f.v[j] = lo[j];
-        f.v[4 + j] = hi[j];
+
+// Fragment of the transposed tile in accumulator order: MFMA row = tile column col0 + lane % 32, slots j < 4 ->
+// k = tile row 16 s + 4 h + j, slots j >= 4 -> tile row 16 s + 8 + 4 h + (j - 4).  Within a group of 16 lanes
+// ds_read_b64_tr_b16 hands lane j the elements D[4 e + j / 4][j % 4], e = 0..3, of the 16 x 4 matrix whose row
+// i is the 8 bytes at lane i's address: lane i points at tile row (first row + i / 4), columns 4 (i % 4) ...
+struct TransposedReader {
+    int base, cx;              // lane constants: byte offset of (row 4 h + i / 4, within-chunk part), swizzled chunk
+    typedef short v4s __attribute__((ext_vector_type(4)));
+    typedef __attribute__((address_space(3))) v4s lds_v4s;
+    __device__ __forceinline__ TransposedReader() {
+        const int lane = threadIdx.x & 63, i = lane & 15, half = (lane >> 4) & 1, h = lane >> 5, q = i >> 2;
+        const int col = 16 * half + 4 * (i & 3);                  // + col0 (0 or 32: chunk + 0 or 4)
+        base = (4 * h + q) * ROW_BYTES + (col & 7) * 2;
+        cx = (col >> 3) ^ ((((q >> 1) & 1) << 2) | h);            // aswz(16 s + 4 h + q) = ((q >> 1) & 1) << 2 | h
     }
-    return f;
-}
+    __device__ __forceinline__ frag_t frag(const char *tile, int col0, int s) const {
+        union { v4s h[2]; bf16x8 v; } u;
+        // second read: rows + 8, whose swizzle differs by 2 (aswz low bits = (row >> 2) & 3)
+        u.h[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s *)(tile + base + 16 * s * ROW_BYTES + ((cx ^ (col0 >> 3)) << 4)));
+        u.h[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s *)(tile + base + (16 * s + 8) * ROW_BYTES + ((cx ^ (col0 >> 3) ^ 2) << 4)));
+        frag_t f;
+        f.v = u.v;
+        return f;
+    }
+};
 // 8 rows (one k-step) of an accumulator tile as a B operand
 __device__ __forceinline__ frag_t acc_to_b(const f32x16 &a, int sp) {
     frag_t f;
@@ -69,8 +87,7 @@ __device__ __forceinline__ frag_t load_row_frag(const bf16_t *row_ptr, bool vali
 }
 
 // One [64 rows][64 d] operand tile (memory [row][d], row stride ld) held as two 16-byte vectors per thread
-// (rows 2 * (t / 8) and + 1, d chunk t % 8).  The same registers fill the row-major LDS tile [row][d] and the
-// transposed one [d][row], so a tile that is needed both ways is fetched from global memory once.
+// (rows 2 * (t / 8) and + 1, d chunk t % 8) on its way into the row-major LDS tile.
 struct PairLoader {
     frag_t v[2];
     __device__ __forceinline__ void load(const bf16_t *base, int64_t ld, int64_t rows_left) {
@@ -81,18 +98,7 @@ struct PairLoader {
     __device__ __forceinline__ void store_rows(char *lds) const {
         const int c8 = threadIdx.x & 7, r0 = (threadIdx.x >> 3) * 2;
 #pragma unroll
-        for (int i = 0; i < 2; ++i) *(frag_t *)(lds + (r0 + i) * ROW_BYTES + ((c8 ^ swz(r0 + i)) << 4)) = v[i];
-    }
-    __device__ __forceinline__ void store_transposed(char *lds) const {
-        const int c8 = threadIdx.x & 7, r0 = (threadIdx.x >> 3) * 2;       // r0 is even: both rows share a 4-byte slot
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const int d = c8 * 8 + e;
-            bf16x2 pr;
-            pr[0] = v[0].v[e];
-            pr[1] = v[1].v[e];
-            *(bf16x2 *)(lds + d * ROW_BYTES + (((r0 >> 3) ^ swz(d)) << 4) + (r0 & 7) * 2) = pr;
-        }
+        for (int i = 0; i < 2; ++i) *(frag_t *)(lds + (r0 + i) * ROW_BYTES + ((c8 ^ aswz(r0 + i)) << 4)) = v[i];
     }
 };
 
@@ -119,7 +125,8 @@ template <bool CAUSAL>
 __global__ __launch_bounds__(AT_THREADS, 2) void attn_fwd_kernel(const bf16_t *qkv, const float *mask, bf16_t *out,
                                                             float *lse, int S, int H, float scale) {
     __shared__ __attribute__((aligned(16))) char Ks[TILE_BYTES];
-    __shared__ __attribute__((aligned(16))) char Vts[TILE_BYTES];
+    __shared__ __attribute__((aligned(16))) char Vs[TILE_BYTES];
+    const TransposedReader tr;
     const int E = H * HD, ld = 3 * E;
     const int blk = BlockOrder<CAUSAL>::row_block(true), bh = BlockOrder<CAUSAL>::batch_head();
     const int b = bh / H, hh = bh % H;
@@ -147,7 +154,7 @@ __global__ __launch_bounds__(AT_THREADS, 2) void attn_fwd_kernel(const bf16_t *q
     for (int kv0 = 0; kv0 < kv_end; kv0 += TILE) {
         __syncthreads();                                   // every wave is done with the previous tiles
         lk.store_rows(Ks);
-        lv.store_transposed(Vts);
+        lv.store_rows(Vs);
         __syncthreads();
         if (kv0 + TILE < kv_end) {
             lk.load(K + (int64_t)(kv0 + TILE) * ld, ld, S - kv0 - TILE);
@@ -210,7 +217,7 @@ __global__ __launch_bounds__(AT_THREADS, 2) void attn_fwd_kernel(const bf16_t *q
         for (int s = 0; s < 4; ++s) {
             const frag_t pb = acc_to_b(st[s >> 1], s & 1);
 #pragma unroll
-            for (int u = 0; u < 2; ++u) ot[u] = mma(frag_perm(Vts, u * 32 + c, s, h), pb, ot[u]);
+            for (int u = 0; u < 2; ++u) ot[u] = mma(tr.frag(Vs, u * 32, s), pb, ot[u]);
         }
     }
     const float l = lsum + __shfl_xor(lsum, 32, 64);
@@ -259,7 +266,7 @@ __global__ __launch_bounds__(AT_THREADS, 2) void attn_bwd_dq_kernel(const bf16_t
                                                                int S, int H, float scale) {
     __shared__ __attribute__((aligned(16))) char Ks[TILE_BYTES];
     __shared__ __attribute__((aligned(16))) char Vs[TILE_BYTES];
-    __shared__ __attribute__((aligned(16))) char Kts[TILE_BYTES];
+    const TransposedReader tr;
     const int E = H * HD, ld = 3 * E;
     const int blk = BlockOrder<CAUSAL>::row_block(true), bh = BlockOrder<CAUSAL>::batch_head();
     const int b = bh / H, hh = bh % H;
@@ -289,7 +296,6 @@ __global__ __launch_bounds__(AT_THREADS, 2) void attn_bwd_dq_kernel(const bf16_t
     for (int kv0 = 0; kv0 < kv_end; kv0 += TILE) {
         __syncthreads();
         lk.store_rows(Ks);
-        lk.store_transposed(Kts);
         lv.store_rows(Vs);
         __syncthreads();
         if (kv0 + TILE < kv_end) {
@@ -333,7 +339,7 @@ __global__ __launch_bounds__(AT_THREADS, 2) void attn_bwd_dq_kernel(const bf16_t
             for (int sp = 0; sp < 2; ++sp) {
                 const frag_t db = acc_to_b(dp, sp);
 #pragma unroll
-                for (int u = 0; u < 2; ++u) dqt[u] = mma(frag_perm(Kts, u * 32 + c, t * 2 + sp, h), db, dqt[u]);
+                for (int u = 0; u < 2; ++u) dqt[u] = mma(tr.frag(Ks, u * 32, t * 2 + sp), db, dqt[u]);
             }
         }
     }
@@ -360,8 +366,7 @@ __global__ __launch_bounds__(AT_THREADS, 2) void attn_bwd_dkv_kernel(const bf16_
                                                                 int S, int H, float scale) {
     __shared__ __attribute__((aligned(16))) char Qs[TILE_BYTES];
     __shared__ __attribute__((aligned(16))) char dOs[TILE_BYTES];
-    __shared__ __attribute__((aligned(16))) char Qts[TILE_BYTES];
-    __shared__ __attribute__((aligned(16))) char dOts[TILE_BYTES];
+    const TransposedReader tr;
     __shared__ __attribute__((aligned(16))) float lse_s[TILE], delta_s[TILE];
     const int E = H * HD, ld = 3 * E;
     const int blk = BlockOrder<CAUSAL>::row_block(false), bh = BlockOrder<CAUSAL>::batch_head();
@@ -390,9 +395,7 @@ __global__ __launch_bounds__(AT_THREADS, 2) void attn_bwd_dkv_kernel(const bf16_
     for (int q0 = q_begin; q0 < S; q0 += TILE) {
         __syncthreads();
         lq.store_rows(Qs);
-        lq.store_transposed(Qts);
         ldo.store_rows(dOs);
-        ldo.store_transposed(dOts);
         if (threadIdx.x < TILE) {
             const int qq = q0 + threadIdx.x;
             lse_s[threadIdx.x] = qq < S ? lse_b[qq] : INFINITY;
@@ -435,8 +438,8 @@ __global__ __launch_bounds__(AT_THREADS, 2) void attn_bwd_dkv_kernel(const bf16_
                 const frag_t pb = acc_to_b(sc, sp), db = acc_to_b(dp, sp);
 #pragma unroll
                 for (int u = 0; u < 2; ++u) {
-                    dvt[u] = mma(frag_perm(dOts, u * 32 + c, t * 2 + sp, h), pb, dvt[u]);
-                    dkt[u] = mma(frag_perm(Qts, u * 32 + c, t * 2 + sp, h), db, dkt[u]);
+                    dvt[u] = mma(tr.frag(dOs, u * 32, t * 2 + sp), pb, dvt[u]);
+                    dkt[u] = mma(tr.frag(Qs, u * 32, t * 2 + sp), db, dkt[u]);
                 }
             }
         }
