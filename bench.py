@@ -35,7 +35,7 @@ WORKLOADS = {
 }
 
 
-def build_workload(name, layers_override=None):
+def build_workload(name, layers_override=None, attn="batch", zero=False):
     import torch
     import hap_amd
     from hap_amd import models
@@ -47,7 +47,7 @@ def build_workload(name, layers_override=None):
         x = torch.randint(0, V, (B, S), generator=g)
         masked = torch.rand(B, S, generator=g) < 0.15
         y = torch.where(masked, x, torch.full_like(x, -100))
-        plan = hap_amd.ShardingPlan([RATIOS], 0, ffn="column")
+        plan = hap_amd.ShardingPlan([RATIOS], 0, ffn="column", attn=attn, zero=zero)
         meta = dict(local_batch=12, global_batch=B, seq_len=S, opt=dict(kind="adam", lr=5e-4), batch_sharded=True,
                     ratios=RATIOS)
     elif name == "lm":
@@ -134,6 +134,10 @@ def main():
     ap.add_argument("--relu-mask-in-dgrad", action="store_true",
                     help="mask the next linear's data gradient in the GEMM epilogue instead of running relu's backward "
                          "as its own pass (the step gains 0.1 ms, the GEMM brackets lose 0.5 ms)")
+    ap.add_argument("--attn", default="batch", choices=["batch", "heads"],
+                    help="bert workload only: shard attention over samples (the headline plan) or over heads (6 of 16)")
+    ap.add_argument("--zero", action="store_true",
+                    help="bert workload only: parameters stored as dim-0 shards and gathered at use")
     ap.add_argument("--gemm-plan-file", default=None,
                     help="JSON file of pinned GEMM plans: loaded instead of autotuning when it exists, written after "
                          "autotuning otherwise (a profiler run can then repeat the plan of an unprofiled run)")
@@ -154,7 +158,9 @@ def main():
     from hap_amd._lib import lib
 
     desc, dtype = WORKLOADS[args.workload]
-    gm, x, y, meta = build_workload(args.workload)
+    if (args.attn != "batch" or args.zero) and args.workload != "bert":
+        raise SystemExit("--attn / --zero are options of the bert workload")
+    gm, x, y, meta = build_workload(args.workload, attn=args.attn, zero=args.zero)
     wire = hap_amd.SyntheticWire(seed=39, scale=1.0, grad_scale=1e-3, share_shapes=True)
     ex = hap_amd.compile_program(gm, [x, y], dtype=dtype, wire=wire, rank=0, world_size=len(meta["ratios"]),
                                  overlap_wgrad=args.overlap, relu_mask_in_dgrad=args.relu_mask_in_dgrad)
@@ -232,7 +238,7 @@ def main():
         "config": {"workload": desc, "local_batch": meta["local_batch"], "global_batch": meta["global_batch"],
                    "seq_len": meta["seq_len"], "launch": "hip-graph" if graph is not None else "eager",
                    "wgrad_stream": "side" if args.overlap else "main",
-                   "gemm_plan": plan_source,
+                   "gemm_plan": plan_source, "attention_sharding": args.attn, "zero_sharded_parameters": bool(args.zero),
                    "final_loss": loss},
         "roofline": {"bound": "mfma", "kernel": "gemm_kernel (all GEMM launches of the step)",
                      "achieved": achieved, "peak": peak, "unit": "TFLOP/s", "frac": achieved / peak,
