@@ -143,8 +143,8 @@ typedef struct {
 int hapmi_gemm(const hapmi_gemm_args *args_host, hapmi_stream_t stream);
 
 /* Tuning hook for measurements: force tile configuration `tile_config` (block tile / waves: 0: 128x128 / 2x2,
- * 1: 256x256 / 2x4, 2: 384x192 / 4x2, 3: 192x256 / 2x4, 4: 256x192 / 4x2, 5: 256x128 / 4x2, 6: 128x256 / 2x4;
- * 1..6 take bf16 operands only; -1 = automatic) and `k_splits` (0 = automatic). */
+ * 1: 256x256 / 2x4, 2: 384x192 / 4x2, 3: 192x256 / 2x4, 4: 256x192 / 4x2, 5: 256x128 / 4x2, 6: 128x256 / 2x4,
+ * 7: 192x128 / 2x4; 1..7 take bf16 operands only; -1 = automatic) and `k_splits` (0 = automatic). */
 int hapmi_gemm_tuning(int tile_config, int k_splits);
 
 /* Plan table: pin the tile configuration and K split that hapmi_gemm uses for one problem signature

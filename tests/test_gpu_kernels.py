@@ -246,6 +246,35 @@ def test_optimizers_match_torch(cuda):
     assert abs(coef.item() - want) < 1e-6 * want
 
 
+@pytest.mark.parametrize("cfg", list(range(8)))
+@pytest.mark.parametrize("tA,tB", [(0, 1), (0, 0), (1, 0), (1, 1)])
+def test_gemm_every_tile_configuration_and_layout(cuda, cfg, tA, tB):
+    """bf16 operands in all four storage layouts through every tile configuration: a shape with ragged edges in
+    M, N and K (several tiles of the small configurations, one partial tile of the large ones) and a tile-aligned
+    one, bf16 and float32 outputs, bias and accumulation."""
+    from hap_amd._lib import lib
+    try:
+        lib().hapmi_gemm_tuning(cfg, 1)
+        for (M, N, K) in [(424, 520, 1000), (768, 512, 256)]:
+            g = torch.Generator().manual_seed(M + cfg)
+            A = torch.randn((K, M) if tA else (M, K), generator=g).bfloat16()
+            B = torch.randn((N, K) if tB else (K, N), generator=g).bfloat16()
+            bias = torch.randn(N, generator=g)
+            opA = A.double().t() if tA else A.double()
+            opB = B.double().t() if tB else B.double()
+            want = opA @ opB + bias.double()
+            for out_dtype in (torch.bfloat16, torch.float32):
+                C = torch.full((M, N), float("nan"), dtype=out_dtype, device=cuda)
+                ops.gemm(A.to(cuda), B.to(cuda), C, M, N, K, transA=bool(tA), transB=bool(tB), bias=bias.to(cuda))
+                close(C, want, torch.bfloat16, scale=2.0)
+            start = torch.randn(M, N, generator=g)
+            C = start.clone().to(cuda)
+            ops.gemm(A.to(cuda), B.to(cuda), C, M, N, K, transA=bool(tA), transB=bool(tB), accumulate=True)
+            close(C, want - bias.double() + start.double(), torch.bfloat16, scale=2.0)
+    finally:
+        lib().hapmi_gemm_tuning(-1, 0)
+
+
 @pytest.mark.parametrize("dtype", DT)
 @pytest.mark.parametrize("cfg", [0, 1])
 def test_gemm_split_k_and_tile_configs(cuda, dtype, cfg):
@@ -273,7 +302,7 @@ def test_gemm_split_k_and_tile_configs(cuda, dtype, cfg):
 
 
 @pytest.mark.parametrize("dtype,cfg", [(torch.float32, 0), (torch.bfloat16, 0), (torch.bfloat16, 1), (torch.bfloat16, 2),
-                                       (torch.bfloat16, 3), (torch.bfloat16, 4), (torch.bfloat16, 5), (torch.bfloat16, 6)])
+                                       (torch.bfloat16, 3), (torch.bfloat16, 4), (torch.bfloat16, 5), (torch.bfloat16, 6), (torch.bfloat16, 7)])
 @pytest.mark.parametrize("tB", [False, True])
 def test_gemm_row_sums_of_a_transposed_operand(cuda, dtype, cfg, tB):
     """a_rowsum: the weight-gradient call dW = dY^T X also returns the column sums of dY (the bias gradient),
