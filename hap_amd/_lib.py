@@ -104,10 +104,18 @@ def stop_recording():
     return rec._log if rec is not None else []
 
 
+def host_call(fn) -> None:
+    """Run ``fn()`` now and, while a launch list is being recorded, put it into the list as well: stream
+    forks / joins (event record and wait) between the library calls of a phase replay in their place."""
+    fn()
+    if _recorder is not None:
+        _recorder._log.append((fn, ()))
+
+
 def replay(calls) -> None:
     for fn, args in calls:
         rc = fn(*args)
-        if rc != 0:
+        if isinstance(rc, int) and rc != 0:                      # host calls (stream forks / joins) return nothing
             raise HapmiError(f"libhapmi error {rc} in {fn.__name__}: {_load().hapmi_last_error().decode()}")
 
 

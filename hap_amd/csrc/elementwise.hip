@@ -535,6 +535,29 @@ extern "C" int hapmi_adam_step_dev(float *param, const float *grad, float *exp_a
     return HAPMI_OK;
 }
 
+extern "C" int hapmi_adam_advance(float *state_dev, float beta1, float beta2, hapmi_stream_t stream) {
+    HAPMI_REQUIRE(state_dev, HAPMI_EINVAL, "adam_advance: null state");
+    hipLaunchKernelGGL(adam_advance_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream, state_dev, beta1, beta2);
+    HAPMI_CHECK_LAUNCH("adam_advance");
+    return HAPMI_OK;
+}
+
+extern "C" int hapmi_adam_apply_dev(float *param, const float *grad, float *exp_avg, float *exp_avg_sq, void *shadow,
+                                    int64_t n, float lr, float beta1, float beta2, float eps, const float *state_dev,
+                                    const float *grad_scale_dev, hapmi_stream_t stream) {
+    HAPMI_REQUIRE(n >= 0, HAPMI_EINVAL, "adam_apply_dev: negative size");
+    HAPMI_REQUIRE(state_dev, HAPMI_EINVAL, "adam_apply_dev: null state");
+    if (n == 0) return HAPMI_OK;
+    HAPMI_REQUIRE(param && grad && exp_avg && exp_avg_sq, HAPMI_EINVAL, "adam_apply_dev: null pointer");
+    HAPMI_REQUIRE(aligned16(param) && aligned16(grad) && aligned16(exp_avg) && aligned16(exp_avg_sq) &&
+                      (!shadow || ((uintptr_t)shadow % 8) == 0),
+                  HAPMI_EALIGN, "adam_apply_dev: misaligned buffer");
+    AdamHyper h{lr, beta1, beta2, eps, 1.f, 1.f};
+    hipLaunchKernelGGL(adam_kernel, dim3(ew_grid(hapmi_cdiv(n, 4))), dim3(EW_THREADS), 0, (hipStream_t)stream, param, grad, exp_avg, exp_avg_sq, (bf16_t *)shadow, n, h, grad_scale_dev, state_dev);
+    HAPMI_CHECK_LAUNCH("adam_apply_dev");
+    return HAPMI_OK;
+}
+
 extern "C" int hapmi_sumsq(const float *g, int64_t n, float *out, hapmi_stream_t stream) {
     HAPMI_REQUIRE(n >= 0 && out, HAPMI_EINVAL, "sumsq: bad argument");
     if (n == 0) return HAPMI_OK;

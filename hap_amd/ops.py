@@ -725,6 +725,29 @@ def adam_step_dev(param, grad, exp_avg, exp_avg_sq, shadow, lr, beta1, beta2, ep
                                     _ptr(state), _ptr(grad_scale), _stream()))
 
 
+def adam_advance(state, beta1, beta2):
+    """Advance the device-side step count / bias corrections once (see ``adam_apply_dev``)."""
+    _dev(state)
+    _need(state, 3, "adam_advance state")
+    check(lib().hapmi_adam_advance(_ptr(state), ctypes.c_float(beta1), ctypes.c_float(beta2), _stream()))
+
+
+def adam_apply_dev(param, grad, exp_avg, exp_avg_sq, shadow, lr, beta1, beta2, eps, state, grad_scale=None):
+    """Adam on one piece of the parameters with the device-side state as it is (``adam_advance`` once per step)."""
+    _dev(param, grad, exp_avg, exp_avg_sq, shadow, grad_scale, state)
+    for t_ in (grad, exp_avg, exp_avg_sq):
+        _need(t_, param.numel(), "adam_apply_dev")
+        if t_.dtype != torch.float32:
+            raise TypeError("adam_apply_dev: float32 state expected")
+    _need(shadow, param.numel(), "adam_apply_dev shadow")
+    _need(state, 3, "adam_apply_dev state")
+    if param.dtype != torch.float32 or state.dtype != torch.float32 or (shadow is not None and shadow.dtype != torch.bfloat16):
+        raise TypeError("adam_apply_dev: dtype mismatch")
+    check(lib().hapmi_adam_apply_dev(_ptr(param), _ptr(grad), _ptr(exp_avg), _ptr(exp_avg_sq), _ptr(shadow), param.numel(),
+                                     ctypes.c_float(lr), ctypes.c_float(beta1), ctypes.c_float(beta2), ctypes.c_float(eps),
+                                     _ptr(state), _ptr(grad_scale), _stream()))
+
+
 def sumsq(g, out):
     _dev(g, out)
     check(lib().hapmi_sumsq(_ptr(g), g.numel(), _ptr(out), _stream()))

@@ -289,6 +289,13 @@ int hapmi_adam_step(float *param, const float *grad, float *exp_avg, float *exp_
 int hapmi_adam_step_dev(float *param, const float *grad, float *exp_avg, float *exp_avg_sq, void *shadow, int64_t n,
                         float lr, float beta1, float beta2, float eps, float *state_dev,
                         const float *grad_scale_dev, hapmi_stream_t stream);
+/* The two halves of hapmi_adam_step_dev, for a caller that updates the parameters in several pieces per step
+ * (e.g. each piece as soon as its gradients are final, on another stream): hapmi_adam_advance advances
+ * state_dev once per step, hapmi_adam_apply_dev applies the update to one piece with the state as it is. */
+int hapmi_adam_advance(float *state_dev, float beta1, float beta2, hapmi_stream_t stream);
+int hapmi_adam_apply_dev(float *param, const float *grad, float *exp_avg, float *exp_avg_sq, void *shadow, int64_t n,
+                         float lr, float beta1, float beta2, float eps, const float *state_dev,
+                         const float *grad_scale_dev, hapmi_stream_t stream);
 /* out[0] += sum g^2 (float32 atomics over block partials; out zeroed by the caller) */
 int hapmi_sumsq(const float *g, int64_t n, float *out, hapmi_stream_t stream);
 /* torch.nn.utils.clip_grad_norm_ coefficient (worker.py:74): coef = min(1, max_norm / (sqrt(sumsq) + 1e-6)) */

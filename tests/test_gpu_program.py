@@ -318,6 +318,55 @@ def test_relu_mask_in_the_data_gradient_equals_the_separate_pass(cuda, dtype):
     assert len(a.bwd) == len(b.bwd) - 2                          # one relu-backward launch per layer gone
 
 
+@pytest.mark.parametrize("dtype,opt,zero", [("fp32", ADAM, False), ("bf16", ADAM, False), ("bf16", SGD, False),
+                                            ("bf16", ADAM, True)])
+def test_optimizer_overlapped_with_backward_equals_the_separate_step(cuda, dtype, opt, zero):
+    """train_step() updates every stretch of the flat parameter buffer on a second stream as soon as backward is
+    done with it.  Same losses and parameters as backward followed by one optimizer launch, over several steps,
+    host-launched (first step closures, later steps recorded launch lists) and replayed from a HIP graph."""
+    model = make_lm(vocab=211, S=32, d=64, H=1, F=128, layers=3)
+    x, y = lm_batch(8, 32, 211)
+
+    def build(overlap):
+        gm = hap_amd.build_program(copy.deepcopy(model), hap_amd.ShardingPlan([RATIOS4], 0, zero=zero), 8)
+        ex = hap_amd.compile_program(gm, [x, y], dtype=dtype, wire=hap_amd.SyntheticWire(seed=3, grad_scale=1e-2),
+                                     rank=0, world_size=4, overlap_optimizer=overlap, optimizer_chunk_min=1024)
+        ex.configure_optimizer(**opt)
+        return ex
+
+    a, b = build(True), build(False)
+    assert a._opt_chunks is not None and b._opt_chunks is None
+    assert sum(len(v) for v in a._opt_chunks.values()) >= 3                 # several stretches, several ready points
+    assert len(a._opt_chunks) >= 2
+    a.load_inputs(x, y)
+    b.load_inputs(x, y)
+
+    def same():
+        # Bias and embedding gradients are sums by float atomics and differ in the last bits between two runs, so
+        # the two executors drift apart at rounding level from the second step on; where a gradient is zero up to
+        # rounding (e.g. the key bias of softmax attention) Adam turns that into a step of +-lr.  Compared: the
+        # elements whose gradient is clearly non-zero.
+        torch.cuda.synchronize()
+        for n, rec in a.params.items():
+            pa, pb, g = rec["master"], b.params[n]["master"], b.params[n]["grad"]
+            clear = g.abs() > 1e-3 * g.abs().max()
+            torch.testing.assert_close(pa[clear], pb[clear], rtol=1e-4, atol=2e-6)
+            assert (pa - pb).abs().max().item() <= 2.5 * opt["lr"] * steps_done[0], n   # no element is off by more than Adam can move it
+    steps_done = [0]
+    for _ in range(3):
+        la, lb = a.train_step().item(), b.train_step().item()
+        steps_done[0] += 1
+        assert abs(la - lb) <= 1e-5 * abs(lb)
+        same()
+    ra, rb = a.capture_train_step(), b.capture_train_step()
+    for _ in range(3):
+        la, lb = ra().item(), rb().item()
+        steps_done[0] += 1
+        torch.cuda.synchronize()
+        assert abs(la - lb) <= 1e-5 * abs(lb)
+        same()
+
+
 @pytest.mark.parametrize("family", ["lm", "vit", "moe"])
 def test_recorded_launch_lists_equal_closure_execution(cuda, family):
     """By default the library calls of the first forward / backward / optimizer phase are recorded and later
