@@ -551,11 +551,19 @@ class ShardExecutor:
         store = self._new(lead + (ldc,))
         out = Val("tensor", store, shape=lead + (N,), ld=ldc if ldc != N else None, needs_grad=True)
         bias = b.meta["master"] if b is not None else None
-        self.fwd.append(lambda: ops.gemm(xt, w.t, store, M, N, K, transB=True, lda=lda, ldc=ldc, bias=bias))
+        # a relu that is the only reader of the result is applied by the GEMM's epilogue; its backward masks the
+        # incoming gradient with the stored (activated) output
+        fuse = self._wants_fused_relu(node) and ldc == N
+        if fuse:
+            out.meta["fused_act"] = "relu"
+        self.fwd.append(lambda: ops.gemm(xt, w.t, store, M, N, K, transB=True, lda=lda, ldc=ldc, bias=bias,
+                                         act="relu" if fuse else None))
 
         def emit():
             if out.grad is None:
                 return
+            if fuse:
+                self._relu_backward_through(out)
             dy = out.grad
             gw, accw = self._param_grad_slot(w)
             gb, accb = self._param_grad_slot(b) if b is not None else (None, False)
