@@ -923,6 +923,15 @@ class ShardExecutor:
                 out[src] = self.wire.recv(tag, direction, src, shape, dtype or self.cdt, self.dev, reduction=reduction)
         return out
 
+    def _announce(self, tag, direction, rank, W, buffer_for, sink: List[Callable]):
+        """Tell the wire which static buffer holds the message for every peer; a callable it returns runs in
+        every step right after the preparation kernels (enqueued just before this call) of the collective."""
+        for dst in range(W):
+            if dst != rank:
+                hook = self.wire.send(tag, direction, dst, buffer_for(dst))
+                if hook is not None:
+                    sink.append(hook)
+
     def _emit_gather(self, tag, direction, x_t, dim, L, rank, sink: List[Callable]):
         """pad own shard -> [wire] -> cut pads and concatenate.  Returns the full tensor."""
         m, W = max(L), len(L)
@@ -932,6 +941,7 @@ class ShardExecutor:
         slices = [own if s == rank else peers[s] for s in range(W)]
         full = self._new(ops._with_dim(x_t.shape, dim, sum(L)), x_t.dtype)
         sink.append(lambda: (ops.pad_rows(x_t, dim, m, own), ops.unpad_concat(slices, L, dim, full)))
+        self._announce(tag, direction, rank, W, lambda dst: own, sink)        # the padded shard goes to every peer
         return full
 
     def _emit_scatter(self, tag, direction, full_t, dim, L, rank, sink: List[Callable], out_t=None):
@@ -944,6 +954,7 @@ class ShardExecutor:
         contribs = [c for c in contribs if c is not None]
         out = out_t if out_t is not None else self._new(ops._with_dim(full_t.shape, dim, L[rank]), full_t.dtype)
         sink.append(lambda: (ops.split_pad(full_t, L, dim, m, sent), ops.ragged_reduce(contribs, dim, 0, L[rank], out)))
+        self._announce(tag, direction, rank, W, lambda dst: sent[dst], sink)  # the padded piece that rank dst reduces
         return out
 
     def _all_gather(self, node):
@@ -1028,6 +1039,7 @@ class ShardExecutor:
             sink.append(lambda: ops.concat_rows(parts, cat_dim, out, act))
         else:
             sink.append(lambda: (ops.split_rows(x_t, split_L, split_dim, pieces), ops.concat_rows(parts, cat_dim, out, act)))
+        self._announce(tag, direction, rank, W, lambda dst: pieces[dst], sink)
         return out
 
     def _all_to_all(self, node):
@@ -1057,6 +1069,7 @@ class ShardExecutor:
         contribs = [c.view(1, -1) for c in contribs if c is not None]
         out = out_t if out_t is not None else self._new(x_t.shape, x_t.dtype)
         n = x_t.numel()
+        self._announce(tag, direction, rank, W, lambda dst: x_t, sink)         # before the sum (it may run in place)
         sink.append(lambda: ops.ragged_reduce(contribs, 1, 0, n, out.view(1, -1)))
         return out
 

@@ -29,6 +29,15 @@ class Wire:
     def recv(self, tag: str, direction: str, src: int, shape, dtype, device) -> Optional[torch.Tensor]:
         raise NotImplementedError
 
+    def send(self, tag: str, direction: str, dst: int, buffer: torch.Tensor) -> None:
+        """Called once, when the program is compiled, for every message this rank sends: ``buffer`` is the static
+        GPU tensor that holds the message for rank ``dst`` after the local preparation kernels of collective
+        ``tag`` have run in a step.  A transport would post its sends from these buffers.  May return a callable:
+        the executor then calls it in every step right after those kernels are enqueued (the point at which the
+        message is complete; later launches of the step may reuse the buffer).  The stand-ins send nothing;
+        ``ReplayWire`` snapshots the messages so that tests can compare them with the recorded run."""
+        return None
+
 
 class SilentWire(Wire):
     def __init__(self, gather_fill: float = 0.0):
@@ -70,6 +79,12 @@ class ReplayWire(Wire):
     def __init__(self, log: dict, rank: int):
         self.log, self.rank = log, rank
         self._cache: Dict[Tuple, torch.Tensor] = {}
+        self.sent: Dict[Tuple, torch.Tensor] = {}       # (tag, direction, dst) -> copy of the message this rank sent last
+
+    def send(self, tag, direction, dst, buffer):
+        def snapshot():
+            self.sent[(tag, direction, dst)] = buffer.detach().clone()
+        return snapshot
 
     def recv(self, tag, direction, src, shape, dtype, device, reduction: bool = False):
         key = (tag, direction, src)

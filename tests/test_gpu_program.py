@@ -15,6 +15,27 @@ from helpers import (RATIOS4, RATIOS_E, joint_cpu, lm_batch, make_lm, make_moe, 
 pytestmark = pytest.mark.gpu
 
 
+def _check_sent_messages(ex, log, rank, dtype):
+    """What this rank hands to the wire (padded shards, padded pieces, exchange pieces, all_reduce addends) is what
+    the recorded run of all ranks sent from this rank: layouts exactly (pads included), values within the
+    tolerance of the dtype."""
+    torch.cuda.synchronize()
+    sent = ex.wire.sent
+    tol = 1e-4 if dtype == "fp32" else 3e-2
+    checked = 0
+    for (tag, direction, dst), buf in sent.items():
+        want = log[(tag, direction)][rank][dst].float()
+        got = buf.float().cpu()
+        assert got.shape == want.shape, (tag, direction, dst)
+        finite = torch.isfinite(want)                            # the oracle poisons pads with NaN
+        assert torch.isfinite(got[finite]).all(), (tag, direction, dst)
+        if finite.any() and want[finite].abs().max() > 0:
+            err = ((got[finite] - want[finite]).norm() / want[finite].norm()).item()
+            assert err < tol, (tag, direction, dst, err)
+        checked += 1
+    assert checked == len(sent)
+
+
 def _gpu_rank(model, ratios, rank, B, x, y, log, dtype, opt, **kw):
     m = copy.deepcopy(model)
     plan = hap_amd.ShardingPlan([list(ratios)], rank, ffn=kw.get("ffn", "column"), zero=kw.get("zero", False),
@@ -26,6 +47,7 @@ def _gpu_rank(model, ratios, rank, B, x, y, log, dtype, opt, **kw):
     ex.configure_optimizer(**opt)
     loss = ex.forward(x, y)
     ex.backward()
+    _check_sent_messages(ex, log, rank, dtype)
     grads = {n: rec["grad"].clone().cpu() for n, rec in ex.params.items()}
     ex.step()
     torch.cuda.synchronize()
