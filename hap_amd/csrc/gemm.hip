@@ -27,6 +27,8 @@ HAPMI_GEMM_DECLARE_CFG(4);
 HAPMI_GEMM_DECLARE_CFG(5);
 HAPMI_GEMM_DECLARE_CFG(6);
 HAPMI_GEMM_DECLARE_CFG(7);
+HAPMI_GEMM_DECLARE_CFG(8);
+HAPMI_GEMM_DECLARE_CFG(9);
 
 namespace {
 
@@ -35,8 +37,8 @@ struct TileCfg {
     int bm, bn, wm, wn;
 };
 constexpr TileCfg kCfg[] = {{128, 128, 2, 2}, {256, 256, 2, 4}, {384, 192, 4, 2}, {192, 256, 2, 4}, {256, 192, 4, 2},
-                             {256, 128, 4, 2}, {128, 256, 2, 4}, {192, 128, 2, 4}};
-constexpr int kNumCfg = 8;
+                             {256, 128, 4, 2}, {128, 256, 2, 4}, {192, 128, 2, 4}, {256, 128, 2, 2}, {128, 192, 4, 2}};
+constexpr int kNumCfg = 10;
 constexpr int kNumCU = 256;
 int g_force_cfg = -1;
 int g_force_splits = 0;
@@ -192,6 +194,8 @@ int launch_typed(GemmParams &p, int transA, int transB, int64_t batch, hipStream
         case 5: rc = hapmi_gemm_launch_cfg5(p, in_dtype, out_dtype, transA, transB, batch, st); break;
         case 6: rc = hapmi_gemm_launch_cfg6(p, in_dtype, out_dtype, transA, transB, batch, st); break;
         case 7: rc = hapmi_gemm_launch_cfg7(p, in_dtype, out_dtype, transA, transB, batch, st); break;
+        case 8: rc = hapmi_gemm_launch_cfg8(p, in_dtype, out_dtype, transA, transB, batch, st); break;
+        case 9: rc = hapmi_gemm_launch_cfg9(p, in_dtype, out_dtype, transA, transB, batch, st); break;
         default: rc = hapmi_gemm_launch_cfg0(p, in_dtype, out_dtype, transA, transB, batch, st);
     }
     if (rc || p.splits <= 1) return rc;

@@ -3,6 +3,6 @@
 
 HAPMI_GEMM_DECLARE_CFG(6) {
     if (in_dtype != HAPMI_BF16) return hapmi_set_error(HAPMI_EINVAL, "gemm: tile configuration 6 takes bf16 operands only");
-    if (out_dtype == HAPMI_BF16) return launch_cfg<bf16_t, bf16_t, 128, 256, 2, 4>(p, transA, transB, batch, st);
-    return launch_cfg<bf16_t, float, 128, 256, 2, 4>(p, transA, transB, batch, st);
+    if (out_dtype == HAPMI_BF16) return launch_cfg<bf16_t, bf16_t, 128, 256, 2, 4, 3>(p, transA, transB, batch, st);
+    return launch_cfg<bf16_t, float, 128, 256, 2, 4, 3>(p, transA, transB, batch, st);
 }

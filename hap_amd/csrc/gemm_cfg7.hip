@@ -4,6 +4,6 @@
 
 HAPMI_GEMM_DECLARE_CFG(7) {
     if (in_dtype != HAPMI_BF16) return hapmi_set_error(HAPMI_EINVAL, "gemm: tile configuration 7 takes bf16 operands only");
-    if (out_dtype == HAPMI_BF16) return launch_cfg<bf16_t, bf16_t, 192, 128, 2, 4>(p, transA, transB, batch, st);
-    return launch_cfg<bf16_t, float, 192, 128, 2, 4>(p, transA, transB, batch, st);
+    if (out_dtype == HAPMI_BF16) return launch_cfg<bf16_t, bf16_t, 192, 128, 2, 4, 3>(p, transA, transB, batch, st);
+    return launch_cfg<bf16_t, float, 192, 128, 2, 4, 3>(p, transA, transB, batch, st);
 }

@@ -60,9 +60,9 @@ __device__ __forceinline__ float apply_act(float v, int act) {
     return v;
 }
 
-template <typename TI, typename TO, int BM, int BN, int WAVES_M, int WAVES_N, bool A_KMAJOR, bool B_KMAJOR>
-// four-wave tiles are meant to run two blocks per CU: keep them within 256 registers
-__global__ __launch_bounds__(WAVES_M *WAVES_N * 64, (WAVES_M * WAVES_N <= 4 ? 2 : 1)) void gemm_kernel(GemmParams p) {
+template <typename TI, typename TO, int BM, int BN, int WAVES_M, int WAVES_N, bool A_KMAJOR, bool B_KMAJOR, int NSTAGES>
+// the four-wave 128 x 128 tile is meant to run two blocks per CU: keep it within 256 registers
+__global__ __launch_bounds__(WAVES_M *WAVES_N * 64, ((WAVES_M * WAVES_N <= 4 && BM * BN <= 128 * 128) ? 2 : 1)) void gemm_kernel(GemmParams p) {
     constexpr int THREADS = WAVES_M * WAVES_N * 64;
     constexpr int EPV = 16 / sizeof(TI);
     constexpr int BK = ROW_BYTES / sizeof(TI);
@@ -72,8 +72,8 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, (WAVES_M * WAVES_N <= 4 ? 2 
     constexpr int A_BYTES = BM * ROW_BYTES, B_BYTES = BN * ROW_BYTES;
 
     extern __shared__ __attribute__((aligned(16))) char smem[];
-    char *As = smem;                                              // [2][BM][128 B]
-    char *Bs = smem + 2 * A_BYTES;                                // [2][BN][128 B]
+    char *As = smem;                                              // [NSTAGES][BM][128 B]
+    char *Bs = smem + NSTAGES * A_BYTES;                          // [NSTAGES][BN][128 B]
 
     // tile mapping: blocks go round-robin over the 8 XCDs; give each XCD a contiguous range of tiles and
     // walk it in columns of 8 m-tiles so that concurrently running tiles share A rows / B columns in L2
@@ -229,6 +229,30 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, (WAVES_M * WAVES_N <= 4 ? 2 
             if constexpr (!B_DIRECT) lb.store(Bs + buf * B_BYTES);
             __builtin_amdgcn_s_waitcnt(0x0F70);                   // vmcnt(0): this wave's direct loads have landed
         };
+        if constexpr (NSTAGES == 3) {
+            // Three buffers, two k-tiles in flight: a k-tile's loads are issued two iterations before it is
+            // multiplied, so their round trip (longer than one iteration of a one-block-per-CU tile) is covered.
+            // Both operands go global -> LDS directly (no registers involved); a wave's loads complete in order,
+            // so tile kt has landed once at most the loads of tile kt + 1 are outstanding.
+            static_assert(A_DIRECT && B_DIRECT, "three stages need direct loads for both operands");
+            constexpr int LPT = decltype(la)::LOADS_PER_TILE + decltype(lb)::LOADS_PER_TILE;
+            static_assert(LPT < 64, "vmcnt holds 6 bits");
+            constexpr int WAIT_NEXT = (LPT & 15) | 0x0F70 | ((LPT >> 4) << 14);
+            issue_tile(kt0, 0);
+            if (kt0 + 1 < kt_end) issue_tile(kt0 + 1, 1);
+            int cur = 0;
+            for (int kt = kt0; kt < kt_end; ++kt) {
+                if (kt + 1 < kt_end) __builtin_amdgcn_s_waitcnt(WAIT_NEXT);
+                else __builtin_amdgcn_s_waitcnt(0x0F70);
+                __syncthreads();                                  // tile kt is complete; everyone is done with tile kt - 1
+                const int nxt2 = cur == 0 ? 2 : cur - 1;          // (cur + 2) % 3: the buffer of tile kt - 1
+                if (kt + 2 < kt_end) issue_tile(kt + 2, nxt2);
+                if (do_rs && kt % p.tiles_n == tn) rs_add_lds(As + cur * A_BYTES);
+                compute_tile(As + cur * A_BYTES, Bs + cur * B_BYTES);
+                cur = cur == 2 ? 0 : cur + 1;
+            }
+            __syncthreads();
+        } else {
         issue_tile(kt0, 0);
         commit_tile(0, kt0);
         __syncthreads();
@@ -239,6 +263,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, (WAVES_M * WAVES_N <= 4 ? 2 
             compute_tile(As + cur * A_BYTES, Bs + cur * B_BYTES);
             if (kt + 1 < kt_end) commit_tile(cur ^ 1, kt + 1);
             __syncthreads();
+        }
         }
     }
 
@@ -336,7 +361,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, (WAVES_M * WAVES_N <= 4 ? 2 
         constexpr int G16 = WTN / 8;
         constexpr int NG = 32 * G16 / 64;
         static_assert((32 * G16) % 64 == 0, "wave tile width must be a multiple of 16");
-        static_assert(32 * SROWH * NWAVES <= 2 * (A_BYTES + B_BYTES), "epilogue staging does not fit the operand LDS");
+        static_assert(32 * SROWH * NWAVES <= NSTAGES * (A_BYTES + B_BYTES), "epilogue staging does not fit the operand LDS");
         char *stage = smem + wave * (32 * SROWH);
         int soff[NG], goff[NG];                                   // staged / global offsets of this lane's groups
 #pragma unroll
@@ -399,7 +424,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, (WAVES_M * WAVES_N <= 4 ? 2 
     }
 
     constexpr int SROW = WTN * 4 + 16;                            // staged row: WTN floats + 16 B (bank spread)
-    static_assert(32 * SROW * NWAVES <= 2 * (A_BYTES + B_BYTES), "epilogue staging does not fit the operand LDS");
+    static_assert(32 * SROW * NWAVES <= NSTAGES * (A_BYTES + B_BYTES), "epilogue staging does not fit the operand LDS");
     char *stage = smem + wave * (32 * SROW);
     constexpr int QPR = WTN / 4;                                  // float4 groups per staged row
     constexpr int NQ = 32 * QPR / 64;
@@ -495,16 +520,16 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, (WAVES_M * WAVES_N <= 4 ? 2 
     }
 }
 
-template <typename TI, typename TO, int BM, int BN, int WM, int WN>
+template <typename TI, typename TO, int BM, int BN, int WM, int WN, int NSTAGES = 2>
 int launch_cfg(const GemmParams &p, int transA, int transB, int64_t batch, hipStream_t st) {
     GemmParams q = p;
     q.tiles_m = (int)hapmi_cdiv(p.M, BM);
     q.tiles_n = (int)hapmi_cdiv(p.N, BN);
     dim3 grid((unsigned)(q.tiles_m * q.tiles_n), (unsigned)q.splits, (unsigned)batch), block(WM * WN * 64);
-    const size_t smem = (size_t)2 * (BM + BN) * ROW_BYTES;
+    const size_t smem = (size_t)NSTAGES * (BM + BN) * ROW_BYTES;
 #define HAPMI_GEMM_LAUNCH(AK, BK_)                                                                        \
     do {                                                                                                  \
-        auto kern = gemm_kernel<TI, TO, BM, BN, WM, WN, AK, BK_>;                                         \
+        auto kern = gemm_kernel<TI, TO, BM, BN, WM, WN, AK, BK_, NSTAGES>;                                       \
         if (smem > 64 * 1024) {                                                                           \
             static bool raised = false;                                                                   \
             if (!raised) {                                                                                \

@@ -61,6 +61,7 @@ template <typename TI, int ROWS, int THREADS, bool KMAJOR> struct TileLoader {
     // l / 8, physical chunk l % 8, so it fetches the logical chunk (l % 8) ^ swz(row) of that row.
     static constexpr int NWAVES = THREADS / 64;
     static constexpr int PASSES_D = ROWS / (8 * NWAVES);
+    static constexpr int LOADS_PER_TILE = PASSES_D;               // direct-load instructions per wave and tile
     int doff[KMAJOR ? (PASSES_D > 0 ? PASSES_D : 1) : 1];
 
     __device__ __forceinline__ void init_direct(int64_t ld, int64_t rows_left) {
@@ -191,6 +192,7 @@ template <int ROWS, int THREADS> struct TrTile {
     static constexpr int LINE = ROWS * 2;                         // bytes per k line
     static constexpr int CHUNKS = BK * CPR;
     static constexpr int PASSES = CHUNKS / THREADS;
+    static constexpr int LOADS_PER_TILE = PASSES;                 // direct-load instructions per wave and tile
     static_assert(ROWS % 64 == 0 && CHUNKS % THREADS == 0, "tile does not divide over the block");
     static_assert(CPR % 16 == 0 || CPR % 16 == 8, "no bank swizzle for this line length");
     typedef short v4s __attribute__((ext_vector_type(4)));

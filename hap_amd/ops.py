@@ -342,7 +342,7 @@ def gemm(A: torch.Tensor, B: torch.Tensor, C: torch.Tensor, M: int, N: int, K: i
 
 _gemm_log = None
 _SPLIT_MENU = (1, 2, 3, 4, 5, 6, 7, 8, 10, 12, 16)
-_N_TILE_CONFIGS = 8
+_N_TILE_CONFIGS = 10
 
 
 def record_gemms(on: bool):

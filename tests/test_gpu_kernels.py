@@ -246,7 +246,7 @@ def test_optimizers_match_torch(cuda):
     assert abs(coef.item() - want) < 1e-6 * want
 
 
-@pytest.mark.parametrize("cfg", list(range(8)))
+@pytest.mark.parametrize("cfg", list(range(10)))
 @pytest.mark.parametrize("tA,tB", [(0, 1), (0, 0), (1, 0), (1, 1)])
 def test_gemm_every_tile_configuration_and_layout(cuda, cfg, tA, tB):
     """bf16 operands in all four storage layouts through every tile configuration: a shape with ragged edges in
@@ -302,7 +302,7 @@ def test_gemm_split_k_and_tile_configs(cuda, dtype, cfg):
 
 
 @pytest.mark.parametrize("dtype,cfg", [(torch.float32, 0), (torch.bfloat16, 0), (torch.bfloat16, 1), (torch.bfloat16, 2),
-                                       (torch.bfloat16, 3), (torch.bfloat16, 4), (torch.bfloat16, 5), (torch.bfloat16, 6), (torch.bfloat16, 7)])
+                                       (torch.bfloat16, 3), (torch.bfloat16, 4), (torch.bfloat16, 5), (torch.bfloat16, 6), (torch.bfloat16, 7), (torch.bfloat16, 8), (torch.bfloat16, 9)])
 @pytest.mark.parametrize("tB", [False, True])
 def test_gemm_row_sums_of_a_transposed_operand(cuda, dtype, cfg, tB):
     """a_rowsum: the weight-gradient call dW = dY^T X also returns the column sums of dY (the bias gradient),
