@@ -24,9 +24,38 @@ struct SegmentList {
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 template <typename V> struct ActNone {
+    static constexpr bool MASKED = false;
     __device__ __forceinline__ V operator()(V v) const { return v; }
 };
+// relu's backward fused into a copy: the element is kept where the forward output, which lies `delta` bytes from
+// the source element, is > 0 (NaN counts as not positive, as `y > 0.f` does)
+struct ReluBwdBf16 {
+    static constexpr bool MASKED = true;
+    int64_t delta;
+    __device__ __forceinline__ u32x4 operator()(u32x4 v, u32x4 y) const {
+        u32x4 r;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t lo = y[i] & 0xffffu, hi = y[i] >> 16;
+            const uint32_t klo = (lo - 1u) < 0x7f80u ? 0xffffu : 0u;          // 0x0001..0x7f80: positive, not NaN
+            const uint32_t khi = (hi - 1u) < 0x7f80u ? 0xffff0000u : 0u;
+            r[i] = v[i] & (klo | khi);
+        }
+        return r;
+    }
+};
+struct ReluBwdF32 {
+    static constexpr bool MASKED = true;
+    int64_t delta;
+    __device__ __forceinline__ u32x4 operator()(u32x4 v, u32x4 y) const {
+        u32x4 r;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) r[i] = (y[i] - 1u) < 0x7f800000u ? v[i] : 0u;
+        return r;
+    }
+};
 struct ReluBf16 {
+    static constexpr bool MASKED = false;
     __device__ __forceinline__ u32x4 operator()(u32x4 v) const {
         // a bf16 is negative iff its sign bit is set; -0.0 -> +0.0 matches relu's value
         u32x4 r;
@@ -40,6 +69,7 @@ struct ReluBf16 {
     }
 };
 struct ReluF32 {
+    static constexpr bool MASKED = false;
     __device__ __forceinline__ u32x4 operator()(u32x4 v) const {
         u32x4 r;
 #pragma unroll
@@ -58,7 +88,7 @@ __global__ __launch_bounds__(COPY_THREADS) void segment_copy_kernel(SegmentList 
     const uint64_t total = per_row * (uint64_t)s.rows;
     const uint64_t step = (uint64_t)gridDim.x * COPY_THREADS * COPY_UNROLL;
     for (uint64_t base = (uint64_t)blockIdx.x * COPY_THREADS * COPY_UNROLL + threadIdx.x; base < total; base += step) {
-        V v[COPY_UNROLL];
+        V v[COPY_UNROLL], y[Act::MASKED ? COPY_UNROLL : 1];
         uint64_t doff[COPY_UNROLL];
         bool ok[COPY_UNROLL];
 #pragma unroll
@@ -77,15 +107,25 @@ __global__ __launch_bounds__(COPY_THREADS) void segment_copy_kernel(SegmentList 
                 col = c - row * per_row;
             }
             doff[u] = row * (uint64_t)s.dst_stride + col * sizeof(V);
-            if (ok[u]) v[u] = *(const V *)(s.src + row * (uint64_t)s.src_stride + col * sizeof(V));
+            const char *from = s.src + row * (uint64_t)s.src_stride + col * sizeof(V);
+            if (ok[u]) v[u] = *(const V *)from;
+            if constexpr (Act::MASKED)
+                if (ok[u]) y[u] = *(const V *)(from + act.delta);
         }
 #pragma unroll
-        for (int u = 0; u < COPY_UNROLL; ++u)
-            if (ok[u]) *(V *)(s.dst + doff[u]) = act(v[u]);
+        for (int u = 0; u < COPY_UNROLL; ++u) {
+            if (!ok[u]) continue;
+            if constexpr (Act::MASKED) *(V *)(s.dst + doff[u]) = act(v[u], y[u]);
+            else *(V *)(s.dst + doff[u]) = act(v[u]);
+        }
     }
 }
 
-int launch_segments(const SegmentList &list, int act, int dtype, hipStream_t stream, const char *name) {
+// act: HAPMI_ACT_NONE, HAPMI_ACT_RELU (applied to the copied elements), or ACT_RELU_BWD (elements kept where the
+// element `mask_delta` bytes after the source element is > 0)
+constexpr int ACT_RELU_BWD = -1;
+int launch_segments(const SegmentList &list, int act, int dtype, hipStream_t stream, const char *name,
+                    int64_t mask_delta = 0) {
     if (list.n == 0) return HAPMI_OK;
     // widest vector that divides every address, stride and row length
     uint64_t bits = 0;
@@ -108,7 +148,13 @@ int launch_segments(const SegmentList &list, int act, int dtype, hipStream_t str
     if (gx > cap) gx = cap;
     if (gx < 1) gx = 1;
     dim3 grid((unsigned)gx, (unsigned)list.n), block(COPY_THREADS);
-    if (act != HAPMI_ACT_NONE) {
+    if (act == ACT_RELU_BWD) {
+        HAPMI_REQUIRE(vec == 16 && mask_delta % 16 == 0, HAPMI_EALIGN, "%s: the fused relu backward needs 16-byte aligned pieces", name);
+        if (dtype == HAPMI_BF16)
+            hipLaunchKernelGGL((segment_copy_kernel<u32x4, ReluBwdBf16>), grid, block, 0, stream, list, ReluBwdBf16{mask_delta});
+        else
+            hipLaunchKernelGGL((segment_copy_kernel<u32x4, ReluBwdF32>), grid, block, 0, stream, list, ReluBwdF32{mask_delta});
+    } else if (act != HAPMI_ACT_NONE) {
         HAPMI_REQUIRE(act == HAPMI_ACT_RELU, HAPMI_EINVAL, "%s: only relu can be fused into a concat", name);
         HAPMI_REQUIRE(vec == 16, HAPMI_EALIGN, "%s: fused activation needs 16-byte aligned pieces", name);
         if (dtype == HAPMI_BF16)
@@ -250,6 +296,29 @@ extern "C" int hapmi_split_rows(const void *src, void *const *pieces, const int6
         off += lengths[i];
     }
     return launch_segments(list, HAPMI_ACT_NONE, 0, (hipStream_t)stream, "split_rows");
+}
+
+extern "C" int hapmi_split_rows_relu_bwd(const void *src, const void *fwd_out, void *const *pieces,
+                                         const int64_t *lengths, int n_ranks, int64_t outer, int64_t inner_bytes,
+                                         int dtype, hapmi_stream_t stream) {
+    int64_t total;
+    int rc = check_lengths(lengths, n_ranks, &total, "split_rows_relu_bwd");
+    if (rc) return rc;
+    HAPMI_REQUIRE(outer >= 0 && inner_bytes > 0 && pieces, HAPMI_EINVAL, "split_rows_relu_bwd: bad argument");
+    HAPMI_REQUIRE(hapmi_dtype_ok(dtype), HAPMI_EINVAL, "split_rows_relu_bwd: bad dtype %d", dtype);
+    SegmentList list;
+    list.n = 0;
+    int64_t off = 0;
+    for (int i = 0; i < n_ranks; ++i) {
+        if (lengths[i] > 0 && outer > 0 && pieces[i]) {
+            HAPMI_REQUIRE(src && fwd_out, HAPMI_EINVAL, "split_rows_relu_bwd: null pointer");
+            list.seg[list.n++] = {(const char *)src + off * inner_bytes, (char *)pieces[i], outer,
+                                  lengths[i] * inner_bytes, total * inner_bytes, lengths[i] * inner_bytes};
+        }
+        off += lengths[i];
+    }
+    return launch_segments(list, ACT_RELU_BWD, dtype, (hipStream_t)stream, "split_rows_relu_bwd",
+                           (int64_t)((const char *)fwd_out - (const char *)src));
 }
 
 extern "C" int hapmi_concat_rows(const void *const *pieces, const int64_t *lengths, int n_ranks, void *dst,

@@ -60,7 +60,8 @@ class ShardExecutor:
     def __init__(self, gm: torch.fx.GraphModule, example_inputs, dtype: str = "fp32", wire: Optional[Wire] = None,
                  rank: int = 0, world_size: int = 1, device: str = "cuda:0", fused_attention: bool = True,
                  overlap_wgrad: bool = False, launch_lists: bool = True, relu_mask_in_dgrad: bool = False,
-                 overlap_optimizer: bool = False, optimizer_chunk_min: int = 1 << 20):
+                 overlap_optimizer: bool = False, optimizer_chunk_min: int = 1 << 20,
+                 relu_bwd_in_split: bool = True):
         """``example_inputs``: the program's inputs (global batch) as tensors or shapes; activations are
         sized from them.  ``rank`` / ``world_size`` are only needed by all_reduce / replicate, whose node
         forms do not carry them (collectives.py:86, 182)."""
@@ -97,6 +98,9 @@ class ShardExecutor:
         # step replayed from a HIP graph, so it is off by default.
         self.overlap_wgrad = overlap_wgrad
         self.relu_mask_in_dgrad = relu_mask_in_dgrad
+        # relu's backward behind an all_to_all rides on the copying split of the backward exchange (one pass over
+        # the gradient less per layer); False keeps the separate pass, for comparison
+        self.relu_bwd_in_split = relu_bwd_in_split
         # Optional: train_step() applies the optimizer to each stretch of the flat parameter buffer as soon as
         # backward has finished with it, on a second stream.  Measured on the BERT-large shard the step takes the
         # same time either way (27.1 against 27.0 ms): the GEMMs that run next to the update slow down by what the
@@ -1017,7 +1021,10 @@ class ShardExecutor:
         self._tape.append(emit)
         return out
 
-    def _emit_exchange(self, tag, direction, x_t, split_dim, cat_dim, split_L, cat_L, rank, sink, act=None):
+    def _emit_exchange(self, tag, direction, x_t, split_dim, cat_dim, split_L, cat_L, rank, sink, act=None,
+                       relu_of=None):
+        """The local half of an all_to_all.  ``act``: activation applied while concatenating.  ``relu_of``: forward
+        output of a relu whose backward is applied to ``x_t`` while splitting (only for a split that copies)."""
         W = len(split_L)
         # pieces along the slowest dimension are contiguous ranges of the input: views, as torch.split gives the
         # reference (collectives.py:156); any other dimension needs the strided copy
@@ -1038,9 +1045,22 @@ class ShardExecutor:
         if views:
             sink.append(lambda: ops.concat_rows(parts, cat_dim, out, act))
         else:
-            sink.append(lambda: (ops.split_rows(x_t, split_L, split_dim, pieces), ops.concat_rows(parts, cat_dim, out, act)))
+            sink.append(lambda: (ops.split_rows(x_t, split_L, split_dim, pieces, relu_of=relu_of),
+                                 ops.concat_rows(parts, cat_dim, out, act)))
         self._announce(tag, direction, rank, W, lambda dst: pieces[dst], sink)
         return out
+
+    @staticmethod
+    def _split_can_mask(grad, fwd_out, dim, lengths):
+        """The masked split works on 16-byte vectors: every piece's rows and both base addresses must be aligned."""
+        if not (grad.is_contiguous() and fwd_out.is_contiguous() and grad.shape == fwd_out.shape and grad.dtype == fwd_out.dtype):
+            return False
+        inner = 1
+        for d in grad.shape[dim + 1:]:
+            inner *= d
+        es = grad.element_size()
+        return (grad.data_ptr() % 16 == 0 and fwd_out.data_ptr() % 16 == 0
+                and all((l * inner * es) % 16 == 0 for l in lengths))
 
     def _all_to_all(self, node):
         x, sd, cd = self._val(node.args[0]), node.args[1], node.args[2]
@@ -1056,9 +1076,14 @@ class ShardExecutor:
         def emit():
             if out.grad is None or not x.needs_grad:
                 return
-            if fuse:
+            # the backward exchange splits along the forward's concat dimension; where that split copies, relu's
+            # backward rides on the copy instead of a pass of its own over the gradient
+            in_split = (fuse and self.relu_bwd_in_split and not out.meta.get("relu_bwd_done") and not (cd == 0 and out.grad.is_contiguous())
+                        and self._split_can_mask(out.grad, out.t, cd, cL))
+            if fuse and not in_split:
                 self._relu_backward_through(out)
-            g = self._emit_exchange(node.name, "bwd", out.grad, cd, sd, cL, sL, rank, self.bwd)
+            g = self._emit_exchange(node.name, "bwd", out.grad, cd, sd, cL, sL, rank, self.bwd,
+                                    relu_of=out.t if in_split else None)
             self._accumulate_into(x, g)
         self._tape.append(emit)
         return out

@@ -165,7 +165,10 @@ def place_rows(src: torch.Tensor, dst: torch.Tensor, dim: int, offset: int) -> t
 
 
 def split_rows(src: torch.Tensor, lengths: Sequence[int], dim: int,
-               outs: Optional[Sequence[Optional[torch.Tensor]]] = None) -> List[torch.Tensor]:
+               outs: Optional[Sequence[Optional[torch.Tensor]]] = None,
+               relu_of: Optional[torch.Tensor] = None) -> List[torch.Tensor]:
+    """Pieces of ``src`` along ``dim``; with ``relu_of`` (a relu's forward output of src's shape) the pieces
+    are those of ``src * (relu_of > 0)``."""
     _dev(src)
     assert src.is_contiguous()
     outer, total, inner = _oli(src.shape, dim)
@@ -177,6 +180,12 @@ def split_rows(src: torch.Tensor, lengths: Sequence[int], dim: int,
             _dev(o)
             _need(o, outer * l * inner, "split_rows piece")
     if src.numel() == 0:
+        return list(outs)
+    if relu_of is not None:
+        _dev(relu_of)
+        assert relu_of.is_contiguous() and relu_of.shape == src.shape and relu_of.dtype == src.dtype
+        check(lib().hapmi_split_rows_relu_bwd(_ptr(src), _ptr(relu_of), _ptrs(outs), _i64(lengths), len(lengths),
+                                              outer, inner * src.element_size(), dtype_code(src), _stream()))
         return list(outs)
     check(lib().hapmi_split_rows(_ptr(src), _ptrs(outs), _i64(lengths), len(lengths), outer,
                                  inner * src.element_size(), _stream()))

@@ -84,6 +84,14 @@ int hapmi_place_rows(const void *src, void *dst, int64_t outer, int64_t dst_len,
 int hapmi_split_rows(const void *src, void *const *pieces_host, const int64_t *lengths_host, int n_ranks,
                      int64_t outer, int64_t inner_bytes, hapmi_stream_t stream);
 
+/* hapmi_split_rows of src * (fwd_out > 0), fwd_out having src's shape and dtype: the backward of a relu whose
+ * only reader's gradient goes straight into an all_to_all (models.py:283 after collectives.py:156-165 in the
+ * column-sharded FFN), without a separate pass over the gradient.  Every piece, src and fwd_out 16-byte aligned
+ * with inner_bytes * lengths a multiple of 16. */
+int hapmi_split_rows_relu_bwd(const void *src, const void *fwd_out, void *const *pieces_host,
+                              const int64_t *lengths_host, int n_ranks, int64_t outer, int64_t inner_bytes,
+                              int dtype, hapmi_stream_t stream);
+
 /* collectives.py:159 / :166: concatenate W contiguous pieces [outer, lengths[i], inner]
  * into dst[outer, sum(lengths), inner]; `act` != NONE applies the activation to
  * every element on the way (dtype needed then). */

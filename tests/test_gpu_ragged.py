@@ -77,6 +77,32 @@ def test_concat_with_fused_relu(cuda, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("shape,dim,L", [((6, 5, 128), 2, [48, 48, 16, 16]), ((3, 40, 8), 1, [18, 18, 2, 2]),
+                                         ((16, 64), 1, [64]), ((520, 1040), 1, [392, 392, 128, 128])])
+def test_split_with_fused_relu_backward(cuda, dtype, shape, dim, L):
+    """Pieces of dy * (y > 0), y the output of a relu (with exact zeros, negative zeros and NaN among its values),
+    against F.relu's own backward (threshold_backward) on the CPU."""
+    g = torch.Generator().manual_seed(5)
+    pre = torch.randn(shape, generator=g)
+    pre.view(-1)[::7] = 0.0
+    y = torch.relu(pre).to(dtype)
+    y.view(-1)[3] = float("nan")
+    y.view(-1)[5] = -0.0
+    y.view(-1)[11] = float("inf")
+    dy = torch.randn(shape, generator=g).to(dtype)
+    want = torch.where(y > 0, dy, torch.zeros_like(dy))
+    pieces = ops.split_rows(dy.to(cuda), L, dim, relu_of=y.to(cuda))
+    for got, ref in zip(pieces, torch.split(want, L, dim=dim)):
+        assert torch.equal(got.cpu().view(torch.int16 if dtype == torch.bfloat16 else torch.int32),
+                           ref.contiguous().view(torch.int16 if dtype == torch.bfloat16 else torch.int32))
+    # autograd's relu backward agrees wherever y is a number
+    yy = pre.clone().requires_grad_(True)
+    torch.relu(yy).backward(dy.float())
+    ok = ~torch.isnan(y.float()) & (y.float() == torch.relu(pre).to(dtype).float())
+    assert torch.equal(torch.cat([p.cpu() for p in pieces], dim=dim).float()[ok], yy.grad.to(dtype).float()[ok])
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("W", [1, 2, 3, 4, 8])
 @pytest.mark.parametrize("shape,dim,off,length", [((40, 64), 0, 7, 20), ((4, 10, 24), 1, 3, 4), ((5, 9, 7), 1, 0, 9),
                                                   ((3, 64), 1, 8, 48)])
