@@ -12,6 +12,7 @@ _lib = None
 F32, BF16 = 0, 1
 ACT_NONE, ACT_RELU, ACT_GELU = 0, 1, 2
 MAX_RANKS = 64
+GEMM_MAX_LIST = 16
 
 
 class HapmiError(RuntimeError):
@@ -34,6 +35,9 @@ class GemmArgs(ctypes.Structure):
         ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_int64),
         ("a_rowsum", ctypes.c_void_p),
         ("c_relu_mask", ctypes.c_void_p),
+        ("c_addend", ctypes.c_void_p),
+        ("A_list", ctypes.c_void_p), ("B_list", ctypes.c_void_p), ("C_list", ctypes.c_void_p),
+        ("a_rowsum_list", ctypes.c_void_p),
     ]
 
 

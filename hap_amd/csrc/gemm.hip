@@ -109,7 +109,7 @@ Choice choose(int64_t M, int64_t N, int64_t K, int64_t batch, int bk, bool wide,
 template <typename TO>
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *ws, TO *C, int64_t M, int64_t N, int64_t ws_ld,
                                                           int64_t ldc, int splits, int accumulate, int act,
-                                                          const TO *relu_mask) {
+                                                          const TO *relu_mask, const TO *addend) {
     // the partial sums of one output group are independent loads: they are issued eight at a time and added in
     // split order afterwards (the order fixes the float32 result)
     constexpr int U = 8;
@@ -133,11 +133,12 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *ws, TO 
                 }
         }
         TO *dst = C + m * ldc + n;
+        const TO *prev = addend ? addend + m * ldc + n : dst;     // what an accumulating call adds to
         if (n + 4 <= N && (ldc & 3) == 0 && !relu_mask) {
             typedef TO out4_t __attribute__((ext_vector_type(4)));
             out4_t o;
             if (accumulate) {
-                const out4_t old = *(const out4_t *)dst;
+                const out4_t old = *(const out4_t *)prev;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) o[e] = (TO)(apply_act(acc[e], act) + (float)old[e]);
             } else {
@@ -152,7 +153,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *ws, TO 
             if (n + e < N) {
                 float x = apply_act(acc[e], act);
                 if (relu_mask && !((float)relu_mask[m * ldc + n + e] > 0.f)) x = 0.f;
-                if (accumulate) x += (float)dst[e];
+                if (accumulate) x += (float)prev[e];
                 dst[e] = (TO)x;
             }
         }
@@ -202,7 +203,8 @@ int launch_typed(GemmParams &p, int transA, int transB, int64_t batch, hipStream
     int64_t gx = hapmi_cdiv(p.M * (p.ws_ld / 4), 256);
     if (gx > 256 * 16) gx = 256 * 16;
     hipLaunchKernelGGL((splitk_reduce_kernel<TO>), dim3((unsigned)gx), dim3(256), 0, st, (const float *)p.ws, (TO *)p.C,
-                       p.M, p.N, p.ws_ld, p.ldc, p.splits, p.accumulate, p.act, (const TO *)p.relu_mask);
+                       p.M, p.N, p.ws_ld, p.ldc, p.splits, p.accumulate, p.act, (const TO *)p.relu_mask,
+                       (const TO *)p.addend);
     return HAPMI_OK;
 }
 
@@ -214,7 +216,23 @@ extern "C" int hapmi_gemm(const hapmi_gemm_args *a, hapmi_stream_t stream) {
     HAPMI_REQUIRE(a->M >= 0 && a->N >= 0 && a->K >= 0 && a->batch1 >= 1 && a->batch2 >= 1, HAPMI_EINVAL,
                   "gemm: bad shape M=%lld N=%lld K=%lld", (long long)a->M, (long long)a->N, (long long)a->K);
     if (a->M == 0 || a->N == 0) return HAPMI_OK;
-    HAPMI_REQUIRE(a->A && a->B && a->C, HAPMI_EINVAL, "gemm: null pointer");
+    const bool lists = a->A_list || a->B_list || a->C_list || a->a_rowsum_list;
+    if (lists) {
+        HAPMI_REQUIRE(a->A_list && a->B_list && a->C_list, HAPMI_EINVAL, "gemm: A_list, B_list and C_list go together");
+        HAPMI_REQUIRE(a->batch1 <= HAPMI_GEMM_MAX_LIST && a->batch2 == 1, HAPMI_ELIMIT,
+                      "gemm: pointer lists hold at most %d problems (batch2 = 1)", HAPMI_GEMM_MAX_LIST);
+        HAPMI_REQUIRE(!a->A && !a->B && !a->C && !a->a_rowsum && !a->c_relu_mask && !a->c_addend, HAPMI_EINVAL,
+                      "gemm: A, B, C, a_rowsum, c_relu_mask and c_addend must be NULL next to pointer lists");
+        HAPMI_REQUIRE(!a->a_rowsum_list || a->transA, HAPMI_EINVAL, "gemm: a_rowsum_list needs transA = 1");
+        for (int64_t z = 0; z < a->batch1; ++z) {
+            HAPMI_REQUIRE(a->A_list[z] && a->B_list[z] && a->C_list[z], HAPMI_EINVAL, "gemm: null pointer in a list");
+            HAPMI_REQUIRE(((uintptr_t)a->A_list[z] % 16) == 0 && ((uintptr_t)a->B_list[z] % 16) == 0 &&
+                              ((uintptr_t)a->C_list[z] % (4 * hapmi_elem_size(a->out_dtype))) == 0,
+                          HAPMI_EALIGN, "gemm: misaligned pointer in a list");
+        }
+    } else {
+        HAPMI_REQUIRE(a->A && a->B && a->C, HAPMI_EINVAL, "gemm: null pointer");
+    }
     HAPMI_REQUIRE(a->act == HAPMI_ACT_NONE || a->act == HAPMI_ACT_RELU || a->act == HAPMI_ACT_GELU, HAPMI_EINVAL,
                   "gemm: unknown activation %d", a->act);
     const int64_t epv = a->in_dtype == HAPMI_F32 ? 4 : 8;
@@ -249,6 +267,18 @@ extern "C" int hapmi_gemm(const hapmi_gemm_args *a, hapmi_stream_t stream) {
     p.rowsum = a->a_rowsum;
     HAPMI_REQUIRE(!a->a_rowsum || (a->transA && a->batch1 * a->batch2 == 1), HAPMI_EINVAL,
                   "gemm: a_rowsum needs transA = 1 (A stored [K, M]) and a single problem");
+    p.addend = a->c_addend;
+    HAPMI_REQUIRE(!a->c_addend || (a->accumulate && a->batch1 * a->batch2 == 1 &&
+                                   ((uintptr_t)a->c_addend % (4 * osz)) == 0),
+                  HAPMI_EINVAL, "gemm: c_addend needs accumulate = 1, a single problem and C's alignment");
+    p.n_list = lists ? (int)a->batch1 : 0;
+    for (int z = 0; z < HAPMI_GEMM_MAX_LIST; ++z) {
+        const bool on = z < p.n_list;
+        p.listA[z] = on ? a->A_list[z] : nullptr;
+        p.listB[z] = on ? a->B_list[z] : nullptr;
+        p.listC[z] = on ? a->C_list[z] : nullptr;
+        p.listRS[z] = on && a->a_rowsum_list ? a->a_rowsum_list[z] : nullptr;
+    }
     p.relu_mask = a->c_relu_mask;
     HAPMI_REQUIRE(!a->c_relu_mask || (a->batch1 * a->batch2 == 1 && ((uintptr_t)a->c_relu_mask % 16) == 0), HAPMI_EINVAL,
                   "gemm: c_relu_mask needs a single problem and a 16-byte aligned pointer");

@@ -36,6 +36,11 @@ struct GemmParams {
     float *rowsum;             // optional: rowsum[m] += sum_k op(A)[m, k] (float32 atomics; A stored [K, M] only)
     const void *relu_mask;     // optional: [M][ldc] in C's element type; result elements whose mask is <= 0 become 0
     int64_t ws_ld;
+    const void *addend;        // optional (accumulate): the old values are read here instead of from C
+    int n_list;                // > 0: problem blockIdx.z takes its pointers from the lists below
+    const void *listA[HAPMI_GEMM_MAX_LIST], *listB[HAPMI_GEMM_MAX_LIST];
+    void *listC[HAPMI_GEMM_MAX_LIST];
+    float *listRS[HAPMI_GEMM_MAX_LIST];
 };
 
 namespace {
@@ -91,13 +96,23 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, ((WAVES_M * WAVES_N <= 4 && 
     const TI *A = (const TI *)p.A;
     const TI *B = (const TI *)p.B;
     TO *C = (TO *)p.C;
-    if (gridDim.z > 1) {                                          // batch index: at most 65535, 32-bit division
+    float *rowsum = p.rowsum;
+    if (p.n_list > 0) {                                           // uniform: scalar loads from the argument block
+        const int z = (int)blockIdx.z;
+        A = (const TI *)p.listA[z];
+        B = (const TI *)p.listB[z];
+        C = (TO *)p.listC[z];
+        rowsum = p.listRS[z];
+    } else if (gridDim.z > 1) {                                   // batch index: at most 65535, 32-bit division
         const int b2 = (int)p.batch2;
         const int64_t z1 = (int)blockIdx.z / b2, z2 = (int)blockIdx.z % b2;
         A += z1 * p.sA1 + z2 * p.sA2;
         B += z1 * p.sB1 + z2 * p.sB2;
         C += z1 * p.sC1 + z2 * p.sC2;
     }
+
+    // accumulate reads the old values `old_delta` bytes from where the result goes (0: in place)
+    const int64_t old_delta = p.addend ? (int64_t)((const char *)p.addend - (const char *)C) : 0;
 
     const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
     const int64_t m_left = p.M - m0, n_left = p.N - n0;
@@ -173,7 +188,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, ((WAVES_M * WAVES_N <= 4 && 
     // they are complete (rs_add_lds).  Every block of a tile row sees the same A tiles, so the k-tiles are
     // dealt round-robin over the tiles_n blocks of the row: each block adds 1/tiles_n of the work instead of
     // one block in tiles_n doing all of it.
-    const bool do_rs = !A_KMAJOR && p.rowsum != nullptr;
+    const bool do_rs = !A_KMAJOR && rowsum != nullptr;
     constexpr int RS_N = A_KMAJOR ? 1 : (A_TR ? 8 : TileLoader<TI, BM, THREADS, false>::PASSES_T * EPV);
     float rs[RS_N];
 #pragma unroll
@@ -292,7 +307,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, ((WAVES_M * WAVES_N <= 4 && 
         }
         __syncthreads();
         for (int t = threadIdx.x; t < BM; t += THREADS)
-            if (t < m_left) atomicAdd(p.rowsum + m0 + t, red[t]);
+            if (t < m_left) atomicAdd(rowsum + m0 + t, red[t]);
         __syncthreads();
     }
 
@@ -464,7 +479,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, ((WAVES_M * WAVES_N <= 4 && 
                     for (int e = 0; e < 4; ++e) v[e] = (float)mk[e] > 0.f ? v[e] : 0.f;
                 }
                 if (p.accumulate) {
-                    const out4_t old = *(const out4_t *)dst;
+                    const out4_t old = *(const out4_t *)((const char *)dst + old_delta);
 #pragma unroll
                     for (int e = 0; e < 4; ++e) v[e] += (float)old[e];
                 }
@@ -498,7 +513,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, ((WAVES_M * WAVES_N <= 4 && 
             if (n + 4 <= p.N && ((p.ldc & 3) == 0)) {
                 f32x4 x = vm;
                 if (p.accumulate) {
-                    const out4_t old = *(const out4_t *)dst;
+                    const out4_t old = *(const out4_t *)((const char *)dst + old_delta);
 #pragma unroll
                     for (int e = 0; e < 4; ++e) x[e] += (float)old[e];
                 }
@@ -511,7 +526,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, ((WAVES_M * WAVES_N <= 4 && 
                 for (int e = 0; e < 4; ++e) {
                     if (n + e < p.N) {
                         float x = vm[e];
-                        if (p.accumulate) x += (float)dst[e];
+                        if (p.accumulate) x += (float)*(const TO *)((const char *)(dst + e) + old_delta);
                         dst[e] = (TO)x;
                     }
                 }

@@ -293,12 +293,14 @@ def gemm(A: torch.Tensor, B: torch.Tensor, C: torch.Tensor, M: int, N: int, K: i
          lda=None, ldb=None, ldc=None, bias: Optional[torch.Tensor] = None, accumulate=False, act=None, alpha=1.0,
          batch1=1, batch2=1, strideA=(0, 0), strideB=(0, 0), strideC=(0, 0),
          offA=0, offB=0, offC=0, workspace: Optional[torch.Tensor] = None,
-         a_rowsum: Optional[torch.Tensor] = None, relu_mask: Optional[torch.Tensor] = None):
+         a_rowsum: Optional[torch.Tensor] = None, relu_mask: Optional[torch.Tensor] = None,
+         addend: Optional[torch.Tensor] = None):
     """C = alpha * op(A) @ op(B) (+bias)(act)(+C).  Offsets and strides are in elements.  ``workspace`` (or
     the buffer installed with ``set_gemm_workspace``) lets the library split a long reduction over K.
     ``a_rowsum`` (float32[M], transA only): the sums over k of op(A)'s rows are added into it.
-    ``relu_mask`` ([M, ldc] like C): result elements whose mask is <= 0 are zero (relu backward)."""
-    _dev(A, B, C, bias, a_rowsum, relu_mask)
+    ``relu_mask`` ([M, ldc] like C): result elements whose mask is <= 0 are zero (relu backward).
+    ``addend`` ([M, ldc] like C, with ``accumulate``): C = addend + result; C itself is only written."""
+    _dev(A, B, C, bias, a_rowsum, relu_mask, addend)
     if A.dtype != B.dtype:
         raise TypeError("gemm operands must share a dtype")
     a = GemmArgs()
@@ -341,12 +343,60 @@ def gemm(A: torch.Tensor, B: torch.Tensor, C: torch.Tensor, M: int, N: int, K: i
             raise TypeError("gemm relu_mask: C's element type and a single problem expected")
         _need(relu_mask, _span(M, N, a.ldc), "gemm relu_mask")
     a.c_relu_mask = relu_mask.data_ptr() if relu_mask is not None else 0
+    if addend is not None:
+        if addend.dtype != C.dtype or not accumulate or batch1 * batch2 != 1:
+            raise TypeError("gemm addend: C's element type, accumulate and a single problem expected")
+        _need(addend, _span(M, N, a.ldc), "gemm addend")
+    a.c_addend = addend.data_ptr() if addend is not None else 0
     if min(strideA + strideB + strideC) < 0:
         raise _lib.HapmiError("gemm: negative batch stride")
     if _gemm_log is not None:
-        _gemm_log.append((a, (A, B, C, bias, ws, a_rowsum, relu_mask)))          # the tensors keep the recorded pointers alive
+        _gemm_log.append((a, (A, B, C, bias, ws, a_rowsum, relu_mask, addend)))  # the tensors keep the recorded pointers alive
     check(lib().hapmi_gemm(ctypes.byref(a), _stream()))
     return C
+
+
+def gemm_group(As: Sequence[torch.Tensor], Bs: Sequence[torch.Tensor], Cs: Sequence[torch.Tensor], M: int, N: int,
+               K: int, *, transA=False, transB=False, lda=None, ldb=None, ldc=None, accumulate=False, alpha=1.0,
+               a_rowsums: Optional[Sequence[Optional[torch.Tensor]]] = None):
+    """``Cs[z] = alpha * op(As[z]) @ op(Bs[z]) (+ Cs[z])`` for up to 16 problems of one shape in one launch
+    (pointer lists of the C ABI; no K split).  ``a_rowsums[z]`` as ``a_rowsum`` of ``gemm``."""
+    n = len(As)
+    if not (1 <= n <= _lib.GEMM_MAX_LIST and len(Bs) == n and len(Cs) == n and (a_rowsums is None or len(a_rowsums) == n)):
+        raise ValueError(f"gemm_group: 1..{_lib.GEMM_MAX_LIST} problems with one entry per list expected")
+    _dev(*As, *Bs, *Cs, *(a_rowsums or ()))
+    a = GemmArgs()
+    a.M, a.N, a.K = M, N, K
+    a.lda = lda if lda is not None else (M if transA else K)
+    a.ldb = ldb if ldb is not None else (K if transB else N)
+    a.ldc = ldc if ldc is not None else N
+    a.transA, a.transB = int(transA), int(transB)
+    a.in_dtype, a.out_dtype = dtype_code(As[0]), dtype_code(Cs[0])
+    a.accumulate, a.act, a.alpha = int(accumulate), 0, float(alpha)
+    a.batch1, a.batch2 = n, 1
+    epv = 16 // As[0].element_size()
+    up = lambda v: (v + epv - 1) // epv * epv
+    for A, B, C in zip(As, Bs, Cs):
+        if A.dtype != As[0].dtype or B.dtype != As[0].dtype or C.dtype != Cs[0].dtype:
+            raise TypeError("gemm_group: every problem must have the element types of the first")
+        _need(A, _span(K if transA else M, up(M) if transA else K, a.lda), "gemm_group A")
+        _need(B, _span(N if transB else K, K if transB else up(N), a.ldb), "gemm_group B")
+        _need(C, _span(M, N, a.ldc), "gemm_group C")
+    for r in a_rowsums or ():
+        if r is not None:
+            if r.dtype != torch.float32 or not transA:
+                raise TypeError("gemm_group a_rowsums: float32 vectors and transA expected")
+            _need(r, M, "gemm_group a_rowsum")
+    arr = lambda ts: (ctypes.c_void_p * n)(*[t.data_ptr() if t is not None else None for t in ts])
+    la, lb, lc = arr(As), arr(Bs), arr(Cs)
+    lr = arr(a_rowsums) if a_rowsums is not None else None
+    a.A_list, a.B_list, a.C_list = ctypes.addressof(la), ctypes.addressof(lb), ctypes.addressof(lc)
+    a.a_rowsum_list = ctypes.addressof(lr) if lr is not None else 0
+    a._keep = (la, lb, lc, lr)                       # the argument block points into these host arrays
+    if _gemm_log is not None:
+        _gemm_log.append((a, (tuple(As), tuple(Bs), tuple(Cs), tuple(a_rowsums or ()))))
+    check(lib().hapmi_gemm(ctypes.byref(a), _stream()))
+    return Cs
 
 
 _gemm_log = None

@@ -147,7 +147,19 @@ typedef struct {
                                   * whose mask value is <= 0 are written as 0: the backward of F.relu
                                   * (hap.rs:1417) when the call is the data gradient of the next F.linear and
                                   * the mask is relu's output.  Needs batch 1; NULL = off */
+    const void *c_addend;        /* optional, with accumulate = 1: the result is added to c_addend[M][ldc] (out_dtype)
+                                  * instead of C's old content, and C is only written: a gradient contribution
+                                  * added to a buffer that other launches still read.  Needs batch 1; NULL = off */
+    /* Several problems of one shape behind arbitrary pointers in ONE launch (the same linear's weight gradient
+     * for a run of layers: each is too small to fill the chip without splitting K, together they are not):
+     * host arrays of batch1 device pointers (batch1 <= HAPMI_GEMM_MAX_LIST, batch2 = 1); problem z uses
+     * A_list[z], B_list[z], C_list[z] and, if a_rowsum_list is given, a_rowsum_list[z] (entries may be NULL).
+     * A, B, C, the batch strides, a_rowsum, c_relu_mask and c_addend must be NULL / 0 then.  NULL = off */
+    const void *const *A_list, *const *B_list;
+    void *const *C_list;
+    float *const *a_rowsum_list;
 } hapmi_gemm_args;
+#define HAPMI_GEMM_MAX_LIST 16
 int hapmi_gemm(const hapmi_gemm_args *args_host, hapmi_stream_t stream);
 
 /* Tuning hook for measurements: force tile configuration `tile_config` (block tile / waves: 0: 128x128 / 2x2,

@@ -362,6 +362,75 @@ def test_gemm_relu_mask_on_the_result(cuda, dtype, out_dtype, cfg, splits, accum
         lib().hapmi_gemm_tuning(-1, 0)
 
 
+@pytest.mark.parametrize("dtype,out_dtype,cfg,splits", [
+    (torch.bfloat16, torch.bfloat16, 0, 1), (torch.bfloat16, torch.bfloat16, 7, 1), (torch.bfloat16, torch.float32, 5, 1),
+    (torch.bfloat16, torch.bfloat16, 1, 3), (torch.float32, torch.float32, 0, 1), (torch.float32, torch.float32, 0, 2)])
+@pytest.mark.parametrize("shape", [(256, 512, 192), (328, 520, 1000)])
+def test_gemm_accumulates_onto_a_separate_addend(cuda, dtype, out_dtype, cfg, splits, shape):
+    """c_addend: C = addend + A B with C only written, bit-equal to accumulating in place into a copy of the
+    addend, in every store path; the addend itself is left untouched."""
+    from hap_amd._lib import lib
+    M, N, K = shape
+    g = torch.Generator().manual_seed(M + cfg + splits)
+    A = torch.randn(M, K, generator=g).to(dtype).to(cuda)
+    B = torch.randn(K, N, generator=g).to(dtype).to(cuda)
+    R = torch.randn(M, N, generator=g).to(out_dtype).to(cuda)
+    ws = torch.empty(8 * M * 520, dtype=torch.float32, device=cuda)
+    try:
+        lib().hapmi_gemm_tuning(cfg, splits)
+        in_place = R.clone()
+        ops.gemm(A, B, in_place, M, N, K, workspace=ws, accumulate=True)
+        keep = R.clone()
+        C = torch.full((M, N), 7.0, dtype=out_dtype, device=cuda)
+        ops.gemm(A, B, C, M, N, K, workspace=ws, accumulate=True, addend=R)
+        assert torch.equal(C, in_place) and torch.equal(R, keep)
+        close(C, A.double().cpu() @ B.double().cpu() + keep.double().cpu(), dtype if out_dtype == torch.float32 else out_dtype, scale=2.0)
+    finally:
+        lib().hapmi_gemm_tuning(-1, 0)
+    with pytest.raises(TypeError):
+        ops.gemm(A, B, C, M, N, K, addend=R)                               # without accumulate
+
+
+@pytest.mark.parametrize("cfg", [0, 1, 5, 6, 7, 9])
+@pytest.mark.parametrize("n,accumulate", [(1, False), (3, True), (8, False), (16, False)])
+def test_gemm_group_of_weight_gradients_behind_pointer_lists(cuda, cfg, n, accumulate):
+    """A_list / B_list / C_list / a_rowsum_list: n weight gradients dW = dY^T X (+ column sums of dY) of one
+    shape in one launch, bit-equal to n single launches of the same tile configuration, and close to float64."""
+    from hap_amd._lib import lib
+    rows, d_out, d_in = 520, 200, 328                                      # ragged against every tile size
+    g = torch.Generator().manual_seed(cfg * 31 + n)
+    dY = [torch.randn(rows, d_out, generator=g).bfloat16().to(cuda) for _ in range(n)]
+    X = [torch.randn(rows, d_in, generator=g).bfloat16().to(cuda) for _ in range(n)]
+    start = [torch.randn(d_out, d_in, generator=g).to(cuda) for _ in range(n)]
+    try:
+        lib().hapmi_gemm_tuning(cfg, 1)
+        single, single_b = [t.clone() for t in start], [torch.zeros(d_out, device=cuda) for _ in range(n)]
+        for z in range(n):
+            ops.gemm(dY[z], X[z], single[z], d_out, d_in, rows, transA=True, accumulate=accumulate, a_rowsum=single_b[z])
+        W, b = [t.clone() for t in start], [torch.zeros(d_out, device=cuda) if z != 1 else None for z in range(n)]
+        ops.gemm_group(dY, X, W, d_out, d_in, rows, transA=True, accumulate=accumulate, a_rowsums=b)
+    finally:
+        lib().hapmi_gemm_tuning(-1, 0)
+    for z in range(n):
+        assert torch.equal(W[z], single[z]), z
+        want = dY[z].double().t() @ X[z].double() + (start[z].double() if accumulate else 0)
+        close(W[z], want.cpu(), torch.bfloat16, scale=2.0)
+        if b[z] is not None:
+            torch.testing.assert_close(b[z].cpu(), dY[z].float().sum(0).cpu(), rtol=1e-4, atol=1e-3)
+    with pytest.raises(ValueError):
+        ops.gemm_group(dY * 17, X * 17, W * 17, d_out, d_in, rows, transA=True)
+
+
+def test_gemm_group_float32_and_plain_layout(cuda):
+    g = torch.Generator().manual_seed(5)
+    A = [torch.randn(70, 96, generator=g).to(cuda) for _ in range(4)]
+    B = [torch.randn(40, 96, generator=g).to(cuda) for _ in range(4)]
+    C = [torch.empty(70, 40, device=cuda) for _ in range(4)]
+    ops.gemm_group(A, B, C, 70, 40, 96, transB=True, alpha=0.5)
+    for z in range(4):
+        torch.testing.assert_close(C[z].cpu(), 0.5 * (A[z].double() @ B[z].double().t()).float().cpu(), rtol=2e-5, atol=2e-5)
+
+
 @pytest.mark.parametrize("S,causal", [(16, True), (128, True), (197, False), (512, False), (200, True), (64, False),
                                       (16, "flag"), (128, "flag"), (200, "flag"), (512, "flag"), (129, "flag")])
 def test_fused_attention_forward_backward(cuda, S, causal):
