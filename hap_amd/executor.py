@@ -61,7 +61,7 @@ class ShardExecutor:
                  rank: int = 0, world_size: int = 1, device: str = "cuda:0", fused_attention: bool = True,
                  overlap_wgrad: bool = False, launch_lists: bool = True, relu_mask_in_dgrad: bool = False,
                  overlap_optimizer: bool = False, optimizer_chunk_min: int = 1 << 20,
-                 relu_bwd_in_split: bool = True):
+                 relu_bwd_in_split: bool = True, wgrad_group: int = 8):
         """``example_inputs``: the program's inputs (global batch) as tensors or shapes; activations are
         sized from them.  ``rank`` / ``world_size`` are only needed by all_reduce / replicate, whose node
         forms do not carry them (collectives.py:86, 182)."""
@@ -112,6 +112,15 @@ class ShardExecutor:
         self.optimizer_chunk_min = int(optimizer_chunk_min)      # smallest stretch (elements) worth a launch of its own
         self._touched: Optional[list] = None
         self._grad_final_idx: Dict[str, int] = {}
+        # The weight gradient of one linear has a small output and a long reduction (BERT-large shard: [1024, 1024]
+        # to [1024, 4096] outputs over 6144-16384 tokens): alone it fills the chip only with its reduction split
+        # 2-8 ways through float32 partial sums.  The same linear's weight gradients of `wgrad_group` consecutive
+        # layers go into ONE launch instead (pointer lists, no split): measured 153 us against 247 us per layer.
+        # They are held back until the group is full (or backward ends); their operands are per-layer buffers
+        # that nothing overwrites before (see _grad_slot / _guard_write).  1 = every weight gradient at once.
+        self.wgrad_group = 1 if (overlap_wgrad or self.overlap_optimizer) else max(1, min(int(wgrad_group), ops._lib.GEMM_MAX_LIST))
+        self._pending_wgrads: Dict[tuple, list] = {}
+        self._deferred_reads: Dict[int, int] = {}          # storage -> launches held back that read it
         self._side_stream = torch.cuda.Stream(device=self.dev) if overlap_wgrad else None
         self._side_join = torch.cuda.Event() if overlap_wgrad else None
         self._side_used = False
@@ -225,6 +234,64 @@ class ShardExecutor:
         self._guard_write(v.grad)
         return v.grad, True
 
+    def _grad_slot_addend(self, v: Val):
+        """``_grad_slot`` for a GEMM: (buffer, accumulate, addend).  When the gradient exists but weight-gradient
+        launches that are held back still read its buffer, the sum goes to a new buffer (C = addend + A B) and
+        the old one stays as it is."""
+        if v.grad is not None and self._is_read_later(v.grad):
+            old = v.grad
+            v.grad = self._new(old.shape, old.dtype)
+            return v.grad, True, old
+        g, acc = self._grad_slot(v)
+        return g, acc, None
+
+    def _is_read_later(self, t: Optional[torch.Tensor]) -> bool:
+        return t is not None and self._deferred_reads.get(t.untyped_storage().data_ptr(), 0) > 0
+
+    def _emit_wgrad(self, dy, xt, gw, gb, n_out, n_in, rows, ld_dy, ld_x, acc, params):
+        """dW[n_out, n_in] (+)= dy[rows, n_out]^T x[rows, n_in], the bias gradient gb (column sums of dy) taken by
+        the same kernel.  Launched at once, or held back to share a launch with the same linear of the next
+        layers (only for parameters with a single use: their gradient is written once, order does not matter)."""
+        single_use = all(v is None or v.meta.get("name") in self._single_use_params for v in params)
+        if self.wgrad_group <= 1 or not single_use:
+            self.bwd.append(lambda: ops.gemm(dy, xt, gw, n_out, n_in, rows, transA=True, lda=ld_dy, ldb=ld_x,
+                                             accumulate=acc, a_rowsum=gb))
+            return
+        sig = (n_out, n_in, rows, ld_dy, ld_x, bool(acc), dy.dtype, gw.dtype)
+        q = self._pending_wgrads.setdefault(sig, [])
+        q.append((dy, xt, gw, gb, [v.meta["name"] for v in params if v is not None]))
+        for t in (dy, xt):
+            k = t.untyped_storage().data_ptr()
+            self._deferred_reads[k] = self._deferred_reads.get(k, 0) + 1
+        if len(q) >= self.wgrad_group:
+            self._flush_wgrads(sig)
+
+    def _flush_wgrads(self, sig=None):
+        """Append the launches of the weight gradients held back (of one signature, or all)."""
+        for key in ([sig] if sig is not None else list(self._pending_wgrads)):
+            q = self._pending_wgrads.pop(key, [])
+            if not q:
+                continue
+            n_out, n_in, rows, ld_dy, ld_x, acc = key[:6]
+            for dy, xt, _, _, _ in q:
+                for t in (dy, xt):
+                    self._deferred_reads[t.untyped_storage().data_ptr()] -= 1
+            self.bwd.append(self._wgrad_launch(q, n_out, n_in, rows, ld_dy, ld_x, acc))
+            for e in q:
+                for name in e[4]:
+                    self._grad_final_idx[name] = len(self.bwd)
+
+    @staticmethod
+    def _wgrad_launch(q, n_out, n_in, rows, ld_dy, ld_x, acc):
+        if len(q) == 1:
+            dy, xt, gw, gb, _ = q[0]
+            return lambda: ops.gemm(dy, xt, gw, n_out, n_in, rows, transA=True, lda=ld_dy, ldb=ld_x, accumulate=acc,
+                                    a_rowsum=gb)
+        dys, xts, gws = [e[0] for e in q], [e[1] for e in q], [e[2] for e in q]
+        gbs = [e[3] for e in q] if any(e[3] is not None for e in q) else None
+        return lambda: ops.gemm_group(dys, xts, gws, n_out, n_in, rows, transA=True, lda=ld_dy, ldb=ld_x,
+                                      accumulate=acc, a_rowsums=gbs)
+
     def _param_grad_slot(self, v: Val):
         if self._touched is not None and v.meta.get("name") is not None:
             self._touched.append(v.meta["name"])
@@ -282,7 +349,10 @@ class ShardExecutor:
 
     def _guard_write(self, t: Optional[torch.Tensor]):
         """Called while the backward list is built, right before a launch that writes into ``t`` is appended:
-        when a side-stream launch appended earlier reads ``t``'s storage, the main stream waits for it first."""
+        when a side-stream launch appended earlier reads ``t``'s storage, the main stream waits for it first;
+        when weight-gradient launches that are held back read it, they are appended first."""
+        if self._is_read_later(t):
+            self._flush_wgrads()             # weight gradients held back read t: they go first
         if t is None or not self._side_readers:
             return
         done = self._side_readers.pop(t.untyped_storage().data_ptr(), None)
@@ -346,6 +416,7 @@ class ShardExecutor:
             emit()
             for name in self._touched:
                 self._grad_final_idx[name] = len(self.bwd)
+        self._flush_wgrads()
         self._touched = None
         self._tape = []
 
@@ -484,6 +555,11 @@ class ShardExecutor:
         program order, hence follow it in backward order."""
         if v.grad is None:
             v.grad = src
+        elif self._is_read_later(v.grad):
+            g = v.grad
+            v.grad = self._new(g.shape, g.dtype)         # weight gradients held back still read g
+            out = v.grad
+            self.bwd.append(lambda: ops.add(g, src, out))
         else:
             g = v.grad
             self._guard_write(g)
@@ -580,7 +656,7 @@ class ShardExecutor:
             if side:
                 self._emit_side(wgrad, (dy, xt))
             else:
-                self.bwd.append(wgrad)
+                self._emit_wgrad(dy, xt, gw, gb, N, K, M, ldc, lda, accw, (w, b))
             if x.kind == "cls_view":
                 src = x.meta["src"]
                 if src.grad is None:
@@ -588,9 +664,10 @@ class ShardExecutor:
                     g = src.grad
                     self.bwd.append(lambda: ops.fill_zero(g))
                 g = src.grad
+                self._guard_write(g)
                 self.bwd.append(lambda: ops.gemm(dy, w.t, g, M, K, N, lda=ldc, ldc=lda, accumulate=True))
             elif x.needs_grad:
-                g, acc = self._grad_slot(x)
+                g, acc, addend = self._grad_slot_addend(x)
                 # x is the output of a producer that applied relu itself and this linear is its only reader:
                 # the data gradient leaves the GEMM already masked and the separate relu-backward pass is skipped
                 mask = None
@@ -598,7 +675,8 @@ class ShardExecutor:
                         and not x.meta.get("relu_bwd_done")):
                     mask = x.t
                     x.meta["relu_bwd_done"] = True
-                self.bwd.append(lambda: ops.gemm(dy, w.t, g, M, K, N, lda=ldc, ldc=lda, accumulate=acc, relu_mask=mask))
+                self.bwd.append(lambda: ops.gemm(dy, w.t, g, M, K, N, lda=ldc, ldc=lda, accumulate=acc, relu_mask=mask,
+                                                 addend=addend))
         self._tape.append(emit)
         return out
 
@@ -624,6 +702,7 @@ class ShardExecutor:
                 self.bwd.append(lambda: ops.act_bwd(out.grad, ref, g, kind))
             else:
                 tmp, g = self._new(x.t.shape), x.grad
+                self._guard_write(g)
                 self.bwd.append(lambda: (ops.act_bwd(out.grad, ref, tmp, kind), ops.add(g, tmp, g)))
         self._tape.append(emit)
         return out
@@ -743,8 +822,11 @@ class ShardExecutor:
             do = out_bsd.grad
             dctx = self._scratch("attn_dctx", (b, S, Ea))
             side = self._side_ok(w_out, b_out, w_in, b_in)
-            # the in-projection's weight gradient reads dqkv from the side stream, so it cannot be shared scratch
-            dqkv = self._new((b, S, 3 * Ea)) if side else self._scratch("attn_dqkv", (b, S, 3 * Ea))
+            held = (not side and self.wgrad_group > 1
+                    and all(v is None or v.meta.get("name") in self._single_use_params for v in (w_in, b_in)))
+            # the in-projection's weight gradient reads dqkv from the side stream, or later together with the next
+            # layers' (wgrad_group), so it cannot be shared scratch then
+            dqkv = self._new((b, S, 3 * Ea)) if (side or held) else self._scratch("attn_dqkv", (b, S, 3 * Ea))
             if fused:
                 delta = self._scratch("attn_delta", (b, H, S), torch.float32)
             else:
@@ -753,7 +835,14 @@ class ShardExecutor:
             gbo, acc_bo = self._param_grad_slot(b_out) if b_out is not None else (None, False)
             gwi, acc_wi = self._param_grad_slot(w_in)
             gbi, acc_bi = self._param_grad_slot(b_in)
-            gx, acc_x = self._grad_slot(x) if x.needs_grad else (None, False)
+            if side:
+                gx, acc_x = self._grad_slot(x) if x.needs_grad else (None, False)
+                addend_x = None
+            else:
+                # first in the list (as before); held back, it keeps reading `do`, which d(x) usually aliases (the
+                # residual add hands one buffer to both): the in-projection's data gradient then goes to a new buffer
+                self._emit_wgrad(do, ctx, gwo, gbo, d_out, Ea, M, d_out, Ea, acc_wo, (w_out, b_out))
+                gx, acc_x, addend_x = self._grad_slot_addend(x) if x.needs_grad else (None, False, None)
 
             ws = self.side_workspace if side else None
 
@@ -764,8 +853,6 @@ class ShardExecutor:
                 ops.gemm(dqkv, x.t, gwi, 3 * Ea, d, M, transA=True, accumulate=acc_wi, workspace=ws, a_rowsum=gbi)
 
             def backward():
-                if not side:
-                    wgrad_out()
                 ops.gemm(do, w_out.t, dctx, M, Ea, d_out)
                 if fused:
                     ops.attention_bwd(qkv, ctx, dctx, lse, fused_mask, dqkv, delta, b, S, H, scale, causal)
@@ -781,11 +868,9 @@ class ShardExecutor:
                              strideA=sP, strideB=sQ, strideC=sQ, offB=Ea)
                     ops.gemm(dP, qkv, dqkv, S, hd, S, transA=True, lda=Sp, ldb=3 * Ea, ldc=3 * Ea, alpha=scale, batch1=b,
                              batch2=H, strideA=sP, strideB=sQ, strideC=sQ, offC=Ea)
-                if not side:
-                    wgrad_in()
 
             def dgrad_in():
-                ops.gemm(dqkv, w_in.t, gx, M, d, 3 * Ea, accumulate=acc_x)
+                ops.gemm(dqkv, w_in.t, gx, M, d, 3 * Ea, accumulate=acc_x, addend=addend_x)
             if side:
                 # do is final here; dqkv is final once `backward` is enqueued.  d(x) usually aliases do (the
                 # residual add hands one buffer to both), so the in-projection's data gradient, which
@@ -795,8 +880,9 @@ class ShardExecutor:
                 self._emit_side(wgrad_in, (dqkv, x.t))
             else:
                 self.bwd.append(backward)
+                self._emit_wgrad(dqkv, x.t, gwi, gbi, 3 * Ea, d, M, 3 * Ea, d, acc_wi, (w_in, b_in))
             if gx is not None:
-                if acc_x:
+                if acc_x and addend_x is None:
                     self._guard_write(gx)
                 self.bwd.append(dgrad_in)
         self._tape.append(emit)
@@ -910,6 +996,7 @@ class ShardExecutor:
                     self.bwd.append(lambda: ops.slice_rows(g, 1, 1, T, gx))
                 else:
                     tmp, gx = self._new(x.t.shape), x.grad
+                    self._guard_write(gx)
                     self.bwd.append(lambda: (ops.slice_rows(g, 1, 1, T, tmp), ops.add(gx, tmp, gx)))
         self._tape.append(emit)
         return out
@@ -977,8 +1064,7 @@ class ShardExecutor:
                 x.grad = self._emit_scatter(node.name, "bwd", out.grad, dim, L, rank, self.bwd)
             else:
                 part = self._emit_scatter(node.name, "bwd", out.grad, dim, L, rank, self.bwd)
-                g = x.grad
-                self.bwd.append(lambda: ops.add(g, part, g))
+                self._accumulate_into(x, part)
         self._tape.append(emit)
         return out
 
@@ -1002,6 +1088,7 @@ class ShardExecutor:
             x.meta["grad_written"] = True
             if self._touched is not None:
                 self._touched.append(x.meta["name"])
+            self._flush_wgrads()                         # the consumers' weight gradients write full_grad
             self._emit_scatter(node.name, "bwd", full_grad, 0, L, rank, self.bwd, out_t=x.meta["grad"])
         self._tape.append(emit)
         return out
