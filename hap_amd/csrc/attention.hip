@@ -19,6 +19,9 @@
 
 namespace {
 
+constexpr float LOG2E = 1.4426950408889634f;
+
+
 constexpr int HD = 64;                 // head dimension (bf16: one 128-byte LDS row)
 constexpr int TILE = 64;               // rows of the streamed operand per iteration
 constexpr int AT_THREADS = 256;        // 4 waves, 32 rows of the stationary operand each
@@ -87,18 +90,34 @@ __device__ __forceinline__ frag_t load_row_frag(const bf16_t *row_ptr, bool vali
 }
 
 // One [64 rows][64 d] operand tile (memory [row][d], row stride ld) held as two 16-byte vectors per thread
-// (rows 2 * (t / 8) and + 1, d chunk t % 8) on its way into the row-major LDS tile.
+// (rows 2 * (t / 8) and + 1, d chunk t % 8) on its way into the row-major LDS tile.  The thread's element offsets
+// inside a tile and its LDS byte offsets are fixed for the kernel's lifetime; `base` (the tile's first element) is
+// the same for every thread, so a load is one instruction on a scalar base and a constant vector offset, and
+// full tiles skip the row checks.
 struct PairLoader {
     frag_t v[2];
-    __device__ __forceinline__ void load(const bf16_t *base, int64_t ld, int64_t rows_left) {
+    int goff[2], soff[2];
+    __device__ __forceinline__ PairLoader(int ld) {
         const int c8 = threadIdx.x & 7, r0 = (threadIdx.x >> 3) * 2;
 #pragma unroll
-        for (int i = 0; i < 2; ++i) v[i] = load_row_frag(base + (int64_t)(r0 + i) * ld + c8 * 8, r0 + i < rows_left, 0, 0);
+        for (int i = 0; i < 2; ++i) {
+            goff[i] = (r0 + i) * ld + c8 * 8;
+            soff[i] = (r0 + i) * ROW_BYTES + ((c8 ^ aswz(r0 + i)) << 4);
+        }
+    }
+    __device__ __forceinline__ void load(const bf16_t *base, int rows_left) {
+        if (rows_left >= TILE) {
+#pragma unroll
+            for (int i = 0; i < 2; ++i) v[i] = *(const frag_t *)(base + goff[i]);
+        } else {
+            const int r0 = (threadIdx.x >> 3) * 2;
+#pragma unroll
+            for (int i = 0; i < 2; ++i) v[i] = load_row_frag(base + goff[i], r0 + i < rows_left, 0, 0);
+        }
     }
     __device__ __forceinline__ void store_rows(char *lds) const {
-        const int c8 = threadIdx.x & 7, r0 = (threadIdx.x >> 3) * 2;
 #pragma unroll
-        for (int i = 0; i < 2; ++i) *(frag_t *)(lds + (r0 + i) * ROW_BYTES + ((c8 ^ aswz(r0 + i)) << 4)) = v[i];
+        for (int i = 0; i < 2; ++i) *(frag_t *)(lds + soff[i]) = v[i];
     }
 };
 
@@ -142,23 +161,28 @@ __global__ __launch_bounds__(AT_THREADS, 2) void attn_fwd_kernel(const bf16_t *q
 
     f32x16 ot[2] = {zero16(), zero16()};
     float m = -INFINITY, lsum = 0.f;
-    PairLoader lk, lv;
+    PairLoader lk(ld), lv(ld);
     const bool vec_mask = mask && ((S & 3) == 0);
+    // Softmax is VALU work next to the MFMAs (32 scores per lane and kv tile), so the common tile (no additive
+    // mask, every query and key of the tile valid and, if causal, visible) takes a short path: maximum over the raw
+    // scores, then one fused multiply-add and one exp2 per score.
+    const float sl2 = scale * LOG2E;
+    const bool plain_block = !mask && blk * 128 + 128 <= S;
 
     // The next tile's global loads are issued before the current tile is multiplied, so their latency is
     // covered by the MFMA / softmax work; the registers are written to LDS at the top of the next iteration.
     const int q_blk_end = blk * 128 + 128;
     const int kv_end = (CAUSAL && q_blk_end < S) ? q_blk_end : S;
-    lk.load(K, ld, S);
-    lv.load(V, ld, S);
+    lk.load(K, S);
+    lv.load(V, S);
     for (int kv0 = 0; kv0 < kv_end; kv0 += TILE) {
         __syncthreads();                                   // every wave is done with the previous tiles
         lk.store_rows(Ks);
         lv.store_rows(Vs);
         __syncthreads();
         if (kv0 + TILE < kv_end) {
-            lk.load(K + (int64_t)(kv0 + TILE) * ld, ld, S - kv0 - TILE);
-            lv.load(V + (int64_t)(kv0 + TILE) * ld, ld, S - kv0 - TILE);
+            lk.load(K + (int64_t)(kv0 + TILE) * ld, S - kv0 - TILE);
+            lv.load(V + (int64_t)(kv0 + TILE) * ld, S - kv0 - TILE);
         }
 
         f32x16 st[2] = {zero16(), zero16()};
@@ -167,52 +191,75 @@ __global__ __launch_bounds__(AT_THREADS, 2) void attn_fwd_kernel(const bf16_t *q
 #pragma unroll
             for (int s = 0; s < 4; ++s) st[t] = mma(frag_rowk(Ks, t * 32 + c, s, h), qf[s], st[t]);
 
-        float mx = -INFINITY;
+        float alpha, psum = 0.f;
+        if (plain_block && kv0 + TILE <= S && (!CAUSAL || kv0 + TILE - 1 <= blk * 128)) {
+            float mx = st[0][0];
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
+            for (int t = 0; t < 2; ++t)
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const int kv = kv0 + t * 32 + g * 8 + h * 4;
-                float mk[4] = {0.f, 0.f, 0.f, 0.f};
-                if (mask && qok) {
-                    if (vec_mask && kv + 4 <= S) {
-                        const f32x4 mv = *(const f32x4 *)(mask + (int64_t)q * S + kv);
+                for (int r = 0; r < 16; ++r) mx = fmaxf(mx, st[t][r]);
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            const float m_new = fmaxf(m, mx * scale);            // finite: every score of the tile is
+            const float nm = -m_new * LOG2E;
+            alpha = __builtin_amdgcn_exp2f(fmaf(m, LOG2E, nm));   // m = -inf before the first tile: 0
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) mk[e] = mv[e];
-                    } else {
+            for (int t = 0; t < 2; ++t)
 #pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            if (kv + e < S) mk[e] = mask[(int64_t)q * S + kv + e];
+                for (int r = 0; r < 16; ++r) {
+                    const float p = __builtin_amdgcn_exp2f(fmaf(st[t][r], sl2, nm));
+                    st[t][r] = p;
+                    psum += p;
+                }
+            m = m_new;
+        } else {
+            float mx = -INFINITY;
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int kv = kv0 + t * 32 + g * 8 + h * 4;
+                    float mk[4] = {0.f, 0.f, 0.f, 0.f};
+                    if (mask && qok) {
+                        if (vec_mask && kv + 4 <= S) {
+                            const f32x4 mv = *(const f32x4 *)(mask + (int64_t)q * S + kv);
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) mk[e] = mv[e];
+                        } else {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e)
+                                if (kv + e < S) mk[e] = mask[(int64_t)q * S + kv + e];
+                        }
+                    }
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        float v = st[t][g * 4 + e] * scale + mk[e];
+                        if (kv + e >= S || (CAUSAL && kv + e > q)) v = -INFINITY;
+                        st[t][g * 4 + e] = v;
+                        mx = fmaxf(mx, v);
                     }
                 }
+            }
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            const float m_new = fmaxf(m, mx);
+            const float msub = (m_new == -INFINITY) ? 0.f : m_new;
+            alpha = (m_new == -INFINITY) ? 1.f : __expf(m - m_new);
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    float v = st[t][g * 4 + e] * scale + mk[e];
-                    if (kv + e >= S || (CAUSAL && kv + e > q)) v = -INFINITY;
-                    st[t][g * 4 + e] = v;
-                    mx = fmaxf(mx, v);
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const float p = __expf(st[t][r] - msub);
+                    st[t][r] = p;
+                    psum += p;
                 }
-            }
+            m = m_new;
         }
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-        const float m_new = fmaxf(m, mx);
-        const float msub = (m_new == -INFINITY) ? 0.f : m_new;
-        const float alpha = (m_new == -INFINITY) ? 1.f : __expf(m - m_new);
-        float psum = 0.f;
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const float p = __expf(st[t][r] - msub);
-                st[t][r] = p;
-                psum += p;
-            }
         lsum = lsum * alpha + psum;
-        m = m_new;
+        if (__builtin_amdgcn_ballot_w64(alpha != 1.f)) {          // the running maximum moved for some query
 #pragma unroll
-        for (int u = 0; u < 2; ++u)
+            for (int u = 0; u < 2; ++u)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) ot[u][r] *= alpha;
+                for (int r = 0; r < 16; ++r) ot[u][r] *= alpha;
+        }
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
             const frag_t pb = acc_to_b(st[s >> 1], s & 1);
@@ -286,22 +333,26 @@ __global__ __launch_bounds__(AT_THREADS, 2) void attn_bwd_dq_kernel(const bf16_t
     const float lse_q = qok ? lse[((int64_t)b * H + hh) * S + q] : 0.f;
     const float delta_q = qok ? delta[((int64_t)b * H + hh) * S + q] : 0.f;
     f32x16 dqt[2] = {zero16(), zero16()};
-    PairLoader lk, lv;
+    PairLoader lk(ld), lv(ld);
     const bool vec_mask = mask && ((S & 3) == 0);
+    // dS is kept without its factor `scale`, which the result gets once at the end; plain tiles (see the forward
+    // kernel) take p = exp2(s * scale * log2 e - lse * log2 e) in two operations
+    const float sl2 = scale * LOG2E, nl = -lse_q * LOG2E;
+    const bool plain_block = !mask && blk * 128 + 128 <= S;
 
     const int q_blk_end = blk * 128 + 128;
     const int kv_end = (CAUSAL && q_blk_end < S) ? q_blk_end : S;
-    lk.load(K, ld, S);
-    lv.load(V, ld, S);
+    lk.load(K, S);
+    lv.load(V, S);
     for (int kv0 = 0; kv0 < kv_end; kv0 += TILE) {
         __syncthreads();
         lk.store_rows(Ks);
         lv.store_rows(Vs);
         __syncthreads();
         if (kv0 + TILE < kv_end) {
-            const int64_t nx = kv0 + TILE;
-            lk.load(K + nx * ld, ld, S - nx);
-            lv.load(V + nx * ld, ld, S - nx);
+            const int nx = kv0 + TILE;
+            lk.load(K + (int64_t)nx * ld, S - nx);
+            lv.load(V + (int64_t)nx * ld, S - nx);
         }
 
         // one 32-row kv block at a time keeps only one score / dP accumulator pair live
@@ -313,26 +364,32 @@ __global__ __launch_bounds__(AT_THREADS, 2) void attn_bwd_dq_kernel(const bf16_t
                 st = mma(frag_rowk(Ks, t * 32 + c, s, h), qf[s], st);
                 dp = mma(frag_rowk(Vs, t * 32 + c, s, h), dof[s], dp);
             }
+            if (plain_block && kv0 + TILE <= S && (!CAUSAL || kv0 + TILE - 1 <= blk * 128)) {
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const int kv = kv0 + t * 32 + g * 8 + h * 4;
-                float mk[4] = {0.f, 0.f, 0.f, 0.f};
-                if (mask && qok) {
-                    if (vec_mask && kv + 4 <= S) {
-                        const f32x4 mv = *(const f32x4 *)(mask + (int64_t)q * S + kv);
+                for (int r = 0; r < 16; ++r)
+                    dp[r] = __builtin_amdgcn_exp2f(fmaf(st[r], sl2, nl)) * (dp[r] - delta_q);
+            } else {
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) mk[e] = mv[e];
-                    } else {
+                for (int g = 0; g < 4; ++g) {
+                    const int kv = kv0 + t * 32 + g * 8 + h * 4;
+                    float mk[4] = {0.f, 0.f, 0.f, 0.f};
+                    if (mask && qok) {
+                        if (vec_mask && kv + 4 <= S) {
+                            const f32x4 mv = *(const f32x4 *)(mask + (int64_t)q * S + kv);
 #pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            if (kv + e < S) mk[e] = mask[(int64_t)q * S + kv + e];
+                            for (int e = 0; e < 4; ++e) mk[e] = mv[e];
+                        } else {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e)
+                                if (kv + e < S) mk[e] = mask[(int64_t)q * S + kv + e];
+                        }
                     }
-                }
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int r = g * 4 + e;
-                    float p = (qok && kv + e < S && !(CAUSAL && kv + e > q)) ? __expf(st[r] * scale + mk[e] - lse_q) : 0.f;
-                    dp[r] = p * (dp[r] - delta_q) * scale;
+                    for (int e = 0; e < 4; ++e) {
+                        const int r = g * 4 + e;
+                        float p = (qok && kv + e < S && !(CAUSAL && kv + e > q)) ? __expf(st[r] * scale + mk[e] - lse_q) : 0.f;
+                        dp[r] = p * (dp[r] - delta_q);
+                    }
                 }
             }
 #pragma unroll
@@ -351,7 +408,7 @@ __global__ __launch_bounds__(AT_THREADS, 2) void attn_bwd_dq_kernel(const bf16_t
             for (int g = 0; g < 4; ++g) {
                 bf16x4 o;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) o[e] = (bf16_t)dqt[u][g * 4 + e];
+                for (int e = 0; e < 4; ++e) o[e] = (bf16_t)(dqt[u][g * 4 + e] * scale);
                 *(bf16x4 *)(drow + u * 32 + g * 8 + h * 4) = o;
             }
     }
@@ -386,26 +443,28 @@ __global__ __launch_bounds__(AT_THREADS, 2) void attn_bwd_dkv_kernel(const bf16_
         vf[s] = load_row_frag(V + (int64_t)kv * ld, kok, s, h);
     }
     f32x16 dvt[2] = {zero16(), zero16()}, dkt[2] = {zero16(), zero16()};
-    PairLoader lq, ldo;
+    PairLoader lq(ld), ldo(E);
+    // log-sum-exps are staged times log2 e and dS is kept without its factor `scale` (applied once at the end)
+    const float sl2 = scale * LOG2E;
 
     // causal: queries before the block's first key see none of its keys
     const int q_begin = CAUSAL ? blk * 128 : 0;
-    lq.load(Q + (int64_t)q_begin * ld, ld, S - q_begin);
-    ldo.load(dO + (int64_t)q_begin * E, E, S - q_begin);
+    lq.load(Q + (int64_t)q_begin * ld, S - q_begin);
+    ldo.load(dO + (int64_t)q_begin * E, S - q_begin);
     for (int q0 = q_begin; q0 < S; q0 += TILE) {
         __syncthreads();
         lq.store_rows(Qs);
         ldo.store_rows(dOs);
         if (threadIdx.x < TILE) {
             const int qq = q0 + threadIdx.x;
-            lse_s[threadIdx.x] = qq < S ? lse_b[qq] : INFINITY;
+            lse_s[threadIdx.x] = qq < S ? lse_b[qq] * LOG2E : INFINITY;
             delta_s[threadIdx.x] = qq < S ? delta_b[qq] : 0.f;
         }
         __syncthreads();
         if (q0 + TILE < S) {
-            const int64_t nx = q0 + TILE;
-            lq.load(Q + nx * ld, ld, S - nx);
-            ldo.load(dO + nx * E, E, S - nx);
+            const int nx = q0 + TILE;
+            lq.load(Q + (int64_t)nx * ld, S - nx);
+            ldo.load(dO + (int64_t)nx * E, S - nx);
         }
 
         // one 32-row query block at a time keeps only one score / dP accumulator pair live; the loop is kept
@@ -418,19 +477,32 @@ __global__ __launch_bounds__(AT_THREADS, 2) void attn_bwd_dkv_kernel(const bf16_
                 sc = mma(frag_rowk(Qs, t * 32 + c, s, h), kf[s], sc);
                 dp = mma(frag_rowk(dOs, t * 32 + c, s, h), vf[s], dp);
             }
+            // without a mask, query rows beyond S carry lse = +inf (p = 0); causal tiles below the diagonal of the
+            // block's 128 keys need no comparison
+            const bool plain = !mask && (!CAUSAL || blk * 128 + 127 <= q0);
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
                 // accumulator registers 4 g .. 4 g + 3 are query rows ql .. ql + 3
                 const int ql = t * 32 + g * 8 + h * 4;
                 const f32x4 l4 = *(const f32x4 *)(lse_s + ql), d4 = *(const f32x4 *)(delta_s + ql);
+                if (plain) {
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int r = g * 4 + e;
-                    float x = sc[r] * scale - l4[e];                 // rows beyond S carry lse = +inf: p = 0
-                    if (mask) x += (kok && q0 + ql + e < S) ? mask[(int64_t)(q0 + ql + e) * S + kv] : 0.f;
-                    const float p = (CAUSAL && kv > q0 + ql + e) ? 0.f : __expf(x);
-                    sc[r] = p;
-                    dp[r] = p * (dp[r] - d4[e]) * scale;
+                    for (int e = 0; e < 4; ++e) {
+                        const int r = g * 4 + e;
+                        const float p = __builtin_amdgcn_exp2f(fmaf(sc[r], sl2, -l4[e]));
+                        sc[r] = p;
+                        dp[r] = p * (dp[r] - d4[e]);
+                    }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int r = g * 4 + e;
+                        float x = fmaf(sc[r], sl2, -l4[e]);
+                        if (mask) x += (kok && q0 + ql + e < S) ? mask[(int64_t)(q0 + ql + e) * S + kv] * LOG2E : 0.f;
+                        const float p = (CAUSAL && kv > q0 + ql + e) ? 0.f : __builtin_amdgcn_exp2f(x);
+                        sc[r] = p;
+                        dp[r] = p * (dp[r] - d4[e]);
+                    }
                 }
             }
 #pragma unroll
@@ -453,7 +525,7 @@ __global__ __launch_bounds__(AT_THREADS, 2) void attn_bwd_dkv_kernel(const bf16_
                 bf16x4 ok_, ov;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    ok_[e] = (bf16_t)dkt[u][g * 4 + e];
+                    ok_[e] = (bf16_t)(dkt[u][g * 4 + e] * scale);
                     ov[e] = (bf16_t)dvt[u][g * 4 + e];
                 }
                 *(bf16x4 *)(drow + E + u * 32 + g * 8 + h * 4) = ok_;
