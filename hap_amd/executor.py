@@ -59,7 +59,7 @@ def _round_up(n, m):
 class ShardExecutor:
     def __init__(self, gm: torch.fx.GraphModule, example_inputs, dtype: str = "fp32", wire: Optional[Wire] = None,
                  rank: int = 0, world_size: int = 1, device: str = "cuda:0", fused_attention: bool = True,
-                 overlap_wgrad: bool = False, launch_lists: bool = True, relu_mask_in_dgrad: bool = False,
+                 overlap_wgrad: bool = False, launch_lists: bool = True, relu_mask_in_dgrad: bool = True,
                  overlap_optimizer: bool = False, optimizer_chunk_min: int = 1 << 20,
                  relu_bwd_in_split: bool = True, wgrad_group: int = 8):
         """``example_inputs``: the program's inputs (global batch) as tensors or shapes; activations are
@@ -672,7 +672,7 @@ class ShardExecutor:
                 # the data gradient leaves the GEMM already masked and the separate relu-backward pass is skipped
                 mask = None
                 if (self.relu_mask_in_dgrad and x.meta.get("fused_act") == "relu" and not acc and x.ld is None and self._only_reader(node, x)
-                        and not x.meta.get("relu_bwd_done")):
+                        and not x.meta.get("relu_bwd_done") and not x.meta.get("relu_bwd_in_split")):
                     mask = x.t
                     x.meta["relu_bwd_done"] = True
                 self.bwd.append(lambda: ops.gemm(dy, w.t, g, M, K, N, lda=ldc, ldc=lda, accumulate=acc, relu_mask=mask,
@@ -1159,13 +1159,15 @@ class ShardExecutor:
         out = Val("tensor", t, needs_grad=x.needs_grad)
         if fuse:
             out.meta["fused_act"] = "relu"
+            # the backward exchange splits along the forward's concat dimension; where that split copies, relu's
+            # backward rides on the copy instead of a pass of its own over the gradient (or a mask read in the
+            # next linear's data-gradient GEMM)
+            out.meta["relu_bwd_in_split"] = self.relu_bwd_in_split and cd != 0 and self._split_can_mask(t, t, cd, cL)
 
         def emit():
             if out.grad is None or not x.needs_grad:
                 return
-            # the backward exchange splits along the forward's concat dimension; where that split copies, relu's
-            # backward rides on the copy instead of a pass of its own over the gradient
-            in_split = (fuse and self.relu_bwd_in_split and not out.meta.get("relu_bwd_done") and not (cd == 0 and out.grad.is_contiguous())
+            in_split = (fuse and out.meta["relu_bwd_in_split"] and not out.meta.get("relu_bwd_done")
                         and self._split_can_mask(out.grad, out.t, cd, cL))
             if fuse and not in_split:
                 self._relu_backward_through(out)

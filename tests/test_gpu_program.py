@@ -350,7 +350,7 @@ def test_relu_backward_in_the_split_of_the_exchange_equals_the_separate_pass(cud
     def build(in_split):
         gm = hap_amd.build_program(copy.deepcopy(model), hap_amd.ShardingPlan([RATIOS4], 0), 8)
         return hap_amd.compile_program(gm, [x, y], dtype=dtype, wire=hap_amd.SyntheticWire(seed=3, grad_scale=1e-2),
-                                       rank=0, world_size=4, relu_bwd_in_split=in_split)
+                                       rank=0, world_size=4, relu_bwd_in_split=in_split, relu_mask_in_dgrad=False)
 
     a, b = build(True), build(False)
     la = a.forward(x, y).item()
