@@ -359,6 +359,7 @@ int g_red_variant = 0;      // measurement hook: bit0 nontemporal loads, bit1 no
 struct ReduceOut {
     void *dst;
     int64_t offset, len;       // rows [offset, offset + len) of the sharded dimension
+    const void *addend;        // optional, dst's layout: added to the sum last (dst may be the addend itself)
 };
 struct ReduceOuts {
     int n;
@@ -388,6 +389,7 @@ __global__ __launch_bounds__(RED_THREADS) void ragged_reduce_kernel(ReduceArgs a
     constexpr bool NTL = VAR & 1, NTS = VAR & 2;
     const ReduceOut od = outs.out[blockIdx.y];
     T *dst = (T *)od.dst;
+    const T *addend = (const T *)od.addend;
     const int64_t offset = od.offset, len = od.len;
     const uint64_t vec_per_row = (uint64_t)(len * inner) / EPV;     // contiguous run per outer index
     const uint64_t total = vec_per_row * (uint64_t)outer;
@@ -442,6 +444,11 @@ __global__ __launch_bounds__(RED_THREADS) void ragged_reduce_kernel(ReduceArgs a
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             if (!ok[u]) continue;
+            if (addend) {
+                const Vec16<T> g = ldv(addend + doff[u], NTL);
+#pragma unroll
+                for (int e = 0; e < EPV; ++e) acc[u][e] += g.get(e);
+            }
             Vec16<T> r;
 #pragma unroll
             for (int e = 0; e < EPV; ++e) r.set(e, acc[u][e]);
@@ -451,9 +458,9 @@ __global__ __launch_bounds__(RED_THREADS) void ragged_reduce_kernel(ReduceArgs a
 }
 
 template <typename T>
-__global__ __launch_bounds__(RED_THREADS) void ragged_reduce_scalar_kernel(ReduceArgs a, T *dst, int64_t outer,
-                                                                          int64_t src_len, int64_t offset,
-                                                                          int64_t len, int64_t inner) {
+__global__ __launch_bounds__(RED_THREADS) void ragged_reduce_scalar_kernel(ReduceArgs a, T *dst, const T *addend,
+                                                                          int64_t outer, int64_t src_len,
+                                                                          int64_t offset, int64_t len, int64_t inner) {
     const uint64_t per = (uint64_t)(len * inner);
     const uint64_t total = per * (uint64_t)outer;
     const uint64_t step = (uint64_t)gridDim.x * RED_THREADS;
@@ -462,6 +469,7 @@ __global__ __launch_bounds__(RED_THREADS) void ragged_reduce_scalar_kernel(Reduc
         const uint64_t soff = (o * (uint64_t)src_len + (uint64_t)offset) * (uint64_t)inner + col;
         float acc = ld_f((const T *)a.src[0], soff);
         for (int w = 1; w < a.n; ++w) acc += ld_f((const T *)a.src[w], soff);
+        if (addend) acc += ld_f(addend, c);
         st_f(dst, c, acc);
     }
 }
@@ -495,7 +503,8 @@ int launch_reduce(const ReduceArgs &a, const ReduceOuts &outs, int64_t outer, in
     int64_t max_len = 0;
     for (int r = 0; r < outs.n; ++r) {
         const ReduceOut &o = outs.out[r];
-        vec_ok = vec_ok && ((o.len * inner) % EPV == 0) && ((o.offset * inner) % EPV == 0) && ((uintptr_t)o.dst % 16 == 0);
+        vec_ok = vec_ok && ((o.len * inner) % EPV == 0) && ((o.offset * inner) % EPV == 0) && ((uintptr_t)o.dst % 16 == 0) &&
+                 ((uintptr_t)o.addend % 16 == 0);
         if (o.len > max_len) max_len = o.len;
     }
     for (int w = 0; w < a.n; ++w) vec_ok = vec_ok && ((uintptr_t)a.src[w] % 16 == 0);
@@ -525,7 +534,7 @@ int launch_reduce(const ReduceArgs &a, const ReduceOuts &outs, int64_t outer, in
             int64_t gx = hapmi_cdiv(total, RED_THREADS);
             if (gx > 256 * 16) gx = 256 * 16;
             hipLaunchKernelGGL((ragged_reduce_scalar_kernel<T>), dim3((unsigned)gx), dim3(RED_THREADS), 0, stream, a,
-                               (T *)o.dst, outer, src_len, o.offset, o.len, inner);
+                               (T *)o.dst, (const T *)o.addend, outer, src_len, o.offset, o.len, inner);
         }
     }
     HAPMI_CHECK_LAUNCH("ragged_reduce");
@@ -534,18 +543,42 @@ int launch_reduce(const ReduceArgs &a, const ReduceOuts &outs, int64_t outer, in
 
 }  // namespace
 
+namespace {
+int reduce_multi(const void *const *contribs, int n_ranks, void *const *dsts, const void *const *addends,
+                 const int64_t *offsets, const int64_t *lengths, int n_outputs, int64_t outer, int64_t src_len,
+                 int64_t inner, int dtype, hapmi_stream_t stream);
+}
+
 extern "C" int hapmi_ragged_reduce(const void *const *contribs, int n_ranks, void *dst, int64_t outer,
                                    int64_t src_len, int64_t offset, int64_t len, int64_t inner, int dtype,
                                    hapmi_stream_t stream) {
     void *dsts[1] = {dst};
     const int64_t offs[1] = {offset}, lens[1] = {len};
-    return hapmi_ragged_reduce_multi(contribs, n_ranks, dsts, offs, lens, 1, outer, src_len, inner, dtype, stream);
+    return reduce_multi(contribs, n_ranks, dsts, nullptr, offs, lens, 1, outer, src_len, inner, dtype, stream);
+}
+
+extern "C" int hapmi_ragged_reduce_add(const void *const *contribs, int n_ranks, void *dst, const void *addend,
+                                       int64_t outer, int64_t src_len, int64_t offset, int64_t len, int64_t inner,
+                                       int dtype, hapmi_stream_t stream) {
+    HAPMI_REQUIRE(addend, HAPMI_EINVAL, "ragged_reduce_add: null addend");
+    void *dsts[1] = {dst};
+    const void *adds[1] = {addend};
+    const int64_t offs[1] = {offset}, lens[1] = {len};
+    return reduce_multi(contribs, n_ranks, dsts, adds, offs, lens, 1, outer, src_len, inner, dtype, stream);
 }
 
 extern "C" int hapmi_ragged_reduce_multi(const void *const *contribs, int n_ranks, void *const *dsts,
                                          const int64_t *offsets, const int64_t *lengths, int n_outputs,
                                          int64_t outer, int64_t src_len, int64_t inner, int dtype,
                                          hapmi_stream_t stream) {
+    return reduce_multi(contribs, n_ranks, dsts, nullptr, offsets, lengths, n_outputs, outer, src_len, inner, dtype,
+                        stream);
+}
+
+namespace {
+int reduce_multi(const void *const *contribs, int n_ranks, void *const *dsts, const void *const *addends,
+                 const int64_t *offsets, const int64_t *lengths, int n_outputs, int64_t outer, int64_t src_len,
+                 int64_t inner, int dtype, hapmi_stream_t stream) {
     HAPMI_REQUIRE(n_ranks >= 1 && n_ranks <= HAPMI_MAX_RANKS && contribs, HAPMI_EINVAL,
                   "ragged_reduce: n_ranks %d outside 1..%d", n_ranks, HAPMI_MAX_RANKS);
     HAPMI_REQUIRE(n_outputs >= 1 && n_outputs <= HAPMI_MAX_RANKS && dsts && offsets && lengths, HAPMI_EINVAL,
@@ -560,7 +593,7 @@ extern "C" int hapmi_ragged_reduce_multi(const void *const *contribs, int n_rank
                       (long long)(offsets[r] + lengths[r]), (long long)src_len);
         if (lengths[r] == 0 || outer == 0) continue;
         HAPMI_REQUIRE(dsts[r], HAPMI_EINVAL, "ragged_reduce: null destination");
-        outs.out[outs.n++] = ReduceOut{dsts[r], offsets[r], lengths[r]};
+        outs.out[outs.n++] = ReduceOut{dsts[r], offsets[r], lengths[r], addends ? addends[r] : nullptr};
     }
     if (outs.n == 0) return HAPMI_OK;
     ReduceArgs a;
@@ -572,6 +605,7 @@ extern "C" int hapmi_ragged_reduce_multi(const void *const *contribs, int n_rank
     if (dtype == HAPMI_F32) return launch_reduce<float>(a, outs, outer, src_len, inner, (hipStream_t)stream);
     return launch_reduce<bf16_t>(a, outs, outer, src_len, inner, (hipStream_t)stream);
 }
+}  // namespace
 
 extern "C" int hapmi_pad_rows_multi(const void *const *srcs, void *const *dsts, const int64_t *lengths, int n_shards,
                                     int64_t outer, int64_t padded_len, int64_t inner_bytes, hapmi_stream_t stream) {

@@ -1035,8 +1035,9 @@ class ShardExecutor:
         self._announce(tag, direction, rank, W, lambda dst: own, sink)        # the padded shard goes to every peer
         return full
 
-    def _emit_scatter(self, tag, direction, full_t, dim, L, rank, sink: List[Callable], out_t=None):
-        """split + pad -> [wire] -> rank-ordered float32 sum of the pieces for this rank, pad cut off."""
+    def _emit_scatter(self, tag, direction, full_t, dim, L, rank, sink: List[Callable], out_t=None, addend=None):
+        """split + pad -> [wire] -> rank-ordered float32 sum of the pieces for this rank, pad cut off; ``addend``
+        (the output's shape) is added to the sum in the same pass."""
         m, W = max(L), len(L)
         pshape = ops._with_dim(full_t.shape, dim, m)
         sent = [self._new(pshape, full_t.dtype) for _ in range(W)]
@@ -1044,7 +1045,8 @@ class ShardExecutor:
         contribs = [sent[rank] if s == rank else peers[s] for s in range(W)]
         contribs = [c for c in contribs if c is not None]
         out = out_t if out_t is not None else self._new(ops._with_dim(full_t.shape, dim, L[rank]), full_t.dtype)
-        sink.append(lambda: (ops.split_pad(full_t, L, dim, m, sent), ops.ragged_reduce(contribs, dim, 0, L[rank], out)))
+        sink.append(lambda: (ops.split_pad(full_t, L, dim, m, sent),
+                             ops.ragged_reduce(contribs, dim, 0, L[rank], out, addend=addend)))
         self._announce(tag, direction, rank, W, lambda dst: sent[dst], sink)  # the padded piece that rank dst reduces
         return out
 
@@ -1063,8 +1065,14 @@ class ShardExecutor:
             if x.grad is None:
                 x.grad = self._emit_scatter(node.name, "bwd", out.grad, dim, L, rank, self.bwd)
             else:
-                part = self._emit_scatter(node.name, "bwd", out.grad, dim, L, rank, self.bwd)
-                self._accumulate_into(x, part)
+                # d(x) += the reduced piece, in the reduction's own pass: in place, or into a new buffer while
+                # weight gradients that are held back still read the old one
+                g = x.grad
+                if self._is_read_later(g):
+                    x.grad = self._new(g.shape, g.dtype)
+                else:
+                    self._guard_write(g)
+                self._emit_scatter(node.name, "bwd", out.grad, dim, L, rank, self.bwd, out_t=x.grad, addend=g)
         self._tape.append(emit)
         return out
 

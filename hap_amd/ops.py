@@ -213,9 +213,10 @@ def concat_rows(pieces: Sequence[torch.Tensor], dim: int, out: Optional[torch.Te
 
 
 def ragged_reduce(contribs: Sequence[torch.Tensor], dim: int, offset: int, length: int,
-                  out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """out = sum_w contribs[w].narrow(dim, offset, length) in rank order, float32 accumulation."""
-    _dev(*contribs, out)
+                  out: Optional[torch.Tensor] = None, addend: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out = sum_w contribs[w].narrow(dim, offset, length) in rank order, float32 accumulation; ``addend`` (out's
+    shape, may be ``out``) is added to the sum last."""
+    _dev(*contribs, out, addend)
     ref = contribs[0]
     outer, src_len, inner = _oli(ref.shape, dim)
     if out is None:
@@ -227,7 +228,15 @@ def ragged_reduce(contribs: Sequence[torch.Tensor], dim: int, offset: int, lengt
     _need(out, outer * length * inner, "ragged_reduce dst")
     if out.dtype != ref.dtype:
         raise TypeError("ragged_reduce: dtype mismatch")
+    if addend is not None:
+        _need(addend, outer * length * inner, "ragged_reduce addend")
+        if addend.dtype != ref.dtype:
+            raise TypeError("ragged_reduce: dtype mismatch")
     if out.numel() == 0:
+        return out
+    if addend is not None:
+        check(lib().hapmi_ragged_reduce_add(_ptrs(contribs), len(contribs), _ptr(out), _ptr(addend), outer, src_len,
+                                            offset, length, inner, dtype_code(ref), _stream()))
         return out
     check(lib().hapmi_ragged_reduce(_ptrs(contribs), len(contribs), _ptr(out), outer, src_len, offset, length, inner,
                                     dtype_code(ref), _stream()))

@@ -104,6 +104,13 @@ int hapmi_concat_rows(const void *const *pieces_host, const int64_t *lengths_hos
 int hapmi_ragged_reduce(const void *const *contribs_host, int n_ranks, void *dst, int64_t outer, int64_t src_len,
                         int64_t offset, int64_t len, int64_t inner, int dtype, hapmi_stream_t stream);
 
+/* hapmi_ragged_reduce with one more term, added last: dst = addend + sum_w contribs[w][...]; addend has dst's
+ * layout and may be dst itself.  The gradient that all_gather's backward (collectives.py:63-68) contributes
+ * to a value that already holds a gradient from another consumer, in one pass. */
+int hapmi_ragged_reduce_add(const void *const *contribs_host, int n_ranks, void *dst, const void *addend,
+                            int64_t outer, int64_t src_len, int64_t offset, int64_t len, int64_t inner, int dtype,
+                            hapmi_stream_t stream);
+
 /* The same sum for several output shards in ONE launch (every rank's piece of a reduce_scatter when the
  * ranks' tensors share one device): dsts[r][outer, lengths[r], inner] = sum_w contribs[w][:, offsets[r]:offsets[r]+lengths[r], :]. */
 int hapmi_ragged_reduce_multi(const void *const *contribs_host, int n_ranks, void *const *dsts_host,

@@ -112,6 +112,17 @@ def test_ragged_reduce_bit_exact(cuda, dtype, W, shape, dim, off, length):
     got = ops.ragged_reduce([p.to(cuda) for p in parts], dim, off, length)
     want = _accumulate([p.narrow(dim, off, length) for p in parts])
     assert torch.equal(got.cpu(), want)
+    # one more term of the output's shape, added last: into a separate output and in place
+    g0 = torch.randn(want.shape, generator=g).to(dtype)
+    acc = parts[0].narrow(dim, off, length).float()
+    for p in parts[1:]:
+        acc = acc + p.narrow(dim, off, length).float()
+    want_add = (acc + g0.float()).to(dtype)
+    got_add = ops.ragged_reduce([p.to(cuda) for p in parts], dim, off, length, addend=g0.to(cuda))
+    assert torch.equal(got_add.cpu(), want_add)
+    inplace = g0.to(cuda)
+    ops.ragged_reduce([p.to(cuda) for p in parts], dim, off, length, out=inplace, addend=inplace)
+    assert torch.equal(inplace.cpu(), want_add)
 
 
 def test_config5_shapes_round_trip_and_reduce(cuda):
