@@ -284,33 +284,13 @@ __global__ __launch_bounds__(AT_THREADS, 2) void attn_fwd_kernel(const bf16_t *q
     }
 }
 
-// delta[b, h, q] = sum_d dO[b, q, h, d] * O[b, q, h, d]
-__global__ __launch_bounds__(256) void attn_delta_kernel(const bf16_t *out, const bf16_t *dout, float *delta, int64_t rows,
-                                                       int S, int H) {
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;        // (b, q, h)
-    if (i >= rows * H) return;
-    const int64_t row = i / H;
-    const int hh = (int)(i % H);
-    const frag_t *o = (const frag_t *)(out + row * H * HD + hh * HD);
-    const frag_t *d = (const frag_t *)(dout + row * H * HD + hh * HD);
-    float acc = 0.f;
-#pragma unroll
-    for (int k = 0; k < 8; ++k) {
-        const frag_t a = o[k], g = d[k];
-#pragma unroll
-        for (int e = 0; e < 8; ++e) acc += (float)a.v[e] * (float)g.v[e];
-    }
-    const int64_t bidx = row / S, q = row % S;
-    delta[(bidx * H + hh) * S + q] = acc;
-}
-
 // ---------------------------------------------------------------------------------------------
 // dQ: lanes own query columns, kv tiles are streamed
 // ---------------------------------------------------------------------------------------------
 template <bool CAUSAL>
-__global__ __launch_bounds__(AT_THREADS, 2) void attn_bwd_dq_kernel(const bf16_t *qkv, const bf16_t *dout, const float *lse,
-                                                               const float *delta, const float *mask, bf16_t *dqkv,
-                                                               int S, int H, float scale) {
+__global__ __launch_bounds__(AT_THREADS, 2) void attn_bwd_dq_kernel(const bf16_t *qkv, const bf16_t *out, const bf16_t *dout,
+                                                               const float *lse, float *delta, const float *mask,
+                                                               bf16_t *dqkv, int S, int H, float scale) {
     __shared__ __attribute__((aligned(16))) char Ks[TILE_BYTES];
     __shared__ __attribute__((aligned(16))) char Vs[TILE_BYTES];
     const TransposedReader tr;
@@ -331,7 +311,20 @@ __global__ __launch_bounds__(AT_THREADS, 2) void attn_bwd_dq_kernel(const bf16_t
         dof[s] = load_row_frag(dO + (int64_t)q * E, qok, s, h);
     }
     const float lse_q = qok ? lse[((int64_t)b * H + hh) * S + q] : 0.f;
-    const float delta_q = qok ? delta[((int64_t)b * H + hh) * S + q] : 0.f;
+    // delta[b, h, q] = sum_d dO[q, d] * O[q, d]: each lane holds half of its query's dO row; the dK / dV kernel,
+    // launched after this one, reads the values written here
+    float delta_q = 0.f;
+    {
+        const bf16_t *O = out + (int64_t)b * S * E + hh * HD;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            const frag_t of = load_row_frag(O + (int64_t)q * E, qok, s, h);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) delta_q += (float)of.v[e] * (float)dof[s].v[e];
+        }
+        delta_q += __shfl_xor(delta_q, 32, 64);
+        if (qok && h == 0) delta[((int64_t)b * H + hh) * S + q] = delta_q;
+    }
     f32x16 dqt[2] = {zero16(), zero16()};
     PairLoader lk(ld), lv(ld);
     const bool vec_mask = mask && ((S & 3) == 0);
@@ -575,17 +568,15 @@ extern "C" int hapmi_attention_bwd(const void *qkv, const void *out, const void 
                       ((uintptr_t)dqkv % 16) == 0 && (!mask || ((uintptr_t)mask % 16) == 0),
                   HAPMI_EALIGN, "attention_bwd: pointers must be 16-byte aligned");
     hipStream_t st = (hipStream_t)stream;
-    hipLaunchKernelGGL(attn_delta_kernel, dim3((unsigned)hapmi_cdiv(b * S * H, 256)), dim3(256), 0, st,
-                       (const bf16_t *)out, (const bf16_t *)dout, delta_ws, b * S, (int)S, (int)H);
     dim3 grid((unsigned)hapmi_cdiv(S, 128), (unsigned)(b * H));
     if (causal) {
-        hipLaunchKernelGGL(attn_bwd_dq_kernel<true>, grid, dim3(AT_THREADS), 0, st, (const bf16_t *)qkv, (const bf16_t *)dout,
-                           lse, (const float *)delta_ws, (const float *)nullptr, (bf16_t *)dqkv, (int)S, (int)H, scale);
+        hipLaunchKernelGGL(attn_bwd_dq_kernel<true>, grid, dim3(AT_THREADS), 0, st, (const bf16_t *)qkv, (const bf16_t *)out,
+                           (const bf16_t *)dout, lse, delta_ws, (const float *)nullptr, (bf16_t *)dqkv, (int)S, (int)H, scale);
         hipLaunchKernelGGL(attn_bwd_dkv_kernel<true>, grid, dim3(AT_THREADS), 0, st, (const bf16_t *)qkv, (const bf16_t *)dout,
                            lse, (const float *)delta_ws, (const float *)nullptr, (bf16_t *)dqkv, (int)S, (int)H, scale);
     } else {
-        hipLaunchKernelGGL(attn_bwd_dq_kernel<false>, grid, dim3(AT_THREADS), 0, st, (const bf16_t *)qkv, (const bf16_t *)dout,
-                           lse, (const float *)delta_ws, mask, (bf16_t *)dqkv, (int)S, (int)H, scale);
+        hipLaunchKernelGGL(attn_bwd_dq_kernel<false>, grid, dim3(AT_THREADS), 0, st, (const bf16_t *)qkv, (const bf16_t *)out,
+                           (const bf16_t *)dout, lse, delta_ws, mask, (bf16_t *)dqkv, (int)S, (int)H, scale);
         hipLaunchKernelGGL(attn_bwd_dkv_kernel<false>, grid, dim3(AT_THREADS), 0, st, (const bf16_t *)qkv, (const bf16_t *)dout,
                            lse, (const float *)delta_ws, mask, (bf16_t *)dqkv, (int)S, (int)H, scale);
     }
