@@ -252,19 +252,24 @@ class ShardExecutor:
         """dW[n_out, n_in] (+)= dy[rows, n_out]^T x[rows, n_in], the bias gradient gb (column sums of dy) taken by
         the same kernel.  Launched at once, or held back to share a launch with the same linear of the next
         layers (only for parameters with a single use: their gradient is written once, order does not matter)."""
-        single_use = all(v is None or v.meta.get("name") in self._single_use_params for v in params)
-        if self.wgrad_group <= 1 or not single_use:
+        if not self._holds_back_wgrad(params):
             self.bwd.append(lambda: ops.gemm(dy, xt, gw, n_out, n_in, rows, transA=True, lda=ld_dy, ldb=ld_x,
                                              accumulate=acc, a_rowsum=gb))
             return
         sig = (n_out, n_in, rows, ld_dy, ld_x, bool(acc), dy.dtype, gw.dtype)
         q = self._pending_wgrads.setdefault(sig, [])
-        q.append((dy, xt, gw, gb, [v.meta["name"] for v in params if v is not None]))
+        q.append((dy, xt, gw, gb, [v.meta.get("name") or v.meta.get("shard_of") for v in params if v is not None], []))
         for t in (dy, xt):
             k = t.untyped_storage().data_ptr()
             self._deferred_reads[k] = self._deferred_reads.get(k, 0) + 1
         if len(q) >= self.wgrad_group:
             self._flush_wgrads(sig)
+
+    def _holds_back_wgrad(self, params) -> bool:
+        """Whether the weight gradient of these parameters (weight, bias) is held back for a shared launch: only when
+        each is used once in the program, so that its gradient is written once and the order does not matter."""
+        return self.wgrad_group > 1 and all(
+            v is None or v.meta.get("name") in self._single_use_params or v.meta.get("single_use") for v in params)
 
     def _flush_wgrads(self, sig=None):
         """Append the launches of the weight gradients held back (of one signature, or all)."""
@@ -273,18 +278,32 @@ class ShardExecutor:
             if not q:
                 continue
             n_out, n_in, rows, ld_dy, ld_x, acc = key[:6]
-            for dy, xt, _, _, _ in q:
+            for dy, xt, _, _, _, _ in q:
                 for t in (dy, xt):
                     self._deferred_reads[t.untyped_storage().data_ptr()] -= 1
             self.bwd.append(self._wgrad_launch(q, n_out, n_in, rows, ld_dy, ld_x, acc))
             for e in q:
+                for hook in e[5]:
+                    hook()                               # launches that wait for this weight gradient
+            for e in q:
                 for name in e[4]:
                     self._grad_final_idx[name] = len(self.bwd)
+
+    def _after_wgrad(self, grad_t: torch.Tensor, fn: Callable[[], None]):
+        """Run ``fn`` (which appends launches that read the gradient buffer ``grad_t``) once the weight gradient
+        that writes ``grad_t`` has been appended: now, or when the group that holds it back is launched."""
+        key = grad_t.data_ptr()                          # gradient buffers are views of one flat buffer
+        for q in self._pending_wgrads.values():
+            for e in q:
+                if any(t is not None and t.data_ptr() == key for t in (e[2], e[3])):
+                    e[5].append(fn)
+                    return
+        fn()
 
     @staticmethod
     def _wgrad_launch(q, n_out, n_in, rows, ld_dy, ld_x, acc):
         if len(q) == 1:
-            dy, xt, gw, gb, _ = q[0]
+            dy, xt, gw, gb = q[0][:4]
             return lambda: ops.gemm(dy, xt, gw, n_out, n_in, rows, transA=True, lda=ld_dy, ldb=ld_x, accumulate=acc,
                                     a_rowsum=gb)
         dys, xts, gws = [e[0] for e in q], [e[1] for e in q], [e[2] for e in q]
@@ -822,8 +841,7 @@ class ShardExecutor:
             do = out_bsd.grad
             dctx = self._scratch("attn_dctx", (b, S, Ea))
             side = self._side_ok(w_out, b_out, w_in, b_in)
-            held = (not side and self.wgrad_group > 1
-                    and all(v is None or v.meta.get("name") in self._single_use_params for v in (w_in, b_in)))
+            held = not side and self._holds_back_wgrad((w_in, b_in))
             # the in-projection's weight gradient reads dqkv from the side stream, or later together with the next
             # layers' (wgrad_group), so it cannot be shared scratch then
             dqkv = self._new((b, S, 3 * Ea)) if (side or held) else self._scratch("attn_dqkv", (b, S, 3 * Ea))
@@ -1088,7 +1106,8 @@ class ShardExecutor:
         src = x.meta["master"] if vector else x.t
         full = self._emit_gather(node.name, "fwd", src, 0, L, rank, self.fwd)
         full_grad = self._gathered_grads[x.meta["name"]]
-        out = Val("param", full, master=full if vector else None, grad=full_grad, needs_grad=True, shard_of=x.meta["name"])
+        out = Val("param", full, master=full if vector else None, grad=full_grad, needs_grad=True, shard_of=x.meta["name"],
+                  single_use=len(node.users) == 1)
 
         def emit():
             if not out.meta.get("grad_written"):
@@ -1096,8 +1115,9 @@ class ShardExecutor:
             x.meta["grad_written"] = True
             if self._touched is not None:
                 self._touched.append(x.meta["name"])
-            self._flush_wgrads()                         # the consumers' weight gradients write full_grad
-            self._emit_scatter(node.name, "bwd", full_grad, 0, L, rank, self.bwd, out_t=x.meta["grad"])
+            # the consumer's weight gradient writes full_grad; it may be held back to share a launch with later layers
+            self._after_wgrad(full_grad, lambda: self._emit_scatter(node.name, "bwd", full_grad, 0, L, rank, self.bwd,
+                                                                    out_t=x.meta["grad"]))
         self._tape.append(emit)
         return out
 

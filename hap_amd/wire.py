@@ -16,6 +16,7 @@ exact (unpadded) extents; that transport is not part of this package.
 """
 from __future__ import annotations
 
+import zlib
 from typing import Dict, Optional, Tuple
 
 import torch
@@ -58,7 +59,7 @@ class SyntheticWire(Wire):
                  share_shapes: bool = False):
         """``share_shapes``: messages of equal shape, direction and sender reuse one buffer (a benchmark with
         many identical layers then needs one set of peer buffers instead of one per layer)."""
-        self.gen = torch.Generator().manual_seed(seed)
+        self.seed = int(seed)
         self.scale, self.grad_scale = scale, grad_scale
         self.reduce_params = reduce_params
         self.share_shapes = share_shapes
@@ -70,7 +71,10 @@ class SyntheticWire(Wire):
         key = (direction, src, tuple(shape), dtype) if self.share_shapes else (tag, direction, src)
         if key not in self._cache:
             s = self.scale if direction == "fwd" else self.grad_scale
-            t = torch.randn(tuple(shape), generator=self.gen, dtype=torch.float32) * s
+            # one stream of random numbers per message, so that the content does not depend on the order in which
+            # the executor asks for its buffers
+            gen = torch.Generator().manual_seed((self.seed * 1000003 + zlib.crc32(repr(key).encode())) % (1 << 63))
+            t = torch.randn(tuple(shape), generator=gen, dtype=torch.float32) * s
             self._cache[key] = t.to(dtype).to(device)
         return self._cache[key]
 
