@@ -1045,11 +1045,16 @@ class ShardExecutor:
         """pad own shard -> [wire] -> cut pads and concatenate.  Returns the full tensor."""
         m, W = max(L), len(L)
         pshape = ops._with_dim(x_t.shape, dim, m)
-        own = self._new(pshape, x_t.dtype)
+        # a shard of the longest length needs no padding: the tensor itself is the message
+        unpadded = L[rank] == m and x_t.is_contiguous() and tuple(x_t.shape) == tuple(pshape)
+        own = x_t if unpadded else self._new(pshape, x_t.dtype)
         peers = self._peers(tag, direction, rank, W, pshape, False, x_t.dtype)
         slices = [own if s == rank else peers[s] for s in range(W)]
         full = self._new(ops._with_dim(x_t.shape, dim, sum(L)), x_t.dtype)
-        sink.append(lambda: (ops.pad_rows(x_t, dim, m, own), ops.unpad_concat(slices, L, dim, full)))
+        if unpadded:
+            sink.append(lambda: ops.unpad_concat(slices, L, dim, full))
+        else:
+            sink.append(lambda: (ops.pad_rows(x_t, dim, m, own), ops.unpad_concat(slices, L, dim, full)))
         self._announce(tag, direction, rank, W, lambda dst: own, sink)        # the padded shard goes to every peer
         return full
 
