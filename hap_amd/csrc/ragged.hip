@@ -334,8 +334,12 @@ extern "C" int hapmi_concat_rows(const void *const *pieces, const int64_t *lengt
     for (int i = 0; i < n_ranks; ++i) {
         if (lengths[i] > 0 && outer > 0) {
             HAPMI_REQUIRE(pieces[i] && dst, HAPMI_EINVAL, "concat_rows: null pointer");
-            list.seg[list.n++] = {(const char *)pieces[i], (char *)dst + off * inner_bytes, outer,
-                                  lengths[i] * inner_bytes, lengths[i] * inner_bytes, total * inner_bytes};
+            // a piece that was produced at its place in dst (outer = 1: the place is one contiguous range) stays
+            const bool in_place = act == HAPMI_ACT_NONE && outer == 1 &&
+                                  (const char *)pieces[i] == (const char *)dst + off * inner_bytes;
+            if (!in_place)
+                list.seg[list.n++] = {(const char *)pieces[i], (char *)dst + off * inner_bytes, outer,
+                                      lengths[i] * inner_bytes, lengths[i] * inner_bytes, total * inner_bytes};
         }
         off += lengths[i];
     }

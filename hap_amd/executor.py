@@ -1149,10 +1149,15 @@ class ShardExecutor:
         # pieces along the slowest dimension are contiguous ranges of the input: views, as torch.split gives the
         # reference (collectives.py:156); any other dimension needs the strided copy
         views = split_dim == 0 and x_t.is_contiguous()
+        own_shape = ops._with_dim(x_t.shape, split_dim, split_L[rank])
+        out = self._new(ops._with_dim(own_shape, cat_dim, sum(cat_L)))
         if views:
             pieces = list(torch.split(x_t, list(split_L), 0))
         else:
             pieces = [self._new(ops._with_dim(x_t.shape, split_dim, l)) for l in split_L]
+            if cat_dim == 0:
+                # the copying split writes this rank's own piece straight to its rows of the concatenation
+                pieces[rank] = out.narrow(0, sum(cat_L[:rank]), cat_L[rank])
         own = pieces[rank]
         parts = []
         for src in range(W):
@@ -1161,7 +1166,6 @@ class ShardExecutor:
             else:
                 shape = ops._with_dim(own.shape, cat_dim, cat_L[src])
                 parts.append(self.wire.recv(tag, direction, src, shape, self.cdt, self.dev, reduction=False))
-        out = self._new(ops._with_dim(own.shape, cat_dim, sum(cat_L)))
         if views:
             sink.append(lambda: ops.concat_rows(parts, cat_dim, out, act))
         else:

@@ -94,7 +94,8 @@ int hapmi_split_rows_relu_bwd(const void *src, const void *fwd_out, void *const 
 
 /* collectives.py:159 / :166: concatenate W contiguous pieces [outer, lengths[i], inner]
  * into dst[outer, sum(lengths), inner]; `act` != NONE applies the activation to
- * every element on the way (dtype needed then). */
+ * every element on the way (dtype needed then).  A piece that already lies at its place in dst
+ * (act = NONE, outer = 1 and pieces[i] == dst + offset of piece i) is left where it is. */
 int hapmi_concat_rows(const void *const *pieces_host, const int64_t *lengths_host, int n_ranks, void *dst,
                       int64_t outer, int64_t inner_bytes, int act, int dtype, hapmi_stream_t stream);
 

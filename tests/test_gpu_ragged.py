@@ -68,6 +68,22 @@ def test_pad_split_concat_slice_layouts(cuda, dtype, shape, dim, L):
         assert torch.equal(back.cpu(), want)
 
 
+def test_concat_leaves_a_piece_that_is_already_in_place(cuda):
+    g = torch.Generator().manual_seed(4)
+    pieces = [torch.randn(n, 24, generator=g).bfloat16().to(cuda) for n in (3, 5, 2)]
+    out = torch.full((10, 24), 7.0, dtype=torch.bfloat16, device=cuda)
+    mine = out.narrow(0, 3, 5)
+    mine.copy_(pieces[1])
+    ops.concat_rows([pieces[0], mine, pieces[2]], 0, out)
+    assert torch.equal(out, torch.cat(pieces, dim=0))
+    # with an activation the piece in place is processed like the others
+    out2 = torch.empty(10, 24, dtype=torch.bfloat16, device=cuda)
+    mine2 = out2.narrow(0, 3, 5)
+    mine2.copy_(pieces[1])
+    ops.concat_rows([pieces[0], mine2, pieces[2]], 0, out2, act="relu")
+    assert torch.equal(out2, torch.relu(torch.cat(pieces, dim=0)))
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 def test_concat_with_fused_relu(cuda, dtype):
     g = torch.Generator().manual_seed(3)
