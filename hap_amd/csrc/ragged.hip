@@ -6,6 +6,7 @@
 namespace {
 
 int g_grid_shift = 2;      // grid cap = 4096 << shift blocks (hapmi_ragged_tuning changes it for measurements)
+bool g_copy_nt = false;    // measurement hook: streaming loads in the plain 16-byte segment copy
 
 struct Segment {
     const char *src;
@@ -81,7 +82,7 @@ struct ReluF32 {
 constexpr int COPY_THREADS = 256;
 constexpr int COPY_UNROLL = 4;
 
-template <typename V, typename Act>
+template <typename V, typename Act, bool NT = false>
 __global__ __launch_bounds__(COPY_THREADS) void segment_copy_kernel(SegmentList list, Act act) {
     const Segment s = list.seg[blockIdx.y];
     const uint64_t per_row = (uint64_t)s.row_bytes / sizeof(V);
@@ -108,7 +109,10 @@ __global__ __launch_bounds__(COPY_THREADS) void segment_copy_kernel(SegmentList 
             }
             doff[u] = row * (uint64_t)s.dst_stride + col * sizeof(V);
             const char *from = s.src + row * (uint64_t)s.src_stride + col * sizeof(V);
-            if (ok[u]) v[u] = *(const V *)from;
+            if (ok[u]) {
+                if constexpr (NT) v[u] = __builtin_nontemporal_load((const V *)from);
+                else v[u] = *(const V *)from;
+            }
             if constexpr (Act::MASKED)
                 if (ok[u]) y[u] = *(const V *)(from + act.delta);
         }
@@ -161,6 +165,8 @@ int launch_segments(const SegmentList &list, int act, int dtype, hipStream_t str
             hipLaunchKernelGGL((segment_copy_kernel<u32x4, ReluBf16>), grid, block, 0, stream, list, ReluBf16());
         else
             hipLaunchKernelGGL((segment_copy_kernel<u32x4, ReluF32>), grid, block, 0, stream, list, ReluF32());
+    } else if (vec == 16 && g_copy_nt) {
+        hipLaunchKernelGGL((segment_copy_kernel<u32x4, ActNone<u32x4>, true>), grid, block, 0, stream, list, ActNone<u32x4>());
     } else if (vec == 16) {
         hipLaunchKernelGGL((segment_copy_kernel<u32x4, ActNone<u32x4>>), grid, block, 0, stream, list, ActNone<u32x4>());
     } else if (vec == 4) {
@@ -358,7 +364,10 @@ struct ReduceArgs {
 
 constexpr int RED_THREADS = 256;
 
-int g_red_variant = 0;      // measurement hook: bit0 nontemporal loads, bit1 nontemporal store, bit2 two vectors per thread
+// bit0 nontemporal loads, bit1 nontemporal store, bit2 two vectors per thread.  Measured on eight contributions of
+// 131 MB: plain 5.2 TB/s, streaming loads 5.7-6.0, with two vectors per thread 6.1; streaming stores lose 0.2
+constexpr int RED_VARIANT_DEFAULT = 5;
+int g_red_variant = RED_VARIANT_DEFAULT;
 
 struct ReduceOut {
     void *dst;
@@ -370,17 +379,19 @@ struct ReduceOuts {
     ReduceOut out[HAPMI_MAX_RANKS];
 };
 
-template <typename T> __device__ __forceinline__ Vec16<T> ldv(const T *p, bool nt) {
+// NT is a template parameter on purpose: a run-time choice between the two kinds of access compiles to the plain one
+template <typename T, bool NT> __device__ __forceinline__ Vec16<T> ldv(const T *p) {
     typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
     union { u32x4 u; Vec16<T> v; } x;
-    x.u = nt ? __builtin_nontemporal_load((const u32x4 *)p) : *(const u32x4 *)p;
+    if constexpr (NT) x.u = __builtin_nontemporal_load((const u32x4 *)p);
+    else x.u = *(const u32x4 *)p;
     return x.v;
 }
-template <typename T> __device__ __forceinline__ void stv(T *p, const Vec16<T> &v, bool nt) {
+template <typename T, bool NT> __device__ __forceinline__ void stv(T *p, const Vec16<T> &v) {
     typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
     union { u32x4 u; Vec16<T> v; } x;
     x.v = v;
-    if (nt) __builtin_nontemporal_store(x.u, (u32x4 *)p);
+    if constexpr (NT) __builtin_nontemporal_store(x.u, (u32x4 *)p);
     else *(u32x4 *)p = x.u;
 }
 
@@ -421,7 +432,7 @@ __global__ __launch_bounds__(RED_THREADS) void ragged_reduce_kernel(ReduceArgs a
             for (int u = 0; u < U; ++u)
 #pragma unroll
                 for (int w = 0; w < NW; ++w)
-                    if (ok[u]) v[u][w] = ldv((const T *)a.src[w] + soff[u], NTL);
+                    if (ok[u]) v[u][w] = ldv<T, NTL>((const T *)a.src[w] + soff[u]);
 #pragma unroll
             for (int u = 0; u < U; ++u) {
 #pragma unroll
@@ -435,11 +446,11 @@ __global__ __launch_bounds__(RED_THREADS) void ragged_reduce_kernel(ReduceArgs a
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 if (!ok[u]) continue;
-                Vec16<T> v = ldv((const T *)a.src[0] + soff[u], NTL);
+                Vec16<T> v = ldv<T, NTL>((const T *)a.src[0] + soff[u]);
 #pragma unroll
                 for (int e = 0; e < EPV; ++e) acc[u][e] = v.get(e);
                 for (int w = 1; w < nw; ++w) {
-                    v = ldv((const T *)a.src[w] + soff[u], NTL);
+                    v = ldv<T, NTL>((const T *)a.src[w] + soff[u]);
 #pragma unroll
                     for (int e = 0; e < EPV; ++e) acc[u][e] += v.get(e);
                 }
@@ -449,14 +460,14 @@ __global__ __launch_bounds__(RED_THREADS) void ragged_reduce_kernel(ReduceArgs a
         for (int u = 0; u < U; ++u) {
             if (!ok[u]) continue;
             if (addend) {
-                const Vec16<T> g = ldv(addend + doff[u], NTL);
+                const Vec16<T> g = ldv<T, NTL>(addend + doff[u]);
 #pragma unroll
                 for (int e = 0; e < EPV; ++e) acc[u][e] += g.get(e);
             }
             Vec16<T> r;
 #pragma unroll
             for (int e = 0; e < EPV; ++e) r.set(e, acc[u][e]);
-            stv(dst + doff[u], r, NTS);
+            stv<T, NTS>(dst + doff[u], r);
         }
     }
 }
@@ -632,7 +643,8 @@ extern "C" int hapmi_pad_rows_multi(const void *const *srcs, void *const *dsts, 
 }
 
 extern "C" int hapmi_ragged_tuning(int reduce_variant, int grid_shift) {
-    g_red_variant = reduce_variant < 0 ? 0 : (reduce_variant & 7);
+    g_red_variant = reduce_variant < 0 ? RED_VARIANT_DEFAULT : (reduce_variant & 7);
+    g_copy_nt = reduce_variant >= 0 && (reduce_variant & 8);
     g_grid_shift = grid_shift < 0 ? 2 : (grid_shift & 7);
     return HAPMI_OK;
 }

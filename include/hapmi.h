@@ -123,7 +123,8 @@ int hapmi_pad_rows_multi(const void *const *srcs_host, void *const *dsts_host, c
                          int64_t outer, int64_t padded_len, int64_t inner_bytes, hapmi_stream_t stream);
 
 /* Tuning hook for measurements of the kernels above: reduce_variant bit 0 / 1 = non-temporal loads / stores,
- * bit 2 = two vectors per thread; grid_shift caps the grid at 4096 << shift blocks; -1 = defaults (0, 2). */
+ * bit 2 = two vectors per thread, bit 3 = non-temporal loads in the plain 16-byte segment copy; grid_shift caps the
+ * grid at 4096 << shift blocks; -1 = defaults (reduce: non-temporal loads, two vectors per thread; copy: plain; 2). */
 int hapmi_ragged_tuning(int reduce_variant, int grid_shift);
 
 /* ---- GEMM: F.linear (hap.rs:1032) and the expert einsums (hap.rs:2273) --
