@@ -270,7 +270,9 @@ def test_hip_graph_replays_equal_eager_steps(cuda, dtype, opt):
         torch.cuda.synchronize()
         losses.append(replay().item())
         assert torch.isfinite(junk).all()
-    assert losses == pytest.approx(ref_losses, rel=1e-6)
+    # the two executors are separate runs: their atomically summed bias / embedding gradients differ in the last bits,
+    # and Adam's updates of near-zero-gradient elements then differ by +-lr, which the later losses see at this level
+    assert losses == pytest.approx(ref_losses, rel=1e-6 if dtype == "fp32" else 2e-5)
     # Bias and embedding gradients are summed with float atomics, so two runs agree only up to summation order;
     # Adam turns that rounding noise into +-lr where the true gradient is zero (the key bias), so those elements
     # are left out of the parameter comparison.
