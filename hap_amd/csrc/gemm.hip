@@ -280,8 +280,8 @@ extern "C" int hapmi_gemm(const hapmi_gemm_args *a, hapmi_stream_t stream) {
         p.listRS[z] = on && a->a_rowsum_list ? a->a_rowsum_list[z] : nullptr;
     }
     p.relu_mask = a->c_relu_mask;
-    HAPMI_REQUIRE(!a->c_relu_mask || (a->batch1 * a->batch2 == 1 && ((uintptr_t)a->c_relu_mask % 16) == 0), HAPMI_EINVAL,
-                  "gemm: c_relu_mask needs a single problem and a 16-byte aligned pointer");
+    HAPMI_REQUIRE(!a->c_relu_mask || (!lists && ((uintptr_t)a->c_relu_mask % 16) == 0), HAPMI_EINVAL,
+                  "gemm: c_relu_mask needs a 16-byte aligned pointer and no pointer lists");
 
     hipStream_t st = (hipStream_t)stream;
     hipEvent_t e0 = nullptr, e1 = nullptr;

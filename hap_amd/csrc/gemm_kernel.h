@@ -97,6 +97,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, ((WAVES_M * WAVES_N <= 4 && 
     const TI *B = (const TI *)p.B;
     TO *C = (TO *)p.C;
     float *rowsum = p.rowsum;
+    const TO *rmask = (const TO *)p.relu_mask;                    // laid out like C, batch strides included
     if (p.n_list > 0) {                                           // uniform: scalar loads from the argument block
         const int z = (int)blockIdx.z;
         A = (const TI *)p.listA[z];
@@ -109,6 +110,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, ((WAVES_M * WAVES_N <= 4 && 
         A += z1 * p.sA1 + z2 * p.sA2;
         B += z1 * p.sB1 + z2 * p.sB2;
         C += z1 * p.sC1 + z2 * p.sC2;
+        if (rmask) rmask += z1 * p.sC1 + z2 * p.sC2;
     }
 
     // accumulate reads the old values `old_delta` bytes from where the result goes (0: in place)
@@ -397,7 +399,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, ((WAVES_M * WAVES_N <= 4 && 
                     *(bf16x4 *)(stage + (lane & 31) * SROWH + (j * 32 + q * 8 + (lane >> 5) * 4) * 2) = o;
                 }
             bf16_t *band = (bf16_t *)C + (m0 + wm + i * 32) * p.ldc + n0 + wn;
-            const bf16_t *mband = p.relu_mask ? (const bf16_t *)p.relu_mask + (m0 + wm + i * 32) * p.ldc + n0 + wn : nullptr;
+            const bf16_t *mband = rmask ? (const bf16_t *)rmask + (m0 + wm + i * 32) * p.ldc + n0 + wn : nullptr;
             if (interior && mband) {
                 // the producer of this operand's gradient applied relu itself: its output is the mask
 #pragma unroll
@@ -473,8 +475,8 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, ((WAVES_M * WAVES_N <= 4 && 
                     continue;
                 }
                 TO *dst = band + row * (int)p.ldc + qc * 4;
-                if (p.relu_mask) {
-                    const out4_t mk = *(const out4_t *)((const TO *)p.relu_mask + (mb + row) * p.ldc + nb + qc * 4);
+                if (rmask) {
+                    const out4_t mk = *(const out4_t *)(rmask + (mb + row) * p.ldc + nb + qc * 4);
 #pragma unroll
                     for (int e = 0; e < 4; ++e) v[e] = (float)mk[e] > 0.f ? v[e] : 0.f;
                 }
@@ -504,8 +506,8 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, ((WAVES_M * WAVES_N <= 4 && 
             }
             TO *dst = C + m * p.ldc + n;
             f32x4 vm = v;
-            if (p.relu_mask) {
-                const TO *mk = (const TO *)p.relu_mask + m * p.ldc + n;
+            if (rmask) {
+                const TO *mk = rmask + m * p.ldc + n;
 #pragma unroll
                 for (int e = 0; e < 4; ++e)
                     if (n + e < p.N && !((float)mk[e] > 0.f)) vm[e] = 0.f;

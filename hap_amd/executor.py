@@ -726,10 +726,12 @@ class ShardExecutor:
         self._tape.append(emit)
         return out
 
-    def _only_reader(self, node, x: Val) -> bool:
-        """True when ``node`` is the only consumer of the value ``x``, followed back through the nodes that pass
-        it on unchanged (the relu a producer already applied, dropout with p = 0)."""
-        n = node.args[0]
+    def _only_reader(self, node, x: Val, arg: int = 0) -> bool:
+        """True when ``node`` is the only consumer of the value ``x`` (its argument number ``arg``), followed back
+        through the nodes that pass it on unchanged (the relu a producer already applied, dropout with p = 0)."""
+        n = node.args[arg]
+        if not (isinstance(n, torch.fx.Node) and self.env.get(n) is x):
+            return False
         while isinstance(n, torch.fx.Node) and self.env.get(n) is x:
             if len(n.users) != 1:
                 return False
@@ -1352,8 +1354,15 @@ class ShardExecutor:
                                              accumulate=accw))
             if x.needs_grad:
                 gx, accx = self._grad_slot(x)
+                # the first expert GEMM applied relu itself and this one is its only reader: the data gradient
+                # leaves the GEMM masked (every expert's mask lies at its output's offset)
+                mask = None
+                if (self.relu_mask_in_dgrad and x.meta.get("fused_act") == "relu" and not accx and self._only_reader(node, x, arg=2)
+                        and not x.meta.get("relu_bwd_done")):
+                    mask = x.t
+                    x.meta["relu_bwd_done"] = True
                 self.bwd.append(lambda: ops.gemm(dy, w.t, gx, M, K, N, transB=True, batch1=E_loc, strideA=(M * N, 0),
-                                                 strideB=(K * N, 0), strideC=(M * K, 0), accumulate=accx))
+                                                 strideB=(K * N, 0), strideC=(M * K, 0), accumulate=accx, relu_mask=mask))
         self._tape.append(emit)
         return out
 

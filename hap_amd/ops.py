@@ -348,9 +348,9 @@ def gemm(A: torch.Tensor, B: torch.Tensor, C: torch.Tensor, M: int, N: int, K: i
         _need(a_rowsum, M, "gemm a_rowsum")
     a.a_rowsum = a_rowsum.data_ptr() if a_rowsum is not None else 0
     if relu_mask is not None:
-        if relu_mask.dtype != C.dtype or batch1 * batch2 != 1:
-            raise TypeError("gemm relu_mask: C's element type and a single problem expected")
-        _need(relu_mask, _span(M, N, a.ldc), "gemm relu_mask")
+        if relu_mask.dtype != C.dtype:
+            raise TypeError("gemm relu_mask: C's element type expected")
+        _need(relu_mask, _span(M, N, a.ldc) + zb(strideC), "gemm relu_mask")
     a.c_relu_mask = relu_mask.data_ptr() if relu_mask is not None else 0
     if addend is not None:
         if addend.dtype != C.dtype or not accumulate or batch1 * batch2 != 1:

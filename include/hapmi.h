@@ -155,7 +155,8 @@ typedef struct {
     const void *c_relu_mask;     /* optional: [M][ldc] in out_dtype; elements of the result (before accumulation)
                                   * whose mask value is <= 0 are written as 0: the backward of F.relu
                                   * (hap.rs:1417) when the call is the data gradient of the next F.linear and
-                                  * the mask is relu's output.  Needs batch 1; NULL = off */
+                                  * the mask is relu's output.  With a batch, problem z's mask lies at C's batch
+                                  * offsets from this pointer; NULL = off */
     const void *c_addend;        /* optional, with accumulate = 1: the result is added to c_addend[M][ldc] (out_dtype)
                                   * instead of C's old content, and C is only written: a gradient contribution
                                   * added to a buffer that other launches still read.  Needs batch 1; NULL = off */

@@ -362,6 +362,23 @@ def test_gemm_relu_mask_on_the_result(cuda, dtype, out_dtype, cfg, splits, accum
         lib().hapmi_gemm_tuning(-1, 0)
 
 
+@pytest.mark.parametrize("dtype", DT)
+def test_gemm_relu_mask_with_a_batch(cuda, dtype):
+    """c_relu_mask next to batch strides: problem z's mask lies at C's offset of problem z (the expert FFN's data
+    gradient: every local expert is one problem)."""
+    g = torch.Generator().manual_seed(9)
+    E, M, N, K = 3, 136, 72, 200
+    A = torch.randn(E, M, K, generator=g).to(dtype)
+    B = torch.randn(E, N, K, generator=g).to(dtype)
+    mask = torch.relu(torch.randn(E, M, N, generator=g)).to(dtype)
+    C = torch.empty(E, M, N, dtype=dtype, device=cuda)
+    ops.gemm(A.to(cuda), B.to(cuda), C, M, N, K, transB=True, batch1=E, strideA=(M * K, 0), strideB=(N * K, 0),
+             strideC=(M * N, 0), relu_mask=mask.to(cuda))
+    want = torch.einsum("emk,enk->emn", A.double(), B.double()) * (mask > 0)
+    close(C, want, dtype, scale=2.0)
+    assert (C.cpu()[mask == 0] == 0).all()
+
+
 @pytest.mark.parametrize("dtype,out_dtype,cfg,splits", [
     (torch.bfloat16, torch.bfloat16, 0, 1), (torch.bfloat16, torch.bfloat16, 7, 1), (torch.bfloat16, torch.float32, 5, 1),
     (torch.bfloat16, torch.bfloat16, 1, 3), (torch.float32, torch.float32, 0, 1), (torch.float32, torch.float32, 0, 2)])
