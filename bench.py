@@ -145,6 +145,9 @@ def main():
     ap.add_argument("--gemm-plan-file", default=None,
                     help="JSON file of pinned GEMM plans: loaded instead of autotuning when it exists, written after "
                          "autotuning otherwise (a profiler run can then repeat the plan of an unprofiled run)")
+    ap.add_argument("--no-receive-in-place", action="store_true",
+                    help="receive the backward all_to_all's pieces into buffers of their own and concatenate them with a "
+                         "copy kernel, instead of receiving them into their rows of the result")
     ap.add_argument("--wgrad-group", type=int, default=8,
                     help="the same linear's weight gradients of this many consecutive layers share one launch "
                          "(1: one launch, with its reduction split, per weight gradient)")
@@ -171,7 +174,8 @@ def main():
     wire = hap_amd.SyntheticWire(seed=39, scale=1.0, grad_scale=1e-3, share_shapes=True)
     ex = hap_amd.compile_program(gm, [x, y], dtype=dtype, wire=wire, rank=0, world_size=len(meta["ratios"]),
                                  overlap_wgrad=args.overlap, relu_mask_in_dgrad=not args.no_relu_mask_in_dgrad,
-                                 overlap_optimizer=args.overlap_optimizer, wgrad_group=args.wgrad_group)
+                                 overlap_optimizer=args.overlap_optimizer, wgrad_group=args.wgrad_group,
+                                 receive_in_place=not args.no_receive_in_place)
     ex.configure_optimizer(**meta["opt"])
     ex.load_inputs(x, y)                              # inputs resident in HBM before the timed region
     torch.cuda.synchronize()
@@ -245,7 +249,7 @@ def main():
                    "seq_len": meta["seq_len"], "launch": "hip-graph" if graph is not None else "eager",
                    "wgrad_stream": "side" if args.overlap else "main",
                    "optimizer": "one launch after backward" if ex._opt_chunks is None else "per stretch, overlapped with backward",
-                   "gemm_plan": plan_source, "weight_gradient_group": ex.wgrad_group, "attention_sharding": args.attn, "zero_sharded_parameters": bool(args.zero),
+                   "gemm_plan": plan_source, "weight_gradient_group": ex.wgrad_group, "exchange_pieces_received_in_place": ex.receive_in_place, "attention_sharding": args.attn, "zero_sharded_parameters": bool(args.zero),
                    "final_loss": loss},
         "roofline": {"bound": "mfma", "kernel": "gemm_kernel (all GEMM launches of the step)",
                      "achieved": achieved, "peak": peak, "unit": "TFLOP/s", "frac": achieved / peak,

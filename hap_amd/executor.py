@@ -61,7 +61,7 @@ class ShardExecutor:
                  rank: int = 0, world_size: int = 1, device: str = "cuda:0", fused_attention: bool = True,
                  overlap_wgrad: bool = False, launch_lists: bool = True, relu_mask_in_dgrad: bool = True,
                  overlap_optimizer: bool = False, optimizer_chunk_min: int = 1 << 20,
-                 relu_bwd_in_split: bool = True, wgrad_group: int = 8):
+                 relu_bwd_in_split: bool = True, wgrad_group: int = 8, receive_in_place: bool = True):
         """``example_inputs``: the program's inputs (global batch) as tensors or shapes; activations are
         sized from them.  ``rank`` / ``world_size`` are only needed by all_reduce / replicate, whose node
         forms do not carry them (collectives.py:86, 182)."""
@@ -101,6 +101,10 @@ class ShardExecutor:
         # relu's backward behind an all_to_all rides on the copying split of the backward exchange (one pass over
         # the gradient less per layer); False keeps the separate pass, for comparison
         self.relu_bwd_in_split = relu_bwd_in_split
+        # the backward all_to_all of the column-sharded FFN concatenates along dim 0: every peer's piece is a
+        # contiguous row range of the result, so it is received there (Wire.recv(into=...)) instead of into a
+        # buffer of its own that a copy kernel then moves; False keeps the copy
+        self.receive_in_place = receive_in_place
         # Optional: train_step() applies the optimizer to each stretch of the flat parameter buffer as soon as
         # backward has finished with it, on a second stream.  Measured on the BERT-large shard the step takes the
         # same time either way (27.1 against 27.0 ms): the GEMMs that run next to the update slow down by what the
@@ -119,6 +123,7 @@ class ShardExecutor:
         # They are held back until the group is full (or backward ends); their operands are per-layer buffers
         # that nothing overwrites before (see _grad_slot / _guard_write).  1 = every weight gradient at once.
         self.wgrad_group = 1 if (overlap_wgrad or self.overlap_optimizer) else max(1, min(int(wgrad_group), ops._lib.GEMM_MAX_LIST))
+        self._wire_backed: set = set()                     # storages that peers' messages are received into in place
         self._pending_wgrads: Dict[tuple, list] = {}
         self._deferred_reads: Dict[int, int] = {}          # storage -> launches held back that read it
         self._side_stream = torch.cuda.Stream(device=self.dev) if overlap_wgrad else None
@@ -370,6 +375,8 @@ class ShardExecutor:
         """Called while the backward list is built, right before a launch that writes into ``t`` is appended:
         when a side-stream launch appended earlier reads ``t``'s storage, the main stream waits for it first;
         when weight-gradient launches that are held back read it, they are appended first."""
+        if t is not None and t.untyped_storage().data_ptr() in self._wire_backed:
+            raise RuntimeError("internal: a launch would write into a buffer that peers' messages are received into")
         if self._is_read_later(t):
             self._flush_wgrads()             # weight gradients held back read t: they go first
         if t is None or not self._side_readers:
@@ -1144,9 +1151,11 @@ class ShardExecutor:
         return out
 
     def _emit_exchange(self, tag, direction, x_t, split_dim, cat_dim, split_L, cat_L, rank, sink, act=None,
-                       relu_of=None):
+                       relu_of=None, receive_in_place=False):
         """The local half of an all_to_all.  ``act``: activation applied while concatenating.  ``relu_of``: forward
-        output of a relu whose backward is applied to ``x_t`` while splitting (only for a split that copies)."""
+        output of a relu whose backward is applied to ``x_t`` while splitting (only for a split that copies).
+        ``receive_in_place`` (concatenation along dim 0, no activation): the peers' pieces are received straight
+        into their rows of the result, which nothing may write afterwards; no concat launch is left."""
         W = len(split_L)
         # pieces along the slowest dimension are contiguous ranges of the input: views, as torch.split gives the
         # reference (collectives.py:156); any other dimension needs the strided copy
@@ -1167,7 +1176,11 @@ class ShardExecutor:
                 parts.append(own)
             else:
                 shape = ops._with_dim(own.shape, cat_dim, cat_L[src])
-                parts.append(self.wire.recv(tag, direction, src, shape, self.cdt, self.dev, reduction=False))
+                into = None
+                if receive_in_place and cat_dim == 0 and act is None and not views and cat_L[src] > 0:
+                    into = out.narrow(0, sum(cat_L[:src]), cat_L[src])
+                    self._wire_backed.add(out.untyped_storage().data_ptr())
+                parts.append(self.wire.recv(tag, direction, src, shape, self.cdt, self.dev, reduction=False, into=into))
         if views:
             sink.append(lambda: ops.concat_rows(parts, cat_dim, out, act))
         else:
@@ -1210,8 +1223,13 @@ class ShardExecutor:
                         and self._split_can_mask(out.grad, out.t, cd, cL))
             if fuse and not in_split:
                 self._relu_backward_through(out)
+            # The result is d(x).  When x is a linear's output that only this exchange reads, d(x) is read by that
+            # linear's two gradient GEMMs and written by nobody: the peers' pieces can be received in place.
+            producer = node.args[0]
+            in_place = (self.receive_in_place and x.grad is None and isinstance(producer, torch.fx.Node)
+                        and producer.target is F.linear and len(producer.users) == 1 and not x.meta.get("fused_act"))
             g = self._emit_exchange(node.name, "bwd", out.grad, cd, sd, cL, sL, rank, self.bwd,
-                                    relu_of=out.t if in_split else None)
+                                    relu_of=out.t if in_split else None, receive_in_place=in_place)
             self._accumulate_into(x, g)
         self._tape.append(emit)
         return out

@@ -27,8 +27,22 @@ class Wire:
     ``src`` sent to this rank at collective ``tag`` (``direction`` 'fwd' or 'bwd'), or
     None when that peer contributes nothing."""
 
-    def recv(self, tag: str, direction: str, src: int, shape, dtype, device) -> Optional[torch.Tensor]:
+    def recv(self, tag: str, direction: str, src: int, shape, dtype, device, reduction: bool = False,
+             into: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+        """``into``: a contiguous static GPU tensor of ``shape`` that the message is to be delivered into (zero-copy
+        receive: the executor passes the rows of a concatenation that the piece belongs to); the wire returns it.
+        The stand-ins below deliver once, when the program is compiled; a transport would post its receive into
+        it every step."""
         raise NotImplementedError
+
+    @staticmethod
+    def _deliver(message: Optional[torch.Tensor], into: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
+        if into is None or message is None:
+            return message
+        if tuple(into.shape) != tuple(message.shape) or into.dtype != message.dtype or not into.is_contiguous():
+            raise ValueError("recv(into=...): a contiguous tensor of the message's shape and dtype expected")
+        into.copy_(message)
+        return into
 
     def send(self, tag: str, direction: str, dst: int, buffer: torch.Tensor) -> None:
         """Called once, when the program is compiled, for every message this rank sends: ``buffer`` is the static
@@ -45,13 +59,13 @@ class SilentWire(Wire):
         self.gather_fill = gather_fill
         self._cache: Dict[Tuple, torch.Tensor] = {}
 
-    def recv(self, tag, direction, src, shape, dtype, device, reduction: bool = False):
+    def recv(self, tag, direction, src, shape, dtype, device, reduction: bool = False, into=None):
         if reduction:
             return None
         key = (tuple(shape), dtype)
         if key not in self._cache:
             self._cache[key] = torch.full(tuple(shape), self.gather_fill, dtype=dtype, device=device)
-        return self._cache[key]
+        return self._deliver(self._cache[key], into)
 
 
 class SyntheticWire(Wire):
@@ -65,7 +79,7 @@ class SyntheticWire(Wire):
         self.share_shapes = share_shapes
         self._cache: Dict[Tuple, torch.Tensor] = {}
 
-    def recv(self, tag, direction, src, shape, dtype, device, reduction: bool = False):
+    def recv(self, tag, direction, src, shape, dtype, device, reduction: bool = False, into=None):
         if tag.startswith("replicate") and not self.reduce_params:
             return None
         key = (direction, src, tuple(shape), dtype) if self.share_shapes else (tag, direction, src)
@@ -76,7 +90,7 @@ class SyntheticWire(Wire):
             gen = torch.Generator().manual_seed((self.seed * 1000003 + zlib.crc32(repr(key).encode())) % (1 << 63))
             t = torch.randn(tuple(shape), generator=gen, dtype=torch.float32) * s
             self._cache[key] = t.to(dtype).to(device)
-        return self._cache[key]
+        return self._deliver(self._cache[key], into)
 
 
 class ReplayWire(Wire):
@@ -90,7 +104,7 @@ class ReplayWire(Wire):
             self.sent[(tag, direction, dst)] = buffer.detach().clone()
         return snapshot
 
-    def recv(self, tag, direction, src, shape, dtype, device, reduction: bool = False):
+    def recv(self, tag, direction, src, shape, dtype, device, reduction: bool = False, into=None):
         key = (tag, direction, src)
         if key not in self._cache:
             if (tag, direction) not in self.log:
@@ -100,4 +114,4 @@ class ReplayWire(Wire):
                 raise ValueError(f"recorded message for {tag!r} ({direction}) from rank {src} has shape "
                                  f"{tuple(t.shape)}, the program expects {tuple(shape)}")
             self._cache[key] = t.detach().to(dtype).contiguous().to(device)
-        return self._cache[key]
+        return self._deliver(self._cache[key], into)

@@ -371,6 +371,36 @@ def test_relu_backward_in_the_split_of_the_exchange_equals_the_separate_pass(cud
 
 
 @pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+def test_pieces_received_in_place_equal_the_copied_concatenation(cuda, dtype):
+    """receive_in_place: the backward all_to_all of the column-sharded FFN hands the wire the row ranges of its
+    result (Wire.recv(into=...)) instead of concatenating separate buffers.  Same loss, bit-equal gradients, also
+    on a second step (the peers' rows must have survived the first)."""
+    model = make_lm(vocab=211, S=32, d=64, H=1, F=128, layers=2)
+    x, y = lm_batch(8, 32, 211)
+
+    def build(in_place):
+        gm = hap_amd.build_program(copy.deepcopy(model), hap_amd.ShardingPlan([RATIOS4], 0), 8)
+        return hap_amd.compile_program(gm, [x, y], dtype=dtype, wire=hap_amd.SyntheticWire(seed=3, grad_scale=1e-2),
+                                       rank=0, world_size=4, receive_in_place=in_place)
+
+    a, b = build(True), build(False)
+    assert a._wire_backed and not b._wire_backed
+    for _ in range(2):
+        la = a.forward(x, y).item()
+        a.backward()
+        lb = b.forward(x, y).item()
+        b.backward()
+        torch.cuda.synchronize()
+        assert la == lb
+        for n, rec in a.params.items():
+            ga, gb = rec["grad"], b.params[n]["grad"]
+            if ga.dim() >= 2 and n != "encoder.weight":
+                assert torch.equal(ga, gb), (n, (ga - gb).abs().max().item())
+            else:
+                torch.testing.assert_close(ga, gb, rtol=1e-4, atol=1e-5 * gb.abs().max().item())
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
 @pytest.mark.parametrize("ffn,zero", [("column", False), ("batch", False), ("column", True)])
 def test_weight_gradients_of_consecutive_layers_in_one_launch_equal_single_launches(cuda, dtype, ffn, zero):
     """wgrad_group: the same linear's weight gradients of several layers share a launch (pointer lists) and are
