@@ -272,7 +272,7 @@ def test_hip_graph_replays_equal_eager_steps(cuda, dtype, opt):
         assert torch.isfinite(junk).all()
     # the two executors are separate runs: their atomically summed bias / embedding gradients differ in the last bits,
     # and Adam's updates of near-zero-gradient elements then differ by +-lr, which the later losses see at this level
-    assert losses == pytest.approx(ref_losses, rel=5e-6 if dtype == "fp32" else 2e-5)
+    assert losses == pytest.approx(ref_losses, rel=5e-6 if dtype == "fp32" else 1e-4)
     # Bias and embedding gradients are summed with float atomics, so two runs agree only up to summation order;
     # Adam turns that rounding noise into +-lr where the true gradient is zero (the key bias), so those elements
     # are left out of the parameter comparison.
