@@ -4,6 +4,7 @@ import pytest
 import torch
 
 from hap_amd import ops
+from hap_amd._lib import HapmiError
 from oracle.ops import _accumulate
 
 pytestmark = pytest.mark.gpu
@@ -66,6 +67,30 @@ def test_pad_split_concat_slice_layouts(cuda, dtype, shape, dim, L):
         want = torch.zeros(shape, dtype=dtype)
         want.narrow(dim, off, L[r]).copy_(shards[r])
         assert torch.equal(back.cpu(), want)
+
+
+def test_fused_entry_points_with_empty_shards_and_misaligned_pieces(cuda):
+    g = torch.Generator().manual_seed(6)
+    # zero-length pieces are skipped by the masked split
+    dy = torch.randn(4, 64, generator=g).bfloat16().to(cuda)
+    y = torch.relu(torch.randn(4, 64, generator=g)).bfloat16().to(cuda)
+    pieces = ops.split_rows(dy, [32, 0, 32, 0], 1, relu_of=y)
+    want = torch.where(y > 0, dy, torch.zeros_like(dy))
+    assert [tuple(p.shape) for p in pieces] == [(4, 32), (4, 0), (4, 32), (4, 0)]
+    assert torch.equal(torch.cat(pieces, dim=1), want)
+    # pieces that are not whole 16-byte vectors are refused (the executor then keeps relu's backward as its own pass)
+    with pytest.raises(HapmiError):
+        ops.split_rows(dy, [30, 34], 1, relu_of=y)
+    # an empty output of the reduction with an addend is a no-op
+    parts = [torch.randn(6, 8, generator=g).to(cuda) for _ in range(3)]
+    empty = ops.ragged_reduce(parts, 0, 2, 0, addend=torch.empty(0, 8, device=cuda))
+    assert tuple(empty.shape) == (0, 8)
+    # a misaligned addend takes the scalar path and gives the same sum
+    base = torch.randn(4 * 8 + 1, generator=g).to(cuda)
+    addend = base[1:].view(4, 8)
+    got = ops.ragged_reduce(parts, 0, 1, 4, addend=addend)
+    want = parts[0][1:5] + parts[1][1:5] + parts[2][1:5] + addend
+    assert torch.equal(got, want)
 
 
 def test_concat_leaves_a_piece_that_is_already_in_place(cuda):
