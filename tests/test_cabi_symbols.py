@@ -36,3 +36,31 @@ def test_product_refuses_cpu_tensors():
     from hap_amd._lib import HapmiError
     with pytest.raises(HapmiError):
         ops.add(torch.ones(4), torch.ones(4), torch.ones(4))
+
+
+def test_gemm_argument_checks_run_before_any_launch():
+    """Pointer lists and the addend are validated on the host: these calls return an error without touching a device."""
+    from hap_amd._lib import GemmArgs, _load, BF16, F32
+    lib = _load()
+
+    def args(**kw):
+        a = GemmArgs()
+        a.M, a.N, a.K, a.lda, a.ldb, a.ldc = 64, 64, 64, 64, 64, 64
+        a.in_dtype, a.out_dtype, a.alpha, a.batch1, a.batch2 = BF16, F32, 1.0, 1, 1
+        for k, v in kw.items():
+            setattr(a, k, v)
+        return a
+
+    ptrs = (ctypes.c_void_p * 17)(*([0x1000] * 17))
+    lists = dict(A_list=ctypes.addressof(ptrs), B_list=ctypes.addressof(ptrs), C_list=ctypes.addressof(ptrs))
+    cases = {
+        b"go together": args(A_list=ctypes.addressof(ptrs), batch1=2),
+        b"at most": args(batch1=17, **lists),
+        b"must be NULL": args(A=0x1000, batch1=2, **lists),
+        b"transA": args(a_rowsum_list=ctypes.addressof(ptrs), batch1=2, **lists),
+        b"c_addend": args(A=0x1000, B=0x1000, C=0x1000, c_addend=0x1000),            # without accumulate
+        b"null pointer": args(),
+    }
+    for needle, a in cases.items():
+        rc = lib.hapmi_gemm(ctypes.byref(a), None)
+        assert rc != 0 and needle in lib.hapmi_last_error(), (needle, rc, lib.hapmi_last_error())
