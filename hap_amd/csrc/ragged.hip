@@ -254,6 +254,11 @@ extern "C" int hapmi_unpad_concat(const void *const *slices, const int64_t *leng
                       (long long)lengths[i], (long long)padded_len);
         if (lengths[i] > 0 && outer > 0) {
             HAPMI_REQUIRE(slices[i] && dst, HAPMI_EINVAL, "unpad_concat: null pointer");
+            // a slice that was received at its place in dst (outer = 1: one contiguous range) stays where it is
+            if (outer == 1 && (const char *)slices[i] == (const char *)dst + off * inner_bytes) {
+                off += lengths[i];
+                continue;
+            }
             list.seg[list.n++] = {(const char *)slices[i], (char *)dst + off * inner_bytes, outer,
                                   lengths[i] * inner_bytes, padded_len * inner_bytes, total * inner_bytes};
         }
@@ -274,8 +279,8 @@ extern "C" int hapmi_split_pad(const void *src, void *const *slices, const int64
     for (int i = 0; i < n_ranks; ++i) {
         HAPMI_REQUIRE(lengths[i] <= padded_len, HAPMI_EINVAL, "split_pad: length %lld above padded length %lld",
                       (long long)lengths[i], (long long)padded_len);
-        if (lengths[i] > 0 && outer > 0) {
-            HAPMI_REQUIRE(slices[i] && src, HAPMI_EINVAL, "split_pad: null pointer");
+        if (lengths[i] > 0 && outer > 0 && slices[i]) {       // a NULL slice is skipped (a piece nobody needs)
+            HAPMI_REQUIRE(src, HAPMI_EINVAL, "split_pad: null pointer");
             list.seg[list.n++] = {(const char *)src + off * inner_bytes, (char *)slices[i], outer,
                                   lengths[i] * inner_bytes, total * inner_bytes, padded_len * inner_bytes};
         }

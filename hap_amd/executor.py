@@ -1057,9 +1057,15 @@ class ShardExecutor:
         # a shard of the longest length needs no padding: the tensor itself is the message
         unpadded = L[rank] == m and x_t.is_contiguous() and tuple(x_t.shape) == tuple(pshape)
         own = x_t if unpadded else self._new(pshape, x_t.dtype)
-        peers = self._peers(tag, direction, rank, W, pshape, False, x_t.dtype)
-        slices = [own if s == rank else peers[s] for s in range(W)]
         full = self._new(ops._with_dim(x_t.shape, dim, sum(L)), x_t.dtype)
+        # a peer's shard of the longest length carries no padding either: along dim 0 it is received straight into
+        # its rows of the result (a forward buffer that no launch writes afterwards)
+        into = {}
+        if self.receive_in_place and dim == 0:
+            into = {s: full.narrow(0, sum(L[:s]), m) for s in range(W) if s != rank and L[s] == m}
+        peers = {s: self.wire.recv(tag, direction, s, pshape, x_t.dtype, self.dev, reduction=False, into=into.get(s))
+                 for s in range(W) if s != rank}
+        slices = [own if s == rank else peers[s] for s in range(W)]
         if unpadded:
             sink.append(lambda: ops.unpad_concat(slices, L, dim, full))
         else:
@@ -1072,11 +1078,19 @@ class ShardExecutor:
         (the output's shape) is added to the sum in the same pass."""
         m, W = max(L), len(L)
         pshape = ops._with_dim(full_t.shape, dim, m)
-        sent = [self._new(pshape, full_t.dtype) for _ in range(W)]
         peers = self._peers(tag, direction, rank, W, pshape, True, full_t.dtype)
-        contribs = [sent[rank] if s == rank else peers[s] for s in range(W)]
-        contribs = [c for c in contribs if c is not None]
         out = out_t if out_t is not None else self._new(ops._with_dim(full_t.shape, dim, L[rank]), full_t.dtype)
+        if dim == 0 and full_t.is_contiguous() and L[rank] > 0:
+            # along dim 0 this rank's own piece is a contiguous row range of the full tensor: the sum reads it there
+            # (and the first L[rank] rows of the peers' padded pieces), and no padded copy of it is made
+            sent = [None if s == rank else self._new(pshape, full_t.dtype) for s in range(W)]
+            own = full_t.narrow(0, sum(L[:rank]), L[rank])
+            contribs = [own if s == rank else (peers[s].narrow(0, 0, L[rank]) if peers[s] is not None else None)
+                        for s in range(W)]
+        else:
+            sent = [self._new(pshape, full_t.dtype) for _ in range(W)]
+            contribs = [sent[rank] if s == rank else peers[s] for s in range(W)]
+        contribs = [c for c in contribs if c is not None]
         sink.append(lambda: (ops.split_pad(full_t, L, dim, m, sent),
                              ops.ragged_reduce(contribs, dim, 0, L[rank], out, addend=addend)))
         self._announce(tag, direction, rank, W, lambda dst: sent[dst], sink)  # the padded piece that rank dst reduces

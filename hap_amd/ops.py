@@ -121,7 +121,8 @@ def unpad_concat(slices: Sequence[torch.Tensor], lengths: Sequence[int], dim: in
 
 
 def split_pad(src: torch.Tensor, lengths: Sequence[int], dim: int, padded_len: int,
-              outs: Optional[Sequence[torch.Tensor]] = None) -> List[torch.Tensor]:
+              outs: Optional[Sequence[Optional[torch.Tensor]]] = None) -> List[torch.Tensor]:
+    """Padded pieces of ``src`` along ``dim``; a ``None`` entry of ``outs`` is a piece that is not produced."""
     _dev(src)
     assert src.is_contiguous()
     outer, total, inner = _oli(src.shape, dim)
@@ -129,8 +130,9 @@ def split_pad(src: torch.Tensor, lengths: Sequence[int], dim: int, padded_len: i
     if outs is None:
         outs = [torch.empty(_with_dim(src.shape, dim, padded_len), dtype=src.dtype, device=src.device) for _ in lengths]
     for o in outs:
-        _dev(o)
-        _need(o, outer * padded_len * inner, "split_pad slice")
+        if o is not None:
+            _dev(o)
+            _need(o, outer * padded_len * inner, "split_pad slice")
     if src.numel() == 0:
         return list(outs)
     check(lib().hapmi_split_pad(_ptr(src), _ptrs(outs), _i64(lengths), len(lengths), outer, padded_len,

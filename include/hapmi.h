@@ -61,12 +61,13 @@ int hapmi_pad_rows(const void *src, void *dst, int64_t outer, int64_t len, int64
                    int64_t inner_bytes, hapmi_stream_t stream);
 
 /* collectives.py:20 / :102: cut the pad off W padded slices [outer, padded_len, inner]
- * and concatenate them along the sharded dimension into dst[outer, sum(lengths), inner]. */
+ * and concatenate them along the sharded dimension into dst[outer, sum(lengths), inner].  A slice that already lies at its place in dst (outer = 1 and
+ * slices[i] == dst + offset of shard i) is left where it is. */
 int hapmi_unpad_concat(const void *const *slices_host, const int64_t *lengths_host, int n_ranks, void *dst,
                        int64_t outer, int64_t padded_len, int64_t inner_bytes, hapmi_stream_t stream);
 
 /* collectives.py:24-25 / :92-93: split src[outer, sum(lengths), inner] along the
- * sharded dimension and pad every piece into its own [outer, padded_len, inner] buffer. */
+ * sharded dimension and pad every piece into its own [outer, padded_len, inner] buffer.  A NULL slice is skipped. */
 int hapmi_split_pad(const void *src, void *const *slices_host, const int64_t *lengths_host, int n_ranks,
                     int64_t outer, int64_t padded_len, int64_t inner_bytes, hapmi_stream_t stream);
 

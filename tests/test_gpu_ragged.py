@@ -93,6 +93,22 @@ def test_fused_entry_points_with_empty_shards_and_misaligned_pieces(cuda):
     assert torch.equal(got, want)
 
 
+def test_split_pad_skips_a_missing_slice_and_unpad_concat_a_slice_in_place(cuda):
+    g = torch.Generator().manual_seed(8)
+    L, m = [5, 5, 2], 5
+    full = torch.randn(12, 16, generator=g).bfloat16()
+    outs = [torch.full((m, 16), 7.0, dtype=torch.bfloat16, device=cuda), None,
+            torch.full((m, 16), 7.0, dtype=torch.bfloat16, device=cuda)]
+    ops.split_pad(full.to(cuda), L, 0, m, outs)
+    assert torch.equal(outs[0].cpu(), full[:5]) and torch.equal(outs[2].cpu()[:2], full[10:]) and (outs[2].cpu()[2:] == 7).all()
+    # a slice of the longest length that already lies at its rows of the result is not copied (and not needed elsewhere)
+    dst = torch.full((12, 16), 3.0, dtype=torch.bfloat16, device=cuda)
+    mine = dst.narrow(0, 5, 5)
+    mine.copy_(full[5:10])
+    ops.unpad_concat([outs[0], mine, outs[2]], L, 0, dst)
+    assert torch.equal(dst.cpu(), full)
+
+
 def test_concat_leaves_a_piece_that_is_already_in_place(cuda):
     g = torch.Generator().manual_seed(4)
     pieces = [torch.randn(n, 24, generator=g).bfloat16().to(cuda) for n in (3, 5, 2)]
