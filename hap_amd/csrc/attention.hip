@@ -473,12 +473,13 @@ __global__ __launch_bounds__(AT_THREADS, 2) void attn_bwd_dkv_kernel(const bf16_
             // without a mask, query rows beyond S carry lse = +inf (p = 0); causal tiles below the diagonal of the
             // block's 128 keys need no comparison
             const bool plain = !mask && (!CAUSAL || blk * 128 + 127 <= q0);
+            // accumulator registers 4 g .. 4 g + 3 are query rows ql .. ql + 3; the two paths are whole loops of their
+            // own (a branch per group makes the compiler copy both accumulator tiles at every merge)
+            if (plain) {
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                // accumulator registers 4 g .. 4 g + 3 are query rows ql .. ql + 3
-                const int ql = t * 32 + g * 8 + h * 4;
-                const f32x4 l4 = *(const f32x4 *)(lse_s + ql), d4 = *(const f32x4 *)(delta_s + ql);
-                if (plain) {
+                for (int g = 0; g < 4; ++g) {
+                    const int ql = t * 32 + g * 8 + h * 4;
+                    const f32x4 l4 = *(const f32x4 *)(lse_s + ql), d4 = *(const f32x4 *)(delta_s + ql);
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
                         const int r = g * 4 + e;
@@ -486,7 +487,12 @@ __global__ __launch_bounds__(AT_THREADS, 2) void attn_bwd_dkv_kernel(const bf16_
                         sc[r] = p;
                         dp[r] = p * (dp[r] - d4[e]);
                     }
-                } else {
+                }
+            } else {
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int ql = t * 32 + g * 8 + h * 4;
+                    const f32x4 l4 = *(const f32x4 *)(lse_s + ql), d4 = *(const f32x4 *)(delta_s + ql);
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
                         const int r = g * 4 + e;
