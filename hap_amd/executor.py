@@ -1059,10 +1059,13 @@ class ShardExecutor:
         own = x_t if unpadded else self._new(pshape, x_t.dtype)
         full = self._new(ops._with_dim(x_t.shape, dim, sum(L)), x_t.dtype)
         # a peer's shard of the longest length carries no padding either: along dim 0 it is received straight into
-        # its rows of the result (a forward buffer that no launch writes afterwards)
+        # its rows of the result.  Only in the forward direction, where the result is an activation that no launch
+        # writes afterwards; a gathered gradient may be accumulated into in place by other consumers.
         into = {}
-        if self.receive_in_place and dim == 0:
+        if self.receive_in_place and dim == 0 and direction == "fwd":
             into = {s: full.narrow(0, sum(L[:s]), m) for s in range(W) if s != rank and L[s] == m}
+            if into:
+                self._wire_backed.add(full.untyped_storage().data_ptr())
         peers = {s: self.wire.recv(tag, direction, s, pshape, x_t.dtype, self.dev, reduction=False, into=into.get(s))
                  for s in range(W) if s != rank}
         slices = [own if s == rank else peers[s] for s in range(W)]
