@@ -29,6 +29,8 @@ HAPMI_GEMM_DECLARE_CFG(6);
 HAPMI_GEMM_DECLARE_CFG(7);
 HAPMI_GEMM_DECLARE_CFG(8);
 HAPMI_GEMM_DECLARE_CFG(9);
+HAPMI_GEMM_DECLARE_CFG(10);
+HAPMI_GEMM_DECLARE_CFG(11);
 
 namespace {
 
@@ -37,8 +39,10 @@ struct TileCfg {
     int bm, bn, wm, wn;
 };
 constexpr TileCfg kCfg[] = {{128, 128, 2, 2}, {256, 256, 2, 4}, {384, 192, 4, 2}, {192, 256, 2, 4}, {256, 192, 4, 2},
-                             {256, 128, 4, 2}, {128, 256, 2, 4}, {192, 128, 2, 4}, {256, 128, 2, 2}, {128, 192, 4, 2}};
-constexpr int kNumCfg = 10;
+                             {256, 128, 4, 2}, {128, 256, 2, 4}, {192, 128, 2, 4}, {256, 128, 2, 2}, {128, 192, 4, 2},
+                             {64, 64, 2, 2}, {64, 128, 2, 2}};
+constexpr int kNumCfg = 12;
+constexpr int kFirstF32Cfg = 10;                 // 10, 11: small tiles for float32 operands only
 constexpr int kNumCU = 256;
 int g_force_cfg = -1;
 int g_force_splits = 0;
@@ -77,19 +81,38 @@ struct Choice {
     int cfg, splits;
 };
 
-Choice choose(int64_t M, int64_t N, int64_t K, int64_t batch, int bk, bool wide, int64_t max_splits, bool row_major_operands) {
+// Which tile configurations a call may use: 0 serves every type; 1..9 bf16 operands of calls that allow the large
+// tiles; 10, 11 float32 operands.
+bool cfg_eligible(int c, bool bf16_in, bool wide, bool row_major_operands, bool forced) {
+    if (c == 0) return true;
+    if (c >= kFirstF32Cfg) return !bf16_in;
+    if (!bf16_in || !wide) return false;
+    if (c == 2 && !row_major_operands && !forced) return false;          // 384x192 with a transposing loader spills registers
+    return true;
+}
+
+Choice choose(int64_t M, int64_t N, int64_t K, int64_t batch, int bk, bool bf16_in, bool wide, int64_t max_splits,
+              bool row_major_operands) {
     static const int kSplitMenu[] = {1, 2, 3, 4, 5, 6, 7, 8, 10, 12, 16, 24, 32};
     const int64_t nk = hapmi_cdiv(K, bk);
     Choice best{0, 1};
     double best_t = 1e30;
+    const bool forced = g_force_cfg >= 0 && g_force_cfg < kNumCfg && cfg_eligible(g_force_cfg, bf16_in, wide, row_major_operands, true);
     for (int c = 0; c < kNumCfg; ++c) {
-        if (g_force_cfg >= 0 && g_force_cfg < kNumCfg && c != g_force_cfg && (wide || g_force_cfg == 0)) continue;
-        if (c > 0 && !wide) continue;
-        if (c == 2 && !row_major_operands && g_force_cfg != 2) continue;   // 384x192 with a transposing loader spills registers
+        if (forced ? c != g_force_cfg : !cfg_eligible(c, bf16_in, wide, row_major_operands, false)) continue;
         const int64_t tiles = hapmi_cdiv(M, kCfg[c].bm) * hapmi_cdiv(N, kCfg[c].bn) * batch;
-        const double slots = c == 0 ? 2.0 * kNumCU : 1.0 * kNumCU;
-        const double rate = c == 0 ? 1.75 : 4.1;                         // TFLOP/s per slot in steady state
-        const double fixed = c == 0 ? 2.0 : 3.5;                         // us per tile: first loads + epilogue
+        // co-resident blocks per CU, TFLOP/s per block slot in steady state, us per tile for first loads + epilogue
+        double per_cu, rate, fixed;
+        if (bf16_in) {
+            per_cu = c == 0 ? 2.0 : 1.0;
+            rate = c == 0 ? 1.75 : 4.1;
+            fixed = c == 0 ? 2.0 : 3.5;
+        } else {                                                         // float32 MFMA: 0.61 TFLOP/s per CU at best
+            per_cu = c == 0 ? 2.0 : 4.0;
+            rate = 0.5 / per_cu;
+            fixed = 2.0;
+        }
+        const double slots = per_cu * kNumCU;
         for (int s : kSplitMenu) {
             if (g_force_splits > 0 && s != g_force_splits && !(s == 1 && (max_splits < g_force_splits || batch != 1))) continue;
             if (s > 1 && (s > max_splits || batch != 1 || nk / s < 4)) continue;
@@ -168,14 +191,14 @@ int launch_typed(GemmParams &p, int transA, int transB, int64_t batch, hipStream
     p.ws_ld = (p.N + 3) / 4 * 4;
     const int64_t per_split = p.M * p.ws_ld * 4;
     const int64_t max_splits = (workspace && ((uintptr_t)workspace % 16) == 0 && per_split > 0) ? workspace_bytes / per_split : 0;
-    Choice ch = choose(p.M, p.N, p.K, batch, bk, wide && sizeof(TI) == 2, max_splits, !transA && transB);
+    Choice ch = choose(p.M, p.N, p.K, batch, bk, sizeof(TI) == 2, wide, max_splits, !transA && transB);
     if (g_force_cfg < 0 && g_force_splits <= 0) {
         std::lock_guard<std::mutex> lk(g_plans_mu);
         auto it = g_plans.find(PlanKey(p.M, p.N, p.K, batch, (int)(transA != 0), (int)(transB != 0), sizeof(TI) == 2 ? HAPMI_BF16 : HAPMI_F32,
                                        sizeof(TO) == 2 ? HAPMI_BF16 : HAPMI_F32));
         if (it != g_plans.end()) {
             const int pc = it->second.first, ps = it->second.second;
-            const bool cfg_ok = pc == 0 || (pc < kNumCfg && wide && sizeof(TI) == 2);
+            const bool cfg_ok = pc >= 0 && pc < kNumCfg && cfg_eligible(pc, sizeof(TI) == 2, wide, !transA && transB, true);
             const bool split_ok = ps == 1 || (ps > 1 && ps <= max_splits && batch == 1 && nk / ps >= 1);
             if (cfg_ok && split_ok) ch = Choice{pc, ps};
         }
@@ -197,6 +220,8 @@ int launch_typed(GemmParams &p, int transA, int transB, int64_t batch, hipStream
         case 7: rc = hapmi_gemm_launch_cfg7(p, in_dtype, out_dtype, transA, transB, batch, st); break;
         case 8: rc = hapmi_gemm_launch_cfg8(p, in_dtype, out_dtype, transA, transB, batch, st); break;
         case 9: rc = hapmi_gemm_launch_cfg9(p, in_dtype, out_dtype, transA, transB, batch, st); break;
+        case 10: rc = hapmi_gemm_launch_cfg10(p, in_dtype, out_dtype, transA, transB, batch, st); break;
+        case 11: rc = hapmi_gemm_launch_cfg11(p, in_dtype, out_dtype, transA, transB, batch, st); break;
         default: rc = hapmi_gemm_launch_cfg0(p, in_dtype, out_dtype, transA, transB, batch, st);
     }
     if (rc || p.splits <= 1) return rc;

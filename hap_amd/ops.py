@@ -412,7 +412,8 @@ def gemm_group(As: Sequence[torch.Tensor], Bs: Sequence[torch.Tensor], Cs: Seque
 
 _gemm_log = None
 _SPLIT_MENU = (1, 2, 3, 4, 5, 6, 7, 8, 10, 12, 16)
-_N_TILE_CONFIGS = 10
+_BF16_TILE_CONFIGS = tuple(range(10))
+_F32_TILE_CONFIGS = (0, 10, 11)
 
 
 def record_gemms(on: bool):
@@ -435,7 +436,7 @@ def autotune_gemm(a: "GemmArgs", flush: Optional[torch.Tensor] = None, repeats: 
     per_split = a.M * ((a.N + 3) // 4 * 4) * 4
     max_splits = a.workspace_bytes // per_split if (a.workspace and per_split) else 0
     cands = []
-    for cfg in range(_N_TILE_CONFIGS if bf16_in else 1):
+    for cfg in (_BF16_TILE_CONFIGS if bf16_in else _F32_TILE_CONFIGS):
         for s in _SPLIT_MENU:
             if s > 1 and (s > max_splits or batch != 1 or nk // s < 4):
                 continue

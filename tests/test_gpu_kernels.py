@@ -275,8 +275,35 @@ def test_gemm_every_tile_configuration_and_layout(cuda, cfg, tA, tB):
         lib().hapmi_gemm_tuning(-1, 0)
 
 
+@pytest.mark.parametrize("cfg", [0, 10, 11])
+@pytest.mark.parametrize("tA,tB", [(0, 1), (0, 0), (1, 0), (1, 1)])
+def test_gemm_float32_tile_configurations_and_layouts(cuda, cfg, tA, tB):
+    """float32 operands in all four storage layouts through the three tile configurations that take them (128 x 128
+    and the small 64 x 64 / 64 x 128 tiles): ragged edges in M, N and K and a tile-aligned shape, float32 and bf16
+    outputs, bias and accumulation, against float64."""
+    from hap_amd._lib import lib
+    try:
+        lib().hapmi_gemm_tuning(cfg, 1)
+        for (M, N, K) in [(200, 136, 300), (384, 512, 256)]:
+            g = torch.Generator().manual_seed(M + cfg)
+            A = torch.randn((K, M) if tA else (M, K), generator=g)
+            B = torch.randn((N, K) if tB else (K, N), generator=g)
+            bias = torch.randn(N, generator=g)
+            want = (A.double().t() if tA else A.double()) @ (B.double().t() if tB else B.double()) + bias.double()
+            for out_dtype in (torch.float32, torch.bfloat16):
+                C = torch.full((M, N), float("nan"), dtype=out_dtype, device=cuda)
+                ops.gemm(A.to(cuda), B.to(cuda), C, M, N, K, transA=bool(tA), transB=bool(tB), bias=bias.to(cuda))
+                close(C, want, out_dtype, scale=2.0)
+            start = torch.randn(M, N, generator=g)
+            C = start.clone().to(cuda)
+            ops.gemm(A.to(cuda), B.to(cuda), C, M, N, K, transA=bool(tA), transB=bool(tB), accumulate=True)
+            close(C, want - bias.double() + start.double(), torch.float32, scale=2.0)
+    finally:
+        lib().hapmi_gemm_tuning(-1, 0)
+
+
 @pytest.mark.parametrize("dtype", DT)
-@pytest.mark.parametrize("cfg", [0, 1])
+@pytest.mark.parametrize("cfg", [0, 1, 10, 11])
 def test_gemm_split_k_and_tile_configs(cuda, dtype, cfg):
     """Forced tile configuration and K splits (workspace partial sums + ordered reduction) give the same product."""
     from hap_amd._lib import lib
@@ -301,7 +328,7 @@ def test_gemm_split_k_and_tile_configs(cuda, dtype, cfg):
         lib().hapmi_gemm_tuning(-1, 0)
 
 
-@pytest.mark.parametrize("dtype,cfg", [(torch.float32, 0), (torch.bfloat16, 0), (torch.bfloat16, 1), (torch.bfloat16, 2),
+@pytest.mark.parametrize("dtype,cfg", [(torch.float32, 0), (torch.float32, 10), (torch.float32, 11), (torch.bfloat16, 0), (torch.bfloat16, 1), (torch.bfloat16, 2),
                                        (torch.bfloat16, 3), (torch.bfloat16, 4), (torch.bfloat16, 5), (torch.bfloat16, 6), (torch.bfloat16, 7), (torch.bfloat16, 8), (torch.bfloat16, 9)])
 @pytest.mark.parametrize("tB", [False, True])
 def test_gemm_row_sums_of_a_transposed_operand(cuda, dtype, cfg, tB):
