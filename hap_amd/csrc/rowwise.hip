@@ -5,17 +5,20 @@
 namespace {
 
 constexpr int ROW_WAVES = 4;                 // rows per block, one wave per row
-constexpr int ROW_MAXE = 32;                 // elements per lane -> width <= 2048
+constexpr int ROW_MAXE = 32;                 // most elements per lane -> width <= 2048
+// The kernels are instantiated for 8, 16 and 32 elements per lane (widths up to 512, 1024, 2048): the loops over a
+// lane's elements are unrolled over registers, so a row of 1024 on the 32-element instance would do twice the
+// arithmetic and hold twice the registers.
 
 // A row of `width` elements held across one wave: element e of lane l is
 // column (e / EPV) * 64 * EPV + l * EPV + (e % EPV).
-template <typename T, int EPV> struct RowRegs {
-    float v[ROW_MAXE];
+template <typename T, int EPV, int MAXE> struct RowRegs {
+    float v[MAXE];
     __device__ __forceinline__ static int col(int e, int lane) { return (e / EPV) * 64 * EPV + lane * EPV + (e % EPV); }
 
     __device__ __forceinline__ void load(const T *row, int width, int lane, float fill) {
 #pragma unroll
-        for (int g = 0; g < ROW_MAXE / EPV; ++g) {
+        for (int g = 0; g < MAXE / EPV; ++g) {
             const int c0 = g * 64 * EPV + lane * EPV;
             if (EPV * sizeof(T) == 16) {
                 if (c0 < width) {
@@ -34,7 +37,7 @@ template <typename T, int EPV> struct RowRegs {
     }
     __device__ __forceinline__ void store(T *row, int width, int lane) const {
 #pragma unroll
-        for (int g = 0; g < ROW_MAXE / EPV; ++g) {
+        for (int g = 0; g < MAXE / EPV; ++g) {
             const int c0 = g * 64 * EPV + lane * EPV;
             if (EPV * sizeof(T) == 16) {
                 if (c0 < width) {
@@ -52,19 +55,19 @@ template <typename T, int EPV> struct RowRegs {
     }
 };
 
-template <typename T, int EPV>
+template <typename T, int EPV, int MAXE>
 __global__ __launch_bounds__(ROW_WAVES * 64) void add_layernorm_fwd_kernel(const T *x, const T *res, T *y, float *rstd,
                                                                          int64_t rows, int width, float eps) {
     const int lane = threadIdx.x & 63;
     const int64_t r = (int64_t)blockIdx.x * ROW_WAVES + (threadIdx.x >> 6);
     if (r >= rows) return;
-    RowRegs<T, EPV> a;
+    RowRegs<T, EPV, MAXE> a;
     a.load(x + r * width, width, lane, 0.f);
     if (res) {
-        RowRegs<T, EPV> b;
+        RowRegs<T, EPV, MAXE> b;
         b.load(res + r * width, width, lane, 0.f);
 #pragma unroll
-        for (int e = 0; e < ROW_MAXE; ++e) {
+        for (int e = 0; e < MAXE; ++e) {
             a.v[e] += b.v[e];
             // the sum is a tensor of the storage type in the unfused program: round it the same way
             if (sizeof(T) == 2) a.v[e] = (float)(bf16_t)a.v[e];
@@ -72,96 +75,96 @@ __global__ __launch_bounds__(ROW_WAVES * 64) void add_layernorm_fwd_kernel(const
     }
     float s = 0.f;
 #pragma unroll
-    for (int e = 0; e < ROW_MAXE; ++e) s += a.v[e];
+    for (int e = 0; e < MAXE; ++e) s += a.v[e];
     const float mean = wave_sum(s) / (float)width;
     float q = 0.f;
 #pragma unroll
-    for (int e = 0; e < ROW_MAXE; ++e) {
-        const float d = (RowRegs<T, EPV>::col(e, lane) < width) ? a.v[e] - mean : 0.f;
+    for (int e = 0; e < MAXE; ++e) {
+        const float d = (RowRegs<T, EPV, MAXE>::col(e, lane) < width) ? a.v[e] - mean : 0.f;
         q += d * d;
     }
     const float var = wave_sum(q) / (float)width;
     const float rs = 1.0f / sqrtf(var + eps);
 #pragma unroll
-    for (int e = 0; e < ROW_MAXE; ++e) a.v[e] = (a.v[e] - mean) * rs;
+    for (int e = 0; e < MAXE; ++e) a.v[e] = (a.v[e] - mean) * rs;
     a.store(y + r * width, width, lane);
     if (lane == 0) rstd[r] = rs;
 }
 
-template <typename T, int EPV>
+template <typename T, int EPV, int MAXE>
 __global__ __launch_bounds__(ROW_WAVES * 64) void layernorm_bwd_kernel(const T *dy, const T *y, const float *rstd,
                                                                      const T *dx_add, T *dx, int64_t rows, int width) {
     const int lane = threadIdx.x & 63;
     const int64_t r = (int64_t)blockIdx.x * ROW_WAVES + (threadIdx.x >> 6);
     if (r >= rows) return;
-    RowRegs<T, EPV> g, o;
+    RowRegs<T, EPV, MAXE> g, o;
     g.load(dy + r * width, width, lane, 0.f);
     o.load(y + r * width, width, lane, 0.f);
     float s1 = 0.f, s2 = 0.f;
 #pragma unroll
-    for (int e = 0; e < ROW_MAXE; ++e) {
+    for (int e = 0; e < MAXE; ++e) {
         s1 += g.v[e];
         s2 += g.v[e] * o.v[e];
     }
     const float c1 = wave_sum(s1) / (float)width, c2 = wave_sum(s2) / (float)width;
     const float rs = rstd[r];
 #pragma unroll
-    for (int e = 0; e < ROW_MAXE; ++e) g.v[e] = rs * (g.v[e] - c1 - o.v[e] * c2);
+    for (int e = 0; e < MAXE; ++e) g.v[e] = rs * (g.v[e] - c1 - o.v[e] * c2);
     if (dx_add) {
         o.load(dx_add + r * width, width, lane, 0.f);
 #pragma unroll
-        for (int e = 0; e < ROW_MAXE; ++e) g.v[e] += o.v[e];
+        for (int e = 0; e < MAXE; ++e) g.v[e] += o.v[e];
     }
     g.store(dx + r * width, width, lane);
 }
 
-template <typename T, int EPV>
+template <typename T, int EPV, int MAXE>
 __global__ __launch_bounds__(ROW_WAVES * 64) void softmax_fwd_kernel(const T *x, const float *mask, T *p, int64_t rows,
                                                                    int width, int64_t ld, int64_t mask_rows) {
     const int lane = threadIdx.x & 63;
     const int64_t r = (int64_t)blockIdx.x * ROW_WAVES + (threadIdx.x >> 6);
     if (r >= rows) return;
-    RowRegs<T, EPV> a;
+    RowRegs<T, EPV, MAXE> a;
     a.load(x + r * ld, width, lane, -INFINITY);
     if (mask) {
         const float *mrow = mask + (r % mask_rows) * width;
 #pragma unroll
-        for (int e = 0; e < ROW_MAXE; ++e) {
-            const int c = RowRegs<T, EPV>::col(e, lane);
+        for (int e = 0; e < MAXE; ++e) {
+            const int c = RowRegs<T, EPV, MAXE>::col(e, lane);
             if (c < width) a.v[e] += mrow[c];
         }
     }
     float m = -INFINITY;
 #pragma unroll
-    for (int e = 0; e < ROW_MAXE; ++e) m = fmaxf(m, a.v[e]);
+    for (int e = 0; e < MAXE; ++e) m = fmaxf(m, a.v[e]);
     m = wave_max(m);
     float s = 0.f;
 #pragma unroll
-    for (int e = 0; e < ROW_MAXE; ++e) {
+    for (int e = 0; e < MAXE; ++e) {
         a.v[e] = __expf(a.v[e] - m);
         s += a.v[e];
     }
     const float inv = 1.0f / wave_sum(s);
 #pragma unroll
-    for (int e = 0; e < ROW_MAXE; ++e) a.v[e] *= inv;
+    for (int e = 0; e < MAXE; ++e) a.v[e] *= inv;
     a.store(p + r * ld, width, lane);
 }
 
-template <typename T, int EPV>
+template <typename T, int EPV, int MAXE>
 __global__ __launch_bounds__(ROW_WAVES * 64) void softmax_bwd_kernel(const T *dp, const T *p, T *ds, int64_t rows,
                                                                    int width, int64_t ld) {
     const int lane = threadIdx.x & 63;
     const int64_t r = (int64_t)blockIdx.x * ROW_WAVES + (threadIdx.x >> 6);
     if (r >= rows) return;
-    RowRegs<T, EPV> g, o;
+    RowRegs<T, EPV, MAXE> g, o;
     g.load(dp + r * ld, width, lane, 0.f);
     o.load(p + r * ld, width, lane, 0.f);
     float s = 0.f;
 #pragma unroll
-    for (int e = 0; e < ROW_MAXE; ++e) s += g.v[e] * o.v[e];
+    for (int e = 0; e < MAXE; ++e) s += g.v[e] * o.v[e];
     s = wave_sum(s);
 #pragma unroll
-    for (int e = 0; e < ROW_MAXE; ++e) g.v[e] = o.v[e] * (g.v[e] - s);
+    for (int e = 0; e < MAXE; ++e) g.v[e] = o.v[e] * (g.v[e] - s);
     g.store(ds + r * ld, width, lane);
 }
 
@@ -172,12 +175,23 @@ template <typename T> int row_epv(const void *const *ptrs, int n, int64_t width)
     return ok ? EPV : 1;
 }
 
-#define HAPMI_ROW_DISPATCH(KERNEL, T, epv, grid, stream, ...)                                               \
+#define HAPMI_ROW_LAUNCH(KERNEL, T, EPV_, MAXE_, grid, stream, ...) \
+    hipLaunchKernelGGL((KERNEL<T, EPV_, MAXE_>), grid, dim3(ROW_WAVES * 64), 0, stream, __VA_ARGS__)
+
+// `width` picks the instance with the fewest elements per lane that holds a row
+#define HAPMI_ROW_DISPATCH(KERNEL, T, epv, width, grid, stream, ...)                                        \
     do {                                                                                                    \
-        if ((epv) == 1)                                                                                     \
-            hipLaunchKernelGGL((KERNEL<T, 1>), grid, dim3(ROW_WAVES * 64), 0, stream, __VA_ARGS__);         \
-        else                                                                                                \
-            hipLaunchKernelGGL((KERNEL<T, 16 / sizeof(T)>), grid, dim3(ROW_WAVES * 64), 0, stream, __VA_ARGS__); \
+        constexpr int V_ = 16 / sizeof(T);                                                                  \
+        const int me_ = (width) <= 8 * 64 ? 8 : ((width) <= 16 * 64 ? 16 : 32);                             \
+        if ((epv) == 1) {                                                                                   \
+            if (me_ == 8) HAPMI_ROW_LAUNCH(KERNEL, T, 1, 8, grid, stream, __VA_ARGS__);                     \
+            else if (me_ == 16) HAPMI_ROW_LAUNCH(KERNEL, T, 1, 16, grid, stream, __VA_ARGS__);              \
+            else HAPMI_ROW_LAUNCH(KERNEL, T, 1, 32, grid, stream, __VA_ARGS__);                             \
+        } else {                                                                                            \
+            if (me_ == 8) HAPMI_ROW_LAUNCH(KERNEL, T, V_, 8, grid, stream, __VA_ARGS__);                    \
+            else if (me_ == 16) HAPMI_ROW_LAUNCH(KERNEL, T, V_, 16, grid, stream, __VA_ARGS__);             \
+            else HAPMI_ROW_LAUNCH(KERNEL, T, V_, 32, grid, stream, __VA_ARGS__);                            \
+        }                                                                                                   \
     } while (0)
 
 int check_rows(const char *name, int64_t rows, int64_t width, int dtype) {
@@ -202,11 +216,11 @@ extern "C" int hapmi_add_layernorm_fwd(const void *x, const void *res, void *y, 
     const void *ptrs[3] = {x, y, res};
     if (dtype == HAPMI_F32) {
         int epv = row_epv<float>(ptrs, 3, width);
-        HAPMI_ROW_DISPATCH(add_layernorm_fwd_kernel, float, epv, grid, (hipStream_t)stream, (const float *)x,
+        HAPMI_ROW_DISPATCH(add_layernorm_fwd_kernel, float, epv, width, grid, (hipStream_t)stream, (const float *)x,
                            (const float *)res, (float *)y, rstd, rows, (int)width, eps);
     } else {
         int epv = row_epv<bf16_t>(ptrs, 3, width);
-        HAPMI_ROW_DISPATCH(add_layernorm_fwd_kernel, bf16_t, epv, grid, (hipStream_t)stream, (const bf16_t *)x,
+        HAPMI_ROW_DISPATCH(add_layernorm_fwd_kernel, bf16_t, epv, width, grid, (hipStream_t)stream, (const bf16_t *)x,
                            (const bf16_t *)res, (bf16_t *)y, rstd, rows, (int)width, eps);
     }
     HAPMI_CHECK_LAUNCH("add_layernorm_fwd");
@@ -223,11 +237,11 @@ extern "C" int hapmi_layernorm_bwd(const void *dy, const void *y, const float *r
     const void *ptrs[4] = {dy, y, dx, dx_add};
     if (dtype == HAPMI_F32) {
         int epv = row_epv<float>(ptrs, 4, width);
-        HAPMI_ROW_DISPATCH(layernorm_bwd_kernel, float, epv, grid, (hipStream_t)stream, (const float *)dy,
+        HAPMI_ROW_DISPATCH(layernorm_bwd_kernel, float, epv, width, grid, (hipStream_t)stream, (const float *)dy,
                            (const float *)y, rstd, (const float *)dx_add, (float *)dx, rows, (int)width);
     } else {
         int epv = row_epv<bf16_t>(ptrs, 4, width);
-        HAPMI_ROW_DISPATCH(layernorm_bwd_kernel, bf16_t, epv, grid, (hipStream_t)stream, (const bf16_t *)dy,
+        HAPMI_ROW_DISPATCH(layernorm_bwd_kernel, bf16_t, epv, width, grid, (hipStream_t)stream, (const bf16_t *)dy,
                            (const bf16_t *)y, rstd, (const bf16_t *)dx_add, (bf16_t *)dx, rows, (int)width);
     }
     HAPMI_CHECK_LAUNCH("layernorm_bwd");
@@ -246,11 +260,11 @@ extern "C" int hapmi_softmax_fwd(const void *x, const float *mask, void *p, int6
     const void *ptrs[3] = {x, p, (const void *)(uintptr_t)(ld * hapmi_elem_size(dtype))};
     if (dtype == HAPMI_F32) {
         int epv = row_epv<float>(ptrs, 3, width);
-        HAPMI_ROW_DISPATCH(softmax_fwd_kernel, float, epv, grid, (hipStream_t)stream, (const float *)x, mask,
+        HAPMI_ROW_DISPATCH(softmax_fwd_kernel, float, epv, width, grid, (hipStream_t)stream, (const float *)x, mask,
                            (float *)p, rows, (int)width, ld, mask_rows);
     } else {
         int epv = row_epv<bf16_t>(ptrs, 3, width);
-        HAPMI_ROW_DISPATCH(softmax_fwd_kernel, bf16_t, epv, grid, (hipStream_t)stream, (const bf16_t *)x, mask,
+        HAPMI_ROW_DISPATCH(softmax_fwd_kernel, bf16_t, epv, width, grid, (hipStream_t)stream, (const bf16_t *)x, mask,
                            (bf16_t *)p, rows, (int)width, ld, mask_rows);
     }
     HAPMI_CHECK_LAUNCH("softmax_fwd");
@@ -268,11 +282,11 @@ extern "C" int hapmi_softmax_bwd(const void *dp, const void *p, void *ds, int64_
     const void *ptrs[4] = {dp, p, ds, (const void *)(uintptr_t)(ld * hapmi_elem_size(dtype))};
     if (dtype == HAPMI_F32) {
         int epv = row_epv<float>(ptrs, 4, width);
-        HAPMI_ROW_DISPATCH(softmax_bwd_kernel, float, epv, grid, (hipStream_t)stream, (const float *)dp,
+        HAPMI_ROW_DISPATCH(softmax_bwd_kernel, float, epv, width, grid, (hipStream_t)stream, (const float *)dp,
                            (const float *)p, (float *)ds, rows, (int)width, ld);
     } else {
         int epv = row_epv<bf16_t>(ptrs, 4, width);
-        HAPMI_ROW_DISPATCH(softmax_bwd_kernel, bf16_t, epv, grid, (hipStream_t)stream, (const bf16_t *)dp,
+        HAPMI_ROW_DISPATCH(softmax_bwd_kernel, bf16_t, epv, width, grid, (hipStream_t)stream, (const bf16_t *)dp,
                            (const bf16_t *)p, (bf16_t *)ds, rows, (int)width, ld);
     }
     HAPMI_CHECK_LAUNCH("softmax_bwd");

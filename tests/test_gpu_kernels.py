@@ -72,7 +72,7 @@ def test_gemm_refuses_misaligned(cuda):
 
 
 @pytest.mark.parametrize("dtype", DT)
-@pytest.mark.parametrize("rows,width", [(384, 512), (37, 768), (5, 1024), (9, 100), (3, 2048)])
+@pytest.mark.parametrize("rows,width", [(384, 512), (37, 768), (5, 1024), (9, 100), (3, 2048), (4, 520), (6, 1030), (7, 1032), (2, 8)])
 def test_add_layernorm_forward_backward(cuda, dtype, rows, width):
     g = torch.Generator().manual_seed(rows)
     x, r = torch.randn(rows, width, generator=g).to(dtype), torch.randn(rows, width, generator=g).to(dtype)

@@ -276,11 +276,20 @@ def test_hip_graph_replays_equal_eager_steps(cuda, dtype, opt):
     # Bias and embedding gradients are summed with float atomics, so two runs agree only up to summation order;
     # Adam turns that rounding noise into +-lr where the true gradient is zero (the key bias), so those elements
     # are left out of the parameter comparison.
+    # In bf16 one such flipped update of a key bias changes the rounding of every activation behind it, so from the
+    # next step on all gradients of the two runs agree to bf16 rounding only and the zero-gradient elements are
+    # unrelated noise: there the comparison is the one between two bf16 runs (a replay that went wrong differs by the
+    # size of the values).
     for n, rec in graphed.params.items():
         g = eager.params[n]["grad"]
-        torch.testing.assert_close(rec["grad"], g, rtol=1e-4, atol=1e-5 * g.abs().max().item())
         clear = g.abs() > 1e-3 * g.abs().max()
-        torch.testing.assert_close(rec["master"][clear], eager.params[n]["master"][clear], rtol=1e-4, atol=1e-6)
+        if dtype == "fp32":
+            torch.testing.assert_close(rec["grad"], g, rtol=1e-4, atol=1e-5 * g.abs().max().item())
+            torch.testing.assert_close(rec["master"][clear], eager.params[n]["master"][clear], rtol=1e-4, atol=1e-6)
+        else:
+            assert rel_err(rec["grad"][clear], g[clear]) < 2e-2, n
+            torch.testing.assert_close(rec["master"][clear], eager.params[n]["master"][clear], rtol=1e-2,
+                                       atol=2 * opt["lr"])
 
 
 @pytest.mark.parametrize("dtype", ["fp32", "bf16"])
