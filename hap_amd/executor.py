@@ -1311,7 +1311,7 @@ class ShardExecutor:
         dgate = self._new((B, S, 2), torch.float32)
         route = ops.switch_gate_into if node.target is models.switch_gating else ops.top2_gate_into
         self.fwd.append(lambda: (ops.gemm(x.t, wg.t, logits, B * S, E, d), route(logits, C, r)))
-        v = Val("gating", None, x=x, E=E, C=C, r=r, dgate=dgate, dgate_used=False)
+        v = Val("gating", None, x=x, E=E, C=C, r=r, dgate=dgate, dgate_used=False, logits=logits)
 
         def emit():
             if not v.meta["dgate_used"]:

@@ -145,20 +145,157 @@ class JointCPURun:
         return [l.detach() for l in losses]
 
 
-class PeerlessCPURun(JointCPURun):
-    """One rank only, peers silent: every collective keeps its local half and
-    receives zeros (all_gather / all_to_all) or nothing (reductions) from the
-    other ranks.  Used to time the CPU baseline of a single shard at full
-    size without executing the peers' share of the work."""
+def _rank_ordered_sum(own: torch.Tensor, rank: int, peers: Dict[int, Optional[torch.Tensor]], W: int) -> torch.Tensor:
+    """Sum over ranks in rank order with float32 accumulation (collectives.py:27, :77, :95); a peer that
+    contributes nothing (None) is left out."""
+    parts = [own if s == rank else peers.get(s) for s in range(W)]
+    parts = [p for p in parts if p is not None]
+    acc = parts[0].float().clone()
+    for p in parts[1:]:
+        acc = acc + p.float()
+    return acc.to(own.dtype)
 
-    def __init__(self, program: torch.fx.GraphModule, rank: int, dtype: str = "fp32"):
+
+class SingleRankCPURun(JointCPURun):
+    """ONE rank of the SPMD program on the CPU; what the other ranks would send comes from a wire object with
+    the interface of hap_amd.wire.Wire (``recv(tag, direction, src, shape, dtype, device, reduction)``), asked
+    for exactly the messages, shapes and directions that the product's executor asks its wire for:
+
+    * all_gather (collectives.py:14-29): forward receives every peer's shard padded to the longest length and
+      keeps its first L[src] entries; backward splits the gradient, keeps this rank's piece and adds the peers'
+      padded pieces (first L[rank] entries) in rank order;
+    * reduce_scatter (collectives.py:88-103): the two directions swapped;
+    * all_to_all (collectives.py:152-166): receives from rank src a piece of this rank's split length along the
+      split dimension and cat_L[src] along the concatenation dimension; backward with the roles swapped;
+    * all_reduce (collectives.py:73-84) and the gradient of replicate (collectives.py:176-180): rank-ordered sum
+      with the peers' tensors of the same shape.
+
+    With a ReplayWire over the log of a JointCPURun it reproduces that rank of the joint run (this is what
+    pins it: tests/test_oracle_single_rank.py); with a SyntheticWire the peers' messages are the same seeded
+    tensors the GPU run receives; with a SilentWire the peers send zeros / nothing.
+
+    ``wire_dtype``: element type the messages are made in before they are cast to this run's own type
+    (a float32 CPU run that checks a bf16 GPU run receives the same bf16-rounded messages)."""
+
+    def __init__(self, program: torch.fx.GraphModule, rank: int, world_size: int, wire, dtype: str = "fp32",
+                 wire_dtype: Optional[torch.dtype] = None):
         super().__init__([program], dtype)
-        self.rank = rank
+        self.rank, self.world_size, self.wire = rank, world_size, wire
+        self.wire_dtype = wire_dtype
+
+    # -- wire access -----------------------------------------------------
+    def _recv(self, tag, direction, src, shape, like: torch.Tensor, reduction: bool, dtype=None):
+        dt = dtype or self.wire_dtype or like.dtype
+        t = self.wire.recv(tag, direction, src, tuple(shape), dt, torch.device("cpu"), reduction=reduction)
+        return None if t is None else t.to(like.dtype)
+
+    def _peers(self, tag, direction, shape, like, reduction, dtype=None):
+        return {s: self._recv(tag, direction, s, shape, like, reduction, dtype)
+                for s in range(self.world_size) if s != self.rank}
+
+    # -- the two directions of all_gather / reduce_scatter ---------------
+    def _gather(self, tag, direction, x, dim, L, dtype=None):
+        m = max(L)
+        pshape = list(x.shape)
+        pshape[dim] = m
+        peers = self._peers(tag, direction, pshape, x, False, dtype)
+        return torch.cat([x if s == self.rank else peers[s].narrow(dim, 0, L[s]) for s in range(len(L))], dim=dim)
+
+    def _scatter(self, tag, direction, full, dim, L, dtype=None):
+        m = max(L)
+        own = torch.split(full.contiguous(), list(L), dim=dim)[self.rank]
+        pshape = list(full.shape)
+        pshape[dim] = m
+        peers = self._peers(tag, direction, pshape, full, True, dtype)
+        peers = {s: (p.narrow(dim, 0, L[self.rank]) if p is not None else None) for s, p in peers.items()}
+        return _rank_ordered_sum(own, self.rank, peers, len(L))
+
+    def _exchange(self, tag, direction, x, split_dim, cat_dim, split_L, cat_L):
+        own = torch.split(x.contiguous(), list(split_L), dim=split_dim)[self.rank]
+        parts = []
+        for s in range(len(split_L)):
+            if s == self.rank:
+                parts.append(own)
+            else:
+                shape = list(own.shape)
+                shape[cat_dim] = cat_L[s]
+                parts.append(self._recv(tag, direction, s, shape, x, False))
+        return torch.cat(parts, dim=cat_dim)
+
+    def _sum(self, tag, direction, x, dtype=None):
+        return _rank_ordered_sum(x, self.rank, self._peers(tag, direction, x.shape, x, True, dtype), self.world_size)
+
+    # -- collectives as autograd nodes over this rank's tensor -----------
+    def _collective(self, node, args):
+        run, t, tag = self, node.target, node.name
+        # a gathered parameter (ZeRO form) is not an activation: its shard travels in the type it is stored in and
+        # its gradient comes back in float32, whatever type the activations' messages are made in
+        of_param = node.args[0].op == "get_attr"
+
+        if t in (product_collectives.all_gather, product_collectives.reduce_scatter):
+            xin, dim, L, rank = args
+            assert rank == self.rank
+            gather_fwd = t is product_collectives.all_gather
+            fwd_dtype = xin.dtype if of_param else None
+            bwd_dtype = torch.float32 if (of_param and self.wire_dtype is not None) else fwd_dtype
+
+            class Fn(torch.autograd.Function):
+                @staticmethod
+                def forward(ctx, x):
+                    if gather_fwd:
+                        return run._gather(tag, "fwd", x, dim, list(L), fwd_dtype)
+                    return run._scatter(tag, "fwd", x, dim, list(L))
+
+                @staticmethod
+                def backward(ctx, g):
+                    if gather_fwd:
+                        return run._scatter(tag, "bwd", g, dim, list(L), bwd_dtype)
+                    return run._gather(tag, "bwd", g.contiguous(), dim, list(L))
+            return Fn.apply(xin)
+
+        if t is product_collectives.all_to_all:
+            xin, sd, cd, sL, cL, rank = args
+            assert rank == self.rank
+
+            class Fn(torch.autograd.Function):
+                @staticmethod
+                def forward(ctx, x):
+                    return run._exchange(tag, "fwd", x, sd, cd, sL, cL)
+
+                @staticmethod
+                def backward(ctx, g):
+                    return run._exchange(tag, "bwd", g, cd, sd, cL, sL)
+            return Fn.apply(xin)
+
+        if t is product_collectives.all_reduce:
+            class Fn(torch.autograd.Function):
+                @staticmethod
+                def forward(ctx, x):
+                    return run._sum(tag, "fwd", x.contiguous())
+
+                @staticmethod
+                def backward(ctx, g):
+                    return run._sum(tag, "bwd", g.contiguous())
+            return Fn.apply(args[0])
+
+        if t is product_collectives.replicate:
+            class Fn(torch.autograd.Function):
+                @staticmethod
+                def forward(ctx, x):
+                    return x.view_as(x)
+
+                @staticmethod
+                def backward(ctx, g):
+                    return run._sum(tag, "bwd", g.contiguous(), torch.float32)
+            return Fn.apply(args[0])
+        raise ValueError(t)
 
     def forward(self, x, y):
         env = self.env[0]
         prog = self.programs[0]
         look = lambda a: torch.fx.node.map_arg(a, lambda n: env[n.name])
+        wire_ops = (product_collectives.all_gather, product_collectives.reduce_scatter, product_collectives.all_to_all,
+                    product_collectives.all_reduce, product_collectives.replicate)
         n_inputs = 0
         for node in prog.graph.nodes:
             if node.op == "placeholder":
@@ -171,36 +308,26 @@ class PeerlessCPURun(JointCPURun):
                 env[node.name] = getattr(a[0], node.target)(*a[1:])
             elif node.op == "output":
                 return [look(node.args[0])]
+            elif node.target in wire_ops:
+                env[node.name] = self._collective(node, look(node.args))
             else:
-                t = node.target
-                if t is product_collectives.all_gather:
-                    xin, dim, L, rank = look(node.args)
-                    parts = []
-                    for i, l in enumerate(L):
-                        if i == rank:
-                            parts.append(xin)
-                        else:
-                            shape = list(xin.shape)
-                            shape[dim] = l
-                            parts.append(torch.zeros(shape, dtype=xin.dtype))
-                    env[node.name] = torch.cat(parts, dim=dim)
-                elif t is product_collectives.reduce_scatter:
-                    xin, dim, L, rank = look(node.args)
-                    env[node.name] = torch.split(xin, list(L), dim=dim)[rank].contiguous()
-                elif t is product_collectives.all_to_all:
-                    xin, sd, cd, sL, cL, rank = look(node.args)
-                    own = torch.split(xin, list(sL), dim=sd)[rank]
-                    parts = []
-                    for i, l in enumerate(cL):
-                        if i == rank:
-                            parts.append(own)
-                        else:
-                            shape = list(own.shape)
-                            shape[cd] = l
-                            parts.append(torch.zeros(shape, dtype=own.dtype))
-                    env[node.name] = torch.cat(parts, dim=cd)
-                elif t in (product_collectives.all_reduce, product_collectives.replicate):
-                    env[node.name] = look(node.args[0])
-                else:
-                    env[node.name] = self._call_local(0, node)
+                env[node.name] = self._call_local(0, node)
         raise RuntimeError("program has no output node")
+
+
+class PeerlessCPURun(SingleRankCPURun):
+    """One rank only, peers silent: every collective keeps its local half and receives zeros (all_gather /
+    all_to_all) or nothing (reductions) from the other ranks.  Used to time the CPU baseline of a single
+    shard at full size without executing the peers' share of the work."""
+
+    def __init__(self, program: torch.fx.GraphModule, rank: int, dtype: str = "fp32", world_size: Optional[int] = None):
+        from hap_amd.wire import SilentWire
+        if world_size is None:
+            world_size = 1
+            for node in program.graph.nodes:
+                if node.op == "call_function" and node.target in (product_collectives.all_gather,
+                                                                  product_collectives.reduce_scatter):
+                    world_size = max(world_size, len(node.args[2]))
+                elif node.op == "call_function" and node.target is product_collectives.all_to_all:
+                    world_size = max(world_size, len(node.args[3]))
+        super().__init__(program, rank, world_size, SilentWire(), dtype)

@@ -1,84 +1,241 @@
-"""The benchmark configurations at their full per-kernel shapes (every GEMM, attention, gating, collective
-copy and optimizer launch has the shape it has in the benchmark) with the depth cut to two layers, one rank with
-silent peers on both sides, against the float32 CPU oracle, which is the reference's arithmetic
-(stock PyTorch eager + autograd on the same generated graph).
+"""The benchmark configurations at their full per-kernel shapes (every GEMM, attention, gating, collective copy
+and optimizer launch has the shape it has in the benchmark), one rank whose peers send SEEDED N(0, 1) activations and
+N(0, 1e-3) gradients (hap_amd.SyntheticWire: the same tensors on both sides, so every row of a gathered tensor and
+every column of an exchanged one carries signal), against the CPU oracle (stock PyTorch eager + autograd on the
+same generated graph: the reference's arithmetic), which tests/test_oracle_single_rank.py pins on the CPU.
 
-Tolerances: the bf16 run against the float32 CPU run: 2e-2 on the loss, 3e-2 norm-wise on every gradient
-that carries signal (the margin the small-size bf16 cases use as well), 8e-2 right behind a ReLU mask; the float32 run: 1e-4 on the loss, 3e-4 norm-wise on gradients (sums over 6144-16384 tokens
-in a different order), 8e-4 right behind a ReLU mask, routing indices and slots bit-exact."""
+Tolerances are the stated ones: float32 runs 1e-4, bf16 runs 2e-2, on the loss, norm-wise on every gradient that
+carries signal, and on the updated weights.  One class of gradients is held to a measured bound instead: a
+gradient taken right behind a ReLU mask (linear1.*, the experts' w1).  The mask is a step function of the
+pre-activation, so an element whose pre-activation lies within rounding distance of zero flips it, and the
+gradient's norm-wise error is about the square root of the fraction of such elements, whatever computes it.  The
+test measures that effect on the oracle itself, on the same tensors (the float32 CPU run against the float64
+CPU run; the bf16 CPU run against the float32 CPU run), prints it, and allows the GPU the stated tolerance or 1.5
+times what the oracle shows, whichever is larger.
+"""
 import pytest
 import torch
 
 import bench
 import hap_amd
+from hap_amd import models, ops
 from helpers import rel_err
-from oracle.cpu_executor import PeerlessCPURun
+from oracle import ops as ref_ops
+from oracle.cpu_executor import SingleRankCPURun
 
 pytestmark = pytest.mark.gpu
 
+SEED = 11
 
-def _both(name, dtype, layers=2):
-    gm_ref, x, y, meta = bench.build_workload(name, layers_override=layers)
-    run = PeerlessCPURun(gm_ref, 0, "fp32")
-    torch.set_num_threads(16)
-    want = run.step(x, y)[0].item()
-    ref_grads = {n: p.grad for n, p in gm_ref.named_parameters() if p.grad is not None}
+
+def _cpu_run(name, layers, dtype, wire_dtype, double=False, opt=False):
     gm, x, y, meta = bench.build_workload(name, layers_override=layers)
-    ex = hap_amd.compile_program(gm, [x, y], dtype=dtype, wire=hap_amd.SilentWire(), rank=0,
+    if double:
+        gm = gm.double()
+    run = SingleRankCPURun(gm, 0, len(meta["ratios"]), hap_amd.SyntheticWire(seed=SEED), dtype, wire_dtype=wire_dtype)
+    torch.set_num_threads(16)
+    optim = [torch.optim.Adam(gm.parameters(), lr=meta["opt"]["lr"])] if opt else None
+    before = {n: p.detach().clone() for n, p in gm.named_parameters()} if opt else None
+    loss = run.step(x, y, optimizers=optim)[0].item()
+    grads = {n: p.grad for n, p in gm.named_parameters() if p.grad is not None}
+    return run, gm, loss, grads, before
+
+
+def _gpu_run(name, layers, dtype, opt=False, wire=None):
+    gm, x, y, meta = bench.build_workload(name, layers_override=layers)
+    ex = hap_amd.compile_program(gm, [x, y], dtype=dtype, wire=wire or hap_amd.SyntheticWire(seed=SEED), rank=0,
                                  world_size=len(meta["ratios"]))
+    before = {n: rec["master"].clone() for n, rec in ex.params.items()} if opt else None
+    if opt:
+        ex.configure_optimizer(**meta["opt"])
     loss = ex.forward(x, y)
     ex.backward()
     torch.cuda.synchronize()
-    return ex, run, loss.item(), want, ref_grads
+    grads = {n: rec["grad"].clone() for n, rec in ex.params.items()}
+    if opt:
+        ex.step()
+        torch.cuda.synchronize()
+    return ex, loss.item(), grads, before
 
 
-def _check_grads(ex, ref_grads, tol, tol_relu, floor=1e-4):
-    """Every gradient that carries signal within ``tol`` norm-wise, except the parameters whose gradient passes
-    through the ReLU mask right behind them (linear1.*, the experts' w1): the mask is a step function of the
-    pre-activation, an element within rounding distance eps of zero flips it, a fraction ~eps of the elements
-    does, and the norm-wise error of that gradient is ~sqrt(eps) (5e-2 for bf16, 4e-4 for float32 addends summed
-    in another order): ``tol_relu``."""
-    assert set(ex.params) == set(ref_grads)
-    worst = {False: ("", 0.0), True: ("", 0.0)}
-    scale = max(g.norm().item() for g in ref_grads.values())
-    for n, rec in ex.params.items():
-        ref = ref_grads[n]
-        if ref.norm().item() < floor * scale:      # no signal (key bias of softmax attention): rounding noise on both sides
+def _behind_relu(n):
+    return "linear1" in n or n.endswith(".w1")
+
+
+def _check_grads(grads, want, tol, oracle_pair=None, floor=1e-4):
+    """``oracle_pair`` = (low, high): the oracle's own gradients at this run's precision and at the next higher one;
+    their distance bounds what a gradient behind a ReLU mask can be held to."""
+    assert set(grads) == set(want)
+    scale = max(g.norm().item() for g in want.values())
+    worst, worst_relu, oracle_relu = ("", 0.0), ("", 0.0), 0.0
+    for n, g in grads.items():
+        ref = want[n]
+        if ref.norm().item() < floor * scale:       # no signal (key bias of softmax attention): rounding noise on both sides
             continue
-        err = rel_err(rec["grad"], ref)
-        k = "linear1" in n or n.endswith(".w1")
-        if err > worst[k][1]:
-            worst[k] = (n, err)
-    print("worst gradient error (plain / behind a ReLU mask):", worst[False], worst[True])
-    assert worst[False][1] < tol, worst[False]
-    assert worst[True][1] < tol_relu, worst[True]
+        err = rel_err(g, ref)
+        if _behind_relu(n):
+            own = rel_err(oracle_pair[0][n], oracle_pair[1][n]) if oracle_pair is not None else 0.0
+            oracle_relu = max(oracle_relu, own)
+            if err > worst_relu[1]:
+                worst_relu = (n, err)
+            assert err < max(tol, 1.5 * own), (n, err, own)
+        else:
+            if err > worst[1]:
+                worst = (n, err)
+            assert err < tol, (n, err)
+    print(f"worst gradient error: {worst}; behind a ReLU mask: {worst_relu}, where the oracle's own runs at the two "
+          f"precisions differ by up to {oracle_relu:.2e}")
+
+
+def test_wire_requests_of_gpu_and_cpu_runs_match(cuda):
+    """The executor and the CPU oracle ask the wire for the same messages (tag, direction, sender, shape)."""
+    class Recording(hap_amd.SyntheticWire):
+        def __init__(self):
+            super().__init__(seed=SEED)
+            self.requests = set()
+
+        def recv(self, tag, direction, src, shape, dtype, device, reduction=False, into=None):
+            if not (tag.startswith("replicate") and not self.reduce_params):
+                self.requests.add((tag, direction, src, tuple(shape)))
+            return super().recv(tag, direction, src, shape, dtype, device, reduction=reduction, into=into)
+
+    for name in ("lm", "moe"):
+        wire_gpu, wire_cpu = Recording(), Recording()
+        _gpu_run(name, 2, "fp32", wire=wire_gpu)
+        gm, x, y, meta = bench.build_workload(name, layers_override=2)
+        SingleRankCPURun(gm, 0, len(meta["ratios"]), wire_cpu).step(x, y)
+        assert wire_gpu.requests and wire_gpu.requests == wire_cpu.requests, name
+
+
+def test_lm_config1_full_size_fp32_against_float64_oracle(cuda):
+    """BASELINE config 1 whole (2 layers, float32, SGD): the GPU against the float64 CPU run at 1e-4."""
+    _, gm64, want, grads64, _ = _cpu_run("lm", 2, "fp32", torch.float32, double=True)
+    _, _, loss32, grads32, _ = _cpu_run("lm", 2, "fp32", torch.float32)
+    ex, loss, grads, _ = _gpu_run("lm", 2, "fp32")
+    assert abs(loss - want) <= 1e-4 * abs(want), (loss, want)
+    _check_grads(grads, grads64, 1e-4, (grads32, grads64))
 
 
 def test_bert_large_shard_full_width_bf16(cuda):
-    ex, run, loss, want, ref_grads = _both("bert", "bf16")
+    _, _, want, grads32, _ = _cpu_run("bert", 2, "fp32", torch.bfloat16)
+    _, _, _, grads16, _ = _cpu_run("bert", 2, "bf16", torch.bfloat16)
+    ex, loss, grads, _ = _gpu_run("bert", 2, "bf16")
     assert abs(loss - want) <= 2e-2 * abs(want), (loss, want)
-    _check_grads(ex, ref_grads, 3e-2, 8e-2)
+    _check_grads(grads, grads32, 2e-2, (grads16, grads32))
+
+
+def test_bert_large_shard_full_depth_bf16_adam_step(cuda):
+    """All 24 layers of BASELINE config 2 with one Adam step: loss, gradients and updated weights."""
+    _, gm_ref, want, grads32, before_ref = _cpu_run("bert", 24, "fp32", torch.bfloat16, opt=True)
+    ex, loss, grads, before = _gpu_run("bert", 24, "bf16", opt=True)
+    assert abs(loss - want) <= 2e-2 * abs(want), (loss, want)
+    # the ReLU-mask bound measured at two layers (the test above prints it) holds per layer; here those gradients
+    # are held to twice the stated tolerance instead of repeating the 24-layer CPU run in bf16
+    assert set(grads) == set(grads32)
+    scale = max(g.norm().item() for g in grads32.values())
+    worst = {False: ("", 0.0), True: ("", 0.0)}
+    for n, g in grads.items():
+        if grads32[n].norm().item() < 1e-4 * scale:
+            continue
+        err = rel_err(g, grads32[n])
+        k = _behind_relu(n)
+        if err > worst[k][1]:
+            worst[k] = (n, err)
+    print("24 layers, worst gradient error (plain / behind a ReLU mask):", worst[False], worst[True])
+    assert worst[False][1] < 2e-2, worst[False]
+    assert worst[True][1] < 4e-2, worst[True]
+    ref_after = dict(gm_ref.named_parameters())
+    lr = 5e-4
+    worst_w, worst_u = ("", 0.0), ("", 0.0)
+    for n, rec in ex.params.items():
+        new, old, new_ref = rec["master"], before[n], ref_after[n].detach()
+        torch.testing.assert_close(old.cpu(), before_ref[n], rtol=0, atol=0)
+        err = rel_err(new, new_ref)
+        if err > worst_w[1]:
+            worst_w = (n, err)
+        assert err < 2e-2, (n, err)
+        # the bf16 shadow the next step reads is the rounded master
+        torch.testing.assert_close(rec["shadow"], new.to(torch.bfloat16), rtol=0, atol=0)
+        # Adam's first step is -lr * sign(g) (up to eps): where the oracle's gradient is clearly non-zero the two
+        # updates must agree; elsewhere the sign is rounding noise on both sides
+        g_ref = grads32[n].float()
+        clear = g_ref.abs() > 1e-2 * g_ref.abs().max()
+        if clear.any():
+            du, du_ref = (new - old).cpu()[clear], (new_ref - before_ref[n])[clear]
+            err_u = rel_err(du, du_ref)
+            if err_u > worst_u[1]:
+                worst_u = (n, err_u)
+            assert err_u < 2e-2, (n, err_u)
+            assert (du.abs() - lr).abs().max() < 0.02 * lr, n
+    print("24 layers after one Adam step: worst weight error", worst_w, "worst update error", worst_u)
 
 
 def test_vit_large_shard_full_width_bf16(cuda):
-    ex, run, loss, want, ref_grads = _both("vit", "bf16", layers=1)
+    _, _, want, grads32, _ = _cpu_run("vit", 1, "fp32", torch.bfloat16)
+    _, _, _, grads16, _ = _cpu_run("vit", 1, "bf16", torch.bfloat16)
+    ex, loss, grads, _ = _gpu_run("vit", 1, "bf16")
     assert abs(loss - want) <= 2e-2 * abs(want), (loss, want)
-    _check_grads(ex, ref_grads, 3e-2, 8e-2)
+    _check_grads(grads, grads32, 2e-2, (grads16, grads32))
+
+
+def _routing_of(ex, run):
+    """(node, GPU routing records, GPU float32 logits, oracle's dense dispatch / combine) per gating node."""
+    out = []
+    for node in ex.gm.graph.nodes:
+        if node.op == "call_function" and node.target is models.top_2_gating:
+            v = ex.env[node]
+            out.append((node, v.meta["r"], v.meta["logits"], run.env[0][node.name]))
+    return out
 
 
 def test_moe_shard_full_width_fp32_routing_bit_exact(cuda):
-    ex, run, loss, want, ref_grads = _both("moe", "fp32")
+    run, _, want, grads64, _ = _cpu_run("moe", 2, "fp32", torch.float32, double=True)
+    run32, _, _, grads32, _ = _cpu_run("moe", 2, "fp32", torch.float32)
+    ex, loss, grads, _ = _gpu_run("moe", 2, "fp32")
     assert abs(loss - want) <= 1e-4 * abs(want), (loss, want)
-    _check_grads(ex, ref_grads, 3e-4, 8e-4)
-    # dense dispatch mask and combine weights of the oracle against the GPU's routing records
-    from hap_amd import models, ops
-    n = 0
-    for node in ex.gm.graph.nodes:
-        if node.op == "call_function" and node.target is models.top_2_gating:
-            dispatch, combine = run.env[0][node.name]
-            B, S, E, C = dispatch.shape
-            got_d, got_c = ops.top2_densify(ex.env[node].meta["r"], E, C)
-            assert torch.equal(got_d.cpu().bool(), dispatch.bool())
-            torch.testing.assert_close(got_c.cpu(), combine.detach().float(), rtol=1e-4, atol=1e-6)
-            n += 1
-    assert n == 1
+    _check_grads(grads, grads64, 1e-4, (grads32, grads64))
+    # dense dispatch mask and combine weights of the float32 oracle against the GPU's routing records
+    recs = _routing_of(ex, run32)
+    assert len(recs) == 1
+    for node, r, logits, (dispatch, combine) in recs:
+        B, S, E, C = dispatch.shape
+        got_d, got_c = ops.top2_densify(r, E, C)
+        assert torch.equal(got_d.cpu().bool(), dispatch.bool())
+        torch.testing.assert_close(got_c.cpu(), combine.detach().float(), rtol=1e-4, atol=1e-6)
+
+
+def test_moe_shard_full_width_bf16(cuda):
+    """BASELINE config 4 in its own element type.  Routing is integer work and must be bit-exact on identical float32
+    logits: the oracle's gating is run on the logits the GPU computed.  End to end the bf16 activations move the
+    logits, so a token whose second and third gate probabilities are closer than that movement may pick another
+    expert than in the float32 oracle: those tokens are counted and every routing difference must be one of them."""
+    run32, _, want, grads32, _ = _cpu_run("moe", 2, "fp32", torch.bfloat16)
+    _, _, _, grads16, _ = _cpu_run("moe", 2, "bf16", torch.bfloat16)
+    ex, loss, grads, _ = _gpu_run("moe", 2, "bf16")
+    assert abs(loss - want) <= 2e-2 * abs(want), (loss, want)
+    recs = _routing_of(ex, run32)
+    assert len(recs) == 1
+    for node, r, logits, (dispatch32, combine32) in recs:
+        B, S, E, C = dispatch32.shape
+        lg = logits.cpu()
+        # (a) identical float32 logits -> identical routing, bit for bit
+        d_same, c_same = ref_ops.top_2_gating(lg, E, C, torch.eye(E))
+        got_d, got_c = ops.top2_densify(r, E, C)
+        assert torch.equal(got_d.cpu().bool(), d_same.bool())
+        torch.testing.assert_close(got_c.cpu(), c_same, rtol=1e-5, atol=1e-7)
+        # (b) against the float32 oracle's own routing: differences only where the choice is a near-tie
+        x32 = run32.env[0][node.args[0].name]
+        wg = run32.env[0][node.args[3].name]
+        lg32 = (x32.float() @ wg.float()).detach()
+        p32 = torch.softmax(lg32, dim=2)
+        top3 = p32.topk(3, dim=2).values
+        moved = (torch.softmax(lg, dim=2) - p32).abs().amax(dim=2)            # how far bf16 moved this token's gates
+        near_tie = ((top3[..., 1] - top3[..., 2]) <= 2 * moved) | ((top3[..., 0] - top3[..., 1]) <= 2 * moved)
+        idx32 = p32.topk(2, dim=2).indices
+        differs = (r["index"].cpu().long() != idx32).any(dim=2)
+        print(f"{node.name}: {int(differs.sum())} of {B * S} tokens routed differently from the float32 oracle, "
+              f"{int(near_tie.sum())} tokens with a top-2 margin below twice the bf16 movement of their gates "
+              f"(largest movement {moved.max().item():.2e})")
+        assert not (differs & ~near_tie).any()
+        assert differs.float().mean().item() < 0.05
+    _check_grads(grads, grads32, 2e-2, (grads16, grads32))
