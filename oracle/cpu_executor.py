@@ -58,8 +58,11 @@ class JointCPURun:
         if t in (product_models.top_2_gating, product_models.switch_gating):
             x, n_expert, capacity, wg = args[:4]
             gating = ref.top_2_gating if t is product_models.top_2_gating else ref.switch_gating
-            dispatch, combine = gating(x.float(), n_expert, capacity, wg.float())
-            return dispatch, combine
+            # float32 whatever the activations' type; a float64 run (a model cast with .double(), used to
+            # calibrate tolerances) gates in float64 and needs the dispatch mask in float64 for the einsums
+            hi = torch.float64 if x.dtype == torch.float64 else torch.float32
+            dispatch, combine = gating(x.to(hi), n_expert, capacity, wg.to(hi))
+            return dispatch.to(hi), combine
         if t is product_models.head_parallel_attention:
             return ref.head_parallel_attention(*args, **kwargs)
         if t is product_models.append_cls_token:
@@ -178,10 +181,33 @@ class SingleRankCPURun(JointCPURun):
     (a float32 CPU run that checks a bf16 GPU run receives the same bf16-rounded messages)."""
 
     def __init__(self, program: torch.fx.GraphModule, rank: int, world_size: int, wire, dtype: str = "fp32",
-                 wire_dtype: Optional[torch.dtype] = None):
+                 wire_dtype: Optional[torch.dtype] = None, decisions: Optional[Dict[str, torch.Tensor]] = None):
+        """``decisions``: discrete decisions taken from another run of the same program, by node name -- for an
+        ``F.relu`` node the boolean mask of the elements it lets through, for a ``top_2_gating`` node the expert
+        choices [B, S, 2].  The node then applies those instead of its own (relu(z) becomes z * mask, the gates
+        stay this run's probabilities of the given experts).  A step function turns a rounding-sized difference of
+        its argument into a whole-sized difference of the result; with the decisions shared, what is left between
+        two runs is their continuous arithmetic, which tolerances can bound.  Whether the other run's decisions
+        differ from this run's own only where the argument is within rounding distance of the step is for the
+        caller to check."""
         super().__init__([program], dtype)
         self.rank, self.world_size, self.wire = rank, world_size, wire
         self.wire_dtype = wire_dtype
+        self.decisions = decisions or {}
+
+    def _call_local(self, r, node):
+        forced = self.decisions.get(node.name)
+        if forced is not None:
+            args = self._lookup(r, node.args)
+            if node.target is F.relu:
+                return args[0] * forced.to(args[0].dtype)
+            if node.target is product_models.top_2_gating:
+                x, n_expert, capacity, wg = args[:4]
+                hi = torch.float64 if x.dtype == torch.float64 else torch.float32
+                dispatch, combine = ref.top_2_gating(x.to(hi), n_expert, capacity, wg.to(hi), index=forced.long())
+                return dispatch.to(hi), combine
+            raise ValueError(f"no shared decision is defined for {node.target}")
+        return super()._call_local(r, node)
 
     # -- wire access -----------------------------------------------------
     def _recv(self, tag, direction, src, shape, like: torch.Tensor, reduction: bool, dtype=None):

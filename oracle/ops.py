@@ -85,12 +85,17 @@ def positional_encoding(seqlen: int, emsize: int) -> np.ndarray:
 # top-2 gating
 # --------------------------------------------------------------------------
 
-def top_2_gating(gate_input, n_expert: int, capacity: int, gate_weight, train: bool = True):
+def top_2_gating(gate_input, n_expert: int, capacity: int, gate_weight, train: bool = True, index=None):
     """models.py:477-502, dense form: returns (dispatch, combine), each
-    [B, S, E, C]; dispatch is float32, combine carries the gate dtype."""
+    [B, S, E, C]; dispatch is float32, combine carries the gate dtype.
+    ``index`` (not in the reference): expert choices [B, S, 2] to use instead of topk's own, for a run that must
+    share its discrete decisions with another run; the gates are still this run's probabilities of those experts."""
     logits = gate_input @ gate_weight                                  # :478
     probs = torch.softmax(logits, dim=2)                               # :479
-    gate, index = probs.topk(2, dim=2)                                 # :481  [B,S,2]
+    if index is None:
+        gate, index = probs.topk(2, dim=2)                             # :481  [B,S,2]
+    else:
+        gate = probs.gather(2, index)
     chosen = F.one_hot(index, n_expert)                                # :483  [B,S,2,E] int64
     pos = chosen.cumsum(dim=1) * chosen                                # :485  1-based, per choice
     first_sum = pos[:, :, 0, :].sum(dim=1, keepdim=True)               # :486  sum of positions (n(n+1)/2)

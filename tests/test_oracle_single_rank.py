@@ -169,3 +169,47 @@ def test_single_rank_run_asks_for_every_peer_message_once_per_direction():
     L_F = hap_amd.sharding_lengths(64, RATIOS4)
     assert shapes[(aa, "fwd")] == (3, 16, L_F[2])           # rank 2's columns of this rank's samples
     assert shapes[(aa, "bwd")] == (1, 16, L_F[0])           # this rank's columns of rank 2's samples
+
+
+def _own_decisions(run, prog):
+    """The discrete decisions a finished run took itself: relu masks and expert choices, by node name."""
+    import torch.nn.functional as F
+    out = {}
+    for node in prog.graph.nodes:
+        if node.op != "call_function":
+            continue
+        if node.target is F.relu:
+            out[node.name] = run.env[0][node.args[0].name].detach() > 0
+        elif node.target is hap_amd.models.top_2_gating:
+            x, wg = run.env[0][node.args[0].name], run.env[0][node.args[3].name]
+            out[node.name] = torch.softmax(x.float() @ wg.float(), dim=2).topk(2, dim=2).indices
+    return out
+
+
+@pytest.mark.parametrize("case", ["lm-column", "moe"])
+def test_a_run_given_its_own_decisions_reproduces_itself(case):
+    """SingleRankCPURun(decisions=...): relu as a multiplication with a given mask and gating with given expert
+    choices are the same functions as the run's own when the decisions are its own."""
+    make, ratios, B, batch, kw = CASES[case]
+    model = make()
+    x, y = batch()
+    W = len(ratios)
+    a = rank_programs(model, ratios, B, **kw)[0]
+    free = SingleRankCPURun(a, 0, W, hap_amd.SyntheticWire(seed=3))
+    la = free.step(x, y)[0]
+    decisions = _own_decisions(free, a)
+    assert any(v.dtype == torch.bool for v in decisions.values())
+    if case == "moe":
+        assert any(v.dtype == torch.int64 for v in decisions.values())
+    b = rank_programs(model, ratios, B, **kw)[0]
+    lb = SingleRankCPURun(b, 0, W, hap_amd.SyntheticWire(seed=3), decisions=decisions).step(x, y)[0]
+    torch.testing.assert_close(la, lb, rtol=0, atol=0)
+    ga, gb = _grads(a), _grads(b)
+    for n in ga:
+        torch.testing.assert_close(ga[n], gb[n], rtol=1e-6, atol=1e-9, msg=lambda m, n=n: f"{n}: {m}")
+    # other decisions give another result (the argument is used)
+    flipped = {k: (~v if v.dtype == torch.bool else v.flip(2)) for k, v in decisions.items()}
+    c = rank_programs(model, ratios, B, **kw)[0]
+    SingleRankCPURun(c, 0, W, hap_amd.SyntheticWire(seed=3), decisions=flipped).step(x, y)
+    gc = _grads(c)
+    assert max(rel_err(gc[n], ga[n]) for n in ga if ga[n].norm() > 0) > 0.5
