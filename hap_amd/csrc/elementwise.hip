@@ -132,33 +132,39 @@ __global__ __launch_bounds__(EW_THREADS) void add_bcast_rows_kernel(const T *a, 
     }
 }
 
-// column sums of x[M, N] (row stride ldx): each block owns 64 columns and a slab of rows
-constexpr int CS_ROWS_PER_BLOCK = 256;
+// column sums of x[M, N] (row stride ldx): each block owns 64 columns and a slab of `rows_per_slab` rows and writes
+// its sum to dst[slab][N] (dst = the output itself when there is one slab, else the workspace, whose slabs
+// colsum_final_kernel adds in order): no atomics, so the same call gives the same bits every time
 template <typename T>
-__global__ __launch_bounds__(256) void colsum_kernel(const T *x, float *out, int64_t M, int64_t N, int64_t ldx) {
+__global__ __launch_bounds__(256) void colsum_kernel(const T *x, float *dst, int64_t M, int64_t N, int64_t ldx,
+                                                   int64_t rows_per_slab, int add_to_dst) {
     __shared__ float part[4][64];
     const int c = threadIdx.x & 63, rg = threadIdx.x >> 6;
     const int64_t col = (int64_t)blockIdx.x * 64 + c;
-    const int64_t r0 = (int64_t)blockIdx.y * CS_ROWS_PER_BLOCK;
-    const int64_t r1 = r0 + CS_ROWS_PER_BLOCK < M ? r0 + CS_ROWS_PER_BLOCK : M;
+    const int64_t r0 = (int64_t)blockIdx.y * rows_per_slab;
+    const int64_t r1 = r0 + rows_per_slab < M ? r0 + rows_per_slab : M;
     float s = 0.f;
     if (col < N)
         for (int64_t r = r0 + rg; r < r1; r += 4) s += ld_f(x, r * ldx + col);
     part[rg][c] = s;
     __syncthreads();
-    if (rg == 0 && col < N) atomicAdd(out + col, part[0][c] + part[1][c] + part[2][c] + part[3][c]);
+    if (rg == 0 && col < N) {
+        const float t = part[0][c] + part[1][c] + part[2][c] + part[3][c];
+        float *o = dst + (int64_t)blockIdx.y * N + col;
+        *o = add_to_dst ? *o + t : t;
+    }
 }
 
 // vectorised form: 32 column groups of one 16-byte vector x 8 row groups per block
-constexpr int CSV_ROWS_PER_BLOCK = 128;
 template <typename T>
-__global__ __launch_bounds__(256) void colsum_vec_kernel(const T *x, float *out, int64_t M, int64_t N, int64_t ldx) {
+__global__ __launch_bounds__(256) void colsum_vec_kernel(const T *x, float *dst, int64_t M, int64_t N, int64_t ldx,
+                                                       int64_t rows_per_slab, int add_to_dst) {
     constexpr int EPV = Vec16<T>::N;
     __shared__ float part[8][32 * EPV + 1];
     const int cg = threadIdx.x & 31, rg = threadIdx.x >> 5;
     const int64_t col = ((int64_t)blockIdx.x * 32 + cg) * EPV;
-    const int64_t r0 = (int64_t)blockIdx.y * CSV_ROWS_PER_BLOCK;
-    const int64_t r1 = r0 + CSV_ROWS_PER_BLOCK < M ? r0 + CSV_ROWS_PER_BLOCK : M;
+    const int64_t r0 = (int64_t)blockIdx.y * rows_per_slab;
+    const int64_t r1 = r0 + rows_per_slab < M ? r0 + rows_per_slab : M;
     float s[EPV];
 #pragma unroll
     for (int e = 0; e < EPV; ++e) s[e] = 0.f;
@@ -177,9 +183,19 @@ __global__ __launch_bounds__(256) void colsum_vec_kernel(const T *x, float *out,
             float t = 0.f;
 #pragma unroll
             for (int g = 0; g < 8; ++g) t += part[g][c];
-            atomicAdd(out + gc, t);
+            float *o = dst + (int64_t)blockIdx.y * N + gc;
+            *o = add_to_dst ? *o + t : t;
         }
     }
+}
+
+__global__ __launch_bounds__(256) void colsum_final_kernel(const float *slabs, float *out, int64_t N, int64_t n_slabs,
+                                                         int accumulate) {
+    const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (c >= N) return;
+    float s = accumulate ? out[c] : 0.f;
+    for (int64_t i = 0; i < n_slabs; ++i) s += slabs[i * N + c];
+    out[c] = s;
 }
 
 template <typename TS, typename TD>
@@ -231,27 +247,38 @@ extern "C" int hapmi_fill_zero(void *p, int64_t bytes, hapmi_stream_t stream) {
 }
 
 extern "C" int hapmi_colsum(const void *x, float *out, int64_t M, int64_t N, int64_t ldx, int accumulate, int dtype,
-                            hapmi_stream_t stream) {
-    HAPMI_REQUIRE(hapmi_dtype_ok(dtype) && M >= 0 && N >= 0 && ldx >= N, HAPMI_EINVAL, "colsum: bad argument");
+                            float *workspace, int64_t workspace_elems, hapmi_stream_t stream) {
+    HAPMI_REQUIRE(hapmi_dtype_ok(dtype) && M >= 0 && N >= 0 && ldx >= N && workspace_elems >= 0, HAPMI_EINVAL, "colsum: bad argument");
     if (N == 0) return HAPMI_OK;
     HAPMI_REQUIRE(out && (x || M == 0), HAPMI_EINVAL, "colsum: null pointer");
-    if (!accumulate) {
-        // out may be 4-byte aligned only (a view into a flat gradient buffer)
-        HAPMI_REQUIRE(((uintptr_t)out % 4) == 0, HAPMI_EALIGN, "colsum: out must be 4-byte aligned");
-        hipLaunchKernelGGL(zero_f32_kernel, dim3(ew_grid(N)), dim3(EW_THREADS), 0, (hipStream_t)stream, out, N);
-    }
-    if (M == 0) return HAPMI_OK;
-    const int64_t epv = dtype == HAPMI_F32 ? 4 : 8;
-    if (aligned16(x) && ldx % epv == 0 && N % epv == 0) {
-        dim3 vgrid((unsigned)hapmi_cdiv(N, 32 * epv), (unsigned)hapmi_cdiv(M, CSV_ROWS_PER_BLOCK));
-        if (dtype == HAPMI_F32) hipLaunchKernelGGL((colsum_vec_kernel<float>), vgrid, dim3(256), 0, (hipStream_t)stream, (const float *)x, out, M, N, ldx);
-        else hipLaunchKernelGGL((colsum_vec_kernel<bf16_t>), vgrid, dim3(256), 0, (hipStream_t)stream, (const bf16_t *)x, out, M, N, ldx);
-        HAPMI_CHECK_LAUNCH("colsum");
+    // out may be 4-byte aligned only (a view into a flat gradient buffer)
+    HAPMI_REQUIRE(((uintptr_t)out % 4) == 0 && ((uintptr_t)workspace % 4) == 0, HAPMI_EALIGN, "colsum: out / workspace must be 4-byte aligned");
+    if (M == 0) {
+        if (!accumulate) hipLaunchKernelGGL(zero_f32_kernel, dim3(ew_grid(N)), dim3(EW_THREADS), 0, (hipStream_t)stream, out, N);
         return HAPMI_OK;
     }
-    dim3 grid((unsigned)hapmi_cdiv(N, 64), (unsigned)hapmi_cdiv(M, CS_ROWS_PER_BLOCK));
-    if (dtype == HAPMI_F32) hipLaunchKernelGGL((colsum_kernel<float>), grid, dim3(256), 0, (hipStream_t)stream, (const float *)x, out, M, N, ldx);
-    else hipLaunchKernelGGL((colsum_kernel<bf16_t>), grid, dim3(256), 0, (hipStream_t)stream, (const bf16_t *)x, out, M, N, ldx);
+    // slabs of at least 128 rows, as many as the workspace holds ([slab][N]); one slab writes the result itself
+    int64_t n_slabs = hapmi_cdiv(M, 128);
+    if (!workspace || n_slabs * N > workspace_elems) n_slabs = workspace ? workspace_elems / N : 1;
+    if (n_slabs < 2) n_slabs = 1;
+    if (n_slabs > 65535) n_slabs = 65535;
+    const int64_t rows_per_slab = hapmi_cdiv(M, n_slabs);
+    n_slabs = hapmi_cdiv(M, rows_per_slab);
+    float *dst = n_slabs > 1 ? workspace : out;
+    const int add = n_slabs > 1 ? 0 : accumulate;
+    const int64_t epv = dtype == HAPMI_F32 ? 4 : 8;
+    if (aligned16(x) && ldx % epv == 0 && N % epv == 0) {
+        dim3 vgrid((unsigned)hapmi_cdiv(N, 32 * epv), (unsigned)n_slabs);
+        if (dtype == HAPMI_F32) hipLaunchKernelGGL((colsum_vec_kernel<float>), vgrid, dim3(256), 0, (hipStream_t)stream, (const float *)x, dst, M, N, ldx, rows_per_slab, add);
+        else hipLaunchKernelGGL((colsum_vec_kernel<bf16_t>), vgrid, dim3(256), 0, (hipStream_t)stream, (const bf16_t *)x, dst, M, N, ldx, rows_per_slab, add);
+    } else {
+        dim3 grid((unsigned)hapmi_cdiv(N, 64), (unsigned)n_slabs);
+        if (dtype == HAPMI_F32) hipLaunchKernelGGL((colsum_kernel<float>), grid, dim3(256), 0, (hipStream_t)stream, (const float *)x, dst, M, N, ldx, rows_per_slab, add);
+        else hipLaunchKernelGGL((colsum_kernel<bf16_t>), grid, dim3(256), 0, (hipStream_t)stream, (const bf16_t *)x, dst, M, N, ldx, rows_per_slab, add);
+    }
+    if (n_slabs > 1)
+        hipLaunchKernelGGL(colsum_final_kernel, dim3((unsigned)hapmi_cdiv(N, 256)), dim3(256), 0, (hipStream_t)stream,
+                           (const float *)workspace, out, N, n_slabs, accumulate);
     HAPMI_CHECK_LAUNCH("colsum");
     return HAPMI_OK;
 }
@@ -296,6 +323,11 @@ __global__ __launch_bounds__(256) void embedding_fwd_kernel(const int64_t *ids, 
     }
 }
 
+// dtable[id, :] += sum over the tokens t with ids[t] == id of dout[t, :] * scale, added in token order.  One wave per
+// token; the wave of the FIRST token of an id (no earlier token has the same id) gathers all of that id's rows in
+// registers and adds the sum to the table row, the other waves leave.  No atomics and one writer per table row, so
+// the same call gives the same bits every time.  Rows up to 64 * EB_COLS wide.
+constexpr int EB_COLS = 32;
 template <typename T>
 __global__ __launch_bounds__(256) void embedding_bwd_kernel(const int64_t *ids, const T *dout, float *dtable,
                                                           int64_t n_tokens, int64_t d, int64_t vocab, float scale) {
@@ -304,10 +336,37 @@ __global__ __launch_bounds__(256) void embedding_bwd_kernel(const int64_t *ids, 
     if (t >= n_tokens) return;
     const int64_t id = ids[t];
     if (id < 0 || id >= vocab) return;
-    for (int64_t c = lane; c < d; c += 64) {
-        float g = ld_f(dout + t * d, c) * scale;
-        if (sizeof(T) == 2) g = (float)(bf16_t)g;
-        atomicAdd(dtable + id * d + c, g);
+    // is an earlier token of the same id?  (wave-uniform)
+    for (int64_t u0 = 0; u0 < t; u0 += 64) {
+        const int64_t u = u0 + lane;
+        const bool hit = u < t && ids[u] == id;
+        if (__ballot(hit) != 0ull) return;
+    }
+    float acc[EB_COLS];
+#pragma unroll
+    for (int j = 0; j < EB_COLS; ++j) acc[j] = 0.f;
+    for (int64_t u0 = t / 64 * 64; u0 < n_tokens; u0 += 64) {
+        const int64_t u = u0 + lane;
+        unsigned long long hits = __ballot(u >= t && u < n_tokens && ids[u] == id);
+        while (hits) {                                            // ascending token order
+            const int b = __ffsll((long long)hits) - 1;
+            hits &= hits - 1;
+            const T *row = dout + (u0 + b) * d;
+#pragma unroll
+            for (int j = 0; j < EB_COLS; ++j) {
+                const int64_t c = (int64_t)j * 64 + lane;
+                if ((int64_t)j * 64 < d && c < d) {
+                    float g = ld_f(row, c) * scale;
+                    if (sizeof(T) == 2) g = (float)(bf16_t)g;
+                    acc[j] += g;
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < EB_COLS; ++j) {
+        const int64_t c = (int64_t)j * 64 + lane;
+        if ((int64_t)j * 64 < d && c < d) dtable[id * d + c] += acc[j];
     }
 }
 
@@ -331,6 +390,7 @@ extern "C" int hapmi_embedding_fwd(const int64_t *ids, const void *table, const 
 extern "C" int hapmi_embedding_bwd(const int64_t *ids, const void *dout, float *dtable, int64_t n_tokens, int64_t d,
                                    int64_t vocab, float scale, int dtype, hapmi_stream_t stream) {
     HAPMI_REQUIRE(hapmi_dtype_ok(dtype) && n_tokens >= 0 && d >= 1 && vocab >= 1, HAPMI_EINVAL, "embedding_bwd: bad argument");
+    HAPMI_REQUIRE(d <= 64 * EB_COLS, HAPMI_ELIMIT, "embedding_bwd: rows of at most %d elements", 64 * EB_COLS);
     if (n_tokens == 0) return HAPMI_OK;
     HAPMI_REQUIRE(ids && dout && dtable, HAPMI_EINVAL, "embedding_bwd: null pointer");
     dim3 grid((unsigned)hapmi_cdiv(n_tokens, 4));
@@ -490,13 +550,26 @@ __global__ __launch_bounds__(EW_THREADS) void adam_kernel(float *p, const float 
     }
 }
 
-__global__ __launch_bounds__(EW_THREADS) void sumsq_kernel(const float *g, int64_t n, float *out) {
+// Sum of squares in two deterministic stages: the input is cut into chunks of SUMSQ_CHUNK elements (a partition
+// that does not depend on the grid), partials[c] is chunk c's sum in a fixed order, and one block adds the
+// partials in a fixed order.  No atomics: the same call gives the same bits every time.
+constexpr int64_t SUMSQ_CHUNK = 16384;
+__global__ __launch_bounds__(EW_THREADS) void sumsq_partial_kernel(const float *g, int64_t n, float *partials, int64_t n_chunks) {
+    __shared__ float red[16];
+    for (int64_t c = blockIdx.x; c < n_chunks; c += gridDim.x) {
+        const int64_t i0 = c * SUMSQ_CHUNK, i1 = i0 + SUMSQ_CHUNK < n ? i0 + SUMSQ_CHUNK : n;
+        float s = 0.f;
+        for (int64_t i = i0 + threadIdx.x; i < i1; i += EW_THREADS) s += g[i] * g[i];
+        s = block_sum(s, red);
+        if (threadIdx.x == 0) partials[c] = s;
+    }
+}
+__global__ __launch_bounds__(EW_THREADS) void sumsq_final_kernel(const float *partials, int64_t n_chunks, float *out) {
     __shared__ float red[16];
     float s = 0.f;
-    const int64_t step = (int64_t)gridDim.x * EW_THREADS;
-    for (int64_t i = (int64_t)blockIdx.x * EW_THREADS + threadIdx.x; i < n; i += step) s += g[i] * g[i];
+    for (int64_t i = threadIdx.x; i < n_chunks; i += EW_THREADS) s += partials[i];
     s = block_sum(s, red);
-    if (threadIdx.x == 0) atomicAdd(out, s);
+    if (threadIdx.x == 0) out[0] = s;
 }
 
 __global__ void clip_coef_kernel(const float *sumsq, float max_norm, float *coef) {
@@ -572,15 +645,35 @@ extern "C" int hapmi_adam_apply_dev(float *param, const float *grad, float *exp_
     return HAPMI_OK;
 }
 
-extern "C" int hapmi_sumsq(const float *g, int64_t n, float *out, hapmi_stream_t stream) {
-    HAPMI_REQUIRE(n >= 0 && out, HAPMI_EINVAL, "sumsq: bad argument");
-    if (n == 0) return HAPMI_OK;
-    HAPMI_REQUIRE(g, HAPMI_EINVAL, "sumsq: null pointer");
-    int64_t gx = hapmi_cdiv(n, EW_THREADS * 8);
-    if (gx > 1024) gx = 1024;
-    hipLaunchKernelGGL(sumsq_kernel, dim3((unsigned)gx), dim3(EW_THREADS), 0, (hipStream_t)stream, g, n, out);
+namespace {
+int sumsq_launch(const float *g, int64_t n, float *out, float *partials, hipStream_t st) {
+    const int64_t n_chunks = hapmi_cdiv(n, SUMSQ_CHUNK);
+    int64_t gx = n_chunks < 2048 ? n_chunks : 2048;
+    hipLaunchKernelGGL(sumsq_partial_kernel, dim3((unsigned)gx), dim3(EW_THREADS), 0, st, g, n, partials, n_chunks);
+    hipLaunchKernelGGL(sumsq_final_kernel, dim3(1), dim3(EW_THREADS), 0, st, (const float *)partials, n_chunks, out);
     HAPMI_CHECK_LAUNCH("sumsq");
     return HAPMI_OK;
+}
+}  // namespace
+
+extern "C" int hapmi_sumsq_workspace_elems(int64_t n, int64_t *elems_host) {
+    HAPMI_REQUIRE(n >= 0 && elems_host, HAPMI_EINVAL, "sumsq_workspace_elems: bad argument");
+    *elems_host = hapmi_cdiv(n, SUMSQ_CHUNK);
+    return HAPMI_OK;
+}
+
+extern "C" int hapmi_sumsq(const float *g, int64_t n, float *out, float *workspace, int64_t workspace_elems,
+                           hapmi_stream_t stream) {
+    HAPMI_REQUIRE(n >= 0 && out, HAPMI_EINVAL, "sumsq: bad argument");
+    if (n == 0) {
+        hipLaunchKernelGGL(zero_f32_kernel, dim3(1), dim3(EW_THREADS), 0, (hipStream_t)stream, out, (int64_t)1);
+        return HAPMI_OK;
+    }
+    HAPMI_REQUIRE(g && workspace, HAPMI_EINVAL, "sumsq: null pointer");
+    HAPMI_REQUIRE(workspace_elems >= hapmi_cdiv(n, SUMSQ_CHUNK), HAPMI_ELIMIT,
+                  "sumsq: %lld elements need a workspace of %lld floats, %lld given", (long long)n,
+                  (long long)hapmi_cdiv(n, SUMSQ_CHUNK), (long long)workspace_elems);
+    return sumsq_launch(g, n, out, workspace, (hipStream_t)stream);
 }
 
 extern "C" int hapmi_clip_coef(const float *sumsq, float max_norm, float *coef, hapmi_stream_t stream) {

@@ -183,6 +183,22 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *ws, TO 
     }
 }
 
+// The second half of a_rowsum: out[z][m] += the partial row sums of problem z, row m, added in the order (split, tile
+// column).  One thread per row and problem; the order fixes the float32 result.
+struct RowsumOuts {
+    float *out[HAPMI_GEMM_MAX_LIST];
+};
+__global__ __launch_bounds__(256) void rowsum_reduce_kernel(const float *ws, RowsumOuts outs, int64_t M, int parts) {
+    const int z = blockIdx.y;
+    float *out = outs.out[z];
+    const int64_t m = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (!out || m >= M) return;
+    const float *src = ws + (int64_t)z * parts * M + m;
+    float s = 0.f;
+    for (int q = 0; q < parts; ++q) s += src[(int64_t)q * M];
+    out[m] += s;
+}
+
 template <typename TI, typename TO>
 int launch_typed(GemmParams &p, int transA, int transB, int64_t batch, hipStream_t st, bool wide, void *workspace,
                  int64_t workspace_bytes) {
@@ -190,7 +206,14 @@ int launch_typed(GemmParams &p, int transA, int transB, int64_t batch, hipStream
     const int64_t nk = hapmi_cdiv(p.K, bk);
     p.ws_ld = (p.N + 3) / 4 * 4;
     const int64_t per_split = p.M * p.ws_ld * 4;
-    const int64_t max_splits = (workspace && ((uintptr_t)workspace % 16) == 0 && per_split > 0) ? workspace_bytes / per_split : 0;
+    bool want_rs = p.rowsum != nullptr;
+    for (int z = 0; z < p.n_list; ++z) want_rs = want_rs || p.listRS[z] != nullptr;
+    // with row sums the workspace is shared: split-K partials in its first half, partial row sums in the second
+    const int64_t rs_off = want_rs ? (workspace_bytes / 2) / 16 * 16 : 0;
+    const int64_t split_bytes = want_rs ? rs_off : workspace_bytes;
+    if (want_rs && (!workspace || ((uintptr_t)workspace % 16) != 0))
+        return hapmi_set_error(HAPMI_EINVAL, "gemm: a_rowsum needs a 16-byte aligned workspace for its partial sums");
+    const int64_t max_splits = (workspace && ((uintptr_t)workspace % 16) == 0 && per_split > 0) ? split_bytes / per_split : 0;
     Choice ch = choose(p.M, p.N, p.K, batch, bk, sizeof(TI) == 2, wide, max_splits, !transA && transB);
     if (g_force_cfg < 0 && g_force_splits <= 0) {
         std::lock_guard<std::mutex> lk(g_plans_mu);
@@ -208,6 +231,16 @@ int launch_typed(GemmParams &p, int transA, int transB, int64_t batch, hipStream
     p.ktiles_per_split = (int)hapmi_cdiv(nk, p.splits);
     p.splits = (int)hapmi_cdiv(nk, p.ktiles_per_split);
     p.ws = (float *)workspace;
+    int rs_parts = 0;
+    p.rs_ws = nullptr;
+    if (want_rs) {
+        rs_parts = p.splits * (int)hapmi_cdiv(p.N, kCfg[c].bn);
+        const int64_t need = batch * rs_parts * p.M * 4;
+        if (need > workspace_bytes - rs_off)
+            return hapmi_set_error(HAPMI_ELIMIT, "gemm: a_rowsum needs %lld bytes in the second half of the workspace, %lld given",
+                                   (long long)need, (long long)(workspace_bytes - rs_off));
+        p.rs_ws = (float *)((char *)workspace + rs_off);
+    }
     const int in_dtype = sizeof(TI) == 2 ? HAPMI_BF16 : HAPMI_F32, out_dtype = sizeof(TO) == 2 ? HAPMI_BF16 : HAPMI_F32;
     int rc;
     switch (c) {
@@ -224,7 +257,14 @@ int launch_typed(GemmParams &p, int transA, int transB, int64_t batch, hipStream
         case 11: rc = hapmi_gemm_launch_cfg11(p, in_dtype, out_dtype, transA, transB, batch, st); break;
         default: rc = hapmi_gemm_launch_cfg0(p, in_dtype, out_dtype, transA, transB, batch, st);
     }
-    if (rc || p.splits <= 1) return rc;
+    if (rc) return rc;
+    if (want_rs) {
+        RowsumOuts outs;
+        for (int z = 0; z < HAPMI_GEMM_MAX_LIST; ++z) outs.out[z] = p.n_list > 0 ? p.listRS[z] : (z == 0 ? p.rowsum : nullptr);
+        hipLaunchKernelGGL(rowsum_reduce_kernel, dim3((unsigned)hapmi_cdiv(p.M, 256), (unsigned)batch), dim3(256), 0, st,
+                           (const float *)p.rs_ws, outs, p.M, rs_parts);
+    }
+    if (p.splits <= 1) return HAPMI_OK;
     int64_t gx = hapmi_cdiv(p.M * (p.ws_ld / 4), 256);
     if (gx > 256 * 16) gx = 256 * 16;
     hipLaunchKernelGGL((splitk_reduce_kernel<TO>), dim3((unsigned)gx), dim3(256), 0, st, (const float *)p.ws, (TO *)p.C,

@@ -33,7 +33,9 @@ struct GemmParams {
     int tiles_m, tiles_n;
     int splits, ktiles_per_split;
     float *ws;                 // split-K workspace [splits][M][ws_ld] (float32)
-    float *rowsum;             // optional: rowsum[m] += sum_k op(A)[m, k] (float32 atomics; A stored [K, M] only)
+    float *rowsum;             // optional: rowsum[m] += sum_k op(A)[m, k] (A stored [K, M] only); the blocks write
+                               // partial sums to rs_ws, a second kernel adds them up in a fixed order
+    float *rs_ws;              // [problem][split][tiles_n][M] partial row sums (float32)
     const void *relu_mask;     // optional: [M][ldc] in C's element type; result elements whose mask is <= 0 become 0
     int64_t ws_ld;
     const void *addend;        // optional (accumulate): the old values are read here instead of from C
@@ -285,15 +287,19 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, ((WAVES_M * WAVES_N <= 4 && 
     }
 
     if (do_rs) {
-        // reduce the per-thread sums over the threads that share a row-vector (LDS float atomics), then one
-        // global atomic per row; the operand LDS is idle here (the main loop ended with a barrier)
-        float *red = (float *)smem;
-        for (int t = threadIdx.x; t < BM; t += THREADS) red[t] = 0.f;
-        __syncthreads();
+        // Every thread's sums go to a slot of their own in the (idle) operand LDS, [group][row] with one group per
+        // set of threads that covers all rows once; one thread per row then adds the groups in order and writes the
+        // block's partial sum to its slot of the workspace, [problem][split][tile column][M].  No atomics anywhere:
+        // the second kernel (rowsum_reduce_kernel) adds the slots of a row in a fixed order, so the result does not
+        // depend on the order in which blocks run.
+        float *part = (float *)smem;
+        constexpr int RS_GROUPS = A_TR ? TrA::KP : BK / 4;
+        static_assert(RS_GROUPS * BM * 4 <= NSTAGES * (A_BYTES + B_BYTES), "row-sum staging does not fit the operand LDS");
         if constexpr (A_TR) {
             if ((int)threadIdx.x < TrA::KP * TrA::CPR) {
+                float *dst = part + ((int)threadIdx.x / TrA::CPR) * BM + ((int)threadIdx.x % TrA::CPR) * 8;
 #pragma unroll
-                for (int e = 0; e < 8; ++e) atomicAdd(red + ((int)threadIdx.x % TrA::CPR) * 8 + e, rs[e]);
+                for (int e = 0; e < 8; ++e) dst[e] = rs[e];
             }
         } else if constexpr (!A_KMAJOR) {
             constexpr int RV_ = decltype(la)::RV, BLOCKS_ = decltype(la)::BLOCKS;
@@ -301,15 +307,21 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, ((WAVES_M * WAVES_N <= 4 && 
             for (int pp = 0; pp < decltype(la)::PASSES_T; ++pp) {
                 const int blk = threadIdx.x + pp * THREADS;
                 if (blk < BLOCKS_) {
-                    const int rv = blk % RV_;
+                    float *dst = part + (blk / RV_) * BM + (blk % RV_) * EPV;
 #pragma unroll
-                    for (int e = 0; e < EPV; ++e) atomicAdd(red + rv * EPV + e, rs[pp * EPV + e]);
+                    for (int e = 0; e < EPV; ++e) dst[e] = rs[pp * EPV + e];
                 }
             }
         }
         __syncthreads();
+        float *slot = p.rs_ws + (((int64_t)blockIdx.z * gridDim.y + blockIdx.y) * p.tiles_n + tn) * p.M + m0;
         for (int t = threadIdx.x; t < BM; t += THREADS)
-            if (t < m_left) atomicAdd(rowsum + m0 + t, red[t]);
+            if (t < m_left) {
+                float s = 0.f;
+#pragma unroll
+                for (int g = 0; g < RS_GROUPS; ++g) s += part[g * BM + t];
+                slot[t] = s;
+            }
         __syncthreads();
     }
 

@@ -1494,6 +1494,8 @@ class ShardExecutor:
             self._adam_state = torch.zeros(4, dtype=torch.float32, device=self.dev)   # step, 1-b1^t, 1-b2^t
         if clip_grad_norm is not None:
             self._sumsq = torch.zeros(1, dtype=torch.float32, device=self.dev)
+            self._sumsq_ws = torch.empty(max(1, ops.sumsq_workspace_elems(self.flat_grad.numel())), dtype=torch.float32,
+                                         device=self.dev)
             self._coef = torch.ones(1, dtype=torch.float32, device=self.dev)
         self._step_count = 0
         self._lists = {k: v for k, v in self._lists.items() if k[0] != "bwd_step"}
@@ -1532,8 +1534,7 @@ class ShardExecutor:
         o = self._opt
         coef = None
         if o["clip"] is not None:
-            ops.fill_zero(self._sumsq)
-            ops.sumsq(self.flat_grad, self._sumsq)
+            ops.sumsq(self.flat_grad, self._sumsq, self._sumsq_ws)
             ops.clip_coef(self._sumsq, o["clip"], self._coef)
             coef = self._coef
         if o["kind"] == "sgd":

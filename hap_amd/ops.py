@@ -295,9 +295,18 @@ _gemm_ws: Optional[torch.Tensor] = None
 
 
 def set_gemm_workspace(t: Optional[torch.Tensor]) -> None:
-    """Scratch buffer for split-K partial sums, shared by all GEMM calls that follow (one stream)."""
+    """Scratch buffer for split-K partial sums and the partial sums of the deterministic reductions (bias
+    gradients, column sums), shared by all calls that follow (one stream)."""
     global _gemm_ws
     _gemm_ws = t
+
+
+def _workspace(device) -> torch.Tensor:
+    """The installed workspace, or a 64 MiB one made on first use (calls outside an executor, e.g. tests)."""
+    global _gemm_ws
+    if _gemm_ws is None or _gemm_ws.device != device:
+        _gemm_ws = torch.empty(16 << 20, dtype=torch.float32, device=device)
+    return _gemm_ws
 
 
 def gemm(A: torch.Tensor, B: torch.Tensor, C: torch.Tensor, M: int, N: int, K: int, *, transA=False, transB=False,
@@ -333,6 +342,8 @@ def gemm(A: torch.Tensor, B: torch.Tensor, C: torch.Tensor, M: int, N: int, K: i
     a.strideB1, a.strideB2 = strideB
     a.strideC1, a.strideC2 = strideC
     ws = workspace if workspace is not None else _gemm_ws
+    if ws is None and a_rowsum is not None:
+        ws = _workspace(A.device)                      # the row sums' partial sums need one
     if ws is not None and ws.is_cuda and ws.device == A.device:
         a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel() * ws.element_size()
     else:
@@ -404,6 +415,9 @@ def gemm_group(As: Sequence[torch.Tensor], Bs: Sequence[torch.Tensor], Cs: Seque
     a.A_list, a.B_list, a.C_list = ctypes.addressof(la), ctypes.addressof(lb), ctypes.addressof(lc)
     a.a_rowsum_list = ctypes.addressof(lr) if lr is not None else 0
     a._keep = (la, lb, lc, lr)                       # the argument block points into these host arrays
+    if lr is not None:
+        ws = _workspace(As[0].device)                  # partial row sums
+        a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel() * ws.element_size()
     if _gemm_log is not None:
         _gemm_log.append((a, (tuple(As), tuple(Bs), tuple(Cs), tuple(a_rowsums or ()))))
     check(lib().hapmi_gemm(ctypes.byref(a), _stream()))
@@ -696,8 +710,9 @@ def colsum(x, out, M, N, ldx=None, accumulate=False):
     _need(out, N, "colsum out")
     if out.dtype != torch.float32:
         raise TypeError("colsum: float32 output expected")
+    ws = _workspace(x.device)
     check(lib().hapmi_colsum(_ptr(x), _ptr(out), M, N, ldx if ldx is not None else N, int(accumulate),
-                             dtype_code(x), _stream()))
+                             dtype_code(x), _ptr(ws), ws.numel(), _stream()))
 
 
 def fill_zero(t):
@@ -819,9 +834,19 @@ def adam_apply_dev(param, grad, exp_avg, exp_avg_sq, shadow, lr, beta1, beta2, e
                                      _ptr(state), _ptr(grad_scale), _stream()))
 
 
-def sumsq(g, out):
-    _dev(g, out)
-    check(lib().hapmi_sumsq(_ptr(g), g.numel(), _ptr(out), _stream()))
+def sumsq_workspace_elems(n: int) -> int:
+    need = ctypes.c_int64()
+    check(lib().hapmi_sumsq_workspace_elems(n, ctypes.byref(need)))
+    return need.value
+
+
+def sumsq(g, out, workspace=None):
+    """out[0] = sum of g^2 (deterministic; ``workspace``: float32 scratch of ``sumsq_workspace_elems(n)``)."""
+    ws = workspace if workspace is not None else _workspace(g.device)
+    _dev(g, out, ws)
+    if ws.dtype != torch.float32 or g.dtype != torch.float32 or out.dtype != torch.float32:
+        raise TypeError("sumsq: float32 tensors expected")
+    check(lib().hapmi_sumsq(_ptr(g), g.numel(), _ptr(out), _ptr(ws), ws.numel(), _stream()))
 
 
 def clip_coef(sumsq_t, max_norm, coef):

@@ -147,12 +147,16 @@ typedef struct {
     float alpha;                 /* result scaled before bias */
     int64_t batch1, batch2;      /* >= 1 */
     int64_t strideA1, strideA2, strideB1, strideB2, strideC1, strideC2;
-    void *workspace;             /* optional float32 scratch for split-K (16-byte aligned) or NULL;   */
-    int64_t workspace_bytes;     /* a split needs M * roundup(N, 4) * 4 bytes; unused when batch > 1 */
-    float *a_rowsum;             /* optional: a_rowsum[m] += sum over k of op(A)[m, k] (float32 atomics, so the
-                                  * caller clears it): the bias gradient of F.linear when the call is the weight
-                                  * gradient dW = dY^T X, i.e. the column sum that autograd takes of dY
-                                  * (hap.rs:1032 F.linear with bias).  Needs transA = 1 and batch 1; NULL = off */
+    void *workspace;             /* optional float32 scratch (16-byte aligned) or NULL: partial sums of a split    */
+    int64_t workspace_bytes;     /* reduction (M * roundup(N, 4) * 4 bytes per split; no split when batch > 1), and,
+                                  * with a_rowsum / a_rowsum_list, partial row sums in its second half (at most
+                                  * batch * 32 * ceil(N / 64) * M * 4 bytes; HAPMI_ELIMIT if they do not fit)        */
+    float *a_rowsum;             /* optional: a_rowsum[m] += sum over k of op(A)[m, k]: the bias gradient of F.linear
+                                  * when the call is the weight gradient dW = dY^T X, i.e. the column sum that
+                                  * autograd takes of dY (hap.rs:1032 F.linear with bias).  The blocks write partial
+                                  * sums to the workspace and a second kernel adds them in a fixed order (no atomics:
+                                  * the same call gives the same bits every time).  Needs transA = 1, batch 1 and a
+                                  * workspace; NULL = off */
     const void *c_relu_mask;     /* optional: [M][ldc] in out_dtype; elements of the result (before accumulation)
                                   * whose mask value is <= 0 are written as 0: the backward of F.relu
                                   * (hap.rs:1417) when the call is the data gradient of the next F.linear and
@@ -242,9 +246,11 @@ int hapmi_scale(const void *a, float s, void *out, int64_t n, int dtype, hapmi_s
 /* out[r, :] = a[r, :] + b[r % b_rows, :] (broadcast add of pe / pos_embed, hap.rs:3821-3837) */
 int hapmi_add_bcast_rows(const void *a, const void *b, void *out, int64_t rows, int64_t b_rows, int64_t width,
                          int dtype, hapmi_stream_t stream);
-/* column sums: out[N] (float32) (+)= sum_m x[m, :]; bias gradient of F.linear; also sums over samples */
+/* column sums: out[N] (float32) (+)= sum_m x[m, :]; bias gradient of F.linear; also sums over samples.
+ * Rows are summed in slabs whose partial sums go to `workspace` (float32, up to ceil(M / 128) * N elements are
+ * used; NULL or too small: fewer, longer slabs) and are added in slab order: no atomics, reproducible bits. */
 int hapmi_colsum(const void *x, float *out, int64_t M, int64_t N, int64_t ldx, int accumulate, int dtype,
-                 hapmi_stream_t stream);
+                 float *workspace, int64_t workspace_elems, hapmi_stream_t stream);
 int hapmi_fill_zero(void *p, int64_t bytes, hapmi_stream_t stream);
 int hapmi_cast(const void *src, int src_dtype, void *dst, int dst_dtype, int64_t n, hapmi_stream_t stream);
 
@@ -252,7 +258,8 @@ int hapmi_cast(const void *src, int src_dtype, void *dst, int dst_dtype, int64_t
  * out[t, :] = table[ids[t], :] * scale + pe[t % S, :]   (pe may be NULL) */
 int hapmi_embedding_fwd(const int64_t *ids, const void *table, const void *pe, void *out, int64_t n_tokens,
                         int64_t d, int64_t S, int64_t vocab, float scale, int dtype, hapmi_stream_t stream);
-/* dtable[ids[t], :] += dout[t, :] * scale   (float32 atomics; dtable zeroed by the caller) */
+/* dtable[ids[t], :] += dout[t, :] * scale, the tokens of one id added in token order by one wave (no atomics,
+ * reproducible bits); dtable zeroed by the caller; d <= 2048 */
 int hapmi_embedding_bwd(const int64_t *ids, const void *dout, float *dtable, int64_t n_tokens, int64_t d,
                         int64_t vocab, float scale, int dtype, hapmi_stream_t stream);
 
@@ -329,8 +336,12 @@ int hapmi_adam_advance(float *state_dev, float beta1, float beta2, hapmi_stream_
 int hapmi_adam_apply_dev(float *param, const float *grad, float *exp_avg, float *exp_avg_sq, void *shadow, int64_t n,
                          float lr, float beta1, float beta2, float eps, const float *state_dev,
                          const float *grad_scale_dev, hapmi_stream_t stream);
-/* out[0] += sum g^2 (float32 atomics over block partials; out zeroed by the caller) */
-int hapmi_sumsq(const float *g, int64_t n, float *out, hapmi_stream_t stream);
+/* out[0] = sum g^2, the square of the norm that torch.nn.utils.clip_grad_norm_ takes (worker.py:74), in two
+ * stages through `workspace` (the number of floats that hapmi_sumsq_workspace_elems reports for n: one partial sum per 16384 elements, added in
+ * order by one block): no atomics, reproducible bits */
+int hapmi_sumsq_workspace_elems(int64_t n, int64_t *elems_host);
+int hapmi_sumsq(const float *g, int64_t n, float *out, float *workspace, int64_t workspace_elems,
+                hapmi_stream_t stream);
 /* torch.nn.utils.clip_grad_norm_ coefficient (worker.py:74): coef = min(1, max_norm / (sqrt(sumsq) + 1e-6)) */
 int hapmi_clip_coef(const float *sumsq, float max_norm, float *coef, hapmi_stream_t stream);
 

@@ -239,7 +239,7 @@ def test_optimizers_match_torch(cuda):
     ops.adam_step(p1, grads[0].to(cuda), m1, v1, None, 5e-4, 0.9, 0.999, 1e-8, 1)
     torch.testing.assert_close(p1.cpu(), -5e-4 * torch.sign(grads[0]), rtol=1e-4, atol=1e-9)
     # gradient clipping coefficient (clip_grad_norm_)
-    ss, coef = torch.zeros(1, device=cuda), torch.zeros(1, device=cuda)
+    ss, coef = torch.full((1,), 7.0, device=cuda), torch.zeros(1, device=cuda)     # the old content is overwritten
     ops.sumsq(grads[0].to(cuda), ss)
     ops.clip_coef(ss, 0.5, coef)
     want = min(1.0, 0.5 / (grads[0].norm().item() + 1e-6))
@@ -550,3 +550,70 @@ def test_gemm_plans_round_trip_through_a_file(cuda, tmp_path):
         close(C, A0.double() @ B0.double().t(), torch.bfloat16)
     finally:
         ops.clear_gemm_plans()
+
+
+def test_reductions_give_the_same_bits_every_time(cuda):
+    """The reductions that many blocks share add in a fixed order (no float atomics): the embedding gradient, column
+    sums over several slabs of rows, the gradient norm, and the bias gradient that a weight-gradient GEMM takes
+    along (also with the reduction split over K and for several problems in one launch)."""
+    g = torch.Generator().manual_seed(21)
+    # embedding gradient with heavy collisions: equal to the token-ordered float32 sum, bit for bit
+    V, d, n = 50, 200, 1500
+    ids = torch.randint(0, 7, (n,), generator=g) * 7
+    dout = torch.randn(n, d, generator=g)
+    want = torch.zeros(V, d)
+    for t in range(n):
+        want[ids[t]] += dout[t]
+    runs = []
+    for _ in range(3):
+        dt = torch.zeros(V, d, device=cuda)
+        ops.embedding_bwd(ids.to(cuda), dout.to(cuda), dt, 1.0)
+        runs.append(dt.cpu())
+    assert torch.equal(runs[0], want)
+    assert torch.equal(runs[0], runs[1]) and torch.equal(runs[0], runs[2])
+    # column sums over 3000 rows (24 slabs) and the sum of squares of 1.3 M elements
+    x = torch.randn(3000, 264, generator=g).to(cuda)
+    big = torch.randn(1_300_003, generator=g).to(cuda)
+    outs = []
+    for _ in range(3):
+        cs = torch.empty(264, device=cuda)
+        ops.colsum(x, cs, 3000, 264)
+        ss = torch.empty(1, device=cuda)
+        ops.sumsq(big, ss)
+        outs.append((cs.cpu(), ss.cpu()))
+    torch.testing.assert_close(outs[0][0].double(), x.cpu().double().sum(0), rtol=1e-5, atol=1e-4)
+    torch.testing.assert_close(outs[0][1].double(), big.cpu().double().pow(2).sum().reshape(1), rtol=1e-6, atol=0)
+    for o in outs[1:]:
+        assert torch.equal(o[0], outs[0][0]) and torch.equal(o[1], outs[0][1])
+    # bias gradient as row sums of dY in dW = dY^T X: one problem (with and without a K split), then a group
+    for dtype in (torch.bfloat16, torch.float32):
+        rows, n_out, n_in = 4096, 320, 256
+        dy = torch.randn(rows, n_out, generator=g).to(dtype).to(cuda)
+        xx = torch.randn(rows, n_in, generator=g).to(dtype).to(cuda)
+        ref = dy.double().sum(0).cpu()
+        for splits in (0, 4):
+            ops.lib().hapmi_gemm_tuning(-1, splits)
+            try:
+                got = []
+                for _ in range(3):
+                    gw = torch.empty(n_out, n_in, device=cuda)
+                    gb = torch.zeros(n_out, device=cuda)
+                    ops.gemm(dy, xx, gw, n_out, n_in, rows, transA=True, a_rowsum=gb)
+                    got.append((gw.cpu(), gb.cpu()))
+            finally:
+                ops.lib().hapmi_gemm_tuning(-1, 0)
+            torch.testing.assert_close(got[0][1].double(), ref, rtol=1e-5, atol=1e-3)
+            for o in got[1:]:
+                assert torch.equal(o[0], got[0][0]) and torch.equal(o[1], got[0][1])
+        dys = [torch.randn(rows, n_out, generator=g).to(dtype).to(cuda) for _ in range(3)]
+        xs = [torch.randn(rows, n_in, generator=g).to(dtype).to(cuda) for _ in range(3)]
+        got = []
+        for _ in range(2):
+            gws = [torch.empty(n_out, n_in, device=cuda) for _ in range(3)]
+            gbs = [torch.zeros(n_out, device=cuda), None, torch.ones(n_out, device=cuda)]
+            ops.gemm_group(dys, xs, gws, n_out, n_in, rows, transA=True, a_rowsums=gbs)
+            got.append([t.cpu() for t in gws] + [gbs[0].cpu(), gbs[2].cpu()])
+        torch.testing.assert_close(got[0][3].double(), dys[0].double().sum(0).cpu(), rtol=1e-5, atol=1e-3)
+        torch.testing.assert_close(got[0][4].double(), 1 + dys[2].double().sum(0).cpu(), rtol=1e-5, atol=1e-3)
+        for u, v in zip(got[0], got[1]):
+            assert torch.equal(u, v)
