@@ -123,6 +123,10 @@ class ShardExecutor:
         # They are held back until the group is full (or backward ends); their operands are per-layer buffers
         # that nothing overwrites before (see _grad_slot / _guard_write).  1 = every weight gradient at once.
         self.wgrad_group = 1 if (overlap_wgrad or self.overlap_optimizer) else max(1, min(int(wgrad_group), ops._lib.GEMM_MAX_LIST))
+        self._send_hooks = 0                               # callables the wire asked to run after every message is complete
+        self._grad_sharers: Dict[int, list] = {}           # gradient storage -> values whose gradient aliases it
+        self._emit_pos = -1                                # index of the backward emitter that is running
+        self.shared_gradient_copies = 0                    # times a contribution went to a new buffer because of sharing
         self._wire_backed: set = set()                     # storages that peers' messages are received into in place
         self._pending_wgrads: Dict[tuple, list] = {}
         self._deferred_reads: Dict[int, int] = {}          # storage -> launches held back that read it
@@ -236,6 +240,13 @@ class ShardExecutor:
         if v.grad is None:
             v.grad = self._new(v.t.shape if v.t is not None else v.shape)
             return v.grad, False
+        if self._shared_with_pending(v):
+            # another value's gradient aliases this buffer and its producer has not read it yet: continue in a copy
+            old = v.grad
+            v.grad = self._new(old.shape, old.dtype)
+            new = v.grad
+            self.bwd.append(lambda: ops.scale(old, 1.0, new))
+            return v.grad, True
         self._guard_write(v.grad)
         return v.grad, True
 
@@ -243,7 +254,7 @@ class ShardExecutor:
         """``_grad_slot`` for a GEMM: (buffer, accumulate, addend).  When the gradient exists but weight-gradient
         launches that are held back still read its buffer, the sum goes to a new buffer (C = addend + A B) and
         the old one stays as it is."""
-        if v.grad is not None and self._is_read_later(v.grad):
+        if v.grad is not None and (self._is_read_later(v.grad) or self._shared_with_pending(v)):
             old = v.grad
             v.grad = self._new(old.shape, old.dtype)
             return v.grad, True, old
@@ -428,7 +439,10 @@ class ShardExecutor:
                 h = handlers.get(node.target)
                 if h is None:
                     self._unsupported(node, "this op has no handler")
-                self.env[node] = h(node)
+                val = self.env[node] = h(node)
+                # which backward emitter belongs to the producer of this value (see _shared_with_pending)
+                if isinstance(val, Val) and "tape_idx" not in val.meta:
+                    val.meta["tape_idx"] = len(self._tape) - 1
             elif node.op == "output":
                 out = self._val(node.args[0])
                 if out.kind != "loss":
@@ -437,9 +451,10 @@ class ShardExecutor:
         # backward list: the tape in reverse.  For every parameter remember how many backward launches must have
         # been enqueued before nothing reads its value or writes its gradient any more (all of them are made by
         # the emit of a node that consumes the parameter)
-        for emit in reversed(self._tape):
+        for idx in range(len(self._tape) - 1, -1, -1):
             self._touched = []
-            emit()
+            self._emit_pos = idx
+            self._tape[idx]()
             for name in self._touched:
                 self._grad_final_idx[name] = len(self.bwd)
         self._flush_wgrads()
@@ -575,21 +590,36 @@ class ShardExecutor:
         return out
 
     def _accumulate_into(self, v: Val, src: torch.Tensor):
-        """d(v) += src; when d(v) does not exist yet it ALIASES src.  Safe because every reader of an
-        aliased gradient (the backward of its single producer) is enqueued before any later accumulation
-        into the other owner: accumulating contributions come from consumers that precede that producer in
-        program order, hence follow it in backward order."""
+        """d(v) += src; when d(v) does not exist yet it ALIASES src (the residual add hands one buffer to both of
+        its operands).  A later contribution is added in place only if no other value still needs the buffer as
+        it is (_shared_with_pending, weight gradients held back); otherwise the sum goes to a new buffer."""
         if v.grad is None:
             v.grad = src
-        elif self._is_read_later(v.grad):
+            self._grad_sharers.setdefault(src.untyped_storage().data_ptr(), []).append(v)
+        elif self._is_read_later(v.grad) or self._shared_with_pending(v):
             g = v.grad
-            v.grad = self._new(g.shape, g.dtype)         # weight gradients held back still read g
+            v.grad = self._new(g.shape, g.dtype)         # weight gradients held back, or another value, still read g
             out = v.grad
             self.bwd.append(lambda: ops.add(g, src, out))
         else:
             g = v.grad
             self._guard_write(g)
             self.bwd.append(lambda: ops.add(g, src, g))
+
+    def _shared_with_pending(self, v: Val) -> bool:
+        """True when d(v)'s buffer is also the gradient of another value whose producer has not been through its
+        backward emitter yet: that emitter will read the buffer, so nothing may be added into it in place before.
+        (Emitters run in reverse program order; a value's producer is pending while its index is below the
+        running emitter's.  The generated programs never get here: between the residual add and the producer of
+        its second operand they have no other consumer of the first.)"""
+        if v.grad is None:
+            return False
+        for o in self._grad_sharers.get(v.grad.untyped_storage().data_ptr(), ()):
+            if o is not v and o.grad is not None and o.grad.untyped_storage().data_ptr() == v.grad.untyped_storage().data_ptr() \
+                    and 0 <= o.meta.get("tape_idx", -1) < self._emit_pos:
+                self.shared_gradient_copies += 1
+                return True
+        return False
 
     def _transpose(self, node):
         v, d0, d1 = self._val(node.args[0]), node.args[1], node.args[2]
@@ -689,8 +719,7 @@ class ShardExecutor:
                     src.grad = self._new(src.t.shape)
                     g = src.grad
                     self.bwd.append(lambda: ops.fill_zero(g))
-                g = src.grad
-                self._guard_write(g)
+                g, _ = self._grad_slot(src)
                 self.bwd.append(lambda: ops.gemm(dy, w.t, g, M, K, N, lda=ldc, ldc=lda, accumulate=True))
             elif x.needs_grad:
                 g, acc, addend = self._grad_slot_addend(x)
@@ -727,8 +756,8 @@ class ShardExecutor:
                 g = x.grad
                 self.bwd.append(lambda: ops.act_bwd(out.grad, ref, g, kind))
             else:
-                tmp, g = self._new(x.t.shape), x.grad
-                self._guard_write(g)
+                tmp = self._new(x.t.shape)
+                g, _ = self._grad_slot(x)
                 self.bwd.append(lambda: (ops.act_bwd(out.grad, ref, tmp, kind), ops.add(g, tmp, g)))
         self._tape.append(emit)
         return out
@@ -754,6 +783,13 @@ class ShardExecutor:
         if out.meta.get("relu_bwd_done"):
             return
         g = out.grad
+        if len(self._grad_sharers.get(g.untyped_storage().data_ptr(), ())) > 1 or self._is_read_later(g):
+            # the buffer is also another value's gradient (or a launch that is held back reads it): mask into a new one
+            self.shared_gradient_copies += 1
+            out.grad = self._new(g.shape, g.dtype)
+            masked = out.grad
+            self.bwd.append(lambda: ops.act_bwd(g, out.t, masked, "relu"))
+            return
         self._guard_write(g)
         self.bwd.append(lambda: ops.act_bwd(g, out.t, g, "relu"))
 
@@ -1022,8 +1058,8 @@ class ShardExecutor:
                     gx = x.grad
                     self.bwd.append(lambda: ops.slice_rows(g, 1, 1, T, gx))
                 else:
-                    tmp, gx = self._new(x.t.shape), x.grad
-                    self._guard_write(gx)
+                    tmp = self._new(x.t.shape)
+                    gx, _ = self._grad_slot(x)
                     self.bwd.append(lambda: (ops.slice_rows(g, 1, 1, T, tmp), ops.add(gx, tmp, gx)))
         self._tape.append(emit)
         return out
@@ -1048,7 +1084,9 @@ class ShardExecutor:
             if dst != rank:
                 hook = self.wire.send(tag, direction, dst, buffer_for(dst))
                 if hook is not None:
-                    sink.append(hook)
+                    # through host_call, so that the hook also sits in the recorded launch list that later steps replay
+                    self._send_hooks += 1
+                    sink.append(lambda hook=hook: ops._lib.host_call(hook))
 
     def _emit_gather(self, tag, direction, x_t, dim, L, rank, sink: List[Callable]):
         """pad own shard -> [wire] -> cut pads and concatenate.  Returns the full tensor."""
@@ -1117,7 +1155,7 @@ class ShardExecutor:
                 # d(x) += the reduced piece, in the reduction's own pass: in place, or into a new buffer while
                 # weight gradients that are held back still read the old one
                 g = x.grad
-                if self._is_read_later(g):
+                if self._is_read_later(g) or self._shared_with_pending(x):
                     x.grad = self._new(g.shape, g.dtype)
                 else:
                     self._guard_write(g)
@@ -1595,6 +1633,9 @@ class ShardExecutor:
         allocation, Adam's step count lives on the device), so replays equal eager steps."""
         if self._opt is None:
             raise RuntimeError("configure_optimizer() first")
+        if self._send_hooks:
+            raise RuntimeError("the wire asked to be called after every outgoing message (Wire.send returned callables): "
+                               "host calls are not part of a captured graph, so such a step cannot be replayed from one")
         if self._shadow_stale:
             self.refresh_shadow()
         torch.cuda.synchronize()

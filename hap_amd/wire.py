@@ -49,7 +49,9 @@ class Wire:
         GPU tensor that holds the message for rank ``dst`` after the local preparation kernels of collective
         ``tag`` have run in a step.  A transport would post its sends from these buffers.  May return a callable:
         the executor then calls it in every step right after those kernels are enqueued (the point at which the
-        message is complete; later launches of the step may reuse the buffer).  The stand-ins send nothing;
+        message is complete; later launches of the step may reuse the buffer), whether the step is launched call
+        by call or replayed from its recorded launch list; a step with such callables cannot be captured into a
+        HIP graph (``capture_train_step`` raises).  The stand-ins send nothing;
         ``ReplayWire`` snapshots the messages so that tests can compare them with the recorded run."""
         return None
 

@@ -1,0 +1,91 @@
+"""Programs that hap_amd.program did not generate: hand-built torch.fx graphs in the emitted node forms
+(hap.rs:991-2324), run by the executor and checked against stock PyTorch autograd on the CPU executing the same
+graph (the reference's execution model, worker.py:44-76)."""
+import operator
+
+import pytest
+import torch
+import torch.fx
+import torch.nn as nn
+import torch.nn.functional as F
+
+import hap_amd
+from helpers import rel_err
+
+pytestmark = pytest.mark.gpu
+
+
+class _Holder(nn.Module):
+    def __init__(self, V, d, seed=0):
+        super().__init__()
+        g = torch.Generator().manual_seed(seed)
+        mk = lambda *shape: nn.Parameter(torch.randn(*shape, generator=g) * 0.3)
+        self.emb = mk(V, d)
+        for i in range(4):
+            setattr(self, f"w{i}", mk(d, d))
+            setattr(self, f"b{i}", mk(d))
+        self.dec_w, self.dec_b = mk(V, d), mk(V)
+
+
+def _finish(g, t, y, d):
+    logits = g.call_function(F.linear, (t, g.get_attr("dec_w"), g.get_attr("dec_b")))
+    lp = g.call_function(torch.log_softmax, (logits, 2))
+    lp = g.call_function(torch.transpose, (lp, 1, 2))
+    g.output(g.call_function(F.nll_loss, (lp, y), {"reduction": "sum"}))
+    g.lint()
+
+
+def _run_both(build, V=37, d=32, B=4, S=8):
+    tokens = torch.randint(0, V, (B, S), generator=torch.Generator().manual_seed(1))
+    targets = torch.randint(0, V, (B, S), generator=torch.Generator().manual_seed(2))
+    results = []
+    for device in ("cpu", "gpu"):
+        holder = _Holder(V, d)
+        g = torch.fx.Graph()
+        x, y = g.placeholder("x"), g.placeholder("y")
+        h = g.call_function(F.embedding, (x, g.get_attr("emb")))
+        _finish(g, build(g, h, d), y, d)
+        gm = torch.fx.GraphModule(holder, g)
+        if device == "cpu":
+            loss = gm(tokens, targets)
+            loss.backward()
+            results.append((loss.item(), {n: p.grad.clone() for n, p in gm.named_parameters() if p.grad is not None}))
+        else:
+            ex = hap_amd.compile_program(gm, [tokens, targets], dtype="fp32")
+            loss = ex.forward(tokens, targets)
+            ex.backward()
+            torch.cuda.synchronize()
+            assert ex.shared_gradient_copies > 0           # the case the test is about did occur
+            results.append((loss.item(), {n: rec["grad"].cpu() for n, rec in ex.params.items()}))
+    (want, ref), (got, grads) = results
+    assert abs(got - want) <= 1e-4 * abs(want)
+    assert set(grads) == set(ref)
+    for n in ref:
+        assert rel_err(grads[n], ref[n]) < 1e-4, n
+
+
+def test_second_consumer_between_a_residual_branch_and_its_add(cuda):
+    """a + f(a) followed by layer_norm hands ONE gradient buffer to both a and f(a).  Here another consumer of a
+    lies between f and the add in program order, so its contribution to d(a) arrives before f's backward has read
+    that buffer: it must not be added in place."""
+    def build(g, h, d):
+        lin = lambda x, i: g.call_function(F.linear, (x, g.get_attr(f"w{i}"), g.get_attr(f"b{i}")))
+        a = lin(h, 0)
+        b = lin(a, 1)                       # f(a)
+        c = lin(a, 2)                       # the other consumer of a, after f
+        n = g.call_function(F.layer_norm, (g.call_function(operator.add, (a, b)), (d,)))
+        return g.call_function(operator.add, (n, c))
+    _run_both(build)
+
+
+def test_relu_output_that_shares_its_gradient_buffer(cuda):
+    """relu(linear(h)) + other: the add hands one gradient buffer to both operands; the relu's backward, which
+    the producing linear would apply in place, must leave the other operand's gradient alone."""
+    def build(g, h, d):
+        lin = lambda x, i: g.call_function(F.linear, (x, g.get_attr(f"w{i}"), g.get_attr(f"b{i}")))
+        other = lin(h, 0)
+        r = g.call_function(F.relu, (lin(h, 1),), {"inplace": False})
+        s = g.call_function(operator.add, (r, other))
+        u = lin(s, 2)                       # consumes the sum, so the add is a launch of its own
+        return g.call_function(operator.add, (u, lin(h, 3)))
+    _run_both(build)

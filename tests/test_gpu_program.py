@@ -249,6 +249,34 @@ def test_module_facade_is_a_drop_in(cuda):
         assert rel_err(got[clear], want[clear]) < 1e-3, n
 
 
+@pytest.mark.parametrize("lists", [True, False])
+def test_send_hooks_run_in_every_step(cuda, lists):
+    """Wire.send may return a callable that the executor runs in every step once the message is complete, also in the
+    steps that replay the recorded launch lists.  Three passes on three different batches: what ReplayWire's hooks
+    snapshot after the third pass must be the third batch's messages (the peers' messages are the recorded run's of
+    that batch, so the first two passes compute on mismatched data, which does not matter here)."""
+    model = make_lm()
+    batches = [lm_batch(8, 16, 97, seed=s) for s in (1, 2, 3)]
+    run = joint_cpu(model, RATIOS4, 8)
+    run.step(*batches[2])
+    gm = hap_amd.build_program(copy.deepcopy(model), hap_amd.ShardingPlan([RATIOS4], 0), 8)
+    ex = hap_amd.compile_program(gm, list(batches[0]), wire=hap_amd.ReplayWire(run.world.log, 0), rank=0, world_size=4,
+                                 launch_lists=lists)
+    assert ex._send_hooks > 0
+    first = None
+    for i, (x, y) in enumerate(batches):
+        ex.forward(x, y)
+        ex.backward()
+        torch.cuda.synchronize()
+        if i == 0:
+            first = {k: v.clone() for k, v in ex.wire.sent.items()}
+    _check_sent_messages(ex, run.world.log, 0, "fp32")
+    assert any(not torch.equal(first[k], v) for k, v in ex.wire.sent.items())
+    ex.configure_optimizer(**SGD)
+    with pytest.raises(RuntimeError, match="captured graph"):
+        ex.capture_train_step()
+
+
 def test_unsupported_nodes_raise(cuda):
     model = make_lm()
     model.dropout_p = 0.1
