@@ -1,5 +1,6 @@
 // Elementwise, gather/scatter and optimizer kernels (all HBM-bound).
 #include "common.h"
+#include <mutex>
 
 namespace {
 
@@ -674,6 +675,55 @@ extern "C" int hapmi_sumsq(const float *g, int64_t n, float *out, float *workspa
                   "sumsq: %lld elements need a workspace of %lld floats, %lld given", (long long)n,
                   (long long)hapmi_cdiv(n, SUMSQ_CHUNK), (long long)workspace_elems);
     return sumsq_launch(g, n, out, workspace, (hipStream_t)stream);
+}
+
+// ---- hapmi_sumsq_static: the same sum for callers that cannot allocate -------------------------------------
+// The partial sums live in a file-scope device array instead of a caller workspace.  Each GPU holds its own copy
+// of the array at its own address: the address is looked up once per device (with that device current) and only
+// that pointer is ever handed to kernels -- the array's name is not a device address in host code.
+constexpr int64_t SUMSQ_STATIC_CHUNKS = 65536;                    // 256 KiB per GPU; 2^30 elements at most
+static __device__ __align__(256) float g_sumsq_scratch[SUMSQ_STATIC_CHUNKS];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mu;
+float *g_scratch_ptr[kMaxDevices] = {nullptr};
+
+int sumsq_scratch_of_current_device(float **ptr) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return hapmi_set_error(HAPMI_ELAUNCH, "sumsq_static: hipGetDevice: %s", hipGetErrorString(e));
+    HAPMI_REQUIRE(dev >= 0 && dev < kMaxDevices, HAPMI_ELIMIT, "sumsq_static: device index %d beyond %d", dev, kMaxDevices);
+    std::lock_guard<std::mutex> lk(g_scratch_mu);
+    if (!g_scratch_ptr[dev]) {
+        void *p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(g_sumsq_scratch));
+        if (e != hipSuccess || !p)
+            return hapmi_set_error(HAPMI_ELAUNCH, "sumsq_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+        g_scratch_ptr[dev] = (float *)p;
+    }
+    *ptr = g_scratch_ptr[dev];
+    return HAPMI_OK;
+}
+}  // namespace
+
+extern "C" int hapmi_sumsq_static(const float *g, int64_t n, float *out, hapmi_stream_t stream) {
+    HAPMI_REQUIRE(n >= 0 && out, HAPMI_EINVAL, "sumsq_static: bad argument");
+    if (n == 0) {
+        hipLaunchKernelGGL(zero_f32_kernel, dim3(1), dim3(EW_THREADS), 0, (hipStream_t)stream, out, (int64_t)1);
+        HAPMI_CHECK_LAUNCH("sumsq_static");
+        return HAPMI_OK;
+    }
+    HAPMI_REQUIRE(g, HAPMI_EINVAL, "sumsq_static: null pointer");
+    HAPMI_REQUIRE(hapmi_cdiv(n, SUMSQ_CHUNK) <= SUMSQ_STATIC_CHUNKS, HAPMI_ELIMIT,
+                  "sumsq_static: %lld elements exceed the built-in scratch (at most %lld elements; use hapmi_sumsq "
+                  "with a workspace)", (long long)n, (long long)(SUMSQ_STATIC_CHUNKS * SUMSQ_CHUNK));
+    float *scratch = nullptr;
+    const int rc = sumsq_scratch_of_current_device(&scratch);
+    if (rc) return rc;
+    // every partial sum that the final kernel reads is written by the first kernel of this call: nothing in the
+    // array has to start at zero, whatever an earlier call left there
+    return sumsq_launch(g, n, out, scratch, (hipStream_t)stream);
 }
 
 extern "C" int hapmi_clip_coef(const float *sumsq, float max_norm, float *coef, hapmi_stream_t stream) {

@@ -342,6 +342,13 @@ int hapmi_adam_apply_dev(float *param, const float *grad, float *exp_avg, float 
 int hapmi_sumsq_workspace_elems(int64_t n, int64_t *elems_host);
 int hapmi_sumsq(const float *g, int64_t n, float *out, float *workspace, int64_t workspace_elems,
                 hapmi_stream_t stream);
+/* hapmi_sumsq without a workspace argument and without any allocation.  No counterpart in the reference; it is for
+ * callers that cannot allocate device memory: code under HIP graph capture, tight serving loops, harnesses that
+ * forbid it.  The partial sums go to a 256 KiB array inside the library's device code (each GPU the library runs
+ * on holds its copy until the process ends), so n is limited to 2^30 elements (HAPMI_ELIMIT beyond).  Calls that
+ * overlap on one GPU (different streams) share that array and race; calls on one stream are ordered and give the
+ * bits of hapmi_sumsq. */
+int hapmi_sumsq_static(const float *g, int64_t n, float *out, hapmi_stream_t stream);
 /* torch.nn.utils.clip_grad_norm_ coefficient (worker.py:74): coef = min(1, max_norm / (sqrt(sumsq) + 1e-6)) */
 int hapmi_clip_coef(const float *sumsq, float max_norm, float *coef, hapmi_stream_t stream);
 
