@@ -61,7 +61,8 @@ class ShardExecutor:
                  rank: int = 0, world_size: int = 1, device: str = "cuda:0", fused_attention: bool = True,
                  overlap_wgrad: bool = False, launch_lists: bool = True, relu_mask_in_dgrad: bool = True,
                  overlap_optimizer: bool = False, optimizer_chunk_min: int = 1 << 20,
-                 relu_bwd_in_split: bool = True, wgrad_group: int = 8, receive_in_place: bool = True):
+                 relu_bwd_in_split: bool = True, wgrad_group: int = 8, receive_in_place: bool = True,
+                 dropout_seed: int = 0):
         """``example_inputs``: the program's inputs (global batch) as tensors or shapes; activations are
         sized from them.  ``rank`` / ``world_size`` are only needed by all_reduce / replicate, whose node
         forms do not carry them (collectives.py:86, 182)."""
@@ -136,6 +137,11 @@ class ShardExecutor:
         self._side_readers: Dict[int, torch.cuda.Event] = {}   # storage -> event after its last side-stream reader
         self.side_workspace = torch.empty(64 << 20, dtype=torch.float32, device=self.dev) if overlap_wgrad else None
         self._single_use_params = self._find_single_use_params(gm)
+        # F.dropout with p > 0: keep decisions are a function of (seed, step, node, element); the step count lives on
+        # the device and is advanced by the first launch of every forward pass, so replayed steps draw new masks
+        self.rng_state = torch.tensor([int(dropout_seed), 0], dtype=torch.int64, device=self.dev)
+        self._node_ids = {node: i for i, node in enumerate(gm.graph.nodes)}
+        self._uses_rng = False
         # Every launch of a step is a library call on static buffers with constant arguments, so the calls of
         # the first forward / backward / optimizer phase are recorded and later phases replay the recorded
         # calls directly (no per-call argument marshalling or host-side checks: about 10 us of interpreter
@@ -460,6 +466,8 @@ class ShardExecutor:
         self._flush_wgrads()
         self._touched = None
         self._tape = []
+        if self._uses_rng:
+            self.fwd.insert(0, lambda: ops.rng_advance(self.rng_state))
 
     # ------------------------------------------------------------------ leaves
     def _get_attr(self, node):
@@ -635,9 +643,55 @@ class ShardExecutor:
         return Val("transposed", None, src=v, dims=dims, needs_grad=v.needs_grad)
 
     def _dropout(self, node):
-        if float(node.args[1]) != 0.0:
-            self._unsupported(node, "dropout with p > 0 is not implemented (parity runs use p = 0)")
-        return self._val(node.args[0])
+        """F.dropout(input, p) (hap.rs:1464: training mode).  p = 0 is the identity.  Otherwise one elementwise pass
+        forward and the same pass on the gradient backward; the mask is regenerated, not stored."""
+        p = float(node.args[1])
+        if len(node.args) > 2 or node.kwargs:
+            self._unsupported(node, "the program emits F.dropout(input, p) only")
+        x = self._val(node.args[0])
+        if p == 0.0:
+            return x
+        if not 0.0 < p <= 1.0:
+            self._unsupported(node, f"dropout probability {p}")
+        if x.t is None or x.ld is not None:
+            self._unsupported(node, f"dropout of a {x.kind} value")
+        self._uses_rng = True
+        sid = self._node_ids[node]
+        out = Val("tensor", self._new(x.t.shape), needs_grad=x.needs_grad, dropout=(p, sid))
+        self.fwd.append(lambda: ops.dropout(x.t, out.t, p, self.rng_state, sid))
+
+        def emit():
+            if out.grad is None or not x.needs_grad:
+                return
+            if x.grad is None:
+                x.grad = self._new(x.t.shape)
+                g = x.grad
+                self.bwd.append(lambda: ops.dropout(out.grad, g, p, self.rng_state, sid))
+            else:
+                tmp = self._new(x.t.shape)
+                g, _ = self._grad_slot(x)
+                self.bwd.append(lambda: (ops.dropout(out.grad, tmp, p, self.rng_state, sid), ops.add(g, tmp, g)))
+        self._tape.append(emit)
+        return out
+
+    def dropout_masks(self) -> Dict[str, torch.Tensor]:
+        """The keep decisions of the step that ran last, by node name: for an F.dropout node a bool tensor of its
+        input's shape, for an attention node with dropout_p > 0 a bool tensor [batch, heads, L, S] over its
+        probabilities.  (Tests hand them to the CPU oracle, which cannot share a random stream with the GPU.)"""
+        out = {}
+        for node, v in self.env.items():
+            if not isinstance(node, torch.fx.Node) or node.op != "call_function":
+                continue
+            if isinstance(v, Val) and v.meta.get("dropout") and node.target is F.dropout and float(node.args[1]) > 0:
+                p, sid = v.meta["dropout"]
+                out[node.name] = ops.dropout_mask(v.t.numel(), p, self.rng_state, sid).view(v.t.shape).bool()
+            elif isinstance(v, Val) and v.kind == "mha" and v.meta.get("dropout"):
+                p, sid, shape, S = v.meta["dropout"]
+                n = 1
+                for d in shape:
+                    n *= d
+                out[node.name] = ops.dropout_mask(n, p, self.rng_state, sid).view(shape)[..., :S].bool()
+        return out
 
     def _layer_norm(self, node):
         v, shape = self._val(node.args[0]), tuple(node.args[1])
@@ -803,16 +857,17 @@ class ShardExecutor:
             self._unsupported(node, "expects the (L, N, E) view produced by transpose(0, 1) of a batch-first tensor")
         if kw.get("bias_k") is not None or kw.get("bias_v") is not None or kw.get("add_zero_attn"):
             self._unsupported(node, "bias_k / bias_v / add_zero_attn are not supported")
-        if float(kw.get("dropout_p", 0.0)) != 0.0:
-            self._unsupported(node, "attention dropout with p > 0 is not implemented")
+        p_drop = float(kw.get("dropout_p", 0.0))
+        if not 0.0 <= p_drop <= 1.0:
+            self._unsupported(node, f"attention dropout probability {p_drop}")
         x = q.meta["src"]
         E = x.t.shape[2]
         if kw["embed_dim_to_check"] != E or E % kw["num_heads"]:
             self._unsupported(node, "embed_dim mismatch")
         out_bsd = self._attention_core(node, x, kw["in_proj_weight"], kw["in_proj_bias"], kw["out_proj_weight"],
-                                       kw["out_proj_bias"], kw["num_heads"], kw.get("attn_mask"))
+                                       kw["out_proj_bias"], kw["num_heads"], kw.get("attn_mask"), p_drop)
         out = Val("transposed", None, src=out_bsd, dims=(0, 1), needs_grad=True)
-        return Val("mha", None, out=out)
+        return Val("mha", None, out=out, dropout=out_bsd.meta.get("prob_dropout"))
 
     def _head_parallel_attention(self, node):
         """models.head_parallel_attention(x, in_proj_weight, in_proj_bias, out_proj_weight, num_heads, attn_mask):
@@ -825,9 +880,12 @@ class ShardExecutor:
             self._unsupported(node, "expects a materialised [batch, seq, d] tensor")
         return self._attention_core(node, x, w_in, b_in, w_out, None, H, mask)
 
-    def _attention_core(self, node, x: Val, w_in: Val, b_in: Val, w_out: Val, b_out: Optional[Val], H: int, mask):
+    def _attention_core(self, node, x: Val, w_in: Val, b_in: Val, w_out: Val, b_out: Optional[Val], H: int, mask,
+                        p_drop: float = 0.0):
         """qkv = x W_in^T + b_in over Ea = H * head_dim attention columns (all heads, or this device's heads),
-        softmax attention per head, out = ctx W_out^T (+ b_out).  x is [b, S, d]; W_in [3 Ea, d]; W_out [d_out, Ea]."""
+        softmax attention per head, out = ctx W_out^T (+ b_out).  x is [b, S, d]; W_in [3 Ea, d]; W_out [d_out, Ea].
+        ``p_drop`` > 0 (dropout of the probabilities, torch:nn/functional.py:6591): the probabilities are
+        materialised, as the reference's explicit path does, and the fused kernels are not used."""
         for v in (w_in, b_in, w_out) + ((b_out,) if b_out is not None else ()):
             if v.kind != "param":
                 self._unsupported(node, "attention weights must be parameters")
@@ -846,7 +904,7 @@ class ShardExecutor:
                 self._unsupported(node, "attn_mask must be a float32 [L, S] additive mask")
             mask_t = mask.t
         scale = 1.0 / math.sqrt(hd)
-        fused = self.fused_attention and self.dtype == "bf16" and hd == 64
+        fused = self.fused_attention and self.dtype == "bf16" and hd == 64 and p_drop == 0.0
         # a constant mask (a buffer of the module, not a gathered shard) that is exactly the causal one is
         # applied arithmetically by the fused kernels, which then also skip the key tiles above the diagonal
         causal = False
@@ -863,6 +921,11 @@ class ShardExecutor:
         else:
             P = self._new((b, H, S, Sp))
         out_bsd = Val("tensor", o, needs_grad=True)
+        sid = self._node_ids[node]
+        if p_drop > 0.0:
+            self._uses_rng = True
+            out_bsd.meta["prob_dropout"] = (p_drop, sid, (b, H, S, Sp), S)
+            Pd = self._scratch("attn_Pd", (b, H, S, Sp))          # dropout(P): rebuilt from P wherever it is needed
         M = b * S
         sQ, sP = (S * 3 * Ea, hd), (H * S * Sp, S * Sp)
         bias_out = b_out.meta["master"] if b_out is not None else None
@@ -875,7 +938,11 @@ class ShardExecutor:
                 ops.gemm(qkv, qkv, P, S, S, hd, transB=True, lda=3 * Ea, ldb=3 * Ea, ldc=Sp, alpha=scale, batch1=b,
                          batch2=H, strideA=sQ, strideB=sQ, strideC=sP, offB=Ea)
                 ops.softmax_fwd(P, mask_t, P, b * H * S, S, Sp, S)
-                ops.gemm(P, qkv, ctx, S, hd, S, lda=Sp, ldb=3 * Ea, ldc=Ea, batch1=b, batch2=H, strideA=sP, strideB=sQ,
+                Pv = P
+                if p_drop > 0.0:
+                    ops.dropout(P, Pd, p_drop, self.rng_state, sid)
+                    Pv = Pd
+                ops.gemm(Pv, qkv, ctx, S, hd, S, lda=Sp, ldb=3 * Ea, ldc=Ea, batch1=b, batch2=H, strideA=sP, strideB=sQ,
                          strideC=(S * Ea, hd), offB=2 * Ea)
             ops.gemm(ctx, w_out.t, o, M, d_out, Ea, transB=True, bias=bias_out)
         self.fwd.append(forward)
@@ -923,7 +990,12 @@ class ShardExecutor:
                     # dP = dctx V^T ; dV = P^T dctx
                     ops.gemm(dctx, qkv, dP, S, S, hd, transB=True, lda=Ea, ldb=3 * Ea, ldc=Sp, batch1=b, batch2=H,
                              strideA=(S * Ea, hd), strideB=sQ, strideC=sP, offB=2 * Ea)
-                    ops.gemm(P, dctx, dqkv, S, hd, S, transA=True, lda=Sp, ldb=Ea, ldc=3 * Ea, batch1=b, batch2=H,
+                    Pv = P
+                    if p_drop > 0.0:
+                        ops.dropout(P, Pd, p_drop, self.rng_state, sid)      # the forward's dropped probabilities again
+                        ops.dropout(dP, dP, p_drop, self.rng_state, sid)     # d(P) = d(dropout(P)) * keep / (1 - p)
+                        Pv = Pd
+                    ops.gemm(Pv, dctx, dqkv, S, hd, S, transA=True, lda=Sp, ldb=Ea, ldc=3 * Ea, batch1=b, batch2=H,
                              strideA=sP, strideB=(S * Ea, hd), strideC=sQ, offC=2 * Ea)
                     ops.softmax_bwd(dP, P, dP, b * H * S, S, Sp)
                     # dQ = scale dS K ; dK = scale dS^T Q

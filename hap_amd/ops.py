@@ -715,6 +715,29 @@ def colsum(x, out, M, N, ldx=None, accumulate=False):
                              dtype_code(x), _ptr(ws), ws.numel(), _stream()))
 
 
+def dropout(x, y, p: float, rng_state, stream_id: int):
+    """y = x * keep / (1 - p) (F.dropout in training mode); keep = f(rng_state = [seed, step], stream_id, index)."""
+    _dev(x, y, rng_state)
+    _need(y, x.numel(), "dropout y")
+    if x.dtype != y.dtype or rng_state.dtype != torch.int64 or rng_state.numel() < 2:
+        raise TypeError("dropout: x and y of one type and an int64[2] state expected")
+    check(lib().hapmi_dropout(_ptr(x), _ptr(y), x.numel(), ctypes.c_float(p), _ptr(rng_state), int(stream_id),
+                              dtype_code(x), _stream()))
+
+
+def dropout_mask(n: int, p: float, rng_state, stream_id: int) -> torch.Tensor:
+    """The keep decisions (uint8, 1 = kept) that ``dropout`` takes for n elements with this state and stream id."""
+    _dev(rng_state)
+    mask = torch.empty(n, dtype=torch.uint8, device=rng_state.device)
+    check(lib().hapmi_dropout_mask(_ptr(mask), n, ctypes.c_float(p), _ptr(rng_state), int(stream_id), _stream()))
+    return mask
+
+
+def rng_advance(rng_state):
+    _dev(rng_state)
+    check(lib().hapmi_rng_advance(_ptr(rng_state), _stream()))
+
+
 def fill_zero(t):
     _dev(t)
     check(lib().hapmi_fill_zero(_ptr(t), t.numel() * t.element_size(), _stream()))

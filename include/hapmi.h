@@ -254,6 +254,20 @@ int hapmi_colsum(const void *x, float *out, int64_t M, int64_t N, int64_t ldx, i
 int hapmi_fill_zero(void *p, int64_t bytes, hapmi_stream_t stream);
 int hapmi_cast(const void *src, int src_dtype, void *dst, int dst_dtype, int64_t n, hapmi_stream_t stream);
 
+/* F.dropout(input, p) as the emitted program calls it, i.e. in training mode (hap.rs:1464; also the dropout of the
+ * attention probabilities, hap.rs:1307): y = x * keep / (1 - p), in place allowed.  keep is a counter-based function
+ * of (rng_state_dev[0] = seed, rng_state_dev[1] = step, stream_id, element index): nothing is stored, the
+ * backward of the node is the same call on the gradient, and hapmi_dropout_mask writes the same decisions as
+ * bytes (1 = kept).  stream_id names the dropout node inside a program.  The reference draws from torch's
+ * generator instead; the two streams of random numbers cannot be made equal, so results are compared on exported
+ * masks and statistically. */
+int hapmi_dropout(const void *x, void *y, int64_t n, float p, const int64_t *rng_state_dev, int64_t stream_id,
+                  int dtype, hapmi_stream_t stream);
+int hapmi_dropout_mask(uint8_t *mask, int64_t n, float p, const int64_t *rng_state_dev, int64_t stream_id,
+                       hapmi_stream_t stream);
+/* rng_state_dev[1] += 1: once per training step, as a kernel, so that a step replayed from a HIP graph draws new masks */
+int hapmi_rng_advance(int64_t *rng_state_dev, hapmi_stream_t stream);
+
 /* F.embedding (hap.rs:2041) fused with `* scale` and `+ pe[S, d]` (models.py:79-81):
  * out[t, :] = table[ids[t], :] * scale + pe[t % S, :]   (pe may be NULL) */
 int hapmi_embedding_fwd(const int64_t *ids, const void *table, const void *pe, void *out, int64_t n_tokens,

@@ -184,8 +184,11 @@ class SingleRankCPURun(JointCPURun):
                  wire_dtype: Optional[torch.dtype] = None, decisions: Optional[Dict[str, torch.Tensor]] = None):
         """``decisions``: discrete decisions taken from another run of the same program, by node name -- for an
         ``F.relu`` node the boolean mask of the elements it lets through, for a ``top_2_gating`` node the expert
-        choices [B, S, 2].  The node then applies those instead of its own (relu(z) becomes z * mask, the gates
-        stay this run's probabilities of the given experts).  A step function turns a rounding-sized difference of
+        choices [B, S, 2], for an ``F.dropout`` node the boolean keep mask of its input's shape, for an
+        ``F.multi_head_attention_forward`` node with dropout_p > 0 the keep mask [N, H, L, S] of its probabilities.
+        The node then applies those instead of its own (relu(z) becomes z * mask, the gates stay this run's
+        probabilities of the given experts, dropout becomes x * keep / (1 - p): the GPU's random stream cannot be
+        shared with torch's generator, its masks can).  A step function turns a rounding-sized difference of
         its argument into a whole-sized difference of the result; with the decisions shared, what is left between
         two runs is their continuous arithmetic, which tolerances can bound.  Whether the other run's decisions
         differ from this run's own only where the argument is within rounding distance of the step is for the
@@ -201,6 +204,17 @@ class SingleRankCPURun(JointCPURun):
             args = self._lookup(r, node.args)
             if node.target is F.relu:
                 return args[0] * forced.to(args[0].dtype)
+            if node.target is F.dropout:
+                x, p = args[0], float(args[1])
+                scale = 1.0 / (1.0 - p) if p < 1.0 else 0.0
+                return (x.to(torch.float64 if x.dtype == torch.float64 else torch.float32)
+                        * (forced.to(torch.float32) * scale)).to(x.dtype)
+            if node.target is F.multi_head_attention_forward:
+                kw = self._lookup(r, node.kwargs)
+                out = ref.attention_with_dropped_probabilities(
+                    kw["query"], kw["in_proj_weight"], kw["in_proj_bias"], kw["out_proj_weight"], kw["out_proj_bias"],
+                    kw["num_heads"], kw.get("attn_mask"), forced, float(kw["dropout_p"]))
+                return out, None
             if node.target is product_models.top_2_gating:
                 x, n_expert, capacity, wg = args[:4]
                 hi = torch.float64 if x.dtype == torch.float64 else torch.float32

@@ -10,6 +10,8 @@ Functions and the reference lines they follow:
 * ``positional_encoding``  -- /root/reference/models.py:504-509.
 * ``top_2_gating``         -- /root/reference/models.py:477-502.
 * ``switch_gating``        -- /root/reference/models.py:452-475.
+* ``attention_with_dropped_probabilities`` -- F.multi_head_attention_forward's explicit path
+  (torch:nn/functional.py:6435-6612, the call emitted at hap.rs:1301-1321) with a given dropout mask.
 * ``head_parallel_attention`` -- no reference counterpart (the reference shards
   attention over the batch only): softmax attention of a subset of heads.
 * ``JointWorld`` collectives -- /root/reference/collectives.py:6-29 (padded,
@@ -127,6 +129,73 @@ def head_parallel_attention(x, in_proj_weight, in_proj_bias, out_proj_weight, nu
         scores = scores + attn_mask.to(scores.dtype)
     ctx = (torch.softmax(scores.float(), dim=3).to(v.dtype) @ v).transpose(1, 2).reshape(b, S, Ea)
     return ctx @ out_proj_weight.t()
+
+
+def attention_with_dropped_probabilities(query, in_proj_weight, in_proj_bias, out_proj_weight, out_proj_bias,
+                                         num_heads: int, attn_mask, keep, p: float):
+    """The explicit path of F.multi_head_attention_forward for self-attention (packed in-projection, baddbmm /
+    softmax / dropout / bmm, out-projection: torch:nn/functional.py:6435, 6504-6519, 6576-6612) with the dropout
+    of the probabilities written as a multiplication with a GIVEN keep mask: ``keep`` [N, H, L, S] (bool) and
+    the probability ``p`` it was drawn with, so P becomes P * keep / (1 - p).  ``query`` is (L, N, E) as in the
+    emitted node (hap.rs:1301-1321); returns the attention output (L, N, E).  Pinned by: with keep all ones and
+    p = 0 it is F.multi_head_attention_forward(dropout_p = 0); a dropped probability removes exactly that key's
+    value from that query's output (tests/test_oracle_attention.py)."""
+    L, N, E = query.shape
+    hd = E // num_heads
+    qkv = F.linear(query, in_proj_weight, in_proj_bias)
+    q, k, v = qkv.split(E, dim=2)
+    heads = lambda t: t.reshape(L, N * num_heads, hd).transpose(0, 1)          # [N*H, L, hd]
+    q, k, v = heads(q), heads(k), heads(v)
+    scores = (q * (1.0 / math.sqrt(hd))) @ k.transpose(1, 2)
+    if attn_mask is not None:
+        scores = scores + attn_mask.to(scores.dtype)
+    probs = torch.softmax(scores.float(), dim=2).to(v.dtype)
+    scale = 1.0 / (1.0 - p) if p < 1.0 else 0.0
+    probs = (probs.float() * (keep.reshape(N * num_heads, L, -1).float() * scale)).to(v.dtype)
+    ctx = (probs @ v).transpose(0, 1).reshape(L * N, E)
+    return F.linear(ctx, out_proj_weight, out_proj_bias).view(L, N, E)
+
+
+# --------------------------------------------------------------------------
+# dropout keep decisions (this build's own counter-based definition; the reference draws from torch's generator,
+# hap.rs:1464, whose stream a GPU kernel cannot reproduce)
+# --------------------------------------------------------------------------
+
+def _mix32(x):
+    """numpy uint32 restatement of the multiply-xorshift mixer (wrapping arithmetic)."""
+    x = np.asarray(x, dtype=np.uint64) & 0xFFFFFFFF
+    x ^= x >> np.uint64(16)
+    x = (x * np.uint64(0x7feb352d)) & np.uint64(0xFFFFFFFF)
+    x ^= x >> np.uint64(15)
+    x = (x * np.uint64(0x846ca68b)) & np.uint64(0xFFFFFFFF)
+    x ^= x >> np.uint64(16)
+    return x
+
+
+def dropout_keep(seed: int, step: int, stream_id: int, p: float, n: int) -> torch.Tensor:
+    """Keep decisions (bool[n]) of the product's dropout for elements 0..n-1: element i is kept iff the 16 random
+    bits that the pair i // 2 yields for it (low half: even element, high half: odd element) are >= round(p * 65536);
+    the pair's 32 bits are two rounds of mixing of (pair index, key) and the key is a mix of seed, step and stream id.
+    Pinned by the statistics any dropout mask must have (keep rate within the binomial bound, no correlation
+    between neighbours, between steps, between streams: tests/test_oracle_dropout.py); the GPU kernels must give
+    exactly these bits (tests/test_gpu_dropout.py)."""
+    M = 0xFFFFFFFF
+    seed, step, stream_id = seed & 0xFFFFFFFFFFFFFFFF, step & 0xFFFFFFFFFFFFFFFF, stream_id & 0xFFFFFFFFFFFFFFFF
+    k = int(_mix32((seed & M) ^ 0x9e3779b9))
+    k = int(_mix32(k ^ (seed >> 32)))
+    k = int(_mix32(k ^ (step & M)))
+    k = int(_mix32(k ^ (step >> 32) ^ 0x85ebca6b))
+    k = int(_mix32(k ^ (stream_id & M)))
+    k0 = k
+    k1 = int(_mix32(k ^ 0xc2b2ae35 ^ (stream_id >> 32)))
+    t = float(np.float32(p) * np.float32(65536.0) + np.float32(0.5))
+    thr = 0 if t <= 0 else (65536 if t >= 65536.0 else int(t))
+    j = np.arange((n + 1) // 2, dtype=np.uint64)
+    inner = _mix32(((j & np.uint64(M)) + np.uint64(k0)) & np.uint64(M))
+    hi = (((j >> np.uint64(32)) * np.uint64(0x9e3779b9)) + np.uint64(k1)) & np.uint64(M)
+    bits = _mix32(inner ^ hi)
+    halves = np.stack([bits & np.uint64(0xFFFF), bits >> np.uint64(16)], axis=1).reshape(-1)[:n]
+    return torch.from_numpy(halves >= np.uint64(thr))
 
 
 def switch_gating(gate_input, n_expert: int, capacity: int, gate_weight, train: bool = True):

@@ -64,3 +64,38 @@ def test_one_head_by_brute_force():
         ctx = [sum(e[t] / sum(e) * float(v[t][j]) for t in range(S)) for j in range(hd)]
         for c in range(d):
             assert abs(float(got[s, c]) - sum(float(w_out[c, j]) * ctx[j] for j in range(hd))) < 1e-6      # the restatement takes the softmax in float32
+
+
+@pytest.mark.parametrize("causal", [True, False])
+def test_attention_with_dropped_probabilities_is_the_library_attention_when_nothing_is_dropped(causal):
+    d, H, b, S = 48, 4, 3, 9
+    m = _layer(d, H, 5)
+    xt = torch.randn(S, b, d)
+    mask = torch.triu(torch.full((S, S), float("-inf")), diagonal=1) if causal else None
+    want = F.multi_head_attention_forward(xt, xt, xt, d, H, m.in_proj_weight, m.in_proj_bias, None, None, False, 0.0,
+                                          m.out_proj.weight, m.out_proj.bias, attn_mask=mask)[0]
+    keep = torch.ones(b, H, S, S, dtype=torch.bool)
+    got = ref.attention_with_dropped_probabilities(xt, m.in_proj_weight, m.in_proj_bias, m.out_proj.weight,
+                                                   m.out_proj.bias, H, mask, keep, 0.0)
+    torch.testing.assert_close(got, want, rtol=1e-5, atol=1e-5)
+
+
+def test_a_dropped_probability_removes_that_key_from_that_query():
+    """Brute force on one head: with keep[n, h, l, s] = 0 the value of key s no longer enters query l's output, the
+    kept probabilities are scaled by 1 / (1 - p) and NOT renormalised (torch drops after the softmax)."""
+    import math
+    torch.manual_seed(2)
+    S, d = 5, 4
+    x = torch.randn(S, 1, d, dtype=torch.float64)
+    w_in, b_in = torch.randn(3 * d, d, dtype=torch.float64), torch.randn(3 * d, dtype=torch.float64)
+    w_out, b_out = torch.eye(d, dtype=torch.float64), torch.zeros(d, dtype=torch.float64)
+    keep = torch.ones(1, 1, S, S, dtype=torch.bool)
+    keep[0, 0, 2, 1] = keep[0, 0, 2, 4] = keep[0, 0, 0, 0] = False
+    p = 0.25
+    got = ref.attention_with_dropped_probabilities(x, w_in, b_in, w_out, b_out, 1, None, keep, p)[:, 0]
+    proj = x[:, 0] @ w_in.t() + b_in
+    q, k, v = proj[:, :d], proj[:, d:2 * d], proj[:, 2 * d:]
+    for l in range(S):
+        e = [math.exp(float(q[l] @ k[s]) / math.sqrt(d)) for s in range(S)]
+        want = sum((e[s] / sum(e)) / (1 - p) * v[s] for s in range(S) if keep[0, 0, l, s])
+        torch.testing.assert_close(got[l], want, rtol=1e-5, atol=1e-6)      # the restatement takes the softmax in float32
