@@ -6,7 +6,9 @@
 Default workload (N = 1): the headline configuration -- BERT-large-style encoder, bf16 compute with float32 master
 weights, 24 layers, d 1024, 16 heads, FFN 4096 column-split to a local 1536 slice, seq 512, local batch 12
 of 32, vocab 30522, 15 % masked-LM targets, Adam.  Inputs are synthetic (seeded), resident in HBM before the
-timed region; the peers' halves of the collectives come from a seeded synthetic wire.
+timed region; the peers' halves of the collectives come from a seeded synthetic wire (one set of message buffers per
+layer).  The line's `extra` object carries the other configurations (2-layer float32 LM, ViT-L/16, MoE, the ragged
+collective kernels), each measured the same way with fewer steps.
 Prints ONE JSON line.
 """
 from __future__ import annotations
@@ -35,7 +37,7 @@ WORKLOADS = {
 }
 
 
-def build_workload(name, layers_override=None, attn="batch", zero=False):
+def build_workload(name, layers_override=None, attn="batch", zero=False, dropout=0.0):
     import torch
     import hap_amd
     from hap_amd import models
@@ -80,6 +82,7 @@ def build_workload(name, layers_override=None, attn="batch", zero=False):
     else:
         raise SystemExit(f"unknown workload {name}")
     models.init_normal_(model, 0.02, 39)
+    model.dropout_p = float(dropout)
     gm = hap_amd.build_program(model, plan, meta["global_batch"], batch_sharded=meta["batch_sharded"])
     return gm, x, y, meta
 
@@ -127,6 +130,11 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="bert", choices=list(WORKLOADS) + ["ragged"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extra", action="store_true",
+                    help="headline workload only: skip the `extra` object (the other configurations, measured briefly)")
+    ap.add_argument("--shared-peer-buffers", action="store_true",
+                    help="one set of peer message buffers per message shape (all layers read the same 50 MB, which can "
+                         "stay in the memory-side cache) instead of one per layer, as real receives are")
     ap.add_argument("--eager", action="store_true",
                     help="launch every kernel of the timed steps from the host instead of replaying a captured HIP graph")
     ap.add_argument("--no-autotune", action="store_true",
@@ -140,6 +148,9 @@ def main():
                          "MoE dense layers: the step loses about 1 %)")
     ap.add_argument("--attn", default="batch", choices=["batch", "heads"],
                     help="bert workload only: shard attention over samples (the headline plan) or over heads (6 of 16)")
+    ap.add_argument("--dropout", type=float, default=0.0,
+                    help="dropout probability of the model (the reference's default is 0.1, config.py:33; the headline "
+                         "configuration names none and runs with 0)")
     ap.add_argument("--zero", action="store_true",
                     help="bert workload only: parameters stored as dim-0 shards and gathered at use")
     ap.add_argument("--gemm-plan-file", default=None,
@@ -162,16 +173,52 @@ def main():
         print(json.dumps(ragged_bench.run(args.steps, args.warmup, not args.no_cpu_baseline)))
         return
 
+    headline = measure(args.workload, args, args.steps, args.warmup, share_shapes=args.shared_peer_buffers)
+    result = headline
+    if not args.no_extra and args.workload == "bert" and not args.eager:
+        # the other configurations of the benchmark set, each measured the same way (fewer steps), and the headline
+        # workload with one set of peer buffers per layer instead of one per message shape
+        extra = {}
+        other = measure("bert", args, max(5, args.steps // 2), 3, share_shapes=not args.shared_peer_buffers)
+        key = "bert_peer_buffers_per_layer" if args.shared_peer_buffers else "bert_peer_buffers_shared_by_shape"
+        extra[key] = _brief(other)
+        for name in ("lm", "vit", "moe"):
+            extra[name] = _brief(measure(name, args, max(5, args.steps // 2), 3, share_shapes=args.shared_peer_buffers))
+        from hap_amd import ragged_bench
+        rg = ragged_bench.run(20, 5, False)
+        extra["ragged"] = {"workload": rg["config"]["workload"], "GBps": rg["value"], "ms_per_pass": rg["ms_per_step"],
+                           "per_kernel_GBps": rg["config"]["per_kernel_GBps"],
+                           "per_kernel_frac_of_hbm_peak": {k: v / HBM_PEAK for k, v in rg["config"]["per_kernel_GBps"].items()},
+                           "ragged_reduce_traffic_bytes": rg["roofline"]["traffic"],
+                           "ragged_reduce_algorithmic_bytes": rg["roofline"]["algorithmic_bytes"]}
+        result["extra"] = extra
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(args.workload, headline.pop("_meta"))
+    result.pop("_meta", None)
+    print(json.dumps(result))
+
+
+def _brief(r):
+    return {"workload": r["config"]["workload"], "samples_per_s": r["value"], "ms_per_step": r["ms_per_step"],
+            "dtype": r["dtype"], "gemm_TFLOPs": r["roofline"]["achieved"], "gemm_frac_of_peak": r["roofline"]["frac"],
+            "gemm_ms_per_step": r["roofline"]["gemm_ms_per_step"], "final_loss": r["config"]["final_loss"]}
+
+
+def measure(workload, args, steps, warmup, share_shapes=True):
+    """One workload: compile, autotune the GEMM plans (untimed), warm up, time `steps` steps, bracket the GEMMs."""
+    import ctypes
+    import gc
+
     import torch
     import hap_amd
     from hap_amd import ops, planner
     from hap_amd._lib import lib
 
-    desc, dtype = WORKLOADS[args.workload]
-    if (args.attn != "batch" or args.zero) and args.workload != "bert":
-        raise SystemExit("--attn / --zero are options of the bert workload")
-    gm, x, y, meta = build_workload(args.workload, attn=args.attn, zero=args.zero)
-    wire = hap_amd.SyntheticWire(seed=39, scale=1.0, grad_scale=1e-3, share_shapes=True)
+    desc, dtype = WORKLOADS[workload]
+    bert = workload == "bert"
+    gm, x, y, meta = build_workload(workload, attn=args.attn if bert else "batch", zero=args.zero and bert,
+                                    dropout=args.dropout)
+    wire = hap_amd.SyntheticWire(seed=39, scale=1.0, grad_scale=1e-3, share_shapes=share_shapes)
     ex = hap_amd.compile_program(gm, [x, y], dtype=dtype, wire=wire, rank=0, world_size=len(meta["ratios"]),
                                  overlap_wgrad=args.overlap, relu_mask_in_dgrad=not args.no_relu_mask_in_dgrad,
                                  overlap_optimizer=args.overlap_optimizer, wgrad_group=args.wgrad_group,
@@ -194,7 +241,7 @@ def main():
             ops.save_gemm_plans(args.gemm_plan_file)
 
     graph = None
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         one_step()
     torch.cuda.synchronize()
     if not args.eager:
@@ -212,7 +259,7 @@ def main():
     lib().hapmi_prof_gemm_enable(0 if graph is not None else 1)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(steps):
         if graph is not None:
             graph.replay()
         else:
@@ -221,7 +268,6 @@ def main():
     dt = time.perf_counter() - t0
     loss = float(ex.loss[0].item())
 
-    import ctypes
     ms, n_launch, flops = ctypes.c_double(), ctypes.c_int64(), ctypes.c_double()
     if graph is None:
         lib().hapmi_prof_gemm_collect(ctypes.byref(ms), ctypes.byref(n_launch), ctypes.byref(flops))
@@ -237,33 +283,39 @@ def main():
         lib().hapmi_prof_gemm_enable(0)
     achieved = flops.value / (ms.value * 1e-3) / 1e12 if ms.value > 0 else 0.0
     peak = PEAK[dtype]
-    ms_per_step = dt / args.steps * 1e3
+    ms_per_step = dt / steps * 1e3
     result = {
         "metric": "samples/sec of one GPU's uneven shard (fwd+bwd+step)",
-        "value": meta["local_batch"] * args.steps / dt,
+        "value": meta["local_batch"] * steps / dt,
         "unit": "samples/s",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
+        "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": ms_per_step,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": dtype, "data": "synthetic",
         "config": {"workload": desc, "local_batch": meta["local_batch"], "global_batch": meta["global_batch"],
                    "seq_len": meta["seq_len"], "launch": "hip-graph" if graph is not None else "eager",
                    "wgrad_stream": "side" if args.overlap else "main",
                    "optimizer": "one launch after backward" if ex._opt_chunks is None else "per stretch, overlapped with backward",
-                   "gemm_plan": plan_source, "weight_gradient_group": ex.wgrad_group, "exchange_pieces_received_in_place": ex.receive_in_place, "attention_sharding": args.attn, "zero_sharded_parameters": bool(args.zero),
+                   "gemm_plan": plan_source, "weight_gradient_group": ex.wgrad_group,
+                   "exchange_pieces_received_in_place": ex.receive_in_place,
+                   "peer_buffers": "one set per message shape" if share_shapes else "one set per layer",
+                   "attention_sharding": args.attn if bert else "batch",
+                   "zero_sharded_parameters": bool(args.zero and bert), "dropout": args.dropout,
                    "final_loss": loss},
         "roofline": {"bound": "mfma", "kernel": "gemm_kernel (all GEMM launches of the step)",
                      "achieved": achieved, "peak": peak, "unit": "TFLOP/s", "frac": achieved / peak,
                      "measured_over": "the timed steps" if graph is None else "3 eager steps after the timed graph replays",
-                     "launches_per_step": n_launch.value / max(1, args.steps if graph is None else 3),
-                     "gemm_ms_per_step": ms.value / max(1, args.steps if graph is None else 3), "traffic": None},
+                     "launches_per_step": n_launch.value / max(1, steps if graph is None else 3),
+                     "gemm_ms_per_step": ms.value / max(1, steps if graph is None else 3), "traffic": None},
     }
     # the reference calibrates its planner with hap.stat / (seconds of one training step) (profiler.py:33-39)
     shard_stat = planner.stat(gm, {"input_shape": {"x": tuple(x.shape), "y": tuple(y.shape)}})
     result["config"]["hap_stat_flops_of_shard"] = shard_stat
     result["config"]["device_flops"] = math.floor(shard_stat / (ms_per_step * 1e-3))
-    if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(args.workload, meta)
-    print(json.dumps(result))
+    result["_meta"] = meta
+    del graph, ex, wire, gm
+    gc.collect()
+    torch.cuda.empty_cache()
+    return result
 
 
 if __name__ == "__main__":
