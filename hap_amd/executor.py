@@ -1240,7 +1240,7 @@ class ShardExecutor:
         the shard (bf16 shadow for matrices, float32 master for vectors, which consumers add in float32) is
         gathered every step.  The consumers see a whole parameter whose float32 gradient is a buffer of the
         whole shape; once they have all written it, that gradient is reduce-scattered into the shard's slot
-        of the flat gradient buffer (all_gather's backward, collectives.py:63-68)."""
+        of the flat gradient buffer (AllGather.backward, collectives.py:22-29)."""
         if dim != 0 or x.t.shape[0] != L[rank]:
             self._unsupported(node, "a gathered parameter must be a dim-0 shard of the plan's length")
         vector = x.t.dim() == 1

@@ -86,8 +86,9 @@ int hapmi_split_rows(const void *src, void *const *pieces_host, const int64_t *l
                      int64_t outer, int64_t inner_bytes, hapmi_stream_t stream);
 
 /* hapmi_split_rows of src * (fwd_out > 0), fwd_out having src's shape and dtype: the backward of a relu whose
- * only reader's gradient goes straight into an all_to_all (models.py:283 after collectives.py:156-165 in the
- * column-sharded FFN), without a separate pass over the gradient.  Every piece, src and fwd_out 16-byte aligned
+ * only reader's gradient goes straight into an all_to_all (the FFN's F.relu -- the default activation of the
+ * nn.TransformerEncoderLayer built at models.py:74, emitted at hap.rs:1417 -- behind collectives.py:156-165 in
+ * the column-sharded FFN), without a separate pass over the gradient.  Every piece, src and fwd_out 16-byte aligned
  * with inner_bytes * lengths a multiple of 16. */
 int hapmi_split_rows_relu_bwd(const void *src, const void *fwd_out, void *const *pieces_host,
                               const int64_t *lengths_host, int n_ranks, int64_t outer, int64_t inner_bytes,
@@ -107,7 +108,7 @@ int hapmi_ragged_reduce(const void *const *contribs_host, int n_ranks, void *dst
                         int64_t offset, int64_t len, int64_t inner, int dtype, hapmi_stream_t stream);
 
 /* hapmi_ragged_reduce with one more term, added last: dst = addend + sum_w contribs[w][...]; addend has dst's
- * layout and may be dst itself.  The gradient that all_gather's backward (collectives.py:63-68) contributes
+ * layout and may be dst itself.  The gradient that all_gather's backward (AllGather.backward, collectives.py:22-29) contributes
  * to a value that already holds a gradient from another consumer, in one pass. */
 int hapmi_ragged_reduce_add(const void *const *contribs_host, int n_ranks, void *dst, const void *addend,
                             int64_t outer, int64_t src_len, int64_t offset, int64_t len, int64_t inner, int dtype,
@@ -177,7 +178,13 @@ typedef struct {
 #define HAPMI_GEMM_MAX_LIST 16
 int hapmi_gemm(const hapmi_gemm_args *args_host, hapmi_stream_t stream);
 
-/* Tuning hook for measurements: force tile configuration `tile_config` (block tile / waves: 0: 128x128 / 2x2,
+/* PROCESS-WIDE STATE.  hapmi_gemm_tuning, the plan table below and hapmi_prof_gemm_* keep state inside the library
+ * that every later hapmi_gemm call of the process reads: they are set-up and measurement hooks, not part of a
+ * step.  Calling them while another thread launches GEMMs is safe (the table and the instrumentation are locked)
+ * but changes what that thread's next call does; every other entry point of this header is stateless and
+ * re-entrant (all work goes to the stream passed in, all memory is the caller's).
+ *
+ * Tuning hook for measurements: force tile configuration `tile_config` (block tile / waves: 0: 128x128 / 2x2,
  * 1: 256x256 / 2x4, 2: 384x192 / 4x2, 3: 192x256 / 2x4, 4: 256x192 / 4x2, 5: 256x128 / 4x2, 6: 128x256 / 2x4,
  * 7: 192x128 / 2x4, 8: 256x128 / 2x2, 9: 128x192 / 4x2, 10: 64x64 / 2x2, 11: 64x128 / 2x2; 5..9 keep three
  * k-tiles in LDS (two in flight); 1..9 take bf16 operands only, 10 and 11 float32 operands only; a configuration
