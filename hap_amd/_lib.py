@@ -19,6 +19,14 @@ class HapmiError(RuntimeError):
     pass
 
 
+GEMM_MAX_SEGMENTS = 8
+
+
+class GemmSegments(ctypes.Structure):
+    _fields_ = [("n", ctypes.c_int), ("begin", ctypes.c_int64 * (GEMM_MAX_SEGMENTS + 1)),
+                ("ld", ctypes.c_int64 * GEMM_MAX_SEGMENTS), ("base", ctypes.c_void_p * GEMM_MAX_SEGMENTS)]
+
+
 class GemmArgs(ctypes.Structure):
     _fields_ = [
         ("A", ctypes.c_void_p), ("B", ctypes.c_void_p), ("C", ctypes.c_void_p), ("bias", ctypes.c_void_p),
@@ -38,6 +46,9 @@ class GemmArgs(ctypes.Structure):
         ("c_addend", ctypes.c_void_p),
         ("A_list", ctypes.c_void_p), ("B_list", ctypes.c_void_p), ("C_list", ctypes.c_void_p),
         ("a_rowsum_list", ctypes.c_void_p),
+        ("A_segments", ctypes.c_void_p), ("B_segments", ctypes.c_void_p), ("C_segments", ctypes.c_void_p),
+        ("c_mask_segments", ctypes.c_void_p), ("B_segments_list", ctypes.c_void_p),
+        ("a_relu", ctypes.c_int), ("b_relu", ctypes.c_int),
     ]
 
 

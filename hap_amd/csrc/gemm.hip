@@ -14,6 +14,7 @@
 // holds 4 consecutive n of one m in its accumulators and the epilogue issues 8/16-byte stores along the
 // contiguous dimension of C.
 #include "gemm_kernel.h"
+#include <string.h>
 #include <vector>
 #include <mutex>
 #include <map>
@@ -83,7 +84,17 @@ struct Choice {
 
 // Which tile configurations a call may use: 0 serves every type; 1..9 bf16 operands of calls that allow the large
 // tiles; 10, 11 float32 operands.
-bool cfg_eligible(int c, bool bf16_in, bool wide, bool row_major_operands, bool forced) {
+// A call with operands in pieces narrows the choice further (SegNeeds): A in pieces along K runs on the three-stage
+// configurations only, and the tile's N extent must divide every piece boundary of B / C.
+struct SegNeeds {
+    bool three_stage = false;
+    int64_t n_align = 0;                       // 0: no constraint; else every piece boundary along N is a multiple of it
+};
+constexpr bool kThreeStage[] = {false, false, false, false, false, true, true, true, true, true, false, false};
+
+bool cfg_eligible(int c, bool bf16_in, bool wide, bool row_major_operands, bool forced, const SegNeeds &need = SegNeeds()) {
+    if (need.three_stage && !kThreeStage[c]) return false;
+    if (need.n_align > 0 && need.n_align % kCfg[c].bn != 0) return false;
     if (c == 0) return true;
     if (c >= kFirstF32Cfg) return !bf16_in;
     if (!bf16_in || !wide) return false;
@@ -92,14 +103,14 @@ bool cfg_eligible(int c, bool bf16_in, bool wide, bool row_major_operands, bool 
 }
 
 Choice choose(int64_t M, int64_t N, int64_t K, int64_t batch, int bk, bool bf16_in, bool wide, int64_t max_splits,
-              bool row_major_operands) {
+              bool row_major_operands, const SegNeeds &need) {
     static const int kSplitMenu[] = {1, 2, 3, 4, 5, 6, 7, 8, 10, 12, 16, 24, 32};
     const int64_t nk = hapmi_cdiv(K, bk);
-    Choice best{0, 1};
+    Choice best{-1, 1};
     double best_t = 1e30;
-    const bool forced = g_force_cfg >= 0 && g_force_cfg < kNumCfg && cfg_eligible(g_force_cfg, bf16_in, wide, row_major_operands, true);
+    const bool forced = g_force_cfg >= 0 && g_force_cfg < kNumCfg && cfg_eligible(g_force_cfg, bf16_in, wide, row_major_operands, true, need);
     for (int c = 0; c < kNumCfg; ++c) {
-        if (forced ? c != g_force_cfg : !cfg_eligible(c, bf16_in, wide, row_major_operands, false)) continue;
+        if (forced ? c != g_force_cfg : !cfg_eligible(c, bf16_in, wide, row_major_operands, false, need)) continue;
         const int64_t tiles = hapmi_cdiv(M, kCfg[c].bm) * hapmi_cdiv(N, kCfg[c].bn) * batch;
         // co-resident blocks per CU, TFLOP/s per block slot in steady state, us per tile for first loads + epilogue
         double per_cu, rate, fixed;
@@ -126,6 +137,8 @@ Choice choose(int64_t M, int64_t N, int64_t K, int64_t batch, int bk, bool bf16_
             }
         }
     }
+    // nothing matched the forced split: the 128 x 128 tile without a split serves every call it is eligible for
+    if (best.cfg < 0 && cfg_eligible(0, bf16_in, wide, row_major_operands, false, need)) best = Choice{0, 1};
     return best;
 }
 
@@ -201,7 +214,7 @@ __global__ __launch_bounds__(256) void rowsum_reduce_kernel(const float *ws, Row
 
 template <typename TI, typename TO>
 int launch_typed(GemmParams &p, int transA, int transB, int64_t batch, hipStream_t st, bool wide, void *workspace,
-                 int64_t workspace_bytes) {
+                 int64_t workspace_bytes, const SegNeeds &need) {
     const int bk = ROW_BYTES / (int)sizeof(TI);
     const int64_t nk = hapmi_cdiv(p.K, bk);
     p.ws_ld = (p.N + 3) / 4 * 4;
@@ -213,15 +226,19 @@ int launch_typed(GemmParams &p, int transA, int transB, int64_t batch, hipStream
     const int64_t split_bytes = want_rs ? rs_off : workspace_bytes;
     if (want_rs && (!workspace || ((uintptr_t)workspace % 16) != 0))
         return hapmi_set_error(HAPMI_EINVAL, "gemm: a_rowsum needs a 16-byte aligned workspace for its partial sums");
-    const int64_t max_splits = (workspace && ((uintptr_t)workspace % 16) == 0 && per_split > 0) ? split_bytes / per_split : 0;
-    Choice ch = choose(p.M, p.N, p.K, batch, bk, sizeof(TI) == 2, wide, max_splits, !transA && transB);
+    const bool segmented = p.segA.n > 0 || p.segB.n > 0 || p.segC.n > 0;
+    const int64_t max_splits = (!segmented && workspace && ((uintptr_t)workspace % 16) == 0 && per_split > 0) ? split_bytes / per_split : 0;
+    Choice ch = choose(p.M, p.N, p.K, batch, bk, sizeof(TI) == 2, wide, max_splits, !transA && transB, need);
+    if (ch.cfg < 0)
+        return hapmi_set_error(HAPMI_EINVAL, "gemm: no tile configuration fits the pieces of the operands (boundaries along N "
+                               "must be multiples of a tile's N extent: 64, 128, 192 or 256)");
     if (g_force_cfg < 0 && g_force_splits <= 0) {
         std::lock_guard<std::mutex> lk(g_plans_mu);
         auto it = g_plans.find(PlanKey(p.M, p.N, p.K, batch, (int)(transA != 0), (int)(transB != 0), sizeof(TI) == 2 ? HAPMI_BF16 : HAPMI_F32,
                                        sizeof(TO) == 2 ? HAPMI_BF16 : HAPMI_F32));
         if (it != g_plans.end()) {
             const int pc = it->second.first, ps = it->second.second;
-            const bool cfg_ok = pc >= 0 && pc < kNumCfg && cfg_eligible(pc, sizeof(TI) == 2, wide, !transA && transB, true);
+            const bool cfg_ok = pc >= 0 && pc < kNumCfg && cfg_eligible(pc, sizeof(TI) == 2, wide, !transA && transB, true, need);
             const bool split_ok = ps == 1 || (ps > 1 && ps <= max_splits && batch == 1 && nk / ps >= 1);
             if (cfg_ok && split_ok) ch = Choice{pc, ps};
         }
@@ -275,6 +292,40 @@ int launch_typed(GemmParams &p, int transA, int transB, int64_t batch, hipStream
 
 }  // namespace
 
+namespace {
+int64_t gcd64(int64_t a, int64_t b) {
+    while (b) {
+        const int64_t t = a % b;
+        a = b;
+        b = t;
+    }
+    return a;
+}
+
+// copy a description of pieces into the kernel's parameter block after checking it
+int fill_segments(GemmSegs &g, const hapmi_gemm_segments *s, int64_t extent, int64_t align, int64_t epv, bool need_base,
+                  const char *what) {
+    g.n = 0;
+    if (!s) return HAPMI_OK;
+    HAPMI_REQUIRE(s->n >= 1 && s->n <= HAPMI_GEMM_MAX_SEGMENTS, HAPMI_ELIMIT, "gemm: %s holds 1..%d pieces", what, HAPMI_GEMM_MAX_SEGMENTS);
+    HAPMI_REQUIRE(s->begin[0] == 0 && s->begin[s->n] == extent && extent < (1ll << 31), HAPMI_EINVAL,
+                  "gemm: %s must cover [0, %lld)", what, (long long)extent);
+    for (int i = 0; i < s->n; ++i) {
+        const int64_t len = s->begin[i + 1] - s->begin[i];
+        HAPMI_REQUIRE(len > 0 && s->begin[i] % align == 0, HAPMI_EINVAL, "gemm: %s: piece %d starts at %lld (not a multiple of %lld) or is empty",
+                      what, i, (long long)s->begin[i], (long long)align);
+        HAPMI_REQUIRE(s->ld[i] >= len && s->ld[i] % epv == 0, HAPMI_EALIGN, "gemm: %s: leading dimension of piece %d", what, i);
+        HAPMI_REQUIRE(!need_base || (s->base[i] && ((uintptr_t)s->base[i] % 16) == 0), HAPMI_EALIGN, "gemm: %s: base of piece %d", what, i);
+        g.begin[i] = (int)s->begin[i];
+        g.ld[i] = s->ld[i];
+        g.base[i] = s->base[i];
+    }
+    g.begin[s->n] = (int)extent;
+    g.n = s->n;
+    return HAPMI_OK;
+}
+}  // namespace
+
 extern "C" int hapmi_gemm(const hapmi_gemm_args *a, hapmi_stream_t stream) {
     HAPMI_REQUIRE(a, HAPMI_EINVAL, "gemm: null argument block");
     HAPMI_REQUIRE(hapmi_dtype_ok(a->in_dtype) && hapmi_dtype_ok(a->out_dtype), HAPMI_EINVAL, "gemm: bad dtype");
@@ -296,7 +347,7 @@ extern "C" int hapmi_gemm(const hapmi_gemm_args *a, hapmi_stream_t stream) {
                           HAPMI_EALIGN, "gemm: misaligned pointer in a list");
         }
     } else {
-        HAPMI_REQUIRE(a->A && a->B && a->C, HAPMI_EINVAL, "gemm: null pointer");
+        HAPMI_REQUIRE((a->A || a->A_segments) && (a->B || a->B_segments) && (a->C || a->C_segments), HAPMI_EINVAL, "gemm: null pointer");
     }
     HAPMI_REQUIRE(a->act == HAPMI_ACT_NONE || a->act == HAPMI_ACT_RELU || a->act == HAPMI_ACT_GELU, HAPMI_EINVAL,
                   "gemm: unknown activation %d", a->act);
@@ -348,6 +399,62 @@ extern "C" int hapmi_gemm(const hapmi_gemm_args *a, hapmi_stream_t stream) {
     HAPMI_REQUIRE(!a->c_relu_mask || (!lists && ((uintptr_t)a->c_relu_mask % 16) == 0), HAPMI_EINVAL,
                   "gemm: c_relu_mask needs a 16-byte aligned pointer and no pointer lists");
 
+    // operands / result in pieces
+    SegNeeds need;
+    memset(p.listSegB, 0, sizeof(p.listSegB));
+    p.a_relu = a->a_relu != 0;
+    p.b_relu = a->b_relu != 0;
+    const bool any_seg = a->A_segments || a->B_segments || a->C_segments || a->c_mask_segments || a->B_segments_list;
+    if (any_seg || p.a_relu || p.b_relu)
+        HAPMI_REQUIRE(a->in_dtype == HAPMI_BF16 && a->batch2 == 1, HAPMI_EINVAL, "gemm: pieces and operand relu take bf16 operands");
+    int rc_seg = fill_segments(p.segA, a->A_segments, a->K, 64, 8, true, "A_segments");
+    if (rc_seg) return rc_seg;
+    if (p.segA.n > 0 || p.a_relu) {
+        HAPMI_REQUIRE(!a->transA && a->transB && batch == 1 && a->K % 64 == 0 && !a->a_rowsum, HAPMI_EINVAL,
+                      "gemm: A_segments / a_relu need transA = 0, transB = 1, one problem and K a multiple of 64");
+        need.three_stage = true;
+    }
+    HAPMI_REQUIRE(!p.b_relu || (a->transA && !a->transB), HAPMI_EINVAL, "gemm: b_relu needs transA = 1, transB = 0");
+    const hapmi_gemm_segments *bseg = a->B_segments;
+    if (a->B_segments_list) {
+        HAPMI_REQUIRE(lists && !a->B_segments, HAPMI_EINVAL, "gemm: B_segments_list goes with pointer lists (and without B_segments)");
+        bseg = a->B_segments_list[0];
+        HAPMI_REQUIRE(bseg, HAPMI_EINVAL, "gemm: null entry in B_segments_list");
+    }
+    rc_seg = fill_segments(p.segB, bseg, a->N, 64, 8, true, "B_segments");
+    if (rc_seg) return rc_seg;
+    if (p.segB.n > 0) {
+        HAPMI_REQUIRE(!a->transB && (lists ? a->B_segments_list != nullptr : true), HAPMI_EINVAL,
+                      "gemm: B_segments need transB = 0 (B stored [K, N])");
+        for (int i = 1; i < p.segB.n; ++i) need.n_align = gcd64(need.n_align, p.segB.begin[i]);
+        if (a->B_segments_list)
+            for (int z = 0; z < p.n_list; ++z) {
+                const hapmi_gemm_segments *sz = a->B_segments_list[z];
+                HAPMI_REQUIRE(sz && sz->n == p.segB.n, HAPMI_EINVAL, "gemm: B_segments_list[%d] differs from the first entry", z);
+                for (int i = 0; i < p.segB.n; ++i) {
+                    HAPMI_REQUIRE(sz->begin[i] == bseg->begin[i] && sz->ld[i] == bseg->ld[i] && sz->base[i] &&
+                                      ((uintptr_t)sz->base[i] % 16) == 0, HAPMI_EINVAL,
+                                  "gemm: B_segments_list[%d] differs from the first entry or holds a bad base", z);
+                    p.listSegB[z][i] = sz->base[i];
+                }
+            }
+    }
+    rc_seg = fill_segments(p.segC, a->C_segments, a->N, 64, 4, true, "C_segments");
+    if (rc_seg) return rc_seg;
+    rc_seg = fill_segments(p.segM, a->c_mask_segments, a->N, 64, 4, true, "c_mask_segments");
+    if (rc_seg) return rc_seg;
+    if (p.segC.n > 0) {
+        HAPMI_REQUIRE(batch == 1 && !a->accumulate && !a->c_addend && !a->c_relu_mask, HAPMI_EINVAL,
+                      "gemm: C_segments take one problem without accumulate / c_addend / c_relu_mask");
+        for (int i = 1; i < p.segC.n; ++i) need.n_align = gcd64(need.n_align, p.segC.begin[i]);
+    }
+    if (p.segM.n > 0) {
+        HAPMI_REQUIRE(p.segC.n == p.segM.n, HAPMI_EINVAL, "gemm: c_mask_segments go with C_segments of the same layout");
+        for (int i = 0; i < p.segM.n; ++i)
+            HAPMI_REQUIRE(p.segM.begin[i] == p.segC.begin[i] && p.segM.ld[i] == p.segC.ld[i], HAPMI_EINVAL,
+                          "gemm: c_mask_segments go with C_segments of the same layout");
+    }
+
     hipStream_t st = (hipStream_t)stream;
     hipEvent_t e0 = nullptr, e1 = nullptr;
     bool prof = false;
@@ -362,10 +469,10 @@ extern "C" int hapmi_gemm(const hapmi_gemm_args *a, hapmi_stream_t stream) {
     }
     if (prof) (void)hipEventRecord(e0, st);
     int rc;
-    if (a->in_dtype == HAPMI_BF16 && a->out_dtype == HAPMI_BF16) rc = launch_typed<bf16_t, bf16_t>(p, a->transA, a->transB, batch, st, true, a->workspace, a->workspace_bytes);
-    else if (a->in_dtype == HAPMI_BF16) rc = launch_typed<bf16_t, float>(p, a->transA, a->transB, batch, st, true, a->workspace, a->workspace_bytes);
-    else if (a->out_dtype == HAPMI_F32) rc = launch_typed<float, float>(p, a->transA, a->transB, batch, st, false, a->workspace, a->workspace_bytes);
-    else rc = launch_typed<float, bf16_t>(p, a->transA, a->transB, batch, st, false, a->workspace, a->workspace_bytes);
+    if (a->in_dtype == HAPMI_BF16 && a->out_dtype == HAPMI_BF16) rc = launch_typed<bf16_t, bf16_t>(p, a->transA, a->transB, batch, st, true, a->workspace, a->workspace_bytes, need);
+    else if (a->in_dtype == HAPMI_BF16) rc = launch_typed<bf16_t, float>(p, a->transA, a->transB, batch, st, true, a->workspace, a->workspace_bytes, need);
+    else if (a->out_dtype == HAPMI_F32) rc = launch_typed<float, float>(p, a->transA, a->transB, batch, st, false, a->workspace, a->workspace_bytes, need);
+    else rc = launch_typed<float, bf16_t>(p, a->transA, a->transB, batch, st, false, a->workspace, a->workspace_bytes, need);
     if (prof) {
         (void)hipEventRecord(e1, st);
         std::lock_guard<std::mutex> lk(g_prof.mu);

@@ -20,6 +20,14 @@
 #include "tile.h"
 #include <type_traits>
 
+// an operand or result in pieces along one dimension (hapmi_gemm_segments with 32-bit ranges)
+struct GemmSegs {
+    int n;                                                    // 0 = off
+    int begin[HAPMI_GEMM_MAX_SEGMENTS + 1];
+    int64_t ld[HAPMI_GEMM_MAX_SEGMENTS];
+    const void *base[HAPMI_GEMM_MAX_SEGMENTS];
+};
+
 struct GemmParams {
     const void *A, *B;
     void *C;
@@ -43,7 +51,11 @@ struct GemmParams {
     const void *listA[HAPMI_GEMM_MAX_LIST], *listB[HAPMI_GEMM_MAX_LIST];
     void *listC[HAPMI_GEMM_MAX_LIST];
     float *listRS[HAPMI_GEMM_MAX_LIST];
+    GemmSegs segA, segB, segC, segM;                          // A along K; B, C and the relu mask along N
+    const void *listSegB[HAPMI_GEMM_MAX_LIST][HAPMI_GEMM_MAX_SEGMENTS];   // with pointer lists: the B pieces of problem z
+    int a_relu, b_relu;                                       // relu on op(A) / op(B) fragments as they are read
 };
+static_assert(sizeof(GemmParams) <= 3072, "the parameter block travels as a kernel argument (4 KiB at most)");
 
 namespace {
 
@@ -67,7 +79,23 @@ __device__ __forceinline__ float apply_act(float v, int act) {
     return v;
 }
 
-template <typename TI, typename TO, int BM, int BN, int WAVES_M, int WAVES_N, bool A_KMAJOR, bool B_KMAJOR, int NSTAGES>
+__device__ __forceinline__ bf16x8 relu_frag(bf16x8 v) {
+    // max(x, 0) on bf16 through the signed 16-bit integer order: negative values (sign bit set) become +0
+    typedef short s16x8 __attribute__((ext_vector_type(8)));
+    const s16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+    return __builtin_bit_cast(bf16x8, __builtin_elementwise_max(__builtin_bit_cast(s16x8, v), zero));
+}
+__device__ __forceinline__ f32x4 relu_frag(f32x4 v) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = v[e] > 0.f ? v[e] : 0.f;
+    return v;
+}
+
+// OPMODE 0: plain operands.  1: A in pieces along K (p.segA) with optional relu on its fragments (NT layout, three
+// stages, direct loads).  2: relu on the fragments of op(B) (TN layout: the weight gradient whose B operand is the
+// activation that a relu produced).  The other segment kinds (B, C and the mask along N) only move this block's base
+// pointers and leading dimensions, which costs nothing, so they need no instantiation of their own.
+template <typename TI, typename TO, int BM, int BN, int WAVES_M, int WAVES_N, bool A_KMAJOR, bool B_KMAJOR, int NSTAGES, int OPMODE = 0>
 // the four-wave 128 x 128 tile is meant to run two blocks per CU: keep it within 256 registers
 __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, ((WAVES_M * WAVES_N <= 4 && BM * BN <= 128 * 128) ? 2 : 1)) void gemm_kernel(GemmParams p) {
     constexpr int THREADS = WAVES_M * WAVES_N * 64;
@@ -115,11 +143,29 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, ((WAVES_M * WAVES_N <= 4 && 
         if (rmask) rmask += z1 * p.sC1 + z2 * p.sC2;
     }
 
-    // accumulate reads the old values `old_delta` bytes from where the result goes (0: in place)
-    const int64_t old_delta = p.addend ? (int64_t)((const char *)p.addend - (const char *)C) : 0;
-
     const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
     const int64_t m_left = p.M - m0, n_left = p.N - n0;
+
+    // B, C and the relu mask may exist as pieces along N (no tile straddles a piece): take this block's piece and
+    // address it as if it were the whole matrix (base moved back by the piece's first column)
+    int64_t ldb = p.ldb, ldc = p.ldc;
+    if (p.segB.n > 0) {
+        int s = 0;
+        while (s + 1 < p.segB.n && n0 >= p.segB.begin[s + 1]) ++s;
+        const void *base = p.n_list > 0 ? p.listSegB[(int)blockIdx.z][s] : p.segB.base[s];
+        B = (const TI *)base - p.segB.begin[s];
+        ldb = p.segB.ld[s];
+    }
+    if (p.segC.n > 0) {
+        int s = 0;
+        while (s + 1 < p.segC.n && n0 >= p.segC.begin[s + 1]) ++s;
+        C = (TO *)const_cast<void *>(p.segC.base[s]) - p.segC.begin[s];
+        ldc = p.segC.ld[s];
+        if (p.segM.n > 0) rmask = (const TO *)p.segM.base[s] - p.segC.begin[s];
+    }
+
+    // accumulate reads the old values `old_delta` bytes from where the result goes (0: in place)
+    const int64_t old_delta = p.addend ? (int64_t)((const char *)p.addend - (const char *)C) : 0;
 
     const int nk_total = (int)((p.K + BK - 1) / BK);
     const int kt0 = (int)blockIdx.y * p.ktiles_per_split;
@@ -127,9 +173,9 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, ((WAVES_M * WAVES_N <= 4 && 
     if (kt0 >= kt1) return;                                       // uniform for the whole block
 
     const TI *a_base = A_KMAJOR ? A + m0 * p.lda : A + m0;     // element (m0, k=0)
-    const TI *b_base = B_KMAJOR ? B + n0 * p.ldb : B + n0;
+    const TI *b_base = B_KMAJOR ? B + n0 * ldb : B + n0;
     const int64_t a_kstep = A_KMAJOR ? (int64_t)BK : (int64_t)BK * p.lda;
-    const int64_t b_kstep = B_KMAJOR ? (int64_t)BK : (int64_t)BK * p.ldb;
+    const int64_t b_kstep = B_KMAJOR ? (int64_t)BK : (int64_t)BK * ldb;
 
     // bf16 operands stored [k][row] stay that way in LDS and are transposed by the fragment reads
     constexpr bool A_TR = !A_KMAJOR && sizeof(TI) == 2, B_TR = !B_KMAJOR && sizeof(TI) == 2;
@@ -180,6 +226,18 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, ((WAVES_M * WAVES_N <= 4 && 
                 if constexpr (B_TR) fb[j].v = TrB::read_frag(bs, b_off[j], ks);
                 else fb[j] = *(const Vec16<TI> *)(bs + (b_off[j] ^ (ks << 5)));
             }
+            if constexpr (OPMODE == 1) {
+                if (p.a_relu) {
+#pragma unroll
+                    for (int i = 0; i < TM; ++i) fa[i].v = relu_frag(fa[i].v);
+                }
+            }
+            if constexpr (OPMODE == 2) {
+                if (p.b_relu) {
+#pragma unroll
+                    for (int j = 0; j < TN; ++j) fb[j].v = relu_frag(fb[j].v);
+                }
+            }
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -218,7 +276,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, ((WAVES_M * WAVES_N <= 4 && 
         kt_end = kt1 - 1;
         const int64_t k_left = p.K - (int64_t)kt_end * BK;
         la.load(a_base + (int64_t)kt_end * a_kstep, p.lda, m_left, k_left);
-        lb.load(b_base + (int64_t)kt_end * b_kstep, p.ldb, n_left, k_left);
+        lb.load(b_base + (int64_t)kt_end * b_kstep, ldb, n_left, k_left);
         if (do_rs && kt_end % p.tiles_n == tn) rs_add();
         la.store(As);
         lb.store(Bs);
@@ -234,13 +292,25 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, ((WAVES_M * WAVES_N <= 4 && 
         constexpr bool A_DIRECT = A_KMAJOR || A_TR, B_DIRECT = B_KMAJOR || B_TR;
         if constexpr (A_DIRECT) la.init_direct(p.lda, m_left);
         else la.init_offsets(p.lda, m_left);
-        if constexpr (B_DIRECT) lb.init_direct(p.ldb, n_left);
-        else lb.init_offsets(p.ldb, n_left);
+        if constexpr (B_DIRECT) lb.init_direct(ldb, n_left);
+        else lb.init_offsets(ldb, n_left);
+        // A in pieces along K: k-tiles are issued in increasing order, so the piece index only moves forward
+        int seg_a = 0;
         auto issue_tile = [&](int kt, int buf) {
-            if constexpr (A_DIRECT) la.load_direct(a_base + (int64_t)kt * a_kstep, As + buf * A_BYTES);
+            if constexpr (OPMODE == 1) {
+                if (p.segA.n > 0) {
+                    const int k = kt * BK;
+                    while (seg_a + 1 < p.segA.n && k >= p.segA.begin[seg_a + 1]) ++seg_a;
+                    const int64_t ld = p.segA.ld[seg_a];
+                    la.load_direct_ld((const TI *)p.segA.base[seg_a] + m0 * ld + (k - p.segA.begin[seg_a]), (int)ld,
+                                      As + buf * A_BYTES);
+                } else {
+                    la.load_direct(a_base + (int64_t)kt * a_kstep, As + buf * A_BYTES);
+                }
+            } else if constexpr (A_DIRECT) la.load_direct(a_base + (int64_t)kt * a_kstep, As + buf * A_BYTES);
             else la.load_fast(a_base + (int64_t)kt * a_kstep, p.lda);
             if constexpr (B_DIRECT) lb.load_direct(b_base + (int64_t)kt * b_kstep, Bs + buf * B_BYTES);
-            else lb.load_fast(b_base + (int64_t)kt * b_kstep, p.ldb);
+            else lb.load_fast(b_base + (int64_t)kt * b_kstep, ldb);
         };
         auto commit_tile = [&](int buf, int kt) {
             if (do_rs && kt % p.tiles_n == tn) rs_add();
@@ -254,6 +324,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, ((WAVES_M * WAVES_N <= 4 && 
             // Both operands go global -> LDS directly (no registers involved); a wave's loads complete in order,
             // so tile kt has landed once at most the loads of tile kt + 1 are outstanding.
             static_assert(A_DIRECT && B_DIRECT, "three stages need direct loads for both operands");
+            static_assert(OPMODE != 1 || (A_KMAJOR && sizeof(TI) == 2), "A in pieces: bf16, stored [M, K]");
             constexpr int LPT = decltype(la)::LOADS_PER_TILE + decltype(lb)::LOADS_PER_TILE;
             static_assert(LPT < 64, "vmcnt holds 6 bits");
             constexpr int WAIT_NEXT = (LPT & 15) | 0x0F70 | ((LPT >> 4) << 14);
@@ -272,6 +343,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, ((WAVES_M * WAVES_N <= 4 && 
             }
             __syncthreads();
         } else {
+        static_assert(OPMODE != 1, "A in pieces needs the three-stage loop");
         issue_tile(kt0, 0);
         commit_tile(0, kt0);
         __syncthreads();
@@ -385,7 +457,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, ((WAVES_M * WAVES_N <= 4 && 
     // bf16 output that is neither accumulated into nor a split-K partial: the band is staged as bf16 (half the
     // LDS traffic) and leaves in 16-byte stores.  Needs 16-byte alignment of C, its leading dimension and the
     // tile's column origin.
-    if (sizeof(TO) == 2 && !split && !p.accumulate && (p.ldc & 7) == 0 && ((uintptr_t)C & 15) == 0) {
+    if (sizeof(TO) == 2 && !split && !p.accumulate && (ldc & 7) == 0 && ((uintptr_t)C & 15) == 0) {
         constexpr int SROWH = WTN * 2 + 16;
         constexpr int G16 = WTN / 8;
         constexpr int NG = 32 * G16 / 64;
@@ -397,7 +469,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, ((WAVES_M * WAVES_N <= 4 && 
         for (int g = 0; g < NG; ++g) {
             const int gidx = g * 64 + lane, row = gidx / G16, gc = gidx % G16;
             soff[g] = row * SROWH + gc * 16;
-            goff[g] = row * (int)p.ldc + gc * 8;
+            goff[g] = row * (int)ldc + gc * 8;
         }
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
@@ -410,8 +482,8 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, ((WAVES_M * WAVES_N <= 4 && 
                     for (int e = 0; e < 4; ++e) o[e] = (bf16_t)acc[i][j][q * 4 + e];
                     *(bf16x4 *)(stage + (lane & 31) * SROWH + (j * 32 + q * 8 + (lane >> 5) * 4) * 2) = o;
                 }
-            bf16_t *band = (bf16_t *)C + (m0 + wm + i * 32) * p.ldc + n0 + wn;
-            const bf16_t *mband = rmask ? (const bf16_t *)rmask + (m0 + wm + i * 32) * p.ldc + n0 + wn : nullptr;
+            bf16_t *band = (bf16_t *)C + (m0 + wm + i * 32) * ldc + n0 + wn;
+            const bf16_t *mband = rmask ? (const bf16_t *)rmask + (m0 + wm + i * 32) * ldc + n0 + wn : nullptr;
             if (interior && mband) {
                 // the producer of this operand's gradient applied relu itself: its output is the mask
 #pragma unroll
@@ -459,7 +531,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, ((WAVES_M * WAVES_N <= 4 && 
     constexpr int NQ = 32 * QPR / 64;
     static_assert((32 * QPR) % 64 == 0, "wave tile width must be a multiple of 8");
     typedef TO out4_t __attribute__((ext_vector_type(4)));
-    const bool fast = interior && (p.ldc & 3) == 0;
+    const bool fast = interior && (ldc & 3) == 0;
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
 #pragma unroll
@@ -476,7 +548,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, ((WAVES_M * WAVES_N <= 4 && 
         // up in split order and applies activation / accumulation.
         const int64_t mb = m0 + wm + i * 32, nb = n0 + wn;
         if (fast) {
-            TO *band = C + mb * p.ldc + nb;
+            TO *band = C + mb * ldc + nb;
             float *wband = split ? p.ws + ((int64_t)blockIdx.y * p.M + mb) * p.ws_ld + nb : nullptr;
 #pragma unroll
             for (int g = 0; g < NQ; ++g) {
@@ -486,9 +558,9 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, ((WAVES_M * WAVES_N <= 4 && 
                     *(f32x4 *)(wband + row * (int)p.ws_ld + qc * 4) = v;
                     continue;
                 }
-                TO *dst = band + row * (int)p.ldc + qc * 4;
+                TO *dst = band + row * (int)ldc + qc * 4;
                 if (rmask) {
-                    const out4_t mk = *(const out4_t *)(rmask + (mb + row) * p.ldc + nb + qc * 4);
+                    const out4_t mk = *(const out4_t *)(rmask + (mb + row) * ldc + nb + qc * 4);
 #pragma unroll
                     for (int e = 0; e < 4; ++e) v[e] = (float)mk[e] > 0.f ? v[e] : 0.f;
                 }
@@ -516,15 +588,15 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, ((WAVES_M * WAVES_N <= 4 && 
                 *(f32x4 *)(p.ws + ((int64_t)blockIdx.y * p.M + m) * p.ws_ld + n) = v;
                 continue;
             }
-            TO *dst = C + m * p.ldc + n;
+            TO *dst = C + m * ldc + n;
             f32x4 vm = v;
             if (rmask) {
-                const TO *mk = rmask + m * p.ldc + n;
+                const TO *mk = rmask + m * ldc + n;
 #pragma unroll
                 for (int e = 0; e < 4; ++e)
                     if (n + e < p.N && !((float)mk[e] > 0.f)) vm[e] = 0.f;
             }
-            if (n + 4 <= p.N && ((p.ldc & 3) == 0)) {
+            if (n + 4 <= p.N && ((ldc & 3) == 0)) {
                 f32x4 x = vm;
                 if (p.accumulate) {
                     const out4_t old = *(const out4_t *)((const char *)dst + old_delta);
@@ -556,9 +628,10 @@ int launch_cfg(const GemmParams &p, int transA, int transB, int64_t batch, hipSt
     q.tiles_n = (int)hapmi_cdiv(p.N, BN);
     dim3 grid((unsigned)(q.tiles_m * q.tiles_n), (unsigned)q.splits, (unsigned)batch), block(WM * WN * 64);
     const size_t smem = (size_t)NSTAGES * (BM + BN) * ROW_BYTES;
-#define HAPMI_GEMM_LAUNCH(AK, BK_)                                                                        \
+#define HAPMI_GEMM_LAUNCH(AK, BK_) HAPMI_GEMM_LAUNCH_MODE(AK, BK_, 0)
+#define HAPMI_GEMM_LAUNCH_MODE(AK, BK_, MODE)                                                             \
     do {                                                                                                  \
-        auto kern = gemm_kernel<TI, TO, BM, BN, WM, WN, AK, BK_, NSTAGES>;                                       \
+        auto kern = gemm_kernel<TI, TO, BM, BN, WM, WN, AK, BK_, NSTAGES, MODE>;                                 \
         if (smem > 64 * 1024) {                                                                           \
             static bool raised = false;                                                                   \
             if (!raised) {                                                                                \
@@ -570,11 +643,29 @@ int launch_cfg(const GemmParams &p, int transA, int transB, int64_t batch, hipSt
         }                                                                                                 \
         hipLaunchKernelGGL(kern, grid, block, smem, st, q);                                               \
     } while (0)
+    if constexpr (sizeof(TI) == 2) {
+        // operand modes (A in pieces along K / relu on an operand): own instantiations of the layouts that use them
+        if (p.segA.n > 0 || p.a_relu) {
+            if constexpr (NSTAGES == 3) {
+                if (transA || !transB) return hapmi_set_error(HAPMI_EINVAL, "gemm: A_segments / a_relu need transA = 0, transB = 1");
+                HAPMI_GEMM_LAUNCH_MODE(true, true, 1);
+                return HAPMI_OK;
+            } else {
+                return hapmi_set_error(HAPMI_EINVAL, "gemm: A_segments / a_relu need a three-stage tile configuration");
+            }
+        }
+        if (p.b_relu) {
+            if (!transA || transB) return hapmi_set_error(HAPMI_EINVAL, "gemm: b_relu needs transA = 1, transB = 0");
+            HAPMI_GEMM_LAUNCH_MODE(false, false, 2);
+            return HAPMI_OK;
+        }
+    }
     if (!transA && transB) HAPMI_GEMM_LAUNCH(true, true);
     else if (!transA && !transB) HAPMI_GEMM_LAUNCH(true, false);
     else if (transA && !transB) HAPMI_GEMM_LAUNCH(false, false);
     else HAPMI_GEMM_LAUNCH(false, true);
 #undef HAPMI_GEMM_LAUNCH
+#undef HAPMI_GEMM_LAUNCH_MODE
     return HAPMI_OK;
 }
 

@@ -73,6 +73,8 @@ template <typename TI, int ROWS, int THREADS, bool KMAJOR> struct TileLoader {
             const int row = (p * NWAVES + wave) * 8 + (lane >> 3);
             const int chunk = (lane & 7) ^ swz(row);
             doff[p] = (row < last ? row : last) * (int)ld + chunk * EPV;
+            drow[p] = row < last ? row : last;
+            dchunk[p] = chunk * EPV;
         }
     }
 
@@ -86,6 +88,23 @@ template <typename TI, int ROWS, int THREADS, bool KMAJOR> struct TileLoader {
         for (int p = 0; p < PASSES_D; ++p) {
             const uint32_t lds_addr = (uint32_t)(uintptr_t)(lds_char *)(lds + (p * NWAVES + wave) * 8 * ROW_BYTES);
             const TI *src = base + doff[p];
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                         :
+                         : "s"(lds_addr), "v"(src)
+                         : "memory");
+        }
+    }
+
+    // the same transfer with the leading dimension given per call (an operand that exists in pieces with different
+    // leading dimensions); rows are clamped as in init_direct
+    int drow[KMAJOR ? (PASSES_D > 0 ? PASSES_D : 1) : 1], dchunk[KMAJOR ? (PASSES_D > 0 ? PASSES_D : 1) : 1];
+    __device__ __forceinline__ void load_direct_ld(const TI *base, int ld, char *lds) const {
+        typedef __attribute__((address_space(3))) char lds_char;
+        const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+#pragma unroll
+        for (int p = 0; p < PASSES_D; ++p) {
+            const uint32_t lds_addr = (uint32_t)(uintptr_t)(lds_char *)(lds + (p * NWAVES + wave) * 8 * ROW_BYTES);
+            const TI *src = base + drow[p] * ld + dchunk[p];
             asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
                          :
                          : "s"(lds_addr), "v"(src)

@@ -13,7 +13,7 @@ from typing import List, Optional, Sequence
 import torch
 
 from . import _lib
-from ._lib import ACT_GELU, ACT_NONE, ACT_RELU, BF16, F32, GemmArgs, check, lib
+from ._lib import ACT_GELU, ACT_NONE, ACT_RELU, BF16, F32, GemmArgs, GemmSegments, check, lib
 
 _ACT = {None: ACT_NONE, "none": ACT_NONE, "relu": ACT_RELU, "gelu": ACT_GELU}
 
@@ -309,17 +309,48 @@ def _workspace(device) -> torch.Tensor:
     return _gemm_ws
 
 
-def gemm(A: torch.Tensor, B: torch.Tensor, C: torch.Tensor, M: int, N: int, K: int, *, transA=False, transB=False,
+def _segments(pieces: Sequence[torch.Tensor], rows: int, what: str) -> GemmSegments:
+    """Description of an operand / result that exists as pieces along its column dimension: every piece a 2-d view
+    [rows, len] with unit column stride (its row stride is the piece's leading dimension)."""
+    if not 1 <= len(pieces) <= _lib.GEMM_MAX_SEGMENTS:
+        raise ValueError(f"{what}: 1..{_lib.GEMM_MAX_SEGMENTS} pieces expected")
+    g = GemmSegments()
+    g.n = len(pieces)
+    pos = 0
+    for i, t in enumerate(pieces):
+        _dev(t)
+        if t.dim() != 2 or t.shape[0] != rows or t.stride(1) != 1 or t.dtype != pieces[0].dtype:
+            raise ValueError(f"{what}: piece {i} must be a [rows, len] view with unit column stride of one element type")
+        g.begin[i] = pos
+        g.ld[i] = t.stride(0) if rows > 1 else max(t.stride(0), t.shape[1])
+        g.base[i] = t.data_ptr()
+        # a piece may be a view into a larger buffer: the bound is the storage behind the view's first element
+        room = t.untyped_storage().nbytes() // t.element_size() - t.storage_offset()
+        if _span(rows, t.shape[1], int(g.ld[i])) > room:
+            raise _lib.HapmiError(f"{what}: piece {i} reaches beyond its storage")
+        pos += t.shape[1]
+    g.begin[len(pieces)] = pos
+    return g
+
+
+def gemm(A: Optional[torch.Tensor], B: Optional[torch.Tensor], C: Optional[torch.Tensor], M: int, N: int, K: int, *, transA=False, transB=False,
          lda=None, ldb=None, ldc=None, bias: Optional[torch.Tensor] = None, accumulate=False, act=None, alpha=1.0,
          batch1=1, batch2=1, strideA=(0, 0), strideB=(0, 0), strideC=(0, 0),
          offA=0, offB=0, offC=0, workspace: Optional[torch.Tensor] = None,
          a_rowsum: Optional[torch.Tensor] = None, relu_mask: Optional[torch.Tensor] = None,
-         addend: Optional[torch.Tensor] = None):
+         addend: Optional[torch.Tensor] = None, a_segments=None, b_segments=None, c_segments=None,
+         mask_segments=None, a_relu=False, b_relu=False):
     """C = alpha * op(A) @ op(B) (+bias)(act)(+C).  Offsets and strides are in elements.  ``workspace`` (or
     the buffer installed with ``set_gemm_workspace``) lets the library split a long reduction over K.
     ``a_rowsum`` (float32[M], transA only): the sums over k of op(A)'s rows are added into it.
     ``relu_mask`` ([M, ldc] like C): result elements whose mask is <= 0 are zero (relu backward).
-    ``addend`` ([M, ldc] like C, with ``accumulate``): C = addend + result; C itself is only written."""
+    ``addend`` ([M, ldc] like C, with ``accumulate``): C = addend + result; C itself is only written.
+    ``a_segments`` / ``b_segments`` / ``c_segments`` / ``mask_segments``: the operand / result / relu mask as a list
+    of pieces along K (A, stored [M, K]) or N (B stored [K, N], C, mask) instead of one tensor (pass None for it);
+    ``a_relu`` / ``b_relu``: relu applied to that operand as it is loaded."""
+    if a_segments is not None or b_segments is not None or c_segments is not None or a_relu or b_relu:
+        return _gemm_segmented(A, B, C, M, N, K, transA, transB, lda, ldb, ldc, bias, act, alpha, workspace, a_rowsum,
+                               a_segments, b_segments, c_segments, mask_segments, a_relu, b_relu, accumulate)
     _dev(A, B, C, bias, a_rowsum, relu_mask, addend)
     if A.dtype != B.dtype:
         raise TypeError("gemm operands must share a dtype")
@@ -378,14 +409,96 @@ def gemm(A: torch.Tensor, B: torch.Tensor, C: torch.Tensor, M: int, N: int, K: i
     return C
 
 
+def _gemm_segmented(A, B, C, M, N, K, transA, transB, lda, ldb, ldc, bias, act, alpha, workspace, a_rowsum,
+                    a_segments, b_segments, c_segments, mask_segments, a_relu, b_relu, accumulate):
+    """The forms of ``gemm`` with an operand or the result in pieces (one problem, bf16 operands)."""
+    _dev(A, B, C, bias, a_rowsum)
+    a = GemmArgs()
+    keep = []
+    first = lambda *ts: next(t for t in ts if t is not None)
+    in_t = first(A, a_segments[0] if a_segments else None, B, b_segments[0] if b_segments else None)
+    out_t = first(C, c_segments[0] if c_segments else None)
+    epv = 16 // in_t.element_size()
+    up = lambda n: (n + epv - 1) // epv * epv
+    a.M, a.N, a.K = M, N, K
+    a.lda = lda if lda is not None else (M if transA else K)
+    a.ldb = ldb if ldb is not None else (K if transB else N)
+    a.ldc = ldc if ldc is not None else N
+    a.transA, a.transB = int(transA), int(transB)
+    a.in_dtype, a.out_dtype = dtype_code(in_t), dtype_code(out_t)
+    a.accumulate, a.act, a.alpha = int(accumulate), _ACT[act], float(alpha)
+    a.batch1 = a.batch2 = 1
+    if a_segments is not None:
+        g = _segments(a_segments, M, "gemm a_segments")
+        if int(g.begin[g.n]) != K:
+            raise ValueError("gemm a_segments: the pieces must add up to K")
+        keep.append(g)
+        a.A_segments = ctypes.addressof(g)
+    else:
+        _need(A, _span(K if transA else M, up(M) if transA else K, a.lda), "gemm A")
+        a.A = A.data_ptr()
+    if b_segments is not None:
+        g = _segments(b_segments, K, "gemm b_segments")
+        if int(g.begin[g.n]) != N:
+            raise ValueError("gemm b_segments: the pieces must add up to N")
+        keep.append(g)
+        a.B_segments = ctypes.addressof(g)
+    else:
+        _need(B, _span(N if transB else K, K if transB else up(N), a.ldb), "gemm B")
+        a.B = B.data_ptr()
+    if c_segments is not None:
+        g = _segments(c_segments, M, "gemm c_segments")
+        if int(g.begin[g.n]) != N:
+            raise ValueError("gemm c_segments: the pieces must add up to N")
+        keep.append(g)
+        a.C_segments = ctypes.addressof(g)
+        if mask_segments is not None:
+            gm = _segments(mask_segments, M, "gemm mask_segments")
+            keep.append(gm)
+            a.c_mask_segments = ctypes.addressof(gm)
+    else:
+        _need(C, _span(M, N, a.ldc), "gemm C")
+        a.C = C.data_ptr()
+    a.a_relu, a.b_relu = int(bool(a_relu)), int(bool(b_relu))
+    if bias is not None:
+        if bias.dtype != torch.float32:
+            raise TypeError("gemm bias must be float32")
+        _need(bias, N, "gemm bias")
+        a.bias = bias.data_ptr()
+    if a_rowsum is not None:
+        if a_rowsum.dtype != torch.float32 or not transA:
+            raise TypeError("gemm a_rowsum: float32 vector and transA expected")
+        _need(a_rowsum, M, "gemm a_rowsum")
+        a.a_rowsum = a_rowsum.data_ptr()
+    ws = workspace if workspace is not None else _gemm_ws
+    if ws is None and a_rowsum is not None:
+        ws = _workspace(in_t.device)
+    if ws is not None and ws.is_cuda:
+        a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel() * ws.element_size()
+    a._keep = tuple(keep)                              # the argument block points into these host structures
+    if _gemm_log is not None:
+        _gemm_log.append((a, (A, B, C, bias, a_segments, b_segments, c_segments, mask_segments)))
+    check(lib().hapmi_gemm(ctypes.byref(a), _stream()))
+    return C
+
+
 def gemm_group(As: Sequence[torch.Tensor], Bs: Sequence[torch.Tensor], Cs: Sequence[torch.Tensor], M: int, N: int,
                K: int, *, transA=False, transB=False, lda=None, ldb=None, ldc=None, accumulate=False, alpha=1.0,
-               a_rowsums: Optional[Sequence[Optional[torch.Tensor]]] = None):
+               a_rowsums: Optional[Sequence[Optional[torch.Tensor]]] = None, b_relu=False):
     """``Cs[z] = alpha * op(As[z]) @ op(Bs[z]) (+ Cs[z])`` for up to 16 problems of one shape in one launch
-    (pointer lists of the C ABI; no K split).  ``a_rowsums[z]`` as ``a_rowsum`` of ``gemm``."""
+    (pointer lists of the C ABI; no K split).  ``a_rowsums[z]`` as ``a_rowsum`` of ``gemm``.  An entry of ``Bs`` may
+    be a list of pieces along N (``b_segments`` of ``gemm``; then every entry must be, with equal piece shapes);
+    ``b_relu``: relu applied to op(B) as it is loaded."""
     n = len(As)
     if not (1 <= n <= _lib.GEMM_MAX_LIST and len(Bs) == n and len(Cs) == n and (a_rowsums is None or len(a_rowsums) == n)):
         raise ValueError(f"gemm_group: 1..{_lib.GEMM_MAX_LIST} problems with one entry per list expected")
+    pieces = isinstance(Bs[0], (list, tuple))
+    seg_structs = None
+    if pieces:
+        if not all(isinstance(b, (list, tuple)) for b in Bs) or transB:
+            raise ValueError("gemm_group: either every B is a list of pieces (transB = False) or none")
+        seg_structs = [_segments(b, K, "gemm_group b_segments") for b in Bs]
+        Bs = [b[0] for b in Bs]                           # stands for the operand in the checks below
     _dev(*As, *Bs, *Cs, *(a_rowsums or ()))
     a = GemmArgs()
     a.M, a.N, a.K = M, N, K
@@ -402,7 +515,8 @@ def gemm_group(As: Sequence[torch.Tensor], Bs: Sequence[torch.Tensor], Cs: Seque
         if A.dtype != As[0].dtype or B.dtype != As[0].dtype or C.dtype != Cs[0].dtype:
             raise TypeError("gemm_group: every problem must have the element types of the first")
         _need(A, _span(K if transA else M, up(M) if transA else K, a.lda), "gemm_group A")
-        _need(B, _span(N if transB else K, K if transB else up(N), a.ldb), "gemm_group B")
+        if not pieces:
+            _need(B, _span(N if transB else K, K if transB else up(N), a.ldb), "gemm_group B")
         _need(C, _span(M, N, a.ldc), "gemm_group C")
     for r in a_rowsums or ():
         if r is not None:
@@ -415,6 +529,13 @@ def gemm_group(As: Sequence[torch.Tensor], Bs: Sequence[torch.Tensor], Cs: Seque
     a.A_list, a.B_list, a.C_list = ctypes.addressof(la), ctypes.addressof(lb), ctypes.addressof(lc)
     a.a_rowsum_list = ctypes.addressof(lr) if lr is not None else 0
     a._keep = (la, lb, lc, lr)                       # the argument block points into these host arrays
+    a.b_relu = int(bool(b_relu))
+    if seg_structs is not None:
+        if any(int(g.begin[g.n]) != N for g in seg_structs):
+            raise ValueError("gemm_group b_segments: the pieces must add up to N")
+        ls = (ctypes.c_void_p * n)(*[ctypes.addressof(g) for g in seg_structs])
+        a.B_segments_list = ctypes.addressof(ls)
+        a._keep = a._keep + (ls, tuple(seg_structs))
     if lr is not None:
         ws = _workspace(As[0].device)                  # partial row sums
         a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel() * ws.element_size()

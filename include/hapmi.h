@@ -135,6 +135,18 @@ int hapmi_ragged_tuning(int reduce_variant, int grid_shift);
  * op(B) is [K,N]: transB=0 -> B stored [K,N] (ldb), transB=1 -> B stored [N,K].
  * z = z1 * batch2 + z2 addresses X + z1*strideX1 + z2*strideX2 (elements).
  * Accumulation is float32; in/out element types are given separately. */
+/* An operand or result that exists as SEGMENTS along one of its dimensions instead of as one matrix: the pieces an
+ * all_to_all delivers, which collectives.py:159 / :166 would first concatenate (torch.cat) into one tensor.
+ * Segment s covers the index range [begin[s], begin[s + 1]) of the segmented dimension and is a row-major matrix
+ * [rows, begin[s + 1] - begin[s]] at base[s] with leading dimension ld[s]; begin[0] = 0, begin[n] = the full extent. */
+#define HAPMI_GEMM_MAX_SEGMENTS 8
+typedef struct {
+    int n;                                           /* 1 .. HAPMI_GEMM_MAX_SEGMENTS */
+    int64_t begin[HAPMI_GEMM_MAX_SEGMENTS + 1];
+    int64_t ld[HAPMI_GEMM_MAX_SEGMENTS];
+    const void *base[HAPMI_GEMM_MAX_SEGMENTS];
+} hapmi_gemm_segments;
+
 typedef struct {
     const void *A, *B;
     void *C;
@@ -174,6 +186,22 @@ typedef struct {
     const void *const *A_list, *const *B_list;
     void *const *C_list;
     float *const *a_rowsum_list;
+    /* Segmented operands (bf16 operands, NULL = off).  They let the linear behind an all_to_all (hap.rs:2713-2744,
+     * then F.relu hap.rs:1417, then F.linear hap.rs:1032) read the received pieces where they were received, with
+     * relu applied as the operand is loaded, and let its backward write the pieces of the backward all_to_all
+     * directly, so no concatenating / splitting copy runs on either side:
+     *   A_segments    A stored [M, K] (transA = 0) in pieces along K (begin: multiples of 64; K a multiple of 64,
+     *                 transB = 1, batch 1, no split); A itself is ignored.  The forward of that linear.
+     *   B_segments    B stored [K, N] (transB = 0) in pieces along N; B is ignored.  With pointer lists,
+     *                 B_segments_list[z] describes problem z (all with the same n, begin and ld).  Its weight gradient.
+     *   C_segments    C in pieces along N; C is ignored; c_mask_segments: c_relu_mask in pieces with the same n,
+     *                 begin and ld (piece s of the mask has the layout of piece s of the result).  No accumulate / c_addend.  Its data gradient, written as the backward pieces.
+     *   a_relu / b_relu   max(., 0) applied to op(A) (with A_segments) / op(B) (with transA = 1, transB = 0) on load.
+     * A block tile must not straddle a piece: the tile configuration is chosen among those whose N extent divides
+     * every begin of B_segments / C_segments (HAPMI_EINVAL if none does). */
+    const hapmi_gemm_segments *A_segments, *B_segments, *C_segments, *c_mask_segments;
+    const hapmi_gemm_segments *const *B_segments_list;
+    int a_relu, b_relu;
 } hapmi_gemm_args;
 #define HAPMI_GEMM_MAX_LIST 16
 int hapmi_gemm(const hapmi_gemm_args *args_host, hapmi_stream_t stream);

@@ -617,3 +617,110 @@ def test_reductions_give_the_same_bits_every_time(cuda):
         torch.testing.assert_close(got[0][4].double(), 1 + dys[2].double().sum(0).cpu(), rtol=1e-5, atol=1e-3)
         for u, v in zip(got[0], got[1]):
             assert torch.equal(u, v)
+
+
+def _pieces(full, lengths, cuda, wide_first=True):
+    """Split a [rows, sum(lengths)] CPU tensor into GPU pieces: the first a row-range view of a wider, taller
+    tensor (its leading dimension differs from its length, as the own piece of an all_to_all does), the others
+    contiguous tensors of their own."""
+    out, pos = [], 0
+    for i, l in enumerate(lengths):
+        part = full[:, pos:pos + l]
+        if i == 0 and wide_first:
+            host = torch.full((full.shape[0] + 5, l + 16), float("nan"), dtype=full.dtype)
+            host[3:3 + full.shape[0], :l] = part
+            out.append(host.to(cuda)[3:3 + full.shape[0], :l])
+        else:
+            out.append(part.contiguous().to(cuda))
+        pos += l
+    return out
+
+
+@pytest.mark.parametrize("cfg", [-1, 5, 6, 7, 8, 9])
+def test_gemm_a_in_pieces_along_k_with_relu(cuda, cfg):
+    """The linear behind an all_to_all + relu reads the received pieces in place: A = relu(cat(pieces, dim 1))."""
+    from hap_amd._lib import lib
+    g = torch.Generator().manual_seed(31 + cfg)
+    M, N, lengths = 300, 200, [384, 384, 128, 128]
+    K = sum(lengths)
+    act = torch.randn(M, K, generator=g).bfloat16()
+    W = torch.randn(N, K, generator=g).bfloat16()
+    bias = torch.randn(N, generator=g)
+    pieces = _pieces(act, lengths, cuda)
+    try:
+        lib().hapmi_gemm_tuning(cfg, 1)
+        for relu in (True, False):
+            src = torch.relu(act.double()) if relu else act.double()
+            want = src @ W.double().t() + bias.double()
+            C = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=cuda)
+            ops.gemm(None, W.to(cuda), C, M, N, K, transB=True, bias=bias.to(cuda), a_segments=pieces, a_relu=relu)
+            close(C, want, torch.bfloat16, scale=2.0)
+        # relu on a plain operand
+        C = torch.full((M, N), float("nan"), dtype=torch.float32, device=cuda)
+        ops.gemm(act.to(cuda), W.to(cuda), C, M, N, K, transB=True, a_relu=True)
+        close(C, torch.relu(act.double()) @ W.double().t(), torch.bfloat16, scale=2.0)
+    finally:
+        lib().hapmi_gemm_tuning(-1, 0)
+
+
+@pytest.mark.parametrize("cfg,lengths", [(-1, [384, 384, 128, 128]), (0, [384, 384, 128, 128]), (7, [384, 384, 128, 128]),
+                                         (8, [256, 128, 640]), (1, [768, 256]), (3, [768, 256]), (4, [384, 576]),
+                                         (9, [384, 576]), (6, [512, 512])])
+def test_gemm_result_and_operand_in_pieces_along_n(cuda, cfg, lengths):
+    """Backward of that linear: the data gradient dY W written as the pieces of the backward all_to_all, masked with
+    relu's derivative taken from the forward pieces; the weight gradient dY^T relu(cat(pieces)) with its bias
+    gradient, alone and for several layers in one launch."""
+    from hap_amd._lib import lib
+    g = torch.Generator().manual_seed(41 + max(cfg, 0))
+    rows, d_out = 300, 200
+    F_ = sum(lengths)
+    pre = torch.randn(rows, F_, generator=g).bfloat16()                 # the forward pieces (pre-activation)
+    dy = torch.randn(rows, d_out, generator=g).bfloat16()
+    W = torch.randn(d_out, F_, generator=g).bfloat16()                  # second linear's weight [d_out, F]
+    fwd_pieces = _pieces(pre, lengths, cuda)
+    want_dx = (dy.double() @ W.double()) * (pre.double() > 0)
+    # the result's pieces have the layout of the forward pieces (the mask is read at the result's addresses)
+    outs = _pieces(torch.full((rows, F_), float("nan"), dtype=torch.bfloat16), lengths, cuda)
+    try:
+        lib().hapmi_gemm_tuning(cfg, 1)
+        ops.gemm(dy.to(cuda), W.to(cuda), None, rows, F_, d_out, c_segments=outs, mask_segments=fwd_pieces)
+        close(torch.cat(outs, 1), want_dx, torch.bfloat16, scale=2.0)
+        outs2 = [torch.full((rows, l), float("nan"), dtype=torch.bfloat16, device=cuda) for l in lengths]
+        ops.gemm(dy.to(cuda), W.to(cuda), None, rows, F_, d_out, c_segments=outs2)
+        close(torch.cat(outs2, 1), dy.double() @ W.double(), torch.bfloat16, scale=2.0)
+        # weight gradient [d_out, F] = dY^T relu(pre), bias gradient = column sums of dY
+        want_dw = dy.double().t() @ torch.relu(pre.double())
+        gw = torch.full((d_out, F_), float("nan"), device=cuda)
+        gb = torch.zeros(d_out, device=cuda)
+        ops.gemm(dy.to(cuda), None, gw, d_out, F_, rows, transA=True, b_segments=fwd_pieces, b_relu=True, a_rowsum=gb)
+        close(gw, want_dw, torch.bfloat16, scale=2.0)
+        torch.testing.assert_close(gb.cpu().double(), dy.double().sum(0), rtol=1e-4, atol=1e-3)
+        # three layers in one launch
+        pres = [torch.randn(rows, F_, generator=g).bfloat16() for _ in range(3)]
+        dys = [torch.randn(rows, d_out, generator=g).bfloat16() for _ in range(3)]
+        gws = [torch.full((d_out, F_), float("nan"), device=cuda) for _ in range(3)]
+        ops.gemm_group([t.to(cuda) for t in dys], [_pieces(t, lengths, cuda) for t in pres],
+                       gws, d_out, F_, rows, transA=True, b_relu=True)
+        for z in range(3):
+            close(gws[z], dys[z].double().t() @ torch.relu(pres[z].double()), torch.bfloat16, scale=2.0)
+    finally:
+        lib().hapmi_gemm_tuning(-1, 0)
+
+
+def test_gemm_pieces_are_checked(cuda):
+    from hap_amd._lib import HapmiError
+    x = torch.zeros(64, 96, dtype=torch.bfloat16, device=cuda)
+    y = torch.zeros(64, 160, dtype=torch.bfloat16, device=cuda)
+    W = torch.zeros(32, 256, dtype=torch.bfloat16, device=cuda)
+    C = torch.zeros(64, 32, dtype=torch.bfloat16, device=cuda)
+    with pytest.raises(HapmiError, match="multiple of 64"):            # a piece boundary inside a k-tile
+        ops.gemm(None, W, C, 64, 32, 256, transB=True, a_segments=[x, y])
+    outs = [torch.zeros(64, 96, dtype=torch.bfloat16, device=cuda), torch.zeros(64, 160, dtype=torch.bfloat16, device=cuda)]
+    with pytest.raises(HapmiError, match="multiple of 64"):
+        ops.gemm(C, torch.zeros(32, 256, dtype=torch.bfloat16, device=cuda), None, 64, 256, 32, c_segments=outs)
+    with pytest.raises(ValueError, match="add up"):
+        ops.gemm(None, W, C, 64, 32, 256, transB=True, a_segments=[y])
+    f = torch.zeros(64, 128, device=cuda)
+    with pytest.raises(HapmiError, match="bf16"):
+        ops.gemm(None, torch.zeros(32, 256, device=cuda), torch.zeros(64, 32, device=cuda), 64, 32, 256, transB=True,
+                 a_segments=[f, f])
