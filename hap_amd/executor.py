@@ -62,7 +62,7 @@ class ShardExecutor:
                  overlap_wgrad: bool = False, launch_lists: bool = True, relu_mask_in_dgrad: bool = True,
                  overlap_optimizer: bool = False, optimizer_chunk_min: int = 1 << 20,
                  relu_bwd_in_split: bool = True, wgrad_group: int = 8, receive_in_place: bool = True,
-                 dropout_seed: int = 0):
+                 dropout_seed: int = 0, exchange_in_pieces: bool = True):
         """``example_inputs``: the program's inputs (global batch) as tensors or shapes; activations are
         sized from them.  ``rank`` / ``world_size`` are only needed by all_reduce / replicate, whose node
         forms do not carry them (collectives.py:86, 182)."""
@@ -106,6 +106,11 @@ class ShardExecutor:
         # contiguous row range of the result, so it is received there (Wire.recv(into=...)) instead of into a
         # buffer of its own that a copy kernel then moves; False keeps the copy
         self.receive_in_place = receive_in_place
+        # all_to_all -> relu -> linear (the column-sharded FFN, bf16): the linear reads the exchanged pieces where
+        # they were received (relu applied as the operand is loaded) and its backward writes the pieces of the backward
+        # exchange directly, so neither the concatenating copy forward nor the splitting copy backward runs; False
+        # keeps the copies (which then carry the relu), for comparison
+        self.exchange_in_pieces = exchange_in_pieces
         # Optional: train_step() applies the optimizer to each stretch of the flat parameter buffer as soon as
         # backward has finished with it, on a second stream.  Measured on the BERT-large shard the step takes the
         # same time either way (27.1 against 27.0 ms): the GEMMs that run next to the update slow down by what the
@@ -270,18 +275,25 @@ class ShardExecutor:
     def _is_read_later(self, t: Optional[torch.Tensor]) -> bool:
         return t is not None and self._deferred_reads.get(t.untyped_storage().data_ptr(), 0) > 0
 
-    def _emit_wgrad(self, dy, xt, gw, gb, n_out, n_in, rows, ld_dy, ld_x, acc, params):
+    def _emit_wgrad(self, dy, xt, gw, gb, n_out, n_in, rows, ld_dy, ld_x, acc, params, x_relu=False):
         """dW[n_out, n_in] (+)= dy[rows, n_out]^T x[rows, n_in], the bias gradient gb (column sums of dy) taken by
         the same kernel.  Launched at once, or held back to share a launch with the same linear of the next
-        layers (only for parameters with a single use: their gradient is written once, order does not matter)."""
+        layers (only for parameters with a single use: their gradient is written once, order does not matter).
+        ``xt`` may be a list of pieces [rows, len] along n_in (with ``x_relu``: relu applied as they are loaded)."""
+        pieces = isinstance(xt, (list, tuple))
         if not self._holds_back_wgrad(params):
-            self.bwd.append(lambda: ops.gemm(dy, xt, gw, n_out, n_in, rows, transA=True, lda=ld_dy, ldb=ld_x,
-                                             accumulate=acc, a_rowsum=gb))
+            if pieces:
+                self.bwd.append(lambda: ops.gemm(dy, None, gw, n_out, n_in, rows, transA=True, lda=ld_dy, accumulate=acc,
+                                                 a_rowsum=gb, b_segments=list(xt), b_relu=x_relu))
+            else:
+                self.bwd.append(lambda: ops.gemm(dy, xt, gw, n_out, n_in, rows, transA=True, lda=ld_dy, ldb=ld_x,
+                                                 accumulate=acc, a_rowsum=gb))
             return
-        sig = (n_out, n_in, rows, ld_dy, ld_x, bool(acc), dy.dtype, gw.dtype)
+        layout = tuple((t.shape[1], t.stride(0)) for t in xt) if pieces else None
+        sig = (n_out, n_in, rows, ld_dy, ld_x, bool(acc), dy.dtype, gw.dtype, layout, bool(x_relu))
         q = self._pending_wgrads.setdefault(sig, [])
         q.append((dy, xt, gw, gb, [v.meta.get("name") or v.meta.get("shard_of") for v in params if v is not None], []))
-        for t in (dy, xt):
+        for t in (dy,) + (tuple(xt) if pieces else (xt,)):
             k = t.untyped_storage().data_ptr()
             self._deferred_reads[k] = self._deferred_reads.get(k, 0) + 1
         if len(q) >= self.wgrad_group:
@@ -301,9 +313,9 @@ class ShardExecutor:
                 continue
             n_out, n_in, rows, ld_dy, ld_x, acc = key[:6]
             for dy, xt, _, _, _, _ in q:
-                for t in (dy, xt):
+                for t in (dy,) + (tuple(xt) if isinstance(xt, (list, tuple)) else (xt,)):
                     self._deferred_reads[t.untyped_storage().data_ptr()] -= 1
-            self.bwd.append(self._wgrad_launch(q, n_out, n_in, rows, ld_dy, ld_x, acc))
+            self.bwd.append(self._wgrad_launch(q, n_out, n_in, rows, ld_dy, ld_x, acc, key[9]))
             for e in q:
                 for hook in e[5]:
                     hook()                               # launches that wait for this weight gradient
@@ -323,15 +335,19 @@ class ShardExecutor:
         fn()
 
     @staticmethod
-    def _wgrad_launch(q, n_out, n_in, rows, ld_dy, ld_x, acc):
+    def _wgrad_launch(q, n_out, n_in, rows, ld_dy, ld_x, acc, x_relu=False):
+        pieces = isinstance(q[0][1], (list, tuple))
         if len(q) == 1:
             dy, xt, gw, gb = q[0][:4]
+            if pieces:
+                return lambda: ops.gemm(dy, None, gw, n_out, n_in, rows, transA=True, lda=ld_dy, accumulate=acc, a_rowsum=gb,
+                                        b_segments=list(xt), b_relu=x_relu)
             return lambda: ops.gemm(dy, xt, gw, n_out, n_in, rows, transA=True, lda=ld_dy, ldb=ld_x, accumulate=acc,
                                     a_rowsum=gb)
         dys, xts, gws = [e[0] for e in q], [e[1] for e in q], [e[2] for e in q]
         gbs = [e[3] for e in q] if any(e[3] is not None for e in q) else None
-        return lambda: ops.gemm_group(dys, xts, gws, n_out, n_in, rows, transA=True, lda=ld_dy, ldb=ld_x,
-                                      accumulate=acc, a_rowsums=gbs)
+        return lambda: ops.gemm_group(dys, xts, gws, n_out, n_in, rows, transA=True, lda=ld_dy, ldb=None if pieces else ld_x,
+                                      accumulate=acc, a_rowsums=gbs, b_relu=x_relu)
 
     def _param_grad_slot(self, v: Val):
         if self._touched is not None and v.meta.get("name") is not None:
@@ -723,10 +739,41 @@ class ShardExecutor:
         return out
 
     # ---- linear ---------------------------------------------------------------------------------
+    def _linear_on_pieces(self, node, x: Val, w: Val, b: Optional[Val]):
+        """F.linear whose input is relu(cat(pieces)) of an all_to_all (kind 'pieces'): forward reads the pieces as
+        they lie, the weight gradient does the same, and the data gradient is written, masked with relu's derivative,
+        as the pieces of the backward all_to_all."""
+        pieces = x.meta["pieces2d"]
+        lead = tuple(x.shape[:-1])
+        N, K = w.t.shape
+        M = pieces[0].shape[0]
+        store = self._new(lead + (N,))
+        out = Val("tensor", store, needs_grad=True)
+        bias = b.meta["master"] if b is not None else None
+        relu = bool(x.meta["relu"])
+        self.fwd.append(lambda: ops.gemm(None, w.t, store, M, N, K, transB=True, bias=bias, a_segments=pieces, a_relu=relu))
+
+        def emit():
+            if out.grad is None:
+                return
+            dy = out.grad
+            gw, accw = self._param_grad_slot(w)
+            gb, accb = self._param_grad_slot(b) if b is not None else (None, False)
+            self._emit_wgrad(dy, list(pieces), gw, gb, N, K, M, N, K, accw, (w, b), x_relu=relu)
+            if x.needs_grad:
+                back, finish = x.meta["backward_exchange"]()
+                mask = pieces if relu else None
+                self.bwd.append(lambda: ops.gemm(dy, w.t, None, M, K, N, c_segments=back, mask_segments=mask))
+                finish()
+        self._tape.append(emit)
+        return out
+
     def _linear(self, node):
         x, w, b = self._val(node.args[0]), self._val(node.args[1]), self._val(node.args[2])
         if w.kind != "param" or (b is not None and b.kind != "param"):
             self._unsupported(node, "weight and bias must be parameters")
+        if x.kind == "pieces":
+            return self._linear_on_pieces(node, x, w, b)
         if x.kind == "cls_view":
             xt, lda, lead = x.meta["src"].t, x.meta["row_stride"], (x.meta["src"].t.shape[0],)
         elif x.t is not None:
@@ -794,6 +841,11 @@ class ShardExecutor:
         kind = "relu" if node.target is F.relu else "gelu"
         if node.target is F.gelu and (len(node.args) > 1 or node.kwargs.get("approximate", "none") != "none"):
             self._unsupported(node, "only the erf form of gelu is implemented")
+        if x.kind == "pieces":
+            if kind != "relu" or x.meta["relu"]:
+                self._unsupported(node, "only one relu is applied to the pieces of an exchange")
+            x.meta["relu"] = True                       # applied by the consuming linear as it loads the pieces
+            return x
         if x.meta.get("fused_act") == kind:
             return x                                    # already applied by the producer
         if x.t is None or x.ld is not None:
@@ -1278,15 +1330,18 @@ class ShardExecutor:
         return out
 
     def _emit_exchange(self, tag, direction, x_t, split_dim, cat_dim, split_L, cat_L, rank, sink, act=None,
-                       relu_of=None, receive_in_place=False):
+                       relu_of=None, receive_in_place=False, presplit=False):
         """The local half of an all_to_all.  ``act``: activation applied while concatenating.  ``relu_of``: forward
         output of a relu whose backward is applied to ``x_t`` while splitting (only for a split that copies).
         ``receive_in_place`` (concatenation along dim 0, no activation): the peers' pieces are received straight
-        into their rows of the result, which nothing may write afterwards; no concat launch is left."""
+        into their rows of the result, which nothing may write afterwards; no concat launch is left.
+        ``presplit``: ``x_t`` is only a shape (a meta tensor); the caller writes the pieces itself (a GEMM whose result
+        is laid out in pieces).  Returns (result, pieces, finish): nothing is launched until ``finish()`` appends
+        what is left of the exchange (the concat, the wire's send hooks)."""
         W = len(split_L)
         # pieces along the slowest dimension are contiguous ranges of the input: views, as torch.split gives the
         # reference (collectives.py:156); any other dimension needs the strided copy
-        views = split_dim == 0 and x_t.is_contiguous()
+        views = split_dim == 0 and not presplit and x_t.is_contiguous()
         own_shape = ops._with_dim(x_t.shape, split_dim, split_L[rank])
         out = self._new(ops._with_dim(own_shape, cat_dim, sum(cat_L)))
         if views:
@@ -1308,13 +1363,71 @@ class ShardExecutor:
                     into = out.narrow(0, sum(cat_L[:src]), cat_L[src])
                     self._wire_backed.add(out.untyped_storage().data_ptr())
                 parts.append(self.wire.recv(tag, direction, src, shape, self.cdt, self.dev, reduction=False, into=into))
-        if views:
-            sink.append(lambda: ops.concat_rows(parts, cat_dim, out, act))
-        else:
-            sink.append(lambda: (ops.split_rows(x_t, split_L, split_dim, pieces, relu_of=relu_of),
-                                 ops.concat_rows(parts, cat_dim, out, act)))
-        self._announce(tag, direction, rank, W, lambda dst: pieces[dst], sink)
+
+        def finish():
+            if views or presplit:
+                sink.append(lambda: ops.concat_rows(parts, cat_dim, out, act))
+            else:
+                sink.append(lambda: (ops.split_rows(x_t, split_L, split_dim, pieces, relu_of=relu_of),
+                                     ops.concat_rows(parts, cat_dim, out, act)))
+            self._announce(tag, direction, rank, W, lambda dst: pieces[dst], sink)
+        if presplit:
+            return out, pieces, finish
+        finish()
         return out
+
+    def _exchange_in_pieces(self, node, x: Val, sd, cd, sL, cL, rank):
+        """all_to_all whose result only feeds relu -> linear: nothing is copied.  The value is the list of pieces
+        (this rank's own rows of the input, the peers' messages where the wire delivered them); the linear reads
+        them in place, and its backward writes the pieces of the backward exchange."""
+        W = len(sL)
+        x_t = x.t
+        pieces = list(torch.split(x_t, list(sL), 0))
+        own = pieces[rank]
+        parts = []
+        for src in range(W):
+            shape = ops._with_dim(own.shape, cd, cL[src])
+            parts.append(own if src == rank else
+                         self.wire.recv(node.name, "fwd", src, shape, self.cdt, self.dev, reduction=False))
+        self._announce(node.name, "fwd", rank, W, lambda dst: pieces[dst], self.fwd)
+        live = [t for t, l in zip(parts, cL) if l > 0]
+        out = Val("pieces", None, shape=ops._with_dim(own.shape, cd, sum(cL)), needs_grad=x.needs_grad, relu=False,
+                  pieces=parts, pieces2d=[t.reshape(-1, t.shape[-1]) for t in live])
+
+        def backward_exchange():
+            # the gradient [own rows, sum(cL)] never exists as one tensor: the linear's data-gradient GEMM writes it
+            # as the pieces of the backward exchange (split along cd by cL, concatenated along sd by sL)
+            shape = torch.empty(out.shape, device="meta")
+            # the result is d(x); when x is a linear's output that only this exchange reads, d(x) is read by that
+            # linear's two gradient GEMMs and written by nobody: the peers' pieces can be received in place
+            producer = node.args[0]
+            in_place = (self.receive_in_place and x.grad is None and isinstance(producer, torch.fx.Node)
+                        and producer.target is F.linear and len(producer.users) == 1 and not x.meta.get("fused_act"))
+            g, back, finish = self._emit_exchange(node.name, "bwd", shape, cd, sd, cL, sL, rank, self.bwd,
+                                                  receive_in_place=in_place, presplit=True)
+
+            def done():
+                finish()
+                self._accumulate_into(x, g)
+            return [t.reshape(-1, t.shape[-1]) for t, l in zip(back, cL) if l > 0], done
+        out.meta["backward_exchange"] = backward_exchange
+        return out
+
+    def _feeds_only_relu_linear(self, node) -> bool:
+        """node -> F.relu -> [F.dropout(p = 0)]* -> F.linear (as its input), every link the only user."""
+        users = list(node.users)
+        if len(users) != 1 or users[0].target is not F.relu:
+            return False
+        n = users[0]
+        while True:
+            users = list(n.users)
+            if len(users) != 1:
+                return False
+            u = users[0]
+            if u.target is F.dropout and float(u.args[1]) == 0.0 and u.args[0] is n:
+                n = u
+                continue
+            return u.target is F.linear and u.args[0] is n and u.args[1] is not n and u.args[2] is not n
 
     @staticmethod
     def _split_can_mask(grad, fwd_out, dim, lengths):
@@ -1333,6 +1446,13 @@ class ShardExecutor:
         sL, cL, rank = list(node.args[3]), list(node.args[4]), node.args[5]
         if x.t is None or x.ld is not None:
             self._unsupported(node, f"all_to_all of a {x.kind} value")
+        # piece boundaries: multiples of 64 for the k-tiles of the forward GEMM and of 128, the narrowest bf16 tile,
+        # for the N tiles of the two backward GEMMs
+        bounds = [sum(cL[:i]) for i in range(1, len(cL))]
+        if (self.exchange_in_pieces and self.dtype == "bf16" and sd == 0 and cd == x.t.dim() - 1 and x.t.is_contiguous()
+                and self._feeds_only_relu_linear(node) and all(v % 128 == 0 for v in bounds) and sum(cL) % 64 == 0
+                and sum(1 for l in cL if l > 0) <= ops._lib.GEMM_MAX_SEGMENTS and sL[rank] > 0 and x.t.shape[-1] % 8 == 0):
+            return self._exchange_in_pieces(node, x, sd, cd, sL, cL, rank)
         fuse = self._wants_fused_relu(node)
         t = self._emit_exchange(node.name, "fwd", x.t, sd, cd, sL, cL, rank, self.fwd, "relu" if fuse else None)
         out = Val("tensor", t, needs_grad=x.needs_grad)
@@ -1743,7 +1863,8 @@ class ShardExecutor:
         flush = torch.zeros(512 << 20, dtype=torch.int8, device=self.dev)
         seen, report = set(), []
         for a, keep in log:
-            key = (a.M, a.N, a.K, a.batch1 * a.batch2, a.transA, a.transB, a.in_dtype, a.out_dtype)
+            key = (a.M, a.N, a.K, a.batch1 * a.batch2, a.transA, a.transB, a.in_dtype, a.out_dtype,
+                   bool(a.A_segments), bool(a.B_segments or a.B_segments_list), bool(a.C_segments), a.a_relu, a.b_relu)
             if key in seen:
                 continue
             seen.add(key)

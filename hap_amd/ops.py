@@ -549,6 +549,8 @@ _gemm_log = None
 _SPLIT_MENU = (1, 2, 3, 4, 5, 6, 7, 8, 10, 12, 16)
 _BF16_TILE_CONFIGS = tuple(range(10))
 _F32_TILE_CONFIGS = (0, 10, 11)
+_THREE_STAGE_CONFIGS = (5, 6, 7, 8, 9)
+_TILE_N = {0: 128, 1: 256, 2: 192, 3: 256, 4: 192, 5: 128, 6: 256, 7: 128, 8: 128, 9: 192, 10: 64, 11: 128}
 
 
 def record_gemms(on: bool):
@@ -570,10 +572,25 @@ def autotune_gemm(a: "GemmArgs", flush: Optional[torch.Tensor] = None, repeats: 
     nk = -(-a.K // (64 if bf16_in else 32))
     per_split = a.M * ((a.N + 3) // 4 * 4) * 4
     max_splits = a.workspace_bytes // per_split if (a.workspace and per_split) else 0
+    # calls with an operand or the result in pieces: three-stage configurations only for A in pieces / relu on A,
+    # tiles whose N extent divides every piece boundary for B / C in pieces, and no K split
+    need3 = bool(a.A_segments) or bool(a.a_relu)
+    n_align = 0
+    seg_ptrs = [a.B_segments, a.C_segments]
+    if a.B_segments_list:
+        seg_ptrs.append(ctypes.cast(a.B_segments_list, ctypes.POINTER(ctypes.c_void_p))[0])
+    for ptr in seg_ptrs:
+        if ptr:
+            g = ctypes.cast(ptr, ctypes.POINTER(GemmSegments)).contents
+            for i in range(1, g.n):
+                n_align = math.gcd(n_align, int(g.begin[i]))
+    segmented = need3 or any(seg_ptrs)
     cands = []
     for cfg in (_BF16_TILE_CONFIGS if bf16_in else _F32_TILE_CONFIGS):
+        if (need3 and cfg not in _THREE_STAGE_CONFIGS) or (n_align and n_align % _TILE_N[cfg]):
+            continue
         for s in _SPLIT_MENU:
-            if s > 1 and (s > max_splits or batch != 1 or nk // s < 4):
+            if s > 1 and (segmented or s > max_splits or batch != 1 or nk // s < 4):
                 continue
             cands.append((cfg, s))
     stream = _stream()

@@ -84,7 +84,8 @@ def _masks_from_oracle(ex, step):
             n = shape[0] * shape[1] * shape[2] * shape[3]
             out[node.name] = ref.dropout_keep(seed, step, i, p, n).view(shape)[..., :S]
         elif node.target is F.relu:
-            out[node.name] = (ex.env[node].t > 0).cpu()
+            v = ex.env[node]
+            out[node.name] = (torch.cat([t > 0 for t in v.meta["pieces"]], dim=-1) if v.kind == "pieces" else v.t > 0).cpu()
             continue
         else:
             continue

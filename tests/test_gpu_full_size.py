@@ -79,6 +79,9 @@ def _gpu_decisions(ex):
             continue
         if node.target is F.relu:
             v = ex.env[node]
+            if v.kind == "pieces":                                            # an exchange read in place: relu on load
+                decisions[node.name] = torch.cat([t > 0 for t in v.meta["pieces"]], dim=-1).cpu()
+                continue
             act = v.t.permute(1, 0, 2, 3) if v.kind == "expert" else v.t      # experts are stored expert-major
             decisions[node.name] = (act > 0).cpu()
         elif node.target is models.top_2_gating:
