@@ -58,7 +58,8 @@ struct ProfState {
     std::mutex mu;
     bool on = false;
     std::vector<hipEvent_t> pool;
-    std::vector<std::pair<hipEvent_t, hipEvent_t>> pending;
+    struct Bracket { hipEvent_t e0, e1, e2; };
+    std::vector<Bracket> pending;
     double flops = 0.0;
     int64_t launches = 0;
 };
@@ -413,6 +414,13 @@ extern "C" int hapmi_gemm(const hapmi_gemm_args *a, hapmi_stream_t stream) {
         HAPMI_REQUIRE(!a->transA && a->transB && batch == 1 && a->K % 64 == 0 && !a->a_rowsum, HAPMI_EINVAL,
                       "gemm: A_segments / a_relu need transA = 0, transB = 1, one problem and K a multiple of 64");
         need.three_stage = true;
+        if (p.segA.n == 0) {                                   // relu on a plain A: it travels as one piece
+            p.segA.n = 1;
+            p.segA.begin[0] = 0;
+            p.segA.begin[1] = (int)a->K;
+            p.segA.ld[0] = a->lda;
+            p.segA.base[0] = a->A;
+        }
     }
     HAPMI_REQUIRE(!p.b_relu || (a->transA && !a->transB), HAPMI_EINVAL, "gemm: b_relu needs transA = 1, transB = 0");
     const hapmi_gemm_segments *bseg = a->B_segments;
@@ -456,7 +464,7 @@ extern "C" int hapmi_gemm(const hapmi_gemm_args *a, hapmi_stream_t stream) {
     }
 
     hipStream_t st = (hipStream_t)stream;
-    hipEvent_t e0 = nullptr, e1 = nullptr;
+    hipEvent_t e0 = nullptr, e1 = nullptr, e2 = nullptr;
     bool prof = false;
     {
         std::lock_guard<std::mutex> lk(g_prof.mu);
@@ -464,7 +472,8 @@ extern "C" int hapmi_gemm(const hapmi_gemm_args *a, hapmi_stream_t stream) {
         if (prof) {
             e0 = prof_event();
             e1 = prof_event();
-            prof = e0 && e1;
+            e2 = prof_event();
+            prof = e0 && e1 && e2;
         }
     }
     if (prof) (void)hipEventRecord(e0, st);
@@ -475,8 +484,9 @@ extern "C" int hapmi_gemm(const hapmi_gemm_args *a, hapmi_stream_t stream) {
     else rc = launch_typed<float, bf16_t>(p, a->transA, a->transB, batch, st, false, a->workspace, a->workspace_bytes, need);
     if (prof) {
         (void)hipEventRecord(e1, st);
+        (void)hipEventRecord(e2, st);                 // an empty bracket right behind: what two event records cost by themselves
         std::lock_guard<std::mutex> lk(g_prof.mu);
-        g_prof.pending.emplace_back(e0, e1);
+        g_prof.pending.push_back(ProfState::Bracket{e0, e1, e2});
         g_prof.flops += 2.0 * (double)a->M * (double)a->N * (double)a->K * (double)batch;
         g_prof.launches += 1;
     }
@@ -515,20 +525,23 @@ extern "C" int hapmi_prof_gemm_enable(int on) {
     return HAPMI_OK;
 }
 
-extern "C" int hapmi_prof_gemm_collect(double *ms, int64_t *launches, double *flops) {
+extern "C" int hapmi_prof_gemm_collect(double *ms, int64_t *launches, double *flops, double *empty_ms) {
     std::lock_guard<std::mutex> lk(g_prof.mu);
-    double total = 0.0;
-    for (auto &pr : g_prof.pending) {
-        if (hipEventSynchronize(pr.second) != hipSuccess) return hapmi_set_error(HAPMI_ELAUNCH, "prof: event sync failed");
-        float t = 0.f;
-        if (hipEventElapsedTime(&t, pr.first, pr.second) != hipSuccess)
+    double total = 0.0, empty = 0.0;
+    for (auto &br : g_prof.pending) {
+        if (hipEventSynchronize(br.e2) != hipSuccess) return hapmi_set_error(HAPMI_ELAUNCH, "prof: event sync failed");
+        float t = 0.f, t0 = 0.f;
+        if (hipEventElapsedTime(&t, br.e0, br.e1) != hipSuccess || hipEventElapsedTime(&t0, br.e1, br.e2) != hipSuccess)
             return hapmi_set_error(HAPMI_ELAUNCH, "prof: elapsed time failed");
         total += t;
-        g_prof.pool.push_back(pr.first);
-        g_prof.pool.push_back(pr.second);
+        empty += t0;
+        g_prof.pool.push_back(br.e0);
+        g_prof.pool.push_back(br.e1);
+        g_prof.pool.push_back(br.e2);
     }
     g_prof.pending.clear();
     if (ms) *ms = total;
+    if (empty_ms) *empty_ms = empty;
     if (launches) *launches = g_prof.launches;
     if (flops) *flops = g_prof.flops;
     g_prof.flops = 0.0;

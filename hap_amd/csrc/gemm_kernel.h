@@ -91,10 +91,11 @@ __device__ __forceinline__ f32x4 relu_frag(f32x4 v) {
     return v;
 }
 
-// OPMODE 0: plain operands.  1: A in pieces along K (p.segA) with optional relu on its fragments (NT layout, three
-// stages, direct loads).  2: relu on the fragments of op(B) (TN layout: the weight gradient whose B operand is the
-// activation that a relu produced).  The other segment kinds (B, C and the mask along N) only move this block's base
-// pointers and leading dimensions, which costs nothing, so they need no instantiation of their own.
+// OPMODE bits (compile-time, so that the main loop of every instantiation is free of branches).  1: A is read in
+// pieces along K (p.segA; NT layout, three stages, direct loads; a plain A travels as one piece).  2: relu on the
+// fragments of op(A).  4: relu on the fragments of op(B) (TN layout: the weight gradient whose B operand is the
+// activation that a relu produced).  The other kinds of pieces (B, C and the mask along N) only move this block's
+// base pointers and leading dimensions, which costs nothing, so they need no instantiation of their own.
 template <typename TI, typename TO, int BM, int BN, int WAVES_M, int WAVES_N, bool A_KMAJOR, bool B_KMAJOR, int NSTAGES, int OPMODE = 0>
 // the four-wave 128 x 128 tile is meant to run two blocks per CU: keep it within 256 registers
 __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, ((WAVES_M * WAVES_N <= 4 && BM * BN <= 128 * 128) ? 2 : 1)) void gemm_kernel(GemmParams p) {
@@ -226,17 +227,13 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, ((WAVES_M * WAVES_N <= 4 && 
                 if constexpr (B_TR) fb[j].v = TrB::read_frag(bs, b_off[j], ks);
                 else fb[j] = *(const Vec16<TI> *)(bs + (b_off[j] ^ (ks << 5)));
             }
-            if constexpr (OPMODE == 1) {
-                if (p.a_relu) {
+            if constexpr ((OPMODE & 2) != 0) {
 #pragma unroll
-                    for (int i = 0; i < TM; ++i) fa[i].v = relu_frag(fa[i].v);
-                }
+                for (int i = 0; i < TM; ++i) fa[i].v = relu_frag(fa[i].v);
             }
-            if constexpr (OPMODE == 2) {
-                if (p.b_relu) {
+            if constexpr ((OPMODE & 4) != 0) {
 #pragma unroll
-                    for (int j = 0; j < TN; ++j) fb[j].v = relu_frag(fb[j].v);
-                }
+                for (int j = 0; j < TN; ++j) fb[j].v = relu_frag(fb[j].v);
             }
 #pragma unroll
             for (int i = 0; i < TM; ++i)
@@ -295,18 +292,21 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, ((WAVES_M * WAVES_N <= 4 && 
         if constexpr (B_DIRECT) lb.init_direct(ldb, n_left);
         else lb.init_offsets(ldb, n_left);
         // A in pieces along K: k-tiles are issued in increasing order, so the piece index only moves forward
-        int seg_a = 0;
+        // (the piece's base, end and the loader's row offsets are refreshed only when a k-tile enters the next piece:
+        // a few times per launch, not once per k-tile)
+        int seg_a = 0, seg_end = 0;
+        const TI *seg_base = nullptr;                             // element (m0, k = 0) as if the piece were all of A
         auto issue_tile = [&](int kt, int buf) {
-            if constexpr (OPMODE == 1) {
-                if (p.segA.n > 0) {
-                    const int k = kt * BK;
+            if constexpr ((OPMODE & 1) != 0) {
+                const int k = kt * BK;
+                if (k >= seg_end) {
                     while (seg_a + 1 < p.segA.n && k >= p.segA.begin[seg_a + 1]) ++seg_a;
                     const int64_t ld = p.segA.ld[seg_a];
-                    la.load_direct_ld((const TI *)p.segA.base[seg_a] + m0 * ld + (k - p.segA.begin[seg_a]), (int)ld,
-                                      As + buf * A_BYTES);
-                } else {
-                    la.load_direct(a_base + (int64_t)kt * a_kstep, As + buf * A_BYTES);
+                    la.set_ld((int)ld);
+                    seg_base = (const TI *)p.segA.base[seg_a] + m0 * ld - p.segA.begin[seg_a];
+                    seg_end = p.segA.begin[seg_a + 1];
                 }
+                la.load_direct(seg_base + k, As + buf * A_BYTES);
             } else if constexpr (A_DIRECT) la.load_direct(a_base + (int64_t)kt * a_kstep, As + buf * A_BYTES);
             else la.load_fast(a_base + (int64_t)kt * a_kstep, p.lda);
             if constexpr (B_DIRECT) lb.load_direct(b_base + (int64_t)kt * b_kstep, Bs + buf * B_BYTES);
@@ -324,7 +324,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, ((WAVES_M * WAVES_N <= 4 && 
             // Both operands go global -> LDS directly (no registers involved); a wave's loads complete in order,
             // so tile kt has landed once at most the loads of tile kt + 1 are outstanding.
             static_assert(A_DIRECT && B_DIRECT, "three stages need direct loads for both operands");
-            static_assert(OPMODE != 1 || (A_KMAJOR && sizeof(TI) == 2), "A in pieces: bf16, stored [M, K]");
+            static_assert((OPMODE & 1) == 0 || (A_KMAJOR && sizeof(TI) == 2), "A in pieces: bf16, stored [M, K]");
             constexpr int LPT = decltype(la)::LOADS_PER_TILE + decltype(lb)::LOADS_PER_TILE;
             static_assert(LPT < 64, "vmcnt holds 6 bits");
             constexpr int WAIT_NEXT = (LPT & 15) | 0x0F70 | ((LPT >> 4) << 14);
@@ -343,7 +343,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, ((WAVES_M * WAVES_N <= 4 && 
             }
             __syncthreads();
         } else {
-        static_assert(OPMODE != 1, "A in pieces needs the three-stage loop");
+        static_assert((OPMODE & 1) == 0, "A in pieces needs the three-stage loop");
         issue_tile(kt0, 0);
         commit_tile(0, kt0);
         __syncthreads();
@@ -409,6 +409,23 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, ((WAVES_M * WAVES_N <= 4 && 
     const bool interior = m_left >= BM && n_left >= BN;
     constexpr int NWAVES = WAVES_M * WAVES_N;
 
+    // The plain bf16 store path below masks the result with relu's derivative (rmask) one 32-row band at a time.  The
+    // mask of a band is fetched one band ahead (the first one here, before the accumulators are scaled and staged), so
+    // that its trip to memory overlaps the work on the band before instead of stalling every band's stores.
+    constexpr int MG16 = WTN / 8, MNG = 32 * MG16 / 64;
+    const bool bf16_rows = sizeof(TO) == 2 && !split && !p.accumulate && (ldc & 7) == 0 && ((uintptr_t)C & 15) == 0;
+    const bool mask_ahead = bf16_rows && interior && rmask != nullptr;
+    bf16x8 mask_v[2][MNG];
+    auto fetch_mask = [&](int i) {
+        const bf16_t *mband = (const bf16_t *)rmask + (m0 + wm + i * 32) * ldc + n0 + wn;
+#pragma unroll
+        for (int g = 0; g < MNG; ++g) {
+            const int gidx = g * 64 + lane;
+            mask_v[i & 1][g] = *(const bf16x8 *)(mband + (gidx / MG16) * (int)ldc + (gidx % MG16) * 8);
+        }
+    };
+    if (mask_ahead) fetch_mask(0);
+
     if (p.bias && lead) {
         const bool bias_vec = interior && ((uintptr_t)p.bias & 15) == 0;
 #pragma unroll
@@ -457,7 +474,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, ((WAVES_M * WAVES_N <= 4 && 
     // bf16 output that is neither accumulated into nor a split-K partial: the band is staged as bf16 (half the
     // LDS traffic) and leaves in 16-byte stores.  Needs 16-byte alignment of C, its leading dimension and the
     // tile's column origin.
-    if (sizeof(TO) == 2 && !split && !p.accumulate && (ldc & 7) == 0 && ((uintptr_t)C & 15) == 0) {
+    if (bf16_rows) {
         constexpr int SROWH = WTN * 2 + 16;
         constexpr int G16 = WTN / 8;
         constexpr int NG = 32 * G16 / 64;
@@ -486,10 +503,11 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, ((WAVES_M * WAVES_N <= 4 && 
             const bf16_t *mband = rmask ? (const bf16_t *)rmask + (m0 + wm + i * 32) * ldc + n0 + wn : nullptr;
             if (interior && mband) {
                 // the producer of this operand's gradient applied relu itself: its output is the mask
+                if (i + 1 < TM) fetch_mask(i + 1);
 #pragma unroll
                 for (int g = 0; g < NG; ++g) {
                     bf16x8 sv = *(const bf16x8 *)(stage + soff[g]);
-                    const bf16x8 mv = *(const bf16x8 *)(mband + goff[g]);
+                    const bf16x8 mv = mask_v[i & 1][g];
 #pragma unroll
                     for (int e = 0; e < 8; ++e) sv[e] = (float)mv[e] > 0.f ? sv[e] : (bf16_t)0.f;
                     *(bf16x8 *)(band + goff[g]) = sv;
@@ -645,10 +663,11 @@ int launch_cfg(const GemmParams &p, int transA, int transB, int64_t batch, hipSt
     } while (0)
     if constexpr (sizeof(TI) == 2) {
         // operand modes (A in pieces along K / relu on an operand): own instantiations of the layouts that use them
-        if (p.segA.n > 0 || p.a_relu) {
+        if (p.segA.n > 0) {
             if constexpr (NSTAGES == 3) {
                 if (transA || !transB) return hapmi_set_error(HAPMI_EINVAL, "gemm: A_segments / a_relu need transA = 0, transB = 1");
-                HAPMI_GEMM_LAUNCH_MODE(true, true, 1);
+                if (p.a_relu) HAPMI_GEMM_LAUNCH_MODE(true, true, 3);
+                else HAPMI_GEMM_LAUNCH_MODE(true, true, 1);
                 return HAPMI_OK;
             } else {
                 return hapmi_set_error(HAPMI_EINVAL, "gemm: A_segments / a_relu need a three-stage tile configuration");
@@ -656,7 +675,7 @@ int launch_cfg(const GemmParams &p, int transA, int transB, int64_t batch, hipSt
         }
         if (p.b_relu) {
             if (!transA || transB) return hapmi_set_error(HAPMI_EINVAL, "gemm: b_relu needs transA = 1, transB = 0");
-            HAPMI_GEMM_LAUNCH_MODE(false, false, 2);
+            HAPMI_GEMM_LAUNCH_MODE(false, false, 4);
             return HAPMI_OK;
         }
     }

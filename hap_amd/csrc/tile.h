@@ -95,21 +95,12 @@ template <typename TI, int ROWS, int THREADS, bool KMAJOR> struct TileLoader {
         }
     }
 
-    // the same transfer with the leading dimension given per call (an operand that exists in pieces with different
-    // leading dimensions); rows are clamped as in init_direct
+    // another leading dimension for the rows of init_direct (an operand that exists in pieces with different
+    // leading dimensions): the clamped row and the chunk of every pass are kept for that
     int drow[KMAJOR ? (PASSES_D > 0 ? PASSES_D : 1) : 1], dchunk[KMAJOR ? (PASSES_D > 0 ? PASSES_D : 1) : 1];
-    __device__ __forceinline__ void load_direct_ld(const TI *base, int ld, char *lds) const {
-        typedef __attribute__((address_space(3))) char lds_char;
-        const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    __device__ __forceinline__ void set_ld(int ld) {
 #pragma unroll
-        for (int p = 0; p < PASSES_D; ++p) {
-            const uint32_t lds_addr = (uint32_t)(uintptr_t)(lds_char *)(lds + (p * NWAVES + wave) * 8 * ROW_BYTES);
-            const TI *src = base + drow[p] * ld + dchunk[p];
-            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
-                         :
-                         : "s"(lds_addr), "v"(src)
-                         : "memory");
-        }
+        for (int p = 0; p < PASSES_D; ++p) doff[p] = drow[p] * ld + dchunk[p];
     }
 
     __device__ __forceinline__ void load_fast(const TI *base, int64_t ld) {

@@ -402,11 +402,12 @@ int hapmi_sumsq_static(const float *g, int64_t n, float *out, hapmi_stream_t str
 int hapmi_clip_coef(const float *sumsq, float max_norm, float *coef, hapmi_stream_t stream);
 
 /* ---- instrumentation ---------------------------------------------------
- * When enabled, every hapmi_gemm launch is bracketed by HIP events on its own
- * stream; hapmi_prof_gemm_collect synchronises those events and returns the
- * summed kernel time (ms), launch count and algorithmic FLOPs since enable. */
+ * When enabled, every hapmi_gemm call is bracketed by HIP events on its own stream, followed by an empty bracket
+ * (two event records with nothing between them).  hapmi_prof_gemm_collect synchronises those events and returns,
+ * since enable: the summed bracket time around the calls (ms), the summed time of the empty brackets (ms: what
+ * the event records themselves add to a bracket; NULL = not wanted), the call count and the algorithmic FLOPs. */
 int hapmi_prof_gemm_enable(int on);
-int hapmi_prof_gemm_collect(double *ms_host, int64_t *launches_host, double *flops_host);
+int hapmi_prof_gemm_collect(double *ms_host, int64_t *launches_host, double *flops_host, double *empty_ms_host);
 
 #ifdef __cplusplus
 }
