@@ -10,7 +10,7 @@ _PATH = os.path.join(_HERE, "libhapmi.so")
 _lib = None
 
 F32, BF16 = 0, 1
-ACT_NONE, ACT_RELU, ACT_GELU = 0, 1, 2
+ACT_NONE, ACT_RELU, ACT_GELU, ACT_SIGMOID = 0, 1, 2, 3
 MAX_RANKS = 64
 GEMM_MAX_LIST = 16
 

@@ -64,7 +64,13 @@ struct FRelu { __device__ float operator()(float x) const { return x > 0.f ? x :
 struct FGelu { __device__ float operator()(float x) const { return gelu_f(x); } };
 struct FReluBwd { __device__ float operator()(float dy, float y) const { return y > 0.f ? dy : 0.f; } };
 struct FGeluBwd { __device__ float operator()(float dy, float x) const { return dy * gelu_grad_f(x); } };
+struct FSigmoid { __device__ float operator()(float x) const { return 1.0f / (1.0f + __expf(-x)); } };
+struct FSigmoidBwd { __device__ float operator()(float dy, float y) const { return dy * y * (1.0f - y); } };
 struct FAdd { __device__ float operator()(float a, float b) const { return a + b; } };
+struct FConst {
+    float v;
+    __device__ float operator()(float) const { return v; }
+};
 struct FScale {
     float s;
     __device__ float operator()(float a) const { return a * s; }
@@ -105,16 +111,21 @@ int run_map2(const void *a, const void *b, void *o, int64_t n, int dtype, F f, h
 extern "C" int hapmi_act_fwd(const void *x, void *y, int64_t n, int act, int dtype, hapmi_stream_t stream) {
     if (act == HAPMI_ACT_RELU) return run_map1(x, y, n, dtype, FRelu(), (hipStream_t)stream, "act_fwd(relu)");
     if (act == HAPMI_ACT_GELU) return run_map1(x, y, n, dtype, FGelu(), (hipStream_t)stream, "act_fwd(gelu)");
+    if (act == HAPMI_ACT_SIGMOID) return run_map1(x, y, n, dtype, FSigmoid(), (hipStream_t)stream, "act_fwd(sigmoid)");
     return hapmi_set_error(HAPMI_EINVAL, "act_fwd: unknown activation %d", act);
 }
 extern "C" int hapmi_act_bwd(const void *dy, const void *ref, void *dx, int64_t n, int act, int dtype,
                              hapmi_stream_t stream) {
     if (act == HAPMI_ACT_RELU) return run_map2(dy, ref, dx, n, dtype, FReluBwd(), (hipStream_t)stream, "act_bwd(relu)");
     if (act == HAPMI_ACT_GELU) return run_map2(dy, ref, dx, n, dtype, FGeluBwd(), (hipStream_t)stream, "act_bwd(gelu)");
+    if (act == HAPMI_ACT_SIGMOID) return run_map2(dy, ref, dx, n, dtype, FSigmoidBwd(), (hipStream_t)stream, "act_bwd(sigmoid)");
     return hapmi_set_error(HAPMI_EINVAL, "act_bwd: unknown activation %d", act);
 }
 extern "C" int hapmi_add(const void *a, const void *b, void *out, int64_t n, int dtype, hapmi_stream_t stream) {
     return run_map2(a, b, out, n, dtype, FAdd(), (hipStream_t)stream, "add");
+}
+extern "C" int hapmi_fill_value(void *out, float value, int64_t n, int dtype, hapmi_stream_t stream) {
+    return run_map1(out, out, n, dtype, FConst{value}, (hipStream_t)stream, "fill_value");
 }
 extern "C" int hapmi_scale(const void *a, float s, void *out, int64_t n, int dtype, hapmi_stream_t stream) {
     return run_map1(a, out, n, dtype, FScale{s}, (hipStream_t)stream, "scale");

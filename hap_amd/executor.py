@@ -434,6 +434,7 @@ class ShardExecutor:
             torch.transpose: self._transpose, F.multi_head_attention_forward: self._mha,
             operator.getitem: self._getitem, F.dropout: self._dropout, F.layer_norm: self._layer_norm,
             F.linear: self._linear, F.relu: self._activation, F.gelu: self._activation,
+            torch.sigmoid: self._activation, torch.sum: self._sum,
             torch.log_softmax: self._log_softmax, F.nll_loss: self._nll_loss,
             F.conv2d: self._conv2d, torch.flatten: self._flatten,
             models.append_cls_token: self._append_cls, models.get_cls_token: self._get_cls,
@@ -454,9 +455,9 @@ class ShardExecutor:
                 if node.target != "split":
                     self._unsupported(node, "only Tensor.split is emitted for inputs")
                 src = self._val(node.args[0])
-                if src.kind != "input" or node.args[2] != 0:
-                    self._unsupported(node, "split is only supported on a program input along dim 0")
-                self.env[node] = Val("input_split", src=src, lengths=list(node.args[1]))
+                if src.kind != "input" or len(node.args) != 3:
+                    self._unsupported(node, "split(lengths, dim) is only supported on a program input")
+                self.env[node] = Val("input_split", src=src, lengths=list(node.args[1]), dim=int(node.args[2]))
             elif node.op == "call_function":
                 h = handlers.get(node.target)
                 if h is None:
@@ -468,7 +469,7 @@ class ShardExecutor:
             elif node.op == "output":
                 out = self._val(node.args[0])
                 if out.kind != "loss":
-                    self._unsupported(node, "the program output must be the nll_loss scalar")
+                    self._unsupported(node, "the program output must be the scalar of nll_loss or torch.sum")
                 self.loss = out.t
         # backward list: the tape in reverse.  For every parameter remember how many backward launches must have
         # been enqueued before nothing reads its value or writes its gradient any more (all of them are made by
@@ -510,7 +511,7 @@ class ShardExecutor:
         src, idx = self._val(node.args[0]), node.args[1]
         if src.kind == "input_split":
             L = src.meta["lengths"]
-            return Val("input_slice", src=src.meta["src"], offset=sum(L[:idx]), length=L[idx])
+            return Val("input_slice", src=src.meta["src"], offset=sum(L[:idx]), length=L[idx], dim=src.meta["dim"])
         if src.kind == "mha":
             if idx == 0:
                 return src.meta["out"]
@@ -542,12 +543,19 @@ class ShardExecutor:
             raise ValueError("expected a program input")
         src = v if v.kind == "input" else v.meta["src"]
         rec = self.inputs[src.meta["index"]]
+        full = self._example_inputs[src.meta["index"]]
+        off = v.meta.get("offset") if v.kind == "input_slice" else None
+        dim = v.meta.get("dim", 0) if v.kind == "input_slice" else 0
+        if dim < 0:
+            dim += full.dim()
+        length = v.meta.get("length") if v.kind == "input_slice" else full.shape[0]
         if rec["buf"] is None:
-            full = self._example_inputs[src.meta["index"]]
-            off = v.meta.get("offset") if v.kind == "input_slice" else None
-            length = v.meta.get("length") if v.kind == "input_slice" else full.shape[0]
-            rec.update(offset=off, length=length)
-            rec["buf"] = torch.empty((length,) + tuple(full.shape[1:]), dtype=dtype, device=self.dev)
+            rec.update(offset=off, length=length, dim=dim)
+            shape = list(full.shape)
+            shape[dim] = length
+            rec["buf"] = torch.empty(tuple(shape), dtype=dtype, device=self.dev)
+        elif (rec["offset"], rec["length"], rec.get("dim", 0)) != (off, length, dim) or rec["buf"].dtype != dtype:
+            raise ValueError(f"program input {rec['name']!r} is used as two different slices / types")
         return rec["buf"]
 
     def _mul(self, node):
@@ -774,6 +782,12 @@ class ShardExecutor:
             self._unsupported(node, "weight and bias must be parameters")
         if x.kind == "pieces":
             return self._linear_on_pieces(node, x, w, b)
+        if x.kind in ("input", "input_slice"):
+            # a floating-point program input used as an activation (the MLP models, models.py:19-24): its device
+            # buffer in the compute type; load_inputs converts
+            if "as_tensor" not in x.meta:
+                x.meta["as_tensor"] = Val("tensor", self._input_buffer(x, self.cdt), needs_grad=False)
+            x = x.meta["as_tensor"]
         if x.kind == "cls_view":
             xt, lda, lead = x.meta["src"].t, x.meta["row_stride"], (x.meta["src"].t.shape[0],)
         elif x.t is not None:
@@ -838,7 +852,9 @@ class ShardExecutor:
 
     def _activation(self, node):
         x = self._val(node.args[0])
-        kind = "relu" if node.target is F.relu else "gelu"
+        kind = "relu" if node.target is F.relu else ("sigmoid" if node.target is torch.sigmoid else "gelu")
+        if node.target is torch.sigmoid and (len(node.args) != 1 or node.kwargs):
+            self._unsupported(node, "the program emits torch.sigmoid(input) only")
         if node.target is F.gelu and (len(node.args) > 1 or node.kwargs.get("approximate", "none") != "none"):
             self._unsupported(node, "only the erf form of gelu is implemented")
         if x.kind == "pieces":
@@ -856,7 +872,7 @@ class ShardExecutor:
         def emit():
             if out.grad is None or not x.needs_grad:
                 return
-            ref = out.t if kind == "relu" else x.t
+            ref = x.t if kind == "gelu" else out.t      # relu and sigmoid differentiate through their output
             if x.grad is None:
                 x.grad = self._new(x.t.shape)
                 g = x.grad
@@ -1110,6 +1126,34 @@ class ShardExecutor:
             ops.sum_f32(row_loss, loss)
         self.fwd.append(forward)
         logits.grad = logits.t
+        return Val("loss", loss)
+
+    def _sum(self, node):
+        """torch.sum(input) (hap.rs:1133): the sum of all elements as the program's (partial) loss, the output of
+        the reference's MLP models (models.py:24).  Backward starts from d(input) = 1."""
+        if len(node.args) != 1 or node.kwargs:
+            self._unsupported(node, "the program emits torch.sum(input) only")
+        x = self._val(node.args[0])
+        if x.t is None or x.ld is not None:
+            self._unsupported(node, f"sum of a {x.kind} value")
+        if any(u.op != "output" for u in node.users):
+            self._unsupported(node, "torch.sum is supported as the program's output")
+        width = x.t.shape[-1]
+        rows = x.t.numel() // width
+        cols = self._new((width,), torch.float32)
+        loss = self._new((1,), torch.float32)
+        self.fwd.append(lambda: (ops.colsum(x.t, cols, rows, width), ops.sum_f32(cols, loss)))
+
+        def emit():
+            if not x.needs_grad:
+                return
+            g, acc = self._grad_slot(x)
+            if acc:
+                ones = self._new(x.t.shape)
+                self.bwd.append(lambda: (ops.fill_value(ones, 1.0), ops.add(g, ones, g)))
+            else:
+                self.bwd.append(lambda: ops.fill_value(g, 1.0))
+        self._tape.append(emit)
         return Val("loss", loss)
 
     # ---- ViT leaves -----------------------------------------------------------------------------
@@ -1659,7 +1703,7 @@ class ShardExecutor:
         for rec, a in zip(self.inputs, args):
             if rec["buf"] is None:
                 continue
-            src = a if rec["offset"] is None else a.narrow(0, rec["offset"], rec["length"])
+            src = a if rec["offset"] is None else a.narrow(rec.get("dim", 0), rec["offset"], rec["length"])
             rec["buf"].copy_(src, non_blocking=True)
 
     def refresh_shadow(self):

@@ -15,7 +15,7 @@ import torch
 from . import _lib
 from ._lib import ACT_GELU, ACT_NONE, ACT_RELU, BF16, F32, GemmArgs, GemmSegments, check, lib
 
-_ACT = {None: ACT_NONE, "none": ACT_NONE, "relu": ACT_RELU, "gelu": ACT_GELU}
+_ACT = {None: ACT_NONE, "none": ACT_NONE, "relu": ACT_RELU, "gelu": ACT_GELU, "sigmoid": _lib.ACT_SIGMOID}
 
 
 def dtype_code(t) -> int:
@@ -797,6 +797,13 @@ def sum_f32(x, out):
 # ---------------------------------------------------------------------------
 # elementwise
 # ---------------------------------------------------------------------------
+
+def fill_value(t, value: float):
+    _dev(t)
+    if not t.is_contiguous():
+        raise TypeError("fill_value: contiguous tensor expected")
+    check(lib().hapmi_fill_value(_ptr(t), ctypes.c_float(value), t.numel(), dtype_code(t), _stream()))
+
 
 def act_fwd(x, y, act):
     _dev(x, y)

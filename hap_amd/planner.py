@@ -164,7 +164,7 @@ def _call_shape(node, sh):
         return tuple(s[:start]) + (_prod(s[start:end + 1]),) + tuple(s[end + 1:])
     if t is torch.log_softmax:
         return sh(a[0])
-    if t is F.nll_loss:
+    if t in (F.nll_loss, torch.sum):
         return ()
     if t is models.append_cls_token:
         b, s, d = sh(a[0])
@@ -191,8 +191,8 @@ def _node_flops(node, sh) -> int:
         return 3 * _prod(sh(a[0]))
     if t is F.gelu:                                              # no handler in the reference: priced like relu
         return 3 * _prod(sh(a[0]))
-    if t in (torch.transpose, operator.add, operator.mul, torch.flatten, F.nll_loss):
-        return _prod(sh(a[0]))                                   # hap.rs:1216, 1518, 1566/1609, 1782, 1884
+    if t in (torch.transpose, operator.add, operator.mul, torch.flatten, F.nll_loss, torch.sum):
+        return _prod(sh(a[0]))                                   # hap.rs:1216, 1518, 1566/1609, 1782, 1884, 1136
     if t is F.multi_head_attention_forward:                      # hap.rs:1330-1337
         L, N, E = sh(kw["query"])
         S = sh(kw["key"])[0]

@@ -39,6 +39,16 @@ MoE layers        gating on replicated tokens, experts sharded over the
 ``zero=True``     on top of any of them: every parameter that would be
                   replicated is stored as a dim-0 shard (the reference's
                   ``extra_ps`` / force_zero mode).
+``shard_dim="sequence"``  (language models, ``ffn="batch"``) inputs, embedding,
+                  LayerNorm, FFN, decoder and loss on the device's uneven share
+                  of the POSITIONS of every sample; around attention, which
+                  needs whole sequences, ``all_gather(h, 1, ..)`` before and
+                  ``dynamic_slice(out, 1, ..)`` after (each rank computes the
+                  attention of all samples; ``replicate``'s backward sums the
+                  parameter gradients).
+``embedding="features"``  the embedding table sharded on dim 1 (its output
+                  gathered on dim 2), ``all_gather(.., 2, ..)`` and, for the
+                  batch-sharded plans, ``dynamic_slice(.., 0, ..)`` behind it.
 """
 from __future__ import annotations
 
@@ -139,7 +149,12 @@ def _head_parallel_attention(e: _Emitter, h, prefix: str, emsize: int, nheads: i
     return e.call(F.layer_norm, s, (emsize,))
 
 
-def _attention(e: _Emitter, h, prefix: str, emsize: int, nheads: int, p: float, mask):
+def _attention(e: _Emitter, h, prefix: str, emsize: int, nheads: int, p: float, mask, seq_lengths=None):
+    """``seq_lengths``: h is sharded over positions (dim 1); attention runs on the gathered sequences and its result
+    is cut back to the device's positions."""
+    local = h
+    if seq_lengths is not None:
+        h = e.call(collectives.all_gather, h, 1, seq_lengths, e.rank)
     t = e.call(torch.transpose, h, 0, 1)
     kw = dict(query=t, key=t, value=t,
               in_proj_weight=e.replicated(prefix + "self_attn.in_proj_weight"),
@@ -154,8 +169,10 @@ def _attention(e: _Emitter, h, prefix: str, emsize: int, nheads: int, p: float, 
     out = e.call(operator.getitem, both, 0)
     e.call(operator.getitem, both, 1)            # head-averaged probabilities: bound, never consumed
     out = e.call(torch.transpose, out, 0, 1)
+    if seq_lengths is not None:
+        out = e.call(collectives.dynamic_slice, out, 1, seq_lengths, e.rank)
     out = e.call(F.dropout, out, p)
-    s = e.call(operator.add, h, out)
+    s = e.call(operator.add, local, out)
     return e.call(F.layer_norm, s, (emsize,))
 
 
@@ -224,15 +241,40 @@ def build_program(model: nn.Module, plan: ShardingPlan, global_batch: int,
     p = float(model.dropout_p)
     d = model.emsize
 
+    seq_lengths = None
+    if plan.shard_dim not in ("batch", "sequence") or plan.embedding not in ("rows", "features"):
+        raise ValueError("ShardingPlan: shard_dim is 'batch' or 'sequence', embedding is 'rows' or 'features'")
+    if plan.shard_dim == "sequence" or plan.embedding == "features":
+        if model.family != "lm" or not batch_sharded or plan.attn != "batch":
+            raise ValueError("shard_dim='sequence' / embedding='features' are plans of the batch-attention language models")
+        if plan.shard_dim == "sequence" and (plan.ffn != "batch" or any(isinstance(l, models.Top2TransformerEncoderLayer)
+                                                                           for l in model.layers)):
+            raise ValueError("shard_dim='sequence' goes with ffn='batch' and dense layers")
     if model.family == "lm":
-        if batch_sharded:
-            x = e.sharded_input("x", B)
-            y = e.sharded_input("y", B)
-        else:
+        sdim = 1 if plan.shard_dim == "sequence" else 0
+        extent = model.seqlen if sdim == 1 else B
+        if sdim == 1:
+            seq_lengths = plan.lengths(model.seqlen)
+        if not batch_sharded:
             x, y = e.whole_input("x"), e.whole_input("y")
-        h = e.call(F.embedding, x, e.replicated("encoder.weight"))
+        elif plan.embedding == "features":
+            x, y = e.whole_input("x"), e.sharded_input("y", extent, sdim)
+        else:
+            x, y = e.sharded_input("x", extent, sdim), e.sharded_input("y", extent, sdim)
+        if plan.embedding == "features":
+            # table sharded over the embedding width: whole ids, output gathered on dim 2 (hap.rs:3220-3224), made
+            # whole by an all_gather and cut to the device's samples / positions
+            L_d = plan.lengths(d)
+            h = e.call(F.embedding, x, e.sharded("encoder.weight", d, 1))
+            h = e.call(collectives.all_gather, h, 2, L_d, e.rank)
+            h = e.call(collectives.dynamic_slice, h, sdim, plan.lengths(extent), e.rank)
+        else:
+            h = e.call(F.embedding, x, e.replicated("encoder.weight"))
         h = e.call(operator.mul, h, math.sqrt(d))
-        h = e.call(operator.add, h, e.g.get_attr("pe"))          # [1,S,d]: size-1 dim, never split
+        if sdim == 1:
+            h = e.call(operator.add, h, e.sharded("pe", model.seqlen, 1))     # [1, s, d]: the device's positions
+        else:
+            h = e.call(operator.add, h, e.g.get_attr("pe"))      # [1,S,d]: size-1 dim, never split
         mask = e.replicated("src_mask") if getattr(model, "src_mask", None) is not None else None
     elif model.family == "vit":
         x = e.sharded_input("x", B)
@@ -253,7 +295,7 @@ def build_program(model: nn.Module, plan: ShardingPlan, global_batch: int,
         if plan.attn == "heads" and batch_sharded:
             h1 = _head_parallel_attention(e, h, prefix, d, model.nheads, p, mask, B)
         else:
-            h1 = _attention(e, h, prefix, d, model.nheads, p, mask)
+            h1 = _attention(e, h, prefix, d, model.nheads, p, mask, seq_lengths)
         if isinstance(layer, models.Top2TransformerEncoderLayer):
             # the switch layer takes the top-2 layer's node forms with its own gating leaf (the reference's
             # synthesizer has no handler for models.switch_gating; its models call it at models.py:421)

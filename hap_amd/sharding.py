@@ -73,6 +73,12 @@ class ShardingPlan:
     segment: int = 0
     attn: str = "batch"          # "batch": attention on the device's samples; "heads": on the device's heads of every sample
     zero: bool = False           # parameters stored as dim-0 shards and all_gather-ed at use (hap.rs:2527-2547)
+    shard_dim: str = "batch"     # language models: "batch" shards inputs / activations over samples (dim 0),
+                                 # "sequence" over positions (dim 1: hap.rs:2500-2520 shards a placeholder on any
+                                 # dimension; linear / layer_norm / embedding / add keep a gather on any leading one,
+                                 # hap.rs:2795, 3061, 3214-3218, 2996; attention needs the whole sequence)
+    embedding: str = "rows"      # "rows": ids sharded, table whole; "features": ids whole, table sharded on dim 1,
+                                 # output gathered on dim 2 (hap.rs:3220-3224), then all_gather + dynamic_slice
 
     @property
     def world_size(self) -> int:

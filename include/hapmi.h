@@ -30,7 +30,7 @@ extern "C" {
 typedef void *hapmi_stream_t;
 
 enum { HAPMI_F32 = 0, HAPMI_BF16 = 1 };
-enum { HAPMI_ACT_NONE = 0, HAPMI_ACT_RELU = 1, HAPMI_ACT_GELU = 2 };
+enum { HAPMI_ACT_NONE = 0, HAPMI_ACT_RELU = 1, HAPMI_ACT_GELU = 2, HAPMI_ACT_SIGMOID = 3 };
 enum {
     HAPMI_OK = 0,
     HAPMI_EINVAL = -1,   /* bad shape / argument            */
@@ -270,12 +270,14 @@ int hapmi_logsoftmax_nll(const void *logits, const int64_t *targets, int64_t ign
 int hapmi_sum_f32(const float *x, int64_t n, float *out, hapmi_stream_t stream);
 
 /* ---- elementwise ------------------------------------------------------- */
-/* F.relu (hap.rs:1417) / F.gelu */
+/* F.relu (hap.rs:1417) / F.gelu / torch.sigmoid (hap.rs:1088) */
 int hapmi_act_fwd(const void *x, void *y, int64_t n, int act, int dtype, hapmi_stream_t stream);
-/* relu: ref = y (output); gelu: ref = x (input) */
+/* relu, sigmoid: ref = y (output); gelu: ref = x (input) */
 int hapmi_act_bwd(const void *dy, const void *ref, void *dx, int64_t n, int act, int dtype, hapmi_stream_t stream);
 /* out = a + b (operator.add, hap.rs:1515; also gradient accumulation) */
 int hapmi_add(const void *a, const void *b, void *out, int64_t n, int dtype, hapmi_stream_t stream);
+/* out[i] = value: the gradient of torch.sum(x) (hap.rs:1133) with respect to x */
+int hapmi_fill_value(void *out, float value, int64_t n, int dtype, hapmi_stream_t stream);
 /* out = a * s (operator.mul with a number, hap.rs:1563) */
 int hapmi_scale(const void *a, float s, void *out, int64_t n, int dtype, hapmi_stream_t stream);
 /* out[r, :] = a[r, :] + b[r % b_rows, :] (broadcast add of pe / pos_embed, hap.rs:3821-3837) */

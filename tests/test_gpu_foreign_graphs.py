@@ -89,3 +89,41 @@ def test_relu_output_that_shares_its_gradient_buffer(cuda):
         u = lin(s, 2)                       # consumes the sum, so the add is a launch of its own
         return g.call_function(operator.add, (u, lin(h, 3)))
     _run_both(build)
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+def test_mlp_of_linear_sigmoid_new_segment_and_sum(cuda, dtype):
+    """The reference's MLP model (models.py:8-24): a floating-point input split over the batch, linear -> sigmoid
+    (torch.sigmoid, hap.rs:1088) -> new_segment, the program's output torch.sum (hap.rs:1133)."""
+    d, B, L = 64, 16, [6, 6, 2, 2]
+    g0 = torch.Generator().manual_seed(3)
+    xs = torch.randn(B, d, generator=g0)
+    results = []
+    for device in ("cpu", "gpu"):
+        holder = _Holder(11, d)
+        g = torch.fx.Graph()
+        x, y = g.placeholder("x"), g.placeholder("y")
+        h = g.call_function(operator.getitem, (g.call_method("split", (x, L, 0)), 0))
+        for i in range(3):
+            h = g.call_function(F.linear, (h, g.get_attr(f"w{i}"), g.get_attr(f"b{i}")))
+            h = g.call_function(torch.sigmoid, (h,))
+            h = g.call_function(hap_amd.models.new_segment, (h,))
+        g.output(g.call_function(torch.sum, (h,)))
+        g.lint()
+        gm = torch.fx.GraphModule(holder, g)
+        if device == "cpu":
+            loss = gm(xs, None)
+            loss.backward()
+            results.append((loss.item(), {n: p.grad.clone() for n, p in gm.named_parameters() if p.grad is not None}))
+        else:
+            ex = hap_amd.compile_program(gm, [xs, (B,)], dtype=dtype)
+            loss = ex.forward(xs, None)
+            ex.backward()
+            torch.cuda.synchronize()
+            results.append((loss.item(), {n: rec["grad"].cpu() for n, rec in ex.params.items()}))
+    (want, ref), (got, grads) = results
+    tol = 1e-4 if dtype == "fp32" else 2e-2
+    assert abs(got - want) <= tol * abs(want)
+    assert set(grads) == set(ref)
+    for n in ref:
+        assert rel_err(grads[n], ref[n]) < tol, n

@@ -39,7 +39,8 @@ def _check_sent_messages(ex, log, rank, dtype):
 def _gpu_rank(model, ratios, rank, B, x, y, log, dtype, opt, **kw):
     m = copy.deepcopy(model)
     plan = hap_amd.ShardingPlan([list(ratios)], rank, ffn=kw.get("ffn", "column"), zero=kw.get("zero", False),
-                                attn=kw.get("attn", "batch"))
+                                attn=kw.get("attn", "batch"), shard_dim=kw.get("shard_dim", "batch"),
+                                embedding=kw.get("embedding", "rows"))
     gm = hap_amd.build_program(m, plan, B, activation=kw.get("activation", "relu"),
                                batch_sharded=kw.get("batch_sharded", True))
     ex = hap_amd.compile_program(gm, [x, y], dtype=dtype, wire=hap_amd.ReplayWire(log, rank), rank=rank,
@@ -580,3 +581,27 @@ def test_exchange_read_and_written_in_pieces_bf16(cuda):
             gb = b.params[n]["grad"]
             if gb.norm().item() > 0:
                 assert rel_err(rec["grad"], gb) < 1e-2, n
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+def test_sequence_sharded_program(cuda, dtype):
+    """Inputs, embedding, LayerNorm, FFN, decoder and loss on the device's uneven share of the POSITIONS (placeholder
+    split on dim 1, hap.rs:2500-2520; gathers on dim 1 through linear / layer_norm / embedding / add,
+    hap.rs:2795, 3061, 3214-3218, 2996); all_gather(dim 1) before and dynamic_slice(dim 1) behind attention."""
+    if dtype == "fp32":
+        model = make_lm(S=19)                                          # 19 positions over 4 devices: 7, 7, 2, 3
+        x, y = lm_batch(6, 19, 97)
+        _compare(model, RATIOS4, 6, x, y, dtype, [0, 2, 3], SGD, ffn="batch", shard_dim="sequence")
+    else:
+        model = make_lm(vocab=211, S=32, d=64, H=1, F=128, layers=2, causal=False)
+        x, y = lm_batch(6, 32, 211, mlm=True)
+        _compare(model, RATIOS4, 6, x, y, dtype, [0, 3], SGD, ffn="batch", shard_dim="sequence")
+
+
+@pytest.mark.parametrize("shard_dim,ffn", [("batch", "column"), ("batch", "batch"), ("sequence", "batch")])
+def test_embedding_table_sharded_over_features(cuda, shard_dim, ffn):
+    """F.embedding with whole ids and the table sharded on dim 1 gives its output gathered on dim 2 (hap.rs:3220-3224);
+    all_gather(dim 2) and dynamic_slice behind it."""
+    model = make_lm(d=64, H=4)                                         # 64 columns over 4 devices: 24, 24, 8, 8
+    x, y = lm_batch(8, 16, 97)
+    _compare(model, RATIOS4, 8, x, y, "fp32", [0, 3], ADAM, ffn=ffn, shard_dim=shard_dim, embedding="features")

@@ -27,6 +27,9 @@ CASES = {
     "lm-batch": (lambda: make_lm(), RATIOS4, 8, lambda: lm_batch(8, 16, 97), dict(ffn="batch")),
     "lm-column-zero": (lambda: make_lm(), RATIOS4, 8, lambda: lm_batch(8, 16, 97), dict(ffn="column", zero=True)),
     "lm-heads": (lambda: make_lm(H=8), RATIOS4, 8, lambda: lm_batch(8, 16, 97), dict(ffn="column", attn="heads")),
+    "lm-sequence": (lambda: make_lm(S=19), RATIOS4, 6, lambda: lm_batch(6, 19, 97), dict(ffn="batch", shard_dim="sequence")),
+    "lm-feature-embedding": (lambda: make_lm(d=40, H=4), RATIOS4, 8, lambda: lm_batch(8, 16, 97),
+                             dict(ffn="column", embedding="features")),
     "vit": (lambda: make_vit(), RATIOS4, 8, lambda: vit_batch(8, 16, 10), dict(ffn="batch")),
     "moe": (lambda: make_moe(), RATIOS_E, 16, lambda: lm_batch(16, 16, 61), dict(ffn="batch")),
     "moe-replicated-batch": (lambda: make_moe(), RATIOS_E, 4, lambda: lm_batch(4, 16, 61),

@@ -184,3 +184,31 @@ def test_head_parallel_attention_vit_with_zero_spmd_equals_single_device():
     sharded = _zero_sharded(model, [.25] * 4)
     sharded.update(_head_sharded(2, [1, 1, 1, 1], 8))
     _check(model, run, x, y, sharded, whole_norm=True)
+
+
+@pytest.mark.parametrize("embedding", ["rows", "features"])
+def test_sequence_sharded_lm_spmd_equals_single_device(embedding):
+    """shard_dim='sequence': 19 positions over .375/.375/.125/.125 -> 7, 7, 2, 3 per device."""
+    model = make_lm(S=19, d=40 if embedding == "features" else 32)
+    x, y = lm_batch(6, 19, 97)
+    run = joint_cpu(model, RATIOS4, 6, ffn="batch", shard_dim="sequence", embedding=embedding)
+    assert hap_amd.sharding_lengths(19, RATIOS4) == [7, 7, 2, 3]
+    assert run.programs[2].pe.shape == (1, 2, 40 if embedding == "features" else 32)
+    sharded = {"encoder.weight": (1, hap_amd.sharding_lengths(40, RATIOS4))} if embedding == "features" else {}
+    _check(model, run, x, y, sharded)
+
+
+@pytest.mark.parametrize("ffn", ["column", "batch"])
+def test_feature_sharded_embedding_table_spmd_equals_single_device(ffn):
+    model = make_lm(d=40, H=4)
+    x, y = lm_batch(8, 16, 97)
+    run = joint_cpu(model, RATIOS4, 8, ffn=ffn, embedding="features")
+    L_d = hap_amd.sharding_lengths(40, RATIOS4)
+    assert L_d == [15, 15, 5, 5] and run.programs[3].encoder.weight.shape == (97, 5)
+    sharded = {"encoder.weight": (1, L_d)}
+    if ffn == "column":
+        L_F = hap_amd.sharding_lengths(64, RATIOS4)
+        for i in range(2):
+            sharded[f"layers.{i}.linear1.weight"] = (0, L_F)
+            sharded[f"layers.{i}.linear1.bias"] = (0, L_F)
+    _check(model, run, x, y, sharded)
