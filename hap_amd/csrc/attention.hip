@@ -130,12 +130,20 @@ struct PairLoader {
 // linear index, starts the longest ones first and the short ones fill the tail.
 template <bool CAUSAL> struct BlockOrder {
     __device__ __forceinline__ static int linear() { return (int)(blockIdx.y * gridDim.x + blockIdx.x); }
+    // Without a mask: blocks are dealt round-robin over the 8 XCDs (each with an L2 of its own) in the order of
+    // their linear index.  The row blocks of one (batch, head) stream the same K / V (Q / dO) tiles, so they are
+    // given to the same XCD, next to each other in time: work item w = (XCD) * (items per XCD) + (turn on that XCD),
+    // row block = w % row blocks.  The tiles then come from that XCD's L2 for all but the first of the blocks.
+    __device__ __forceinline__ static int work_item() {
+        const int n = (int)(gridDim.x * gridDim.y), l = linear();
+        return (n % 8 == 0) ? (l % 8) * (n / 8) + l / 8 : l;
+    }
     __device__ __forceinline__ static int row_block(bool work_grows_with_index) {
-        if (!CAUSAL) return (int)blockIdx.x;
+        if (!CAUSAL) return work_item() % (int)gridDim.x;
         const int i = linear() / (int)gridDim.y;
         return work_grows_with_index ? (int)gridDim.x - 1 - i : i;
     }
-    __device__ __forceinline__ static int batch_head() { return CAUSAL ? linear() % (int)gridDim.y : (int)blockIdx.y; }
+    __device__ __forceinline__ static int batch_head() { return CAUSAL ? linear() % (int)gridDim.y : work_item() / (int)gridDim.x; }
 };
 
 // CAUSAL: key j is visible to query i iff j <= i (the additive mask torch.triu(full(-inf), 1), models.py:76),
@@ -143,8 +151,8 @@ template <bool CAUSAL> struct BlockOrder {
 template <bool CAUSAL>
 __global__ __launch_bounds__(AT_THREADS, 2) void attn_fwd_kernel(const bf16_t *qkv, const float *mask, bf16_t *out,
                                                             float *lse, int S, int H, float scale) {
-    __shared__ __attribute__((aligned(16))) char Ks[TILE_BYTES];
-    __shared__ __attribute__((aligned(16))) char Vs[TILE_BYTES];
+    __shared__ __attribute__((aligned(16))) char Ks2[2][TILE_BYTES];   // two tiles each: the next tile is written while
+    __shared__ __attribute__((aligned(16))) char Vs2[2][TILE_BYTES];   // the current one is read (one barrier per tile)
     const TransposedReader tr;
     const int E = H * HD, ld = 3 * E;
     const int blk = BlockOrder<CAUSAL>::row_block(true), bh = BlockOrder<CAUSAL>::batch_head();
@@ -169,27 +177,33 @@ __global__ __launch_bounds__(AT_THREADS, 2) void attn_fwd_kernel(const bf16_t *q
     const float sl2 = scale * LOG2E;
     const bool plain_block = !mask && blk * 128 + 128 <= S;
 
-    // The next tile's global loads are issued before the current tile is multiplied, so their latency is
-    // covered by the MFMA / softmax work; the registers are written to LDS at the top of the next iteration.
+    // Tile i + 1 travels global -> registers while tile i is multiplied and is written to the other LDS buffer at the
+    // end of iteration i (its loads have had the whole iteration to arrive); tile i + 2's loads are issued right after.
     const int q_blk_end = blk * 128 + 128;
     const int kv_end = (CAUSAL && q_blk_end < S) ? q_blk_end : S;
     lk.load(K, S);
     lv.load(V, S);
+    lk.store_rows(Ks2[0]);
+    lv.store_rows(Vs2[0]);
+    if (TILE < kv_end) {
+        lk.load(K + (int64_t)TILE * ld, S - TILE);
+        lv.load(V + (int64_t)TILE * ld, S - TILE);
+    }
+    __syncthreads();
+    int buf = 0;
     for (int kv0 = 0; kv0 < kv_end; kv0 += TILE) {
-        __syncthreads();                                   // every wave is done with the previous tiles
-        lk.store_rows(Ks);
-        lv.store_rows(Vs);
-        __syncthreads();
-        if (kv0 + TILE < kv_end) {
-            lk.load(K + (int64_t)(kv0 + TILE) * ld, S - kv0 - TILE);
-            lv.load(V + (int64_t)(kv0 + TILE) * ld, S - kv0 - TILE);
-        }
-
-        f32x16 st[2] = {zero16(), zero16()};
+        const char *Ks = Ks2[buf], *Vs = Vs2[buf];
+        // all fragment reads of the tile are issued before the first MFMA waits for one
+        frag_t kf[2][4];
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
-            for (int s = 0; s < 4; ++s) st[t] = mma(frag_rowk(Ks, t * 32 + c, s, h), qf[s], st[t]);
+            for (int s = 0; s < 4; ++s) kf[t][s] = frag_rowk(Ks, t * 32 + c, s, h);
+        f32x16 st[2] = {zero16(), zero16()};
+#pragma unroll
+        for (int s = 0; s < 4; ++s)
+#pragma unroll
+            for (int t = 0; t < 2; ++t) st[t] = mma(kf[t][s], qf[s], st[t]);
 
         float alpha, psum = 0.f;
         if (plain_block && kv0 + TILE <= S && (!CAUSAL || kv0 + TILE - 1 <= blk * 128)) {
@@ -266,6 +280,16 @@ __global__ __launch_bounds__(AT_THREADS, 2) void attn_fwd_kernel(const bf16_t *q
 #pragma unroll
             for (int u = 0; u < 2; ++u) ot[u] = mma(tr.frag(Vs, u * 32, s), pb, ot[u]);
         }
+        if (kv0 + TILE < kv_end) {
+            lk.store_rows(Ks2[buf ^ 1]);                   // last read in the iteration before this one
+            lv.store_rows(Vs2[buf ^ 1]);
+            if (kv0 + 2 * TILE < kv_end) {
+                lk.load(K + (int64_t)(kv0 + 2 * TILE) * ld, S - kv0 - 2 * TILE);
+                lv.load(V + (int64_t)(kv0 + 2 * TILE) * ld, S - kv0 - 2 * TILE);
+            }
+        }
+        __syncthreads();
+        buf ^= 1;
     }
     const float l = lsum + __shfl_xor(lsum, 32, 64);
     const float inv = l > 0.f ? 1.0f / l : 0.f;

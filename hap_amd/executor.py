@@ -238,6 +238,35 @@ class ShardExecutor:
     def _val(self, x):
         return self.env[x] if isinstance(x, torch.fx.Node) else x
 
+    def _place_gather_inputs(self):
+        """Which nodes write their result straight into the rows of an all_gather's result.  The gather along dim 0
+        concatenates the ranks' shards; when the shard's producer allocates the whole result and writes its rows of
+        it, the gather has no copy of the own shard left to make (the peers' shards are received at their rows).
+        Producers that do this: layer_norm (the input of the column-sharded FFN's gather)."""
+        self._gather_of: Dict[torch.fx.Node, torch.fx.Node] = {}
+        self._gather_results: Dict[torch.fx.Node, torch.Tensor] = {}
+        if not self.receive_in_place:
+            return
+        for node in self.gm.graph.nodes:
+            if node.op != "call_function" or node.target is not collectives.all_gather or len(node.args) < 4:
+                continue
+            src, dim, L, rank = node.args[0], node.args[1], list(node.args[2]), node.args[3]
+            if (dim == 0 and isinstance(src, torch.fx.Node) and src.op == "call_function" and src.target is F.layer_norm
+                    and src not in self._gather_of and L[rank] > 0):
+                self._gather_of[src] = node
+
+    def _placed_output(self, node, shape):
+        """The buffer for ``node``'s result: new, or its rows of the all_gather result that it feeds."""
+        g = self._gather_of.get(node)
+        if g is None or len(shape) < 1:
+            return self._new(shape)
+        L, rank = list(g.args[2]), g.args[3]
+        if shape[0] != L[rank]:
+            return self._new(shape)
+        full = self._new((sum(L),) + tuple(shape[1:]))
+        self._gather_results[g] = full
+        return full.narrow(0, sum(L[:rank]), L[rank])
+
     def _scratch(self, key, shape, dtype=None):
         """Backward-only temporaries that live inside one node's backward closure are shared between
         nodes of the same shape (the launches of a step are serialised on one stream)."""
@@ -445,6 +474,7 @@ class ShardExecutor:
             collectives.reduce_scatter: self._reduce_scatter, collectives.all_to_all: self._all_to_all,
             collectives.all_reduce: self._all_reduce, collectives.dynamic_slice: self._dynamic_slice,
         }
+        self._place_gather_inputs()
         for node in self.gm.graph.nodes:
             if node.op == "placeholder":
                 self.env[node] = Val("input", name=node.name, index=len(self.inputs))
@@ -729,7 +759,7 @@ class ShardExecutor:
         if len(shape) != 1 or shape[0] != ref_shape[-1]:
             self._unsupported(node, "layer_norm over the last dimension only")
         rows = x.numel() // shape[0]
-        out = Val("tensor", self._new(ref_shape), needs_grad=True)
+        out = Val("tensor", self._placed_output(node, ref_shape), needs_grad=True)
         rstd = self._new((rows,), torch.float32)
         self.fwd.append(lambda: ops.add_layernorm_fwd(x, res, out.t, rstd, _EPS))
 
@@ -1256,29 +1286,35 @@ class ShardExecutor:
                     self._send_hooks += 1
                     sink.append(lambda hook=hook: ops._lib.host_call(hook))
 
-    def _emit_gather(self, tag, direction, x_t, dim, L, rank, sink: List[Callable]):
-        """pad own shard -> [wire] -> cut pads and concatenate.  Returns the full tensor."""
+    def _emit_gather(self, tag, direction, x_t, dim, L, rank, sink: List[Callable], full=None):
+        """pad own shard -> [wire] -> cut pads and concatenate.  Returns the full tensor.  ``full``: the result's
+        buffer when the producer of ``x_t`` already wrote the shard at its rows of it (_place_gather_inputs)."""
         m, W = max(L), len(L)
         pshape = ops._with_dim(x_t.shape, dim, m)
         # a shard of the longest length needs no padding: the tensor itself is the message
         unpadded = L[rank] == m and x_t.is_contiguous() and tuple(x_t.shape) == tuple(pshape)
         own = x_t if unpadded else self._new(pshape, x_t.dtype)
-        full = self._new(ops._with_dim(x_t.shape, dim, sum(L)), x_t.dtype)
-        # a peer's shard of the longest length carries no padding either: along dim 0 it is received straight into
-        # its rows of the result.  Only in the forward direction, where the result is an activation that no launch
-        # writes afterwards; a gathered gradient may be accumulated into in place by other consumers.
+        if full is None:
+            full = self._new(ops._with_dim(x_t.shape, dim, sum(L)), x_t.dtype)
+        # Along dim 0 a peer's shard is received straight into its rows of the result (the payload rows of a shard that
+        # was padded to the longest length).  Only in the forward direction, where the result is an activation that no
+        # launch writes afterwards; a gathered gradient may be accumulated into in place by other consumers.
         into = {}
         if self.receive_in_place and dim == 0 and direction == "fwd":
-            into = {s: full.narrow(0, sum(L[:s]), m) for s in range(W) if s != rank and L[s] == m}
+            into = {s: full.narrow(0, sum(L[:s]), L[s]) for s in range(W) if s != rank and L[s] > 0}
             if into:
                 self._wire_backed.add(full.untyped_storage().data_ptr())
         peers = {s: self.wire.recv(tag, direction, s, pshape, x_t.dtype, self.dev, reduction=False, into=into.get(s))
                  for s in range(W) if s != rank}
-        slices = [own if s == rank else peers[s] for s in range(W)]
-        if unpadded:
+        row = full[0].numel() * full.element_size() if full.dim() > 0 and full.shape[0] > 0 else 0
+        own_placed = dim == 0 and x_t.is_contiguous() and x_t.data_ptr() == full.data_ptr() + sum(L[:rank]) * row
+        slices = [(x_t if (unpadded or own_placed) else own) if s == rank else peers[s] for s in range(W)]
+        placed = all(L[s] == 0 or (dim == 0 and slices[s] is not None and slices[s].is_contiguous()
+                                   and slices[s].data_ptr() == full.data_ptr() + sum(L[:s]) * row) for s in range(W))
+        if not unpadded:
+            sink.append(lambda: ops.pad_rows(x_t, dim, m, own))
+        if not placed:
             sink.append(lambda: ops.unpad_concat(slices, L, dim, full))
-        else:
-            sink.append(lambda: (ops.pad_rows(x_t, dim, m, own), ops.unpad_concat(slices, L, dim, full)))
         self._announce(tag, direction, rank, W, lambda dst: own, sink)        # the padded shard goes to every peer
         return full
 
@@ -1291,18 +1327,23 @@ class ShardExecutor:
         out = out_t if out_t is not None else self._new(ops._with_dim(full_t.shape, dim, L[rank]), full_t.dtype)
         if dim == 0 and full_t.is_contiguous() and L[rank] > 0:
             # along dim 0 this rank's own piece is a contiguous row range of the full tensor: the sum reads it there
-            # (and the first L[rank] rows of the peers' padded pieces), and no padded copy of it is made
-            sent = [None if s == rank else self._new(pshape, full_t.dtype) for s in range(W)]
+            # (and the first L[rank] rows of the peers' padded pieces), and no padded copy of it is made; a peer's
+            # piece of the longest length needs no padding either: its rows of the full tensor are the message
+            in_place = [s != rank and self.receive_in_place and L[s] == m for s in range(W)]
+            sent = [None if (s == rank or in_place[s]) else self._new(pshape, full_t.dtype) for s in range(W)]
+            messages = [full_t.narrow(0, sum(L[:s]), m) if in_place[s] else sent[s] for s in range(W)]
             own = full_t.narrow(0, sum(L[:rank]), L[rank])
             contribs = [own if s == rank else (peers[s].narrow(0, 0, L[rank]) if peers[s] is not None else None)
                         for s in range(W)]
         else:
             sent = [self._new(pshape, full_t.dtype) for _ in range(W)]
+            messages = sent
             contribs = [sent[rank] if s == rank else peers[s] for s in range(W)]
         contribs = [c for c in contribs if c is not None]
-        sink.append(lambda: (ops.split_pad(full_t, L, dim, m, sent),
-                             ops.ragged_reduce(contribs, dim, 0, L[rank], out, addend=addend)))
-        self._announce(tag, direction, rank, W, lambda dst: sent[dst], sink)  # the padded piece that rank dst reduces
+        if any(t is not None for t in sent):
+            sink.append(lambda: ops.split_pad(full_t, L, dim, m, sent))
+        sink.append(lambda: ops.ragged_reduce(contribs, dim, 0, L[rank], out, addend=addend))
+        self._announce(tag, direction, rank, W, lambda dst: messages[dst], sink)  # the padded piece that rank dst reduces
         return out
 
     def _all_gather(self, node):
@@ -1311,7 +1352,7 @@ class ShardExecutor:
             return self._gathered_param(node, x, dim, L, rank)
         if x.t is None or x.ld is not None:
             self._unsupported(node, f"all_gather of a {x.kind} value")
-        full = self._emit_gather(node.name, "fwd", x.t, dim, L, rank, self.fwd)
+        full = self._emit_gather(node.name, "fwd", x.t, dim, L, rank, self.fwd, full=self._gather_results.pop(node, None))
         out = Val("tensor", full, needs_grad=x.needs_grad)
 
         def emit():

@@ -105,13 +105,20 @@ def unpad_concat(slices: Sequence[torch.Tensor], lengths: Sequence[int], dim: in
                  out: Optional[torch.Tensor] = None) -> torch.Tensor:
     _dev(*slices, out)
     ref = slices[0]
-    outer, padded_len, inner = _oli(ref.shape, dim)
+    outer, _, inner = _oli(ref.shape, dim)
+    # a slice that lies at its place in ``out`` may hold its payload only: the padded length is the longest one's
+    padded_len = max([sl.shape[dim] for sl in slices] + [int(n) for n in lengths])
     if out is None:
         out = torch.empty(_with_dim(ref.shape, dim, sum(lengths)), dtype=ref.dtype, device=ref.device)
-    for sl in slices:
-        _need(sl, outer * padded_len * inner, "unpad_concat slice")
+    off = 0
+    for sl, n in zip(slices, lengths):
+        # a slice that already lies at its place in ``out`` (one contiguous range) is left where it is by the kernel
+        # and only has to hold its payload rows
+        in_place = outer == 1 and sl.data_ptr() == out.data_ptr() + off * inner * out.element_size()
+        _need(sl, outer * (n if in_place else padded_len) * inner, "unpad_concat slice")
         if sl.dtype != ref.dtype:
             raise TypeError("unpad_concat: dtype mismatch")
+        off += n
     _need(out, outer * sum(lengths) * inner, "unpad_concat dst")
     if out.numel() == 0:
         return out

@@ -29,8 +29,10 @@ class Wire:
 
     def recv(self, tag: str, direction: str, src: int, shape, dtype, device, reduction: bool = False,
              into: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
-        """``into``: a contiguous static GPU tensor of ``shape`` that the message is to be delivered into (zero-copy
-        receive: the executor passes the rows of a concatenation that the piece belongs to); the wire returns it.
+        """``into``: a contiguous static GPU tensor that the message is to be delivered into (zero-copy receive: the
+        executor passes the rows of a concatenation that the piece belongs to); the wire returns it.  It has the
+        message's ``shape``, or fewer rows along dim 0: then it takes the message's first rows (a shard that was padded
+        to the longest length carries its payload there; a transport that sends exact extents delivers just those).
         The stand-ins below deliver once, when the program is compiled; a transport would post its receive into
         it every step."""
         raise NotImplementedError
@@ -39,9 +41,10 @@ class Wire:
     def _deliver(message: Optional[torch.Tensor], into: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
         if into is None or message is None:
             return message
-        if tuple(into.shape) != tuple(message.shape) or into.dtype != message.dtype or not into.is_contiguous():
-            raise ValueError("recv(into=...): a contiguous tensor of the message's shape and dtype expected")
-        into.copy_(message)
+        rows_ok = into.dim() == message.dim() and into.dim() >= 1 and 0 < into.shape[0] <= message.shape[0]
+        if not rows_ok or tuple(into.shape[1:]) != tuple(message.shape[1:]) or into.dtype != message.dtype or not into.is_contiguous():
+            raise ValueError("recv(into=...): a contiguous tensor of the message's shape (or its first rows) and dtype expected")
+        into.copy_(message[:into.shape[0]])
         return into
 
     def send(self, tag: str, direction: str, dst: int, buffer: torch.Tensor) -> None:

@@ -275,6 +275,35 @@ def test_gemm_every_tile_configuration_and_layout(cuda, cfg, tA, tB):
         lib().hapmi_gemm_tuning(-1, 0)
 
 
+@pytest.mark.parametrize("cfg", [0, 1, 7])
+@pytest.mark.parametrize("act", ["none", "relu", "gelu"])
+def test_gemm_scale_bias_activation_in_every_epilogue(cuda, cfg, act):
+    """alpha, bias and activation applied by the epilogue, bf16 and float32 outputs, with and without bias, ragged
+    and tile-aligned shapes."""
+    from hap_amd._lib import lib
+    fn = {"none": lambda t: t, "relu": torch.relu, "gelu": torch.nn.functional.gelu}[act]
+    try:
+        lib().hapmi_gemm_tuning(cfg, 1)
+        for (M, N, K) in [(424, 520, 328), (512, 512, 128)]:
+            g = torch.Generator().manual_seed(M + cfg)
+            A = torch.randn(M, K, generator=g).bfloat16()
+            B = torch.randn(N, K, generator=g).bfloat16()
+            bias = torch.randn(N, generator=g)
+            for with_bias in (True, False):
+                for alpha in (1.0, 0.25):
+                    want = alpha * (A.double() @ B.double().t())
+                    if with_bias:
+                        want = want + bias.double()
+                    want = fn(want)
+                    for out_dtype in (torch.bfloat16, torch.float32):
+                        C = torch.full((M, N), float("nan"), dtype=out_dtype, device=cuda)
+                        ops.gemm(A.to(cuda), B.to(cuda), C, M, N, K, transB=True, alpha=alpha,
+                                 bias=bias.to(cuda) if with_bias else None, act=act if act != "none" else None)
+                        close(C, want, torch.bfloat16, scale=2.0)
+    finally:
+        lib().hapmi_gemm_tuning(-1, 0)
+
+
 @pytest.mark.parametrize("cfg", [0, 10, 11])
 @pytest.mark.parametrize("tA,tB", [(0, 1), (0, 0), (1, 0), (1, 1)])
 def test_gemm_float32_tile_configurations_and_layouts(cuda, cfg, tA, tB):
