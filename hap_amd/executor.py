@@ -1933,8 +1933,9 @@ class ShardExecutor:
     def autotune_gemms(self, verbose: bool = False):
         """Run one forward + backward with the loaded inputs while recording every GEMM call, then time the
         legal tile configurations / K splits of each distinct problem signature on the recorded operands and
-        pin the winners in the library's plan table (process-wide; other signatures keep the cost model).
-        Buffers that the timed launches overwrite or accumulate into are activations and gradients, which the
+        pin the winners in the library's plan table (process-wide; other signatures keep the cost model).  Returns one
+        row per signature: (signature, configuration, K splits, microseconds of one cold launch, launches per step,
+        problems per step).  Buffers that the timed launches overwrite or accumulate into are activations and gradients, which the
         next step rewrites before reading; parameters and optimizer state are not touched."""
         if any(rec["buf"] is None for rec in self.inputs):
             raise RuntimeError("load_inputs() first")
@@ -1946,15 +1947,22 @@ class ShardExecutor:
             log = ops.record_gemms(False)
         torch.cuda.synchronize()
         flush = torch.zeros(512 << 20, dtype=torch.int8, device=self.dev)
+        def signature(a):
+            return (a.M, a.N, a.K, a.batch1 * a.batch2, a.transA, a.transB, a.in_dtype, a.out_dtype,
+                    bool(a.A_segments), bool(a.B_segments or a.B_segments_list), bool(a.C_segments), a.a_relu, a.b_relu)
+        calls: Dict[tuple, list] = {}
+        for a, keep in log:                              # launches and problems (a launch over pointer lists holds several)
+            c = calls.setdefault(signature(a), [0, 0])
+            c[0] += 1
+            c[1] += int(a.batch1 * a.batch2) if a.A_list else 1
         seen, report = set(), []
         for a, keep in log:
-            key = (a.M, a.N, a.K, a.batch1 * a.batch2, a.transA, a.transB, a.in_dtype, a.out_dtype,
-                   bool(a.A_segments), bool(a.B_segments or a.B_segments_list), bool(a.C_segments), a.a_relu, a.b_relu)
+            key = signature(a)
             if key in seen:
                 continue
             seen.add(key)
             cfg, splits, us = ops.autotune_gemm(a, flush)
-            report.append((key, cfg, splits, us))
+            report.append((key, cfg, splits, us, calls[key][0], calls[key][1]))
             if verbose:
                 print(f"gemm M{a.M} N{a.N} K{a.K} batch{key[3]} tA{a.transA} tB{a.transB}: config {cfg}, "
                       f"{splits} split(s), {us:.1f} us", flush=True)
