@@ -72,3 +72,24 @@ def joint_cpu(model, ratios, B, dtype="fp32", **kw):
 def rel_err(a, b):
     a, b = a.detach().float().cpu(), b.detach().float().cpu()
     return ((a - b).norm() / b.norm().clamp_min(1e-30)).item()
+
+
+def gating_vectors():
+    """The hand-worked routing vectors of tests/golden/gating_vectors.json: the same data for the CPU oracle tests and
+    the GPU kernel tests."""
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(__file__), "golden", "gating_vectors.json")) as f:
+        return json.load(f)
+
+
+def gating_vector_logits(v):
+    """Logits [1, S, E] whose first (and second) choices are the vector's."""
+    import torch
+    lg = torch.full((1, v["S"], v["E"]), v["other_logit"])
+    for s, ch in enumerate(v["choices"]):
+        if isinstance(ch, list):
+            lg[0, s, ch[0]], lg[0, s, ch[1]] = v["first_logit"], v["second_logit"]
+        else:
+            lg[0, s, ch] = v["first_logit"]
+    return lg

@@ -6,7 +6,7 @@ import torch
 
 from hap_amd import ops
 from oracle import ops as ref
-from helpers import rel_err
+from helpers import gating_vector_logits, gating_vectors, rel_err
 
 pytestmark = pytest.mark.gpu
 
@@ -20,14 +20,11 @@ def _logits(B, S, E, seed):
 
 
 def test_hand_worked_vector(cuda):
-    lg = torch.full((1, 4, 2), -4.0)
-    for s, (k0, k1) in enumerate([(0, 1), (0, 1), (1, 0), (0, 1)]):
-        lg[0, s, k0], lg[0, s, k1] = 2.0, 1.0
-    r = ops.top2_gate(lg.to(cuda), 4)
-    assert r["index"].cpu().tolist() == [[[0, 1], [0, 1], [1, 0], [0, 1]]]
-    assert r["slot"].cpu().tolist() == [[[1, 2], [2, 3], [1, 0], [3, 0]]]
-    tos = r["token_of_slot"].cpu()[0].tolist()
-    assert tos == [[-1, 0, 1, 3], [-1, 2, 0, 1]]
+    v = gating_vectors()["top2"]
+    r = ops.top2_gate(gating_vector_logits(v).to(cuda), v["C"])
+    assert r["index"].cpu().tolist() == [v["choices"]]
+    assert r["slot"].cpu().tolist() == [v["slot"]]
+    assert r["token_of_slot"].cpu()[0].tolist() == v["token_of_slot"]
 
 
 @pytest.mark.parametrize("B,S,E,C", SHAPES)
@@ -127,15 +124,14 @@ def test_gate_backward_matches_autograd(cuda):
 # ---- switch (top-1) gating, /root/reference/models.py:452-475 ---------------------------------------------------
 
 def test_switch_hand_worked_vector(cuda):
-    lg = torch.full((1, 6, 3), -4.0)
-    for s, e in enumerate([0, 0, 2, 0, 2, 1]):
-        lg[0, s, e] = 2.0
-    lg = torch.cat([lg, torch.full((1, 6, 1), -9.0)], 2)          # the kernel's GEMM path wants E % 4 == 0; expert 3 unused
-    r = ops.switch_gate(lg.to(cuda), 3)
-    assert r["index"].cpu()[0, :, 0].tolist() == [0, 0, 2, 0, 2, 1]
-    assert r["slot"].cpu()[0].tolist() == [[1, 0], [2, 0], [1, 0], [0, 0], [2, 0], [1, 0]]
-    assert r["gate"].cpu()[0, :, 1].tolist() == [0.0] * 6
-    assert r["token_of_slot"].cpu()[0].tolist() == [[-1, 0, 1], [-1, 5, -1], [-1, 2, 4], [-1, -1, -1]]
+    v = gating_vectors()["switch"]
+    lg = gating_vector_logits(v)
+    lg = torch.cat([lg, torch.full((1, v["S"], 1), -9.0)], 2)     # the kernel's GEMM path wants E % 4 == 0; expert 3 unused
+    r = ops.switch_gate(lg.to(cuda), v["C"])
+    assert r["index"].cpu()[0, :, 0].tolist() == v["choices"]
+    assert r["slot"].cpu()[0].tolist() == v["slot"]
+    assert r["gate"].cpu()[0, :, 1].tolist() == [0.0] * v["S"]
+    assert r["token_of_slot"].cpu()[0].tolist() == v["token_of_slot"] + [[-1] * v["C"]]
 
 
 @pytest.mark.parametrize("B,S,E,C", SHAPES)

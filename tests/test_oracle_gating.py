@@ -4,6 +4,7 @@ algorithm implies."""
 import torch
 
 from oracle import ops as ref
+from helpers import gating_vector_logits, gating_vectors
 
 
 def _logits_for_choices(choices, E):
@@ -21,11 +22,12 @@ def test_hand_worked_vector():
     # B=1, S=4, E=2, C=4; choices t0:(0,1) t1:(0,1) t2:(1,0) t3:(0,1)
     # first-choice positions: e0 {t0:1, t1:2, t3:3}, e1 {t2:1}; sums of positions: e0 = 6, e1 = 1
     # second-choice positions: e1 {t0:1+1, t1:2+1, t3:3+1 -> dropped (>= C)}, e0 {t2:1+6 -> dropped}
-    lg = _logits_for_choices([[(0, 1), (0, 1), (1, 0), (0, 1)]], 2)
-    x = torch.eye(2).repeat(1, 1, 1)            # gate_input @ gate_weight = logits via identity trick
-    d, c = ref.top_2_gating(lg, 2, 4, torch.eye(2))
-    kept = sorted((s, e, k) for _, s, e, k in d.nonzero().tolist())
-    assert kept == [(0, 0, 1), (0, 1, 2), (1, 0, 2), (1, 1, 3), (2, 1, 1), (3, 0, 3)]
+    v = gating_vectors()["top2"]
+    lg = gating_vector_logits(v)
+    assert torch.equal(lg, _logits_for_choices([[tuple(ch) for ch in v["choices"]]], 2))
+    d, c = ref.top_2_gating(lg, v["E"], v["C"], torch.eye(2))   # gate_input @ gate_weight = logits via the identity
+    kept = sorted([s, e, k] for _, s, e, k in d.nonzero().tolist())
+    assert kept == v["kept_token_expert_slot"]
     probs = torch.softmax(lg, dim=2)
     assert torch.equal(c[0, 0, 0, 1], probs[0, 0, 0]) and torch.equal(c[0, 0, 1, 2], probs[0, 0, 1])
     assert torch.equal(c[0, 2, 1, 1], probs[0, 2, 1])
@@ -79,12 +81,11 @@ def test_gradient_flows_through_gates_only():
 def test_switch_hand_worked_vector():
     # B=1, S=6, E=3, C=3; first choices t0:0 t1:0 t2:2 t3:0 t4:2 t5:1
     # positions (1-based, per expert, in token order): e0 {t0:1, t1:2, t3:3 -> dropped (>= C)}, e2 {t2:1, t4:2}, e1 {t5:1}
-    lg = torch.full((1, 6, 3), -4.0)
-    for s, e in enumerate([0, 0, 2, 0, 2, 1]):
-        lg[0, s, e] = 2.0
-    d, c = ref.switch_gating(lg, 3, 3, torch.eye(3))
-    kept = sorted((s, e, k) for _, s, e, k in d.nonzero().tolist())
-    assert kept == [(0, 0, 1), (1, 0, 2), (2, 2, 1), (4, 2, 2), (5, 1, 1)]
+    v = gating_vectors()["switch"]
+    lg = gating_vector_logits(v)
+    d, c = ref.switch_gating(lg, v["E"], v["C"], torch.eye(3))
+    kept = sorted([s, e, k] for _, s, e, k in d.nonzero().tolist())
+    assert kept == v["kept_token_expert_slot"]
     probs = torch.softmax(lg, dim=2)
     assert torch.equal(c[0, 1, 0, 2], probs[0, 1, 0]) and torch.equal(c[0, 5, 1, 1], probs[0, 5, 1])
     assert c[0, 3].sum() == 0                                            # the dropped token reaches no expert
