@@ -547,7 +547,8 @@ class ShardExecutor:
                 return src.meta["out"]
             return Val("dead", why="head-averaged attention probabilities are never consumed by the program")
         if src.kind == "gating":
-            return Val("routing", which="dispatch" if idx == 0 else "combine", gating=src, e_lo=0, E_loc=src.meta["E"])
+            return Val("routing", which="dispatch" if idx == 0 else "combine", gating=src, e_lo=0, E_loc=src.meta["E"],
+                       c_lo=0, C_loc=src.meta["C"])
         self._unsupported(node, f"getitem on a {src.kind} value")
 
     # ------------------------------------------------------------------ ops
@@ -1594,8 +1595,15 @@ class ShardExecutor:
 
     def _dynamic_slice(self, node):
         v, dim, L, rank = self._val(node.args[0]), node.args[1], list(node.args[2]), node.args[3]
-        if v.kind == "routing" and dim == 2:
-            return Val("routing", which=v.meta["which"], gating=v.meta["gating"], e_lo=sum(L[:rank]), E_loc=L[rank])
+        if v.kind == "routing" and dim in (2, 3):
+            # the device's window of the dense [B, S, E, C] tensor: experts (dim 2) and / or capacity slots (dim 3)
+            m = dict(which=v.meta["which"], gating=v.meta["gating"], e_lo=v.meta["e_lo"], E_loc=v.meta["E_loc"],
+                     c_lo=v.meta["c_lo"], C_loc=v.meta["C_loc"])
+            lo, n = ("e_lo", "E_loc") if dim == 2 else ("c_lo", "C_loc")
+            if sum(L) != m[n]:
+                self._unsupported(node, f"the lengths {L} do not add up to the extent {m[n]} of dimension {dim}")
+            m[lo], m[n] = m[lo] + sum(L[:rank]), L[rank]
+            return Val("routing", **m)
         if v.t is None or v.ld is not None:
             self._unsupported(node, f"dynamic_slice of a {v.kind} value")
         off = sum(L[:rank])
@@ -1664,16 +1672,16 @@ class ShardExecutor:
             self._unsupported(node, "expects (tokens, dispatch tensor of top_2_gating)")
         gv = route.meta["gating"]
         r, E, C = gv.meta["r"], gv.meta["E"], gv.meta["C"]
-        e_lo, E_loc = route.meta["e_lo"], route.meta["E_loc"]
+        e_lo, E_loc, c_lo, C_loc = route.meta["e_lo"], route.meta["E_loc"], route.meta["c_lo"], route.meta["C_loc"]
         B, S, d = x.t.shape
-        out = Val("expert", self._new((E_loc, B, C, d)), shape=(B, E_loc, C, d), needs_grad=True)
-        self.fwd.append(lambda: ops.moe_dispatch(x.t, r, out.t, E, C, e_lo, E_loc))
+        out = Val("expert", self._new((E_loc, B, C_loc, d)), shape=(B, E_loc, C_loc, d), needs_grad=True)
+        self.fwd.append(lambda: ops.moe_dispatch(x.t, r, out.t, E, C, e_lo, E_loc, c_lo, C_loc))
 
         def emit():
             if out.grad is None or not x.needs_grad:
                 return
             gx, acc = self._grad_slot(x)
-            self.bwd.append(lambda: ops.moe_dispatch_bwd(out.grad, r, gx, C, e_lo, E_loc, acc))
+            self.bwd.append(lambda: ops.moe_dispatch_bwd(out.grad, r, gx, C, e_lo, E_loc, acc, c_lo, C_loc))
         self._tape.append(emit)
         return out
 
@@ -1684,6 +1692,9 @@ class ShardExecutor:
         El, B, C, Kx = x.t.shape
         if El != E_loc or Kx != K:
             self._unsupported(node, "expert weight / activation shapes do not match")
+        if K % self.epv or N % self.epv:
+            self._unsupported(node, f"expert weight [{K}, {N}]: both extents must be multiples of {self.epv} "
+                                    f"(rows of 16-byte vectors); pick shard widths accordingly")
         M = B * C
         fuse = self._wants_fused_relu(node)
         out = Val("expert", self._new((E_loc, B, C, N)), shape=(B, E_loc, C, N), needs_grad=True)
@@ -1721,11 +1732,14 @@ class ShardExecutor:
             self._unsupported(node, "expects (expert outputs, combine tensor of top_2_gating)")
         gv = route.meta["gating"]
         r, E, C = gv.meta["r"], gv.meta["E"], gv.meta["C"]
-        e_lo, E_loc = route.meta["e_lo"], route.meta["E_loc"]
-        _, B, _, d = eo.t.shape
+        e_lo, E_loc, c_lo, C_loc = route.meta["e_lo"], route.meta["E_loc"], route.meta["c_lo"], route.meta["C_loc"]
+        El, B, Cl, d = eo.t.shape
+        if (El, Cl) != (E_loc, C_loc):
+            self._unsupported(node, f"expert outputs [{El} experts, {Cl} slots] do not match the combine tensor's "
+                                    f"window [{E_loc}, {C_loc}]")
         S = r["index"].shape[1]
         out = Val("tensor", self._new((B, S, d)), needs_grad=True)
-        self.fwd.append(lambda: ops.moe_combine(eo.t, r, out.t, C, e_lo, E_loc))
+        self.fwd.append(lambda: ops.moe_combine(eo.t, r, out.t, C, e_lo, E_loc, c_lo, C_loc))
 
         def emit():
             if out.grad is None:
@@ -1735,7 +1749,7 @@ class ShardExecutor:
             eo.grad = self._new(eo.t.shape)
             gv.meta["dgate_used"] = True
             g, dgate = eo.grad, gv.meta["dgate"]
-            self.bwd.append(lambda: ops.moe_combine_bwd(out.grad, eo.t, r, g, dgate, E, C, e_lo, E_loc))
+            self.bwd.append(lambda: ops.moe_combine_bwd(out.grad, eo.t, r, g, dgate, E, C, e_lo, E_loc, c_lo, C_loc))
         self._tape.append(emit)
         return out
 

@@ -1120,51 +1120,66 @@ def top2_densify(r, E, C):
     return dispatch, combine
 
 
-def moe_dispatch(x, r, expert_in, E, C, e_lo, E_loc):
+def _capacity_window(C, c_lo, C_loc):
+    """(c_lo, C_loc) of the device's capacity slots; None = all of them."""
+    c_lo = 0 if c_lo is None else int(c_lo)
+    C_loc = C - c_lo if C_loc is None else int(C_loc)
+    if c_lo < 0 or C_loc < 0 or c_lo + C_loc > C:
+        raise _lib.HapmiError(f"capacity window [{c_lo}, {c_lo + C_loc}) outside [0, {C})")
+    return c_lo, C_loc
+
+
+def moe_dispatch(x, r, expert_in, E, C, e_lo, E_loc, c_lo=None, C_loc=None):
+    """einsum "bsd,bsec->becd" on the experts [e_lo, e_lo + E_loc) and capacity slots [c_lo, c_lo + C_loc) of the
+    routing ``r``: expert_in[E_loc, B, C_loc, d]."""
     B, S, d = x.shape
     _dev(x, expert_in)
     _check_routing(r, B, S, E, C)
-    _need(expert_in, E_loc * B * C * d, "moe_dispatch expert_in")
+    c_lo, C_loc = _capacity_window(C, c_lo, C_loc)
+    _need(expert_in, E_loc * B * C_loc * d, "moe_dispatch expert_in")
     if expert_in.dtype != x.dtype or not x.is_contiguous():
         raise TypeError("moe_dispatch: dtype / layout mismatch")
     check(lib().hapmi_moe_dispatch(_ptr(x), _ptr(r["token_of_slot"]), _ptr(expert_in), B, S, E, C, d, e_lo, E_loc,
-                                   dtype_code(x), _stream()))
+                                   c_lo, C_loc, dtype_code(x), _stream()))
 
 
-def moe_combine(expert_out, r, out, C, e_lo, E_loc):
+def moe_combine(expert_out, r, out, C, e_lo, E_loc, c_lo=None, C_loc=None):
     B, S, d = out.shape
     _dev(expert_out, out)
     _check_routing(r, B, S)
-    _need(expert_out, E_loc * B * C * d, "moe_combine expert_out")
+    c_lo, C_loc = _capacity_window(C, c_lo, C_loc)
+    _need(expert_out, E_loc * B * C_loc * d, "moe_combine expert_out")
     if expert_out.dtype != out.dtype or not out.is_contiguous():
         raise TypeError("moe_combine: dtype / layout mismatch")
     check(lib().hapmi_moe_combine(_ptr(expert_out), _ptr(r["index"]), _ptr(r["slot"]), _ptr(r["gate"]), _ptr(out),
-                                  B, S, C, d, e_lo, E_loc, dtype_code(out), _stream()))
+                                  B, S, C, d, e_lo, E_loc, c_lo, C_loc, dtype_code(out), _stream()))
 
 
-def moe_combine_bwd(dout, expert_out, r, d_expert_out, dgate, E, C, e_lo, E_loc):
+def moe_combine_bwd(dout, expert_out, r, d_expert_out, dgate, E, C, e_lo, E_loc, c_lo=None, C_loc=None):
     B, S, d = dout.shape
     _dev(dout, expert_out, d_expert_out, dgate)
     _check_routing(r, B, S, E, C)
-    _need(expert_out, E_loc * B * C * d, "moe_combine_bwd expert_out")
-    _need(d_expert_out, E_loc * B * C * d, "moe_combine_bwd d_expert_out")
+    c_lo, C_loc = _capacity_window(C, c_lo, C_loc)
+    _need(expert_out, E_loc * B * C_loc * d, "moe_combine_bwd expert_out")
+    _need(d_expert_out, E_loc * B * C_loc * d, "moe_combine_bwd d_expert_out")
     _need(dgate, B * S * 2, "moe_combine_bwd dgate")
     if not (expert_out.dtype == d_expert_out.dtype == dout.dtype) or dgate.dtype != torch.float32:
         raise TypeError("moe_combine_bwd: dtype mismatch")
     check(lib().hapmi_moe_combine_bwd(_ptr(dout), _ptr(expert_out), _ptr(r["index"]), _ptr(r["slot"]), _ptr(r["gate"]),
                                       _ptr(r["token_of_slot"]), _ptr(d_expert_out), _ptr(dgate), B, S, E, C, d, e_lo,
-                                      E_loc, dtype_code(dout), _stream()))
+                                      E_loc, c_lo, C_loc, dtype_code(dout), _stream()))
 
 
-def moe_dispatch_bwd(d_expert_in, r, dx, C, e_lo, E_loc, accumulate):
+def moe_dispatch_bwd(d_expert_in, r, dx, C, e_lo, E_loc, accumulate, c_lo=None, C_loc=None):
     B, S, d = dx.shape
     _dev(d_expert_in, dx)
     _check_routing(r, B, S)
-    _need(d_expert_in, E_loc * B * C * d, "moe_dispatch_bwd d_expert_in")
+    c_lo, C_loc = _capacity_window(C, c_lo, C_loc)
+    _need(d_expert_in, E_loc * B * C_loc * d, "moe_dispatch_bwd d_expert_in")
     if d_expert_in.dtype != dx.dtype or not dx.is_contiguous():
         raise TypeError("moe_dispatch_bwd: dtype / layout mismatch")
     check(lib().hapmi_moe_dispatch_bwd(_ptr(d_expert_in), _ptr(r["index"]), _ptr(r["slot"]), _ptr(r["gate"]), _ptr(dx),
-                                       B, S, C, d, e_lo, E_loc, int(accumulate), dtype_code(dx), _stream()))
+                                       B, S, C, d, e_lo, E_loc, c_lo, C_loc, int(accumulate), dtype_code(dx), _stream()))
 
 
 # ---------------------------------------------------------------------------

@@ -214,10 +214,29 @@ def _moe_ffn(e: _Emitter, h1, prefix: str, emsize: int, n_expert: int, capacity:
     routed = e.call(gating, tokens, n_expert, capacity, e.replicated(prefix + "gate_weight"))
     dispatch = e.call(operator.getitem, routed, 0)
     combine = e.call(operator.getitem, routed, 1)
-    dispatch = e.call(collectives.dynamic_slice, dispatch, 2, L_E, e.rank)
-    combine = e.call(collectives.dynamic_slice, combine, 2, L_E, e.rank)
-    w1 = e.sharded(prefix + "w1", n_expert, 0)
-    w2 = e.sharded(prefix + "w2", n_expert, 0)
+    if e.plan.moe == "experts":
+        # expert split: (identity, gather(1, 2)) -> gather(0, 1) / (gather(0, 0), gather(1, 1)) -> gather(0, 1) /
+        # (gather(0, 1), gather(1, 2)) -> reduce (hap.rs:3316-3320, 3333-3337, 3363-3367, 3393-3397)
+        dispatch = e.call(collectives.dynamic_slice, dispatch, 2, L_E, e.rank)
+        combine = e.call(collectives.dynamic_slice, combine, 2, L_E, e.rank)
+        w1 = e.sharded(prefix + "w1", n_expert, 0)
+        w2 = e.sharded(prefix + "w2", n_expert, 0)
+    elif e.plan.moe == "capacity":
+        # capacity split: (identity, gather(1, 3)) -> gather(0, 2) / (identity, gather(1, 2)) -> gather(0, 2) /
+        # (gather(0, 2), gather(1, 3)) -> reduce (hap.rs:3322-3326, 3357-3361, 3387-3391, 3399-3403)
+        L_C = e.plan.lengths(capacity)
+        dispatch = e.call(collectives.dynamic_slice, dispatch, 3, L_C, e.rank)
+        combine = e.call(collectives.dynamic_slice, combine, 3, L_C, e.rank)
+        w1 = e.replicated(prefix + "w1")
+        w2 = e.replicated(prefix + "w2")
+    elif e.plan.moe == "hidden":
+        # feature split of the expert FFN: (gather(0, 2), identity) -> gather(0, 3) for the first product,
+        # (gather(0, 1), gather(1, 3)) -> reduce for the second (hap.rs:3345-3349, 3369-3373)
+        nhid = e._shape(prefix + "w1")[2]
+        w1 = e.sharded(prefix + "w1", nhid, 2)
+        w2 = e.sharded(prefix + "w2", nhid, 1)
+    else:
+        raise ValueError(f"unknown MoE split {e.plan.moe!r}")
     x = e.call(torch.einsum, "bsd,bsec->becd", tokens, dispatch)
     x = e.call(torch.einsum, "edh,becd->bech", w1, x)
     x = e.g.call_function(F.relu, (x,), {"inplace": False})

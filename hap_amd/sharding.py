@@ -79,6 +79,11 @@ class ShardingPlan:
                                  # hap.rs:2795, 3061, 3214-3218, 2996; attention needs the whole sequence)
     embedding: str = "rows"      # "rows": ids sharded, table whole; "features": ids whole, table sharded on dim 1,
                                  # output gathered on dim 2 (hap.rs:3220-3224), then all_gather + dynamic_slice
+    moe: str = "experts"         # how the four MoE einsums are split (hap.rs:3285-3419): "experts": dispatch / combine
+                                 # tensors sliced on dim 2, expert weights on dim 0; "capacity": dispatch / combine
+                                 # sliced on dim 3 (every device takes a range of every expert's slots), expert weights
+                                 # whole; "hidden": routing whole, first expert weight sliced on dim 2 and the second on
+                                 # dim 1 (a feature split of the expert FFN; the second product is a partial sum)
 
     @property
     def world_size(self) -> int:

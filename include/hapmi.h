@@ -344,26 +344,31 @@ int hapmi_top2_gate_bwd(const float *probs, const int32_t *index, const int32_t 
 /* dense [B, S, E, C] tensors exactly as models.py:495-500 lays them out */
 int hapmi_top2_densify(const int32_t *index, const int32_t *slot, const float *gate, float *dispatch,
                        float *combine, int64_t B, int64_t S, int64_t E, int64_t C, hapmi_stream_t stream);
-/* einsum "bsd,bsec->becd" with the local expert range [e_lo, e_lo + E_loc) (hap.rs:2273,
- * models.py:356) as a row gather; expert-major output expert_in[E_loc, B, C, d] */
+/* The four MoE einsums (hap.rs:2273, models.py:356-364) on index-form routing.  The device's share of the dense
+ * [B, S, E, C] dispatch / combine tensors is a window of experts [e_lo, e_lo + E_loc) (the expert split of the
+ * einsums, hap.rs:3316-3320, 3333-3337, 3399-3403) and of capacity slots [c_lo, c_lo + C_loc) (the capacity split,
+ * hap.rs:3322-3326, 3357-3361, 3405-3409): dynamic_slice of the gating outputs along dim 2 / dim 3.  Expert-major
+ * activations are [E_loc, B, C_loc, d]; the whole tensor is e_lo = c_lo = 0, E_loc = E, C_loc = C.
+ *
+ * einsum "bsd,bsec->becd" as a row gather into expert_in[E_loc, B, C_loc, d] */
 int hapmi_moe_dispatch(const void *x, const int32_t *token_of_slot, void *expert_in, int64_t B, int64_t S,
-                       int64_t E, int64_t C, int64_t d, int64_t e_lo, int64_t E_loc, int dtype,
-                       hapmi_stream_t stream);
+                       int64_t E, int64_t C, int64_t d, int64_t e_lo, int64_t E_loc, int64_t c_lo, int64_t C_loc,
+                       int dtype, hapmi_stream_t stream);
 /* einsum "becd,bsec->bsd" (models.py:364) as a weighted row gather:
- * out[b, s, :] = sum_k gate_k * expert_out[e_k - e_lo, b, slot_k, :] over kept local choices */
+ * out[b, s, :] = sum_k gate_k * expert_out[e_k - e_lo, b, slot_k - c_lo, :] over kept choices inside the window */
 int hapmi_moe_combine(const void *expert_out, const int32_t *index, const int32_t *slot, const float *gate,
                       void *out, int64_t B, int64_t S, int64_t C, int64_t d, int64_t e_lo, int64_t E_loc,
-                      int dtype, hapmi_stream_t stream);
+                      int64_t c_lo, int64_t C_loc, int dtype, hapmi_stream_t stream);
 /* backward of combine: d_expert_out[e, b, c, :] = gate * dout[b, token, :] (0 for empty slots);
- * dgate[b, s, k] = <dout[b, s, :], expert_out[e_k - e_lo, b, slot_k, :]> (0 if not kept / not local) */
+ * dgate[b, s, k] = <dout[b, s, :], expert_out[e_k - e_lo, b, slot_k - c_lo, :]> (0 if not kept / outside the window) */
 int hapmi_moe_combine_bwd(const void *dout, const void *expert_out, const int32_t *index, const int32_t *slot,
                           const float *gate, const int32_t *token_of_slot, void *d_expert_out, float *dgate,
                           int64_t B, int64_t S, int64_t E, int64_t C, int64_t d, int64_t e_lo, int64_t E_loc,
-                          int dtype, hapmi_stream_t stream);
-/* backward of dispatch: dx[b, s, :] (+)= sum_k d_expert_in[e_k - e_lo, b, slot_k, :] */
+                          int64_t c_lo, int64_t C_loc, int dtype, hapmi_stream_t stream);
+/* backward of dispatch: dx[b, s, :] (+)= sum_k d_expert_in[e_k - e_lo, b, slot_k - c_lo, :] */
 int hapmi_moe_dispatch_bwd(const void *d_expert_in, const int32_t *index, const int32_t *slot, const float *gate,
                            void *dx, int64_t B, int64_t S, int64_t C, int64_t d, int64_t e_lo, int64_t E_loc,
-                           int accumulate, int dtype, hapmi_stream_t stream);
+                           int64_t c_lo, int64_t C_loc, int accumulate, int dtype, hapmi_stream_t stream);
 
 /* ---- optimizer (worker.py:47, 74-76; profiler.py:18) --------------------
  * Flat float32 master parameters and gradients; `shadow` (bf16 copy of the

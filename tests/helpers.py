@@ -59,7 +59,7 @@ def rank_programs(model, ratios, B, **kw):
         m = copy.deepcopy(model)
         plan = hap_amd.ShardingPlan([list(ratios)], r, ffn=kw.get("ffn", "column"), zero=kw.get("zero", False),
                                      attn=kw.get("attn", "batch"), shard_dim=kw.get("shard_dim", "batch"),
-                                     embedding=kw.get("embedding", "rows"))
+                                     embedding=kw.get("embedding", "rows"), moe=kw.get("moe", "experts"))
         progs.append(hap_amd.build_program(m, plan, B, activation=kw.get("activation", "relu"),
                                            batch_sharded=kw.get("batch_sharded", True)))
     return progs

@@ -40,7 +40,7 @@ def _gpu_rank(model, ratios, rank, B, x, y, log, dtype, opt, **kw):
     m = copy.deepcopy(model)
     plan = hap_amd.ShardingPlan([list(ratios)], rank, ffn=kw.get("ffn", "column"), zero=kw.get("zero", False),
                                 attn=kw.get("attn", "batch"), shard_dim=kw.get("shard_dim", "batch"),
-                                embedding=kw.get("embedding", "rows"))
+                                embedding=kw.get("embedding", "rows"), moe=kw.get("moe", "experts"))
     gm = hap_amd.build_program(m, plan, B, activation=kw.get("activation", "relu"),
                                batch_sharded=kw.get("batch_sharded", True))
     ex = hap_amd.compile_program(gm, [x, y], dtype=dtype, wire=hap_amd.ReplayWire(log, rank), rank=rank,
@@ -165,6 +165,20 @@ def test_switch_moe(cuda, dtype, batch_sharded):
     B = 16 if batch_sharded else 4
     x, y = lm_batch(B, 16, 61)
     _compare(model, RATIOS_E, B, x, y, dtype, [0, 2], ADAM, ffn="batch", batch_sharded=batch_sharded)
+
+
+@pytest.mark.parametrize("moe,dtype,batch_sharded", [("capacity", "fp32", True), ("capacity", "fp32", False),
+                                                      ("capacity", "bf16", False), ("hidden", "fp32", True),
+                                                      ("hidden", "bf16", False)])
+def test_moe_capacity_and_hidden_splits(cuda, moe, dtype, batch_sharded):
+    """The capacity split (dispatch / combine tensors sliced on dim 3, whole expert weights: every device works on
+    a range of every expert's slots) and the hidden-feature split of the expert FFN (hap.rs:3285-3419), uneven over
+    the devices, against the CPU run of all ranks."""
+    # hidden widths 40 / 40 / 24 / 24 of 128 (multiples of the 16-byte vector in either type), capacity slots 3 / 3 / 2 / 2
+    model = make_moe(C=10, F=128) if dtype == "fp32" else make_moe(d=64, F=128, C=10, std=0.3)
+    B = 16 if batch_sharded else 4
+    x, y = lm_batch(B, 16, 61)
+    _compare(model, RATIOS_E, B, x, y, dtype, [0, 2], ADAM, ffn="batch", batch_sharded=batch_sharded, moe=moe)
 
 
 def test_moe_bf16_routing_matches(cuda):

@@ -212,3 +212,19 @@ def test_feature_sharded_embedding_table_spmd_equals_single_device(ffn):
             sharded[f"layers.{i}.linear1.weight"] = (0, L_F)
             sharded[f"layers.{i}.linear1.bias"] = (0, L_F)
     _check(model, run, x, y, sharded)
+
+
+@pytest.mark.parametrize("moe", ["capacity", "hidden"])
+def test_moe_capacity_and_hidden_splits_spmd_equal_single_device(moe):
+    """The other legal splits of the four MoE einsums (hap.rs:3285-3419): every device takes a range of every
+    expert's capacity slots with whole expert weights, or every device holds a slice of the experts' hidden
+    features; batch-sharded attention around them as in the expert split."""
+    model = make_moe(C=10, F=48)                                # capacity slots 3 / 3 / 2 / 2, hidden widths 15 / 15 / 9 / 9
+    B = 16
+    x, y = lm_batch(B, 16, 61)
+    run = joint_cpu(model, RATIOS_E, B, ffn="batch", moe=moe)
+    sharded = {}
+    if moe == "hidden":
+        L_F = hap_amd.sharding_lengths(48, RATIOS_E)
+        sharded = {"layers.1.w1": (2, L_F), "layers.1.w2": (1, L_F)}
+    _check(model, run, x, y, sharded)
