@@ -149,7 +149,7 @@ template <bool CAUSAL> struct BlockOrder {
 // CAUSAL: key j is visible to query i iff j <= i (the additive mask torch.triu(full(-inf), 1), models.py:76),
 // applied arithmetically; kv tiles that lie completely above the diagonal of the block's 128 queries are skipped.
 template <bool CAUSAL>
-__global__ __launch_bounds__(AT_THREADS, 2) void attn_fwd_kernel(const bf16_t *qkv, const float *mask, bf16_t *out,
+__global__ __launch_bounds__(AT_THREADS, 3) void attn_fwd_kernel(const bf16_t *qkv, const float *mask, bf16_t *out,
                                                             float *lse, int S, int H, float scale) {
     __shared__ __attribute__((aligned(16))) char Ks2[2][TILE_BYTES];   // two tiles each: the next tile is written while
     __shared__ __attribute__((aligned(16))) char Vs2[2][TILE_BYTES];   // the current one is read (one barrier per tile)
