@@ -121,6 +121,39 @@ struct PairLoader {
     }
 };
 
+// One [64 rows][64 d] operand tile global -> LDS without a stop in registers (global_load_lds_dwordx4: every wave
+// instruction fills 1024 contiguous LDS bytes = 8 tile rows, lane l landing in row l / 8, 16-byte slot l % 8).  The
+// tile's swizzle is applied on the global side: the lane fetches the chunk that belongs in its slot.  Rows beyond the
+// operand's end repeat its last row (finite values; the callers give such keys a probability of zero), since a
+// transfer cannot be zero-filled.  The transfers are asynchronous: the caller counts them with s_waitcnt vmcnt (a
+// wave's loads complete in issue order) and publishes the tile with a barrier.
+struct DirectTileLoader {
+    static constexpr int LOADS = 2;                            // wave instructions per tile (64 rows / 4 waves / 8 rows)
+    int row[LOADS], chunk[LOADS], ld;
+    __device__ __forceinline__ DirectTileLoader(int ld_) : ld(ld_) {
+        const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+#pragma unroll
+        for (int i = 0; i < LOADS; ++i) {
+            row[i] = (i * 4 + wave) * 8 + (lane >> 3);
+            chunk[i] = ((lane & 7) ^ aswz(row[i])) * 8;
+        }
+    }
+    __device__ __forceinline__ void issue(const bf16_t *base, int rows_left, char *lds_tile) const {
+        typedef __attribute__((address_space(3))) char lds_char;
+        const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+#pragma unroll
+        for (int i = 0; i < LOADS; ++i) {
+            const int r = row[i] < rows_left ? row[i] : rows_left - 1;
+            const bf16_t *src = base + r * ld + chunk[i];
+            const uint32_t lds_addr = (uint32_t)(uintptr_t)(lds_char *)(lds_tile + (i * 4 + wave) * 1024);
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                         :
+                         : "s"(lds_addr), "v"(src)
+                         : "memory");
+        }
+    }
+};
+
 // ---------------------------------------------------------------------------------------------
 // forward
 // ---------------------------------------------------------------------------------------------
@@ -151,8 +184,10 @@ template <bool CAUSAL> struct BlockOrder {
 template <bool CAUSAL>
 __global__ __launch_bounds__(AT_THREADS, 3) void attn_fwd_kernel(const bf16_t *qkv, const float *mask, bf16_t *out,
                                                             float *lse, int S, int H, float scale) {
-    __shared__ __attribute__((aligned(16))) char Ks2[2][TILE_BYTES];   // two tiles each: the next tile is written while
-    __shared__ __attribute__((aligned(16))) char Vs2[2][TILE_BYTES];   // the current one is read (one barrier per tile)
+    // three K and three V tiles: one is multiplied while the next two are on their way global -> LDS
+    constexpr int NST = 3;
+    __shared__ __attribute__((aligned(16))) char Ks3[NST][TILE_BYTES];
+    __shared__ __attribute__((aligned(16))) char Vs3[NST][TILE_BYTES];
     const TransposedReader tr;
     const int E = H * HD, ld = 3 * E;
     const int blk = BlockOrder<CAUSAL>::row_block(true), bh = BlockOrder<CAUSAL>::batch_head();
@@ -169,7 +204,7 @@ __global__ __launch_bounds__(AT_THREADS, 3) void attn_fwd_kernel(const bf16_t *q
 
     f32x16 ot[2] = {zero16(), zero16()};
     float m = -INFINITY, lsum = 0.f;
-    PairLoader lk(ld), lv(ld);
+    const DirectTileLoader ldr(ld);
     const bool vec_mask = mask && ((S & 3) == 0);
     // Softmax is VALU work next to the MFMAs (32 scores per lane and kv tile), so the common tile (no additive
     // mask, every query and key of the tile valid and, if causal, visible) takes a short path: maximum over the raw
@@ -177,22 +212,33 @@ __global__ __launch_bounds__(AT_THREADS, 3) void attn_fwd_kernel(const bf16_t *q
     const float sl2 = scale * LOG2E;
     const bool plain_block = !mask && blk * 128 + 128 <= S;
 
-    // Tile i + 1 travels global -> registers while tile i is multiplied and is written to the other LDS buffer at the
-    // end of iteration i (its loads have had the whole iteration to arrive); tile i + 2's loads are issued right after.
+    // K / V tiles go global -> LDS directly, two tiles ahead of the one that is multiplied: a tile's transfers have
+    // two iterations to arrive (the tiles come from the memory-side cache or HBM the first time an XCD touches them,
+    // which takes longer than one iteration).  A wave's transfers complete in issue order, so tile i has landed once
+    // at most the 2 x LOADS transfers of tile i + 1 are outstanding; the barrier then publishes every wave's part and
+    // tells that everyone is done with tile i - 1, whose buffers take tile i + 2.
     const int q_blk_end = blk * 128 + 128;
     const int kv_end = (CAUSAL && q_blk_end < S) ? q_blk_end : S;
-    lk.load(K, S);
-    lv.load(V, S);
-    lk.store_rows(Ks2[0]);
-    lv.store_rows(Vs2[0]);
-    if (TILE < kv_end) {
-        lk.load(K + (int64_t)TILE * ld, S - TILE);
-        lv.load(V + (int64_t)TILE * ld, S - TILE);
-    }
-    __syncthreads();
+    constexpr int PER_TILE = 2 * DirectTileLoader::LOADS;
+    static_assert(PER_TILE == 4, "the wait below is written for four transfers per tile");
+    auto issue_tile = [&](int kv0, int bufi) {
+        ldr.issue(K + (int64_t)kv0 * ld, S - kv0, Ks3[bufi]);
+        ldr.issue(V + (int64_t)kv0 * ld, S - kv0, Vs3[bufi]);
+    };
+    issue_tile(0, 0);
+    if (TILE < kv_end) issue_tile(TILE, 1);
+    // The query fragments are consumed here, before the loop: otherwise the wait for their loads would sit at their
+    // first use inside the loop body, as a wait for ALL outstanding loads in every iteration (the compiler does not
+    // count the transfers above), and no tile would ever be in flight across an iteration.
+#pragma unroll
+    for (int s = 0; s < 4; ++s) asm volatile("" : "+v"(qf[s].v));
     int buf = 0;
     for (int kv0 = 0; kv0 < kv_end; kv0 += TILE) {
-        const char *Ks = Ks2[buf], *Vs = Vs2[buf];
+        if (kv0 + TILE < kv_end) __builtin_amdgcn_s_waitcnt(0x0F74);   // vmcnt(4): only tile i + 1 may be outstanding
+        else __builtin_amdgcn_s_waitcnt(0x0F70);                       // vmcnt(0)
+        __syncthreads();
+        if (kv0 + 2 * TILE < kv_end) issue_tile(kv0 + 2 * TILE, buf == 0 ? 2 : buf - 1);
+        const char *Ks = Ks3[buf], *Vs = Vs3[buf];
         // all fragment reads of the tile are issued before the first MFMA waits for one
         frag_t kf[2][4];
 #pragma unroll
@@ -280,16 +326,7 @@ __global__ __launch_bounds__(AT_THREADS, 3) void attn_fwd_kernel(const bf16_t *q
 #pragma unroll
             for (int u = 0; u < 2; ++u) ot[u] = mma(tr.frag(Vs, u * 32, s), pb, ot[u]);
         }
-        if (kv0 + TILE < kv_end) {
-            lk.store_rows(Ks2[buf ^ 1]);                   // last read in the iteration before this one
-            lv.store_rows(Vs2[buf ^ 1]);
-            if (kv0 + 2 * TILE < kv_end) {
-                lk.load(K + (int64_t)(kv0 + 2 * TILE) * ld, S - kv0 - 2 * TILE);
-                lv.load(V + (int64_t)(kv0 + 2 * TILE) * ld, S - kv0 - 2 * TILE);
-            }
-        }
-        __syncthreads();
-        buf ^= 1;
+        buf = buf == NST - 1 ? 0 : buf + 1;
     }
     const float l = lsum + __shfl_xor(lsum, 32, 64);
     const float inv = l > 0.f ? 1.0f / l : 0.f;
