@@ -32,6 +32,7 @@ HAPMI_GEMM_DECLARE_CFG(8);
 HAPMI_GEMM_DECLARE_CFG(9);
 HAPMI_GEMM_DECLARE_CFG(10);
 HAPMI_GEMM_DECLARE_CFG(11);
+HAPMI_GEMM_DECLARE_CFG(12);
 
 namespace {
 
@@ -41,9 +42,10 @@ struct TileCfg {
 };
 constexpr TileCfg kCfg[] = {{128, 128, 2, 2}, {256, 256, 2, 4}, {384, 192, 4, 2}, {192, 256, 2, 4}, {256, 192, 4, 2},
                              {256, 128, 4, 2}, {128, 256, 2, 4}, {192, 128, 2, 4}, {256, 128, 2, 2}, {128, 192, 4, 2},
-                             {64, 64, 2, 2}, {64, 128, 2, 2}};
-constexpr int kNumCfg = 12;
-constexpr int kFirstF32Cfg = 10;                 // 10, 11: small tiles for float32 operands only
+                             {64, 64, 2, 2}, {64, 128, 2, 2}, {192, 128, 2, 4}};
+constexpr int kNumCfg = 13;
+constexpr int kProbeCfg = 12;                    // operand movement only: a measurement build, never chosen automatically
+constexpr bool is_f32_cfg(int c) { return c == 10 || c == 11; }   // small tiles for float32 operands only
 constexpr int kNumCU = 256;
 int g_force_cfg = -1;
 int g_force_splits = 0;
@@ -84,20 +86,21 @@ struct Choice {
 };
 
 // Which tile configurations a call may use: 0 serves every type; 1..9 bf16 operands of calls that allow the large
-// tiles; 10, 11 float32 operands.
+// tiles; 10, 11 float32 operands; 12 only when forced (a measurement build).
 // A call with operands in pieces narrows the choice further (SegNeeds): A in pieces along K runs on the three-stage
 // configurations only, and the tile's N extent must divide every piece boundary of B / C.
 struct SegNeeds {
     bool three_stage = false;
     int64_t n_align = 0;                       // 0: no constraint; else every piece boundary along N is a multiple of it
 };
-constexpr bool kThreeStage[] = {false, false, false, false, false, true, true, true, true, true, false, false};
+constexpr bool kThreeStage[] = {false, false, false, false, false, true, true, true, true, true, false, false, true};
 
 bool cfg_eligible(int c, bool bf16_in, bool wide, bool row_major_operands, bool forced, const SegNeeds &need = SegNeeds()) {
     if (need.three_stage && !kThreeStage[c]) return false;
     if (need.n_align > 0 && need.n_align % kCfg[c].bn != 0) return false;
     if (c == 0) return true;
-    if (c >= kFirstF32Cfg) return !bf16_in;
+    if (c == kProbeCfg) return forced && bf16_in;
+    if (is_f32_cfg(c)) return !bf16_in;
     if (!bf16_in || !wide) return false;
     if (c == 2 && !row_major_operands && !forced) return false;          // 384x192 with a transposing loader spills registers
     return true;
@@ -273,6 +276,7 @@ int launch_typed(GemmParams &p, int transA, int transB, int64_t batch, hipStream
         case 9: rc = hapmi_gemm_launch_cfg9(p, in_dtype, out_dtype, transA, transB, batch, st); break;
         case 10: rc = hapmi_gemm_launch_cfg10(p, in_dtype, out_dtype, transA, transB, batch, st); break;
         case 11: rc = hapmi_gemm_launch_cfg11(p, in_dtype, out_dtype, transA, transB, batch, st); break;
+        case 12: rc = hapmi_gemm_launch_cfg12(p, in_dtype, out_dtype, transA, transB, batch, st); break;
         default: rc = hapmi_gemm_launch_cfg0(p, in_dtype, out_dtype, transA, transB, batch, st);
     }
     if (rc) return rc;
@@ -506,6 +510,7 @@ extern "C" int hapmi_gemm_plan_set(int64_t M, int64_t N, int64_t K, int64_t batc
     HAPMI_REQUIRE(hapmi_dtype_ok(in_dtype) && hapmi_dtype_ok(out_dtype), HAPMI_EINVAL, "gemm_plan_set: bad dtype");
     HAPMI_REQUIRE(tile_config < kNumCfg && k_splits >= 1 && k_splits <= 64, HAPMI_EINVAL,
                   "gemm_plan_set: configuration %d / splits %d out of range", tile_config, k_splits);
+    HAPMI_REQUIRE(tile_config != kProbeCfg, HAPMI_EINVAL, "gemm_plan_set: configuration %d multiplies nothing (a measurement build) and cannot be pinned", kProbeCfg);
     const PlanKey key(M, N, K, batch, (int)(transA != 0), (int)(transB != 0), in_dtype, out_dtype);
     std::lock_guard<std::mutex> lk(g_plans_mu);
     if (tile_config < 0) g_plans.erase(key);

@@ -215,7 +215,9 @@ int hapmi_gemm(const hapmi_gemm_args *args_host, hapmi_stream_t stream);
  * Tuning hook for measurements: force tile configuration `tile_config` (block tile / waves: 0: 128x128 / 2x2,
  * 1: 256x256 / 2x4, 2: 384x192 / 4x2, 3: 192x256 / 2x4, 4: 256x192 / 4x2, 5: 256x128 / 4x2, 6: 128x256 / 2x4,
  * 7: 192x128 / 2x4, 8: 256x128 / 2x2, 9: 128x192 / 4x2, 10: 64x64 / 2x2, 11: 64x128 / 2x2; 5..9 keep three
- * k-tiles in LDS (two in flight); 1..9 take bf16 operands only, 10 and 11 float32 operands only; a configuration
+ * k-tiles in LDS (two in flight); 1..9 take bf16 operands only, 10 and 11 float32 operands only; 12 is a measurement
+ * build of 7 for bf16 operands and results with transA = 0: it moves the operands of every k-tile into LDS
+ * but multiplies nothing (the result is zeros), so its time is the cost of the operand movement alone; a configuration
  * that does not fit the call's operand type is ignored; -1 = automatic) and `k_splits` (0 = automatic). */
 int hapmi_gemm_tuning(int tile_config, int k_splits);
 

@@ -753,3 +753,33 @@ def test_gemm_pieces_are_checked(cuda):
     with pytest.raises(HapmiError, match="bf16"):
         ops.gemm(None, torch.zeros(32, 256, device=cuda), torch.zeros(64, 32, device=cuda), 64, 32, 256, transB=True,
                  a_segments=[f, f])
+
+
+def test_gemm_operand_movement_only_configuration(cuda):
+    """Tile configuration 12 is a measurement build: it runs the operand movement of configuration 7 and multiplies
+    nothing.  It is reachable through hapmi_gemm_tuning only (result: zeros), refuses layouts and types it has no
+    build for, cannot be pinned as a plan, and leaves the automatic choice untouched."""
+    from hap_amd._lib import lib, HapmiError
+    g = torch.Generator().manual_seed(3)
+    M, N, K = 384, 256, 512
+    A = torch.randn(M, K, generator=g).bfloat16().to(cuda)
+    B = torch.randn(N, K, generator=g).bfloat16().to(cuda)
+    want = A.double().cpu() @ B.double().cpu().t()
+    try:
+        lib().hapmi_gemm_tuning(ops.OPERAND_MOVEMENT_ONLY_CONFIG, 1)
+        C = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=cuda)
+        ops.gemm(A, B, C, M, N, K, transB=True)
+        assert (C == 0).all()
+        Bn = B.t().contiguous()
+        C.fill_(float("nan"))
+        ops.gemm(A, Bn, C, M, N, K)
+        assert (C == 0).all()
+        Cf = torch.empty(M, N, dtype=torch.float32, device=cuda)
+        with pytest.raises(HapmiError):
+            ops.gemm(A, B, Cf, M, N, K, transB=True)
+    finally:
+        lib().hapmi_gemm_tuning(-1, 0)
+    assert lib().hapmi_gemm_plan_set(M, N, K, 1, 0, 1, 1, 1, ops.OPERAND_MOVEMENT_ONLY_CONFIG, 1) != 0
+    C = torch.empty(M, N, dtype=torch.bfloat16, device=cuda)
+    ops.gemm(A, B, C, M, N, K, transB=True)
+    close(C, want, torch.bfloat16, scale=2.0)
