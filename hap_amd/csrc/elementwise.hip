@@ -441,7 +441,7 @@ __global__ __launch_bounds__(EW_THREADS) void append_cls_pos_kernel(const T *pat
     for (int64_t i = (int64_t)blockIdx.x * EW_THREADS + threadIdx.x; i < total; i += step) {
         const int64_t n = i / (T1 * d), r = i - n * T1 * d, t = r / d, c = r - t * d;
         const float v = t == 0 ? ld_f(cls, c) : ld_f(patches, (n * (T1 - 1) + (t - 1)) * d + c);
-        st_f(out, i, v + ld_f(pos, t * d + c));
+        st_f(out, i, pos ? v + ld_f(pos, t * d + c) : v);
     }
 }
 
@@ -463,7 +463,7 @@ extern "C" int hapmi_append_cls_pos(const void *patches, const void *cls, const 
                                     int64_t T, int64_t d, int dtype, hapmi_stream_t stream) {
     HAPMI_REQUIRE(hapmi_dtype_ok(dtype) && b >= 0 && T >= 0 && d >= 1, HAPMI_EINVAL, "append_cls_pos: bad argument");
     if (b == 0) return HAPMI_OK;
-    HAPMI_REQUIRE(patches && cls && pos && out, HAPMI_EINVAL, "append_cls_pos: null pointer");
+    HAPMI_REQUIRE(patches && cls && out, HAPMI_EINVAL, "append_cls_pos: null pointer");
     dim3 grid(ew_grid(b * (T + 1) * d));
     if (dtype == HAPMI_F32)
         hipLaunchKernelGGL((append_cls_pos_kernel<float>), grid, dim3(EW_THREADS), 0, (hipStream_t)stream, (const float *)patches, (const float *)cls, (const float *)pos, (float *)out, b, T + 1, d);

@@ -133,6 +133,7 @@ class ShardExecutor:
         self._grad_sharers: Dict[int, list] = {}           # gradient storage -> values whose gradient aliases it
         self._emit_pos = -1                                # index of the backward emitter that is running
         self.shared_gradient_copies = 0                    # times a contribution went to a new buffer because of sharing
+        self._param_vals: Dict[str, Val] = {}
         self._wire_backed: set = set()                     # storages that peers' messages are received into in place
         self._pending_wgrads: Dict[tuple, list] = {}
         self._deferred_reads: Dict[int, int] = {}          # storage -> launches held back that read it
@@ -520,9 +521,13 @@ class ShardExecutor:
     def _get_attr(self, node):
         name = node.target
         if name in self.params:
-            rec = self.params[name]
-            t = rec["shadow"] if self.dtype == "bf16" else rec["master"]
-            return Val("param", t, name=name, master=rec["master"], grad=rec["grad"], needs_grad=True)
+            # one value per parameter, however many get_attr nodes name it: whether its gradient has had its first
+            # contribution (which overwrites; later ones accumulate) is kept on the value
+            if name not in self._param_vals:
+                rec = self.params[name]
+                t = rec["shadow"] if self.dtype == "bf16" else rec["master"]
+                self._param_vals[name] = Val("param", t, name=name, master=rec["master"], grad=rec["grad"], needs_grad=True)
+            return self._param_vals[name]
         buf = self.buffers[name]
         keep_f32 = name.endswith("src_mask")
         t = buf.detach().to(self.dev, torch.float32 if keep_f32 else self.cdt).contiguous()
@@ -612,7 +617,12 @@ class ShardExecutor:
         a, b = self._val(node.args[0]), self._val(node.args[1])
         users = list(node.users)
         if a.kind == "cls_appended" or b.kind == "cls_appended":
-            return self._append_cls_pos(node, a if a.kind == "cls_appended" else b, b if a.kind == "cls_appended" else a)
+            ac, other = (a, b) if a.kind == "cls_appended" else (b, a)
+            n, T, d = ac.meta["x"].t.shape
+            if other.t is not None and tuple(other.t.shape) == (1, T + 1, d):
+                return self._append_cls_pos(node, ac, other)       # the position embedding's add (models.py:167)
+            done = self._append_cls_pos(node, ac, None)             # some other add: the bare append first
+            a, b = (done, b) if a is ac else (a, done)
         if a.t is None or b.t is None:
             self._unsupported(node, "operands must be materialised tensors")
         if tuple(a.t.shape) == tuple(b.t.shape):
@@ -1229,23 +1239,26 @@ class ShardExecutor:
     def _append_cls(self, node):
         x, cls = self._val(node.args[0]), self._val(node.args[1])
         users = list(node.users)
-        if not (len(users) == 1 and users[0].target is operator.add):
-            self._unsupported(node, "append_cls_token must be followed by the position-embedding add")
-        return Val("cls_appended", None, x=x, cls=cls)
+        if len(users) == 1 and users[0].target is operator.add:
+            return Val("cls_appended", None, x=x, cls=cls)          # decided at the add: fused if it adds [1, T + 1, d]
+        return self._append_cls_pos(node, Val("cls_appended", None, x=x, cls=cls), None)
 
-    def _append_cls_pos(self, node, ac: Val, pos: Val):
+    def _append_cls_pos(self, node, ac: Val, pos: Optional[Val]):
+        """append_cls_token, fused with the position-embedding add that follows it in the reference's ViT
+        (models.py:167) or, ``pos`` None, on its own."""
         x, cls = ac.meta["x"], ac.meta["cls"]
         n, T, d = x.t.shape
-        if tuple(pos.t.shape) != (1, T + 1, d):
+        if pos is not None and tuple(pos.t.shape) != (1, T + 1, d):
             self._unsupported(node, "position embedding must be [1, T+1, d]")
         out = Val("tensor", self._new((n, T + 1, d)), needs_grad=True)
-        self.fwd.append(lambda: ops.append_cls_pos(x.t, cls.t, pos.t, out.t, n, T, d))
+        pos_t = pos.t if pos is not None else None
+        self.fwd.append(lambda: ops.append_cls_pos(x.t, cls.t, pos_t, out.t, n, T, d))
 
         def emit():
             if out.grad is None:
                 return
             g = out.grad
-            if pos.kind == "param":
+            if pos is not None and pos.kind == "param":
                 gp, accp = self._param_grad_slot(pos)
                 self.bwd.append(lambda: ops.colsum(g, gp, n, (T + 1) * d, (T + 1) * d, accp))
             if cls.kind == "param":

@@ -931,14 +931,16 @@ def patchify(x, cols, b, C, gh, gw, ph, pw):
 
 
 def append_cls_pos(patches, cls, pos, out, b, T, d):
+    """``pos`` None: the bare append_cls_token."""
     _dev(patches, cls, pos, out)
     _need(patches, b * T * d, "append_cls_pos patches")
     _need(cls, d, "append_cls_pos cls")
     _need(pos, (T + 1) * d, "append_cls_pos pos")
     _need(out, b * (T + 1) * d, "append_cls_pos out")
-    if not (patches.dtype == cls.dtype == pos.dtype == out.dtype):
+    if not (patches.dtype == cls.dtype == out.dtype) or (pos is not None and pos.dtype != out.dtype):
         raise TypeError("append_cls_pos: dtype mismatch")
-    check(lib().hapmi_append_cls_pos(_ptr(patches), _ptr(cls), _ptr(pos), _ptr(out), b, T, d, dtype_code(out), _stream()))
+    check(lib().hapmi_append_cls_pos(_ptr(patches), _ptr(cls), _ptr(pos) if pos is not None else None, _ptr(out), b, T, d,
+                                     dtype_code(out), _stream()))
 
 
 # ---------------------------------------------------------------------------

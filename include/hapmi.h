@@ -322,7 +322,8 @@ int hapmi_embedding_bwd(const int64_t *ids, const void *dout, float *dtable, int
 int hapmi_patchify(const float *x, void *cols, int64_t b, int64_t C, int64_t gh, int64_t gw, int64_t ph,
                    int64_t pw, int dtype, hapmi_stream_t stream);
 /* models.append_cls_token (models.py:443-445) fused with `+ pos_embed` (models.py:167):
- * out[b, 0, :] = cls + pos[0]; out[b, 1 + t, :] = patches[b, t, :] + pos[1 + t] */
+ * out[b, 0, :] = cls + pos[0]; out[b, 1 + t, :] = patches[b, t, :] + pos[1 + t]; pos may be NULL (the bare
+ * append_cls_token) */
 int hapmi_append_cls_pos(const void *patches, const void *cls, const void *pos, void *out, int64_t b, int64_t T,
                          int64_t d, int dtype, hapmi_stream_t stream);
 

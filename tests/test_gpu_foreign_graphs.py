@@ -127,3 +127,55 @@ def test_mlp_of_linear_sigmoid_new_segment_and_sum(cuda, dtype):
     assert set(grads) == set(ref)
     for n in ref:
         assert rel_err(grads[n], ref[n]) < tol, n
+
+
+@pytest.mark.parametrize("follow", ["linear", "other_add"])
+def test_append_cls_token_without_the_position_embedding_add(cuda, follow):
+    """models.append_cls_token (models.py:443-445) on its own: followed by a linear, or by an add that is not the
+    [1, T + 1, d] position embedding's (a same-shape tensor), then get_cls_token and a linear head with nll_loss;
+    against the same arithmetic in stock PyTorch on the CPU."""
+    d, B, T, C = 32, 6, 5, 7
+    g0 = torch.Generator().manual_seed(5)
+    xs = torch.randn(B, T, d, generator=g0)
+    ys = torch.randint(0, C, (B,), generator=g0)
+
+    def holder():
+        m = _Holder(C, d)
+        m.cls = nn.Parameter(torch.randn(1, 1, d, generator=torch.Generator().manual_seed(9)) * 0.3)
+        return m
+
+    m = holder()
+    h = F.linear(xs, m.w0, m.b0)
+    t = torch.cat((m.cls.expand(B, -1, -1), h), dim=1)
+    if follow == "linear":
+        t = F.linear(t, m.w1, m.b1)
+    else:
+        t = torch.cat((m.cls.expand(B, -1, -1), h), dim=1) + F.linear(t, m.w1, m.b1)
+    want = F.nll_loss(torch.log_softmax(F.linear(t[:, 0, :], m.dec_w, m.dec_b), 1), ys, reduction="sum")
+    want.backward()
+    ref = {n: p.grad.clone() for n, p in m.named_parameters() if p.grad is not None}
+
+    g = torch.fx.Graph()
+    x, y = g.placeholder("x"), g.placeholder("y")
+    h = g.call_function(F.linear, (x, g.get_attr("w0"), g.get_attr("b0")))
+    t = g.call_function(hap_amd.models.append_cls_token, (h, g.get_attr("cls")))
+    if follow == "linear":
+        t = g.call_function(F.linear, (t, g.get_attr("w1"), g.get_attr("b1")))
+    else:
+        u = g.call_function(F.linear, (t, g.get_attr("w1"), g.get_attr("b1")))
+        t2 = g.call_function(hap_amd.models.append_cls_token, (h, g.get_attr("cls")))
+        t = g.call_function(operator.add, (t2, u))
+    c = g.call_function(hap_amd.models.get_cls_token, (t,))
+    logits = g.call_function(F.linear, (c, g.get_attr("dec_w"), g.get_attr("dec_b")))
+    lp = g.call_function(torch.log_softmax, (logits, 1))
+    g.output(g.call_function(F.nll_loss, (lp, y), {"reduction": "sum"}))
+    g.lint()
+    ex = hap_amd.compile_program(torch.fx.GraphModule(holder(), g), [xs, ys], dtype="fp32")
+    got = ex.forward(xs, ys).item()
+    ex.backward()
+    torch.cuda.synchronize()
+    grads = {n: rec["grad"].cpu() for n, rec in ex.params.items()}
+    assert abs(got - want.item()) <= 1e-4 * abs(want.item())
+    assert set(grads) == set(ref)
+    for n in ref:
+        assert rel_err(grads[n], ref[n]) < 1e-4, n
