@@ -15,6 +15,7 @@
 // different 16-byte slots (row & 3 picks the 64-byte quarter, row >> 2 the slot), and the four 64-byte pieces
 // of rows 4a .. 4a + 3 that a half wave touches in a transposing read fall into different quarters.
 #include "common.h"
+#include "dropout.h"
 #include "tile.h"
 
 namespace {
@@ -154,6 +155,15 @@ struct DirectTileLoader {
     }
 };
 
+// One 4-byte word per thread global -> LDS (global_load_lds_dword: a wave instruction fills 256 contiguous LDS bytes,
+// lane l landing in word l), into the thread's own slot lds_words[threadIdx.x]; asynchronous like the tile transfers.
+__device__ __forceinline__ void issue_word(const uint32_t *src, uint32_t *lds_words) {
+    typedef __attribute__((address_space(3))) uint32_t lds_u32;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t lds_addr = (uint32_t)(uintptr_t)(lds_u32 *)(lds_words + wave * 64);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" : : "s"(lds_addr), "v"(src) : "memory");
+}
+
 // ---------------------------------------------------------------------------------------------
 // forward
 // ---------------------------------------------------------------------------------------------
@@ -181,13 +191,21 @@ template <bool CAUSAL> struct BlockOrder {
 
 // CAUSAL: key j is visible to query i iff j <= i (the additive mask torch.triu(full(-inf), 1), models.py:76),
 // applied arithmetically; kv tiles that lie completely above the diagonal of the block's 128 queries are skipped.
-template <bool CAUSAL>
+// DROP: dropout of the probabilities (F.multi_head_attention_forward with dropout_p > 0, hap.rs:1257, 1307).  The
+// keep decisions come as bit words (attn_keep_bits below): the row sums stay those of the undropped probabilities,
+// the probabilities that multiply V are zeroed where the bit is clear, and the factor 1 / (1 - p) is applied to the
+// output once at the end.
+template <bool CAUSAL, bool DROP = false>
 __global__ __launch_bounds__(AT_THREADS, 3) void attn_fwd_kernel(const bf16_t *qkv, const float *mask, bf16_t *out,
-                                                            float *lse, int S, int H, float scale) {
+                                                            float *lse, int S, int H, float scale,
+                                                            const uint32_t *keep_rows = nullptr, float keep_scale = 1.f) {
     // three K and three V tiles: one is multiplied while the next two are on their way global -> LDS
     constexpr int NST = 3;
     __shared__ __attribute__((aligned(16))) char Ks3[NST][TILE_BYTES];
     __shared__ __attribute__((aligned(16))) char Vs3[NST][TILE_BYTES];
+    // DROP: each thread's keep word of a tile travels with the tile (one 4-byte transfer per thread, landing in the
+    // thread's own slot), so it is counted by the same wait and needs no wait of its own
+    __shared__ __attribute__((aligned(16))) uint32_t keep_s[DROP ? NST : 1][AT_THREADS];
     const TransposedReader tr;
     const int E = H * HD, ld = 3 * E;
     const int blk = BlockOrder<CAUSAL>::row_block(true), bh = BlockOrder<CAUSAL>::batch_head();
@@ -219,11 +237,14 @@ __global__ __launch_bounds__(AT_THREADS, 3) void attn_fwd_kernel(const bf16_t *q
     // tells that everyone is done with tile i - 1, whose buffers take tile i + 2.
     const int q_blk_end = blk * 128 + 128;
     const int kv_end = (CAUSAL && q_blk_end < S) ? q_blk_end : S;
-    constexpr int PER_TILE = 2 * DirectTileLoader::LOADS;
-    static_assert(PER_TILE == 4, "the wait below is written for four transfers per tile");
+    constexpr int PER_TILE = 2 * DirectTileLoader::LOADS + (DROP ? 1 : 0);
+    static_assert(2 * DirectTileLoader::LOADS == 4, "the waits below are written for four (five) transfers per tile");
+    const int n_kt = (S + TILE - 1) / TILE;
+    const uint32_t *keep_row = DROP ? keep_rows + ((int64_t)bh * S + (qok ? q : S - 1)) * n_kt * 2 + h : nullptr;
     auto issue_tile = [&](int kv0, int bufi) {
         ldr.issue(K + (int64_t)kv0 * ld, S - kv0, Ks3[bufi]);
         ldr.issue(V + (int64_t)kv0 * ld, S - kv0, Vs3[bufi]);
+        if constexpr (DROP) issue_word(keep_row + (kv0 / TILE) * 2, &keep_s[bufi][0]);
     };
     issue_tile(0, 0);
     if (TILE < kv_end) issue_tile(TILE, 1);
@@ -234,11 +255,13 @@ __global__ __launch_bounds__(AT_THREADS, 3) void attn_fwd_kernel(const bf16_t *q
     for (int s = 0; s < 4; ++s) asm volatile("" : "+v"(qf[s].v));
     int buf = 0;
     for (int kv0 = 0; kv0 < kv_end; kv0 += TILE) {
-        if (kv0 + TILE < kv_end) __builtin_amdgcn_s_waitcnt(0x0F74);   // vmcnt(4): only tile i + 1 may be outstanding
+        if (kv0 + TILE < kv_end) __builtin_amdgcn_s_waitcnt(0x0F70 | PER_TILE);   // vmcnt(4 / 5): only tile i + 1 may be outstanding
         else __builtin_amdgcn_s_waitcnt(0x0F70);                       // vmcnt(0)
         __syncthreads();
         if (kv0 + 2 * TILE < kv_end) issue_tile(kv0 + 2 * TILE, buf == 0 ? 2 : buf - 1);
         const char *Ks = Ks3[buf], *Vs = Vs3[buf];
+        uint32_t keep = 0xffffffffu;                               // this lane's 32 keys of the tile, bit = register index
+        if constexpr (DROP) keep = keep_s[buf][threadIdx.x];
         // all fragment reads of the tile are issued before the first MFMA waits for one
         frag_t kf[2][4];
 #pragma unroll
@@ -314,6 +337,12 @@ __global__ __launch_bounds__(AT_THREADS, 3) void attn_fwd_kernel(const bf16_t *q
             m = m_new;
         }
         lsum = lsum * alpha + psum;
+        if constexpr (DROP) {
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) st[t][r] = (keep & (1u << (t * 16 + r))) ? st[t][r] : 0.f;
+        }
         if (__builtin_amdgcn_ballot_w64(alpha != 1.f)) {          // the running maximum moved for some query
 #pragma unroll
             for (int u = 0; u < 2; ++u)
@@ -329,7 +358,7 @@ __global__ __launch_bounds__(AT_THREADS, 3) void attn_fwd_kernel(const bf16_t *q
         buf = buf == NST - 1 ? 0 : buf + 1;
     }
     const float l = lsum + __shfl_xor(lsum, 32, 64);
-    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    const float inv = (l > 0.f ? 1.0f / l : 0.f) * (DROP ? keep_scale : 1.f);
     if (qok) {
         bf16_t *orow = out + ((int64_t)b * S + q) * E + hh * HD;
 #pragma unroll
@@ -348,10 +377,11 @@ __global__ __launch_bounds__(AT_THREADS, 3) void attn_fwd_kernel(const bf16_t *q
 // ---------------------------------------------------------------------------------------------
 // dQ: lanes own query columns, kv tiles are streamed
 // ---------------------------------------------------------------------------------------------
-template <bool CAUSAL>
+template <bool CAUSAL, bool DROP = false>
 __global__ __launch_bounds__(AT_THREADS, 2) void attn_bwd_dq_kernel(const bf16_t *qkv, const bf16_t *out, const bf16_t *dout,
                                                                const float *lse, float *delta, const float *mask,
-                                                               bf16_t *dqkv, int S, int H, float scale) {
+                                                               bf16_t *dqkv, int S, int H, float scale,
+                                                               const uint32_t *keep_rows = nullptr, float keep_scale = 1.f) {
     __shared__ __attribute__((aligned(16))) char Ks[TILE_BYTES];
     __shared__ __attribute__((aligned(16))) char Vs[TILE_BYTES];
     const TransposedReader tr;
@@ -398,15 +428,21 @@ __global__ __launch_bounds__(AT_THREADS, 2) void attn_bwd_dq_kernel(const bf16_t
     const int kv_end = (CAUSAL && q_blk_end < S) ? q_blk_end : S;
     lk.load(K, S);
     lv.load(V, S);
+    // DROP: the lane's keep word of a tile (bit = register index) is fetched together with the tile
+    const uint32_t *keep_row = DROP ? keep_rows + ((int64_t)bh * S + (qok ? q : S - 1)) * ((S + TILE - 1) / TILE) * 2 + h : nullptr;
+    uint32_t keep = 0xffffffffu, keep_next = 0xffffffffu;
+    if constexpr (DROP) keep_next = keep_row[0];
     for (int kv0 = 0; kv0 < kv_end; kv0 += TILE) {
         __syncthreads();
         lk.store_rows(Ks);
         lv.store_rows(Vs);
+        if constexpr (DROP) keep = keep_next;
         __syncthreads();
         if (kv0 + TILE < kv_end) {
             const int nx = kv0 + TILE;
             lk.load(K + (int64_t)nx * ld, S - nx);
             lv.load(V + (int64_t)nx * ld, S - nx);
+            if constexpr (DROP) keep_next = keep_row[(nx / TILE) * 2];
         }
 
         // one 32-row kv block at a time keeps only one score / dP accumulator pair live
@@ -417,6 +453,10 @@ __global__ __launch_bounds__(AT_THREADS, 2) void attn_bwd_dq_kernel(const bf16_t
             for (int s = 0; s < 4; ++s) {
                 st = mma(frag_rowk(Ks, t * 32 + c, s, h), qf[s], st);
                 dp = mma(frag_rowk(Vs, t * 32 + c, s, h), dof[s], dp);
+            }
+            if constexpr (DROP) {                                  // d(P) = d(dropout(P)) * keep / (1 - p)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) dp[r] = (keep & (1u << (t * 16 + r))) ? dp[r] * keep_scale : 0.f;
             }
             if (plain_block && kv0 + TILE <= S && (!CAUSAL || kv0 + TILE - 1 <= blk * 128)) {
 #pragma unroll
@@ -471,10 +511,11 @@ __global__ __launch_bounds__(AT_THREADS, 2) void attn_bwd_dq_kernel(const bf16_t
 // ---------------------------------------------------------------------------------------------
 // dK, dV: lanes own kv columns, query tiles are streamed
 // ---------------------------------------------------------------------------------------------
-template <bool CAUSAL>
+template <bool CAUSAL, bool DROP = false>
 __global__ __launch_bounds__(AT_THREADS, 2) void attn_bwd_dkv_kernel(const bf16_t *qkv, const bf16_t *dout, const float *lse,
                                                                 const float *delta, const float *mask, bf16_t *dqkv,
-                                                                int S, int H, float scale) {
+                                                                int S, int H, float scale,
+                                                                const uint32_t *keep_cols = nullptr, float keep_scale = 1.f) {
     __shared__ __attribute__((aligned(16))) char Qs[TILE_BYTES];
     __shared__ __attribute__((aligned(16))) char dOs[TILE_BYTES];
     const TransposedReader tr;
@@ -505,10 +546,16 @@ __global__ __launch_bounds__(AT_THREADS, 2) void attn_bwd_dkv_kernel(const bf16_
     const int q_begin = CAUSAL ? blk * 128 : 0;
     lq.load(Q + (int64_t)q_begin * ld, S - q_begin);
     ldo.load(dO + (int64_t)q_begin * E, S - q_begin);
+    // DROP: the lane's two keep words of a query tile (one per 32 queries, bit = query) are fetched with the tile
+    typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+    const u32x2 *keep_col = DROP ? (const u32x2 *)(keep_cols + ((int64_t)bh * S + (kok ? kv : S - 1)) * (2 * ((S + TILE - 1) / TILE))) : nullptr;
+    u32x2 keep2 = {0xffffffffu, 0xffffffffu}, keep2_next = keep2;
+    if constexpr (DROP) keep2_next = keep_col[q_begin / TILE];
     for (int q0 = q_begin; q0 < S; q0 += TILE) {
         __syncthreads();
         lq.store_rows(Qs);
         ldo.store_rows(dOs);
+        if constexpr (DROP) keep2 = keep2_next;
         if (threadIdx.x < TILE) {
             const int qq = q0 + threadIdx.x;
             lse_s[threadIdx.x] = qq < S ? lse_b[qq] * LOG2E : INFINITY;
@@ -519,6 +566,7 @@ __global__ __launch_bounds__(AT_THREADS, 2) void attn_bwd_dkv_kernel(const bf16_
             const int nx = q0 + TILE;
             lq.load(Q + (int64_t)nx * ld, S - nx);
             ldo.load(dO + (int64_t)nx * E, S - nx);
+            if constexpr (DROP) keep2_next = keep_col[nx / TILE];
         }
 
         // one 32-row query block at a time keeps only one score / dP accumulator pair live; the loop is kept
@@ -530,6 +578,14 @@ __global__ __launch_bounds__(AT_THREADS, 2) void attn_bwd_dkv_kernel(const bf16_
             for (int s = 0; s < 4; ++s) {
                 sc = mma(frag_rowk(Qs, t * 32 + c, s, h), kf[s], sc);
                 dp = mma(frag_rowk(dOs, t * 32 + c, s, h), vf[s], dp);
+            }
+            const uint32_t keep = t ? keep2.y : keep2.x;           // this key's 32 queries q0 + 32 t .. + 32, bit = query
+            if constexpr (DROP) {
+#pragma unroll
+                for (int g = 0; g < 4; ++g)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        dp[g * 4 + e] = (keep & (1u << (g * 8 + h * 4 + e))) ? dp[g * 4 + e] * keep_scale : 0.f;
             }
             // without a mask, query rows beyond S carry lse = +inf (p = 0); causal tiles below the diagonal of the
             // block's 128 keys need no comparison
@@ -565,6 +621,13 @@ __global__ __launch_bounds__(AT_THREADS, 2) void attn_bwd_dkv_kernel(const bf16_
                     }
                 }
             }
+            if constexpr (DROP) {                                  // dV takes the dropped probabilities
+#pragma unroll
+                for (int g = 0; g < 4; ++g)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        sc[g * 4 + e] = (keep & (1u << (g * 8 + h * 4 + e))) ? sc[g * 4 + e] * keep_scale : 0.f;
+            }
 #pragma unroll
             for (int sp = 0; sp < 2; ++sp) {
                 const frag_t pb = acc_to_b(sc, sp), db = acc_to_b(dp, sp);
@@ -594,6 +657,65 @@ __global__ __launch_bounds__(AT_THREADS, 2) void attn_bwd_dkv_kernel(const bf16_
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// keep decisions of the probabilities' dropout, as bit words in the two orders the kernels above read them in
+// ---------------------------------------------------------------------------------------------
+// The decision for probability (bh, q, k) is the one F.dropout's kernel takes for element (bh * S + q) * row_len + k
+// of a [b * H, S, row_len] tensor (row_len even, >= S), so the fused kernels and a materialised-probabilities path
+// drop the same entries.  A wave takes 64 queries x 64 keys: lane = query computes its row's 64 decisions (32 hashes),
+//   keep_rows[bh][q][key tile][2]    word h, bit 16 t + 4 g + e  <->  key 64 tile + 32 t + 8 g + 4 h + e
+//                                    (the accumulator register order of a lane of half h in forward and dQ),
+// and a 64 x 64 bit transpose across the lanes (six exchange steps) turns rows into columns: lane = key gets
+//   keep_cols[bh][k][2 * query tile + w]   bit i  <->  query 64 tile + 32 w + i.
+// Rows / columns beyond S are not written (keep_rows) or hold zeros for the missing queries (keep_cols).
+__global__ __launch_bounds__(256) void attn_keep_bits_kernel(uint32_t *keep_rows, uint32_t *keep_cols, int S, int64_t row_len,
+                                                           float p, const int64_t *state, int64_t stream_id) {
+    typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+    const DropKey key = drop_key(state[0], state[1], stream_id, p);
+    const int n_kt = (S + TILE - 1) / TILE;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int kt = blockIdx.x * 4 + wave, qt = blockIdx.y;
+    const int64_t bh = blockIdx.z;
+    if (kt >= n_kt) return;                                        // whole waves leave; no barrier below
+    const int q = qt * TILE + lane;
+    uint64_t nat = 0;                                              // bit k: keep (q, key 64 kt + k)
+    if (q < S) {
+        const uint64_t first = (uint64_t)((bh * S + q) * row_len + (int64_t)kt * TILE);      // even
+#pragma unroll 8
+        for (int j = 0; j < 32; ++j) {
+            const uint32_t bits = drop_pair_bits(key, (first >> 1) + j);
+            nat |= (uint64_t)((bits & 0xffffU) >= key.thr) << (2 * j);
+            nat |= (uint64_t)((bits >> 16) >= key.thr) << (2 * j + 1);
+        }
+        u32x2 w = {0u, 0u};
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                w.x |= (uint32_t)((nat >> (t * 32 + g * 8)) & 0xf) << (t * 16 + g * 4);
+                w.y |= (uint32_t)((nat >> (t * 32 + g * 8 + 4)) & 0xf) << (t * 16 + g * 4);
+            }
+        *(u32x2 *)(keep_rows + (((int64_t)bh * S + q) * n_kt + kt) * 2) = w;
+    }
+    // transpose: after the step for j, bit position and lane number have exchanged their bit j
+    uint64_t x = nat;
+#pragma unroll
+    for (int step = 0; step < 6; ++step) {
+        constexpr uint64_t masks[6] = {0x00000000ffffffffull, 0x0000ffff0000ffffull, 0x00ff00ff00ff00ffull,
+                                       0x0f0f0f0f0f0f0f0full, 0x3333333333333333ull, 0x5555555555555555ull};
+        const int j = 32 >> step;
+        const uint64_t m = masks[step];
+        const uint32_t lo = __shfl_xor((uint32_t)x, j, 64), hi = __shfl_xor((uint32_t)(x >> 32), j, 64);
+        const uint64_t other = ((uint64_t)hi << 32) | lo;
+        x = (lane & j) ? ((x & ~m) | ((other & ~m) >> j)) : ((x & m) | ((other & m) << j));
+    }
+    const int k = kt * TILE + lane;
+    if (k < S) {
+        u32x2 w = {(uint32_t)x, (uint32_t)(x >> 32)};
+        *(u32x2 *)(keep_cols + ((int64_t)bh * S + k) * (2 * n_kt) + 2 * qt) = w;
+    }
+}
+
 int check_attn(const char *name, int64_t b, int64_t S, int64_t H) {
     HAPMI_REQUIRE(b >= 0 && S >= 1 && H >= 1, HAPMI_EINVAL, "%s: bad shape", name);
     HAPMI_REQUIRE(S < (1ll << 24) && b * H <= 65535, HAPMI_ELIMIT, "%s: b*H %lld above 65535 or S too long", name,
@@ -601,52 +723,116 @@ int check_attn(const char *name, int64_t b, int64_t S, int64_t H) {
     return HAPMI_OK;
 }
 
+int attention_fwd(const char *name, const void *qkv, const float *mask, int causal, void *out, float *lse, int64_t b, int64_t S,
+                  int64_t H, float scale, const uint32_t *keep_rows, float p, hipStream_t st) {
+    int rc = check_attn(name, b, S, H);
+    if (rc) return rc;
+    if (b == 0) return HAPMI_OK;
+    HAPMI_REQUIRE(qkv && out && lse, HAPMI_EINVAL, "%s: null pointer", name);
+    HAPMI_REQUIRE(((uintptr_t)qkv % 16) == 0 && ((uintptr_t)out % 16) == 0 && (!mask || ((uintptr_t)mask % 16) == 0) &&
+                      ((uintptr_t)keep_rows % 8) == 0,
+                  HAPMI_EALIGN, "%s: pointers must be 16-byte aligned (keep words: 8)", name);
+    HAPMI_REQUIRE(!(causal && mask), HAPMI_EINVAL, "%s: causal and an explicit mask exclude each other", name);
+    const bf16_t *x = (const bf16_t *)qkv;
+    bf16_t *o = (bf16_t *)out;
+    const float *no_mask = nullptr;
+    const float ks = keep_rows ? 1.0f / (1.0f - p) : 1.0f;
+    dim3 grid((unsigned)hapmi_cdiv(S, 128), (unsigned)(b * H)), block(AT_THREADS);
+    if (causal && keep_rows)
+        hipLaunchKernelGGL((attn_fwd_kernel<true, true>), grid, block, 0, st, x, no_mask, o, lse, (int)S, (int)H, scale, keep_rows, ks);
+    else if (causal)
+        hipLaunchKernelGGL((attn_fwd_kernel<true, false>), grid, block, 0, st, x, no_mask, o, lse, (int)S, (int)H, scale, keep_rows, ks);
+    else if (keep_rows)
+        hipLaunchKernelGGL((attn_fwd_kernel<false, true>), grid, block, 0, st, x, mask, o, lse, (int)S, (int)H, scale, keep_rows, ks);
+    else
+        hipLaunchKernelGGL((attn_fwd_kernel<false, false>), grid, block, 0, st, x, mask, o, lse, (int)S, (int)H, scale, keep_rows, ks);
+    HAPMI_CHECK_LAUNCH(name);
+    return HAPMI_OK;
+}
+
+int attention_bwd(const char *name, const void *qkv, const void *out, const void *dout, const float *lse, const float *mask,
+                  int causal, void *dqkv, float *delta_ws, int64_t b, int64_t S, int64_t H, float scale,
+                  const uint32_t *keep_rows, const uint32_t *keep_cols, float p, hipStream_t st) {
+    int rc = check_attn(name, b, S, H);
+    if (rc) return rc;
+    if (b == 0) return HAPMI_OK;
+    HAPMI_REQUIRE(qkv && out && dout && lse && dqkv && delta_ws, HAPMI_EINVAL, "%s: null pointer", name);
+    HAPMI_REQUIRE(!(causal && mask), HAPMI_EINVAL, "%s: causal and an explicit mask exclude each other", name);
+    HAPMI_REQUIRE(((uintptr_t)qkv % 16) == 0 && ((uintptr_t)out % 16) == 0 && ((uintptr_t)dout % 16) == 0 &&
+                      ((uintptr_t)dqkv % 16) == 0 && (!mask || ((uintptr_t)mask % 16) == 0) &&
+                      ((uintptr_t)keep_rows % 8) == 0 && ((uintptr_t)keep_cols % 8) == 0,
+                  HAPMI_EALIGN, "%s: pointers must be 16-byte aligned (keep words: 8)", name);
+    const bf16_t *x = (const bf16_t *)qkv, *o = (const bf16_t *)out, *d_o = (const bf16_t *)dout;
+    bf16_t *dx = (bf16_t *)dqkv;
+    const float *no_mask = nullptr, *delta_in = delta_ws;
+    const bool drop = keep_rows != nullptr;
+    const float ks = drop ? 1.0f / (1.0f - p) : 1.0f;
+    dim3 grid((unsigned)hapmi_cdiv(S, 128), (unsigned)(b * H)), block(AT_THREADS);
+    if (causal && drop) {
+        hipLaunchKernelGGL((attn_bwd_dq_kernel<true, true>), grid, block, 0, st, x, o, d_o, lse, delta_ws, no_mask, dx, (int)S, (int)H, scale, keep_rows, ks);
+        hipLaunchKernelGGL((attn_bwd_dkv_kernel<true, true>), grid, block, 0, st, x, d_o, lse, delta_in, no_mask, dx, (int)S, (int)H, scale, keep_cols, ks);
+    } else if (causal) {
+        hipLaunchKernelGGL((attn_bwd_dq_kernel<true, false>), grid, block, 0, st, x, o, d_o, lse, delta_ws, no_mask, dx, (int)S, (int)H, scale, keep_rows, ks);
+        hipLaunchKernelGGL((attn_bwd_dkv_kernel<true, false>), grid, block, 0, st, x, d_o, lse, delta_in, no_mask, dx, (int)S, (int)H, scale, keep_cols, ks);
+    } else if (drop) {
+        hipLaunchKernelGGL((attn_bwd_dq_kernel<false, true>), grid, block, 0, st, x, o, d_o, lse, delta_ws, mask, dx, (int)S, (int)H, scale, keep_rows, ks);
+        hipLaunchKernelGGL((attn_bwd_dkv_kernel<false, true>), grid, block, 0, st, x, d_o, lse, delta_in, mask, dx, (int)S, (int)H, scale, keep_cols, ks);
+    } else {
+        hipLaunchKernelGGL((attn_bwd_dq_kernel<false, false>), grid, block, 0, st, x, o, d_o, lse, delta_ws, mask, dx, (int)S, (int)H, scale, keep_rows, ks);
+        hipLaunchKernelGGL((attn_bwd_dkv_kernel<false, false>), grid, block, 0, st, x, d_o, lse, delta_in, mask, dx, (int)S, (int)H, scale, keep_cols, ks);
+    }
+    HAPMI_CHECK_LAUNCH(name);
+    return HAPMI_OK;
+}
+
 }  // namespace
 
 extern "C" int hapmi_attention_fwd(const void *qkv, const float *mask, int causal, void *out, float *lse, int64_t b,
                                    int64_t S, int64_t H, float scale, hapmi_stream_t stream) {
-    int rc = check_attn("attention_fwd", b, S, H);
-    if (rc) return rc;
-    if (b == 0) return HAPMI_OK;
-    HAPMI_REQUIRE(qkv && out && lse, HAPMI_EINVAL, "attention_fwd: null pointer");
-    HAPMI_REQUIRE(((uintptr_t)qkv % 16) == 0 && ((uintptr_t)out % 16) == 0 && (!mask || ((uintptr_t)mask % 16) == 0),
-                  HAPMI_EALIGN, "attention_fwd: pointers must be 16-byte aligned");
-    HAPMI_REQUIRE(!(causal && mask), HAPMI_EINVAL, "attention_fwd: causal and an explicit mask exclude each other");
-    dim3 grid((unsigned)hapmi_cdiv(S, 128), (unsigned)(b * H));
-    if (causal)
-        hipLaunchKernelGGL(attn_fwd_kernel<true>, grid, dim3(AT_THREADS), 0, (hipStream_t)stream, (const bf16_t *)qkv,
-                           (const float *)nullptr, (bf16_t *)out, lse, (int)S, (int)H, scale);
-    else
-        hipLaunchKernelGGL(attn_fwd_kernel<false>, grid, dim3(AT_THREADS), 0, (hipStream_t)stream, (const bf16_t *)qkv, mask,
-                           (bf16_t *)out, lse, (int)S, (int)H, scale);
-    HAPMI_CHECK_LAUNCH("attention_fwd");
-    return HAPMI_OK;
+    return attention_fwd("attention_fwd", qkv, mask, causal, out, lse, b, S, H, scale, nullptr, 0.f, (hipStream_t)stream);
 }
 
 extern "C" int hapmi_attention_bwd(const void *qkv, const void *out, const void *dout, const float *lse,
                                    const float *mask, int causal, void *dqkv, float *delta_ws, int64_t b, int64_t S,
                                    int64_t H, float scale, hapmi_stream_t stream) {
-    int rc = check_attn("attention_bwd", b, S, H);
+    return attention_bwd("attention_bwd", qkv, out, dout, lse, mask, causal, dqkv, delta_ws, b, S, H, scale, nullptr, nullptr, 0.f,
+                         (hipStream_t)stream);
+}
+
+extern "C" int hapmi_attention_keep_bits(uint32_t *keep_rows, uint32_t *keep_cols, int64_t b, int64_t S, int64_t H,
+                                         int64_t row_len, float p, const int64_t *rng_state_dev, int64_t stream_id,
+                                         hapmi_stream_t stream) {
+    int rc = check_attn("attention_keep_bits", b, S, H);
     if (rc) return rc;
+    HAPMI_REQUIRE(p >= 0.f && p < 1.f && row_len >= S && row_len % 2 == 0, HAPMI_EINVAL,
+                  "attention_keep_bits: p = %g must lie in [0, 1) and row_len = %lld must be even and >= S", (double)p, (long long)row_len);
     if (b == 0) return HAPMI_OK;
-    HAPMI_REQUIRE(qkv && out && dout && lse && dqkv && delta_ws, HAPMI_EINVAL, "attention_bwd: null pointer");
-    HAPMI_REQUIRE(!(causal && mask), HAPMI_EINVAL, "attention_bwd: causal and an explicit mask exclude each other");
-    HAPMI_REQUIRE(((uintptr_t)qkv % 16) == 0 && ((uintptr_t)out % 16) == 0 && ((uintptr_t)dout % 16) == 0 &&
-                      ((uintptr_t)dqkv % 16) == 0 && (!mask || ((uintptr_t)mask % 16) == 0),
-                  HAPMI_EALIGN, "attention_bwd: pointers must be 16-byte aligned");
-    hipStream_t st = (hipStream_t)stream;
-    dim3 grid((unsigned)hapmi_cdiv(S, 128), (unsigned)(b * H));
-    if (causal) {
-        hipLaunchKernelGGL(attn_bwd_dq_kernel<true>, grid, dim3(AT_THREADS), 0, st, (const bf16_t *)qkv, (const bf16_t *)out,
-                           (const bf16_t *)dout, lse, delta_ws, (const float *)nullptr, (bf16_t *)dqkv, (int)S, (int)H, scale);
-        hipLaunchKernelGGL(attn_bwd_dkv_kernel<true>, grid, dim3(AT_THREADS), 0, st, (const bf16_t *)qkv, (const bf16_t *)dout,
-                           lse, (const float *)delta_ws, (const float *)nullptr, (bf16_t *)dqkv, (int)S, (int)H, scale);
-    } else {
-        hipLaunchKernelGGL(attn_bwd_dq_kernel<false>, grid, dim3(AT_THREADS), 0, st, (const bf16_t *)qkv, (const bf16_t *)out,
-                           (const bf16_t *)dout, lse, delta_ws, mask, (bf16_t *)dqkv, (int)S, (int)H, scale);
-        hipLaunchKernelGGL(attn_bwd_dkv_kernel<false>, grid, dim3(AT_THREADS), 0, st, (const bf16_t *)qkv, (const bf16_t *)dout,
-                           lse, (const float *)delta_ws, mask, (bf16_t *)dqkv, (int)S, (int)H, scale);
-    }
-    HAPMI_CHECK_LAUNCH("attention_bwd");
+    HAPMI_REQUIRE(keep_rows && keep_cols && rng_state_dev, HAPMI_EINVAL, "attention_keep_bits: null pointer");
+    HAPMI_REQUIRE(((uintptr_t)keep_rows % 8) == 0 && ((uintptr_t)keep_cols % 8) == 0 && ((uintptr_t)rng_state_dev % 8) == 0, HAPMI_EALIGN,
+                  "attention_keep_bits: pointers must be 8-byte aligned");
+    const int64_t n_kt = hapmi_cdiv(S, TILE);
+    HAPMI_REQUIRE(n_kt <= 65535, HAPMI_ELIMIT, "attention_keep_bits: S too long");
+    dim3 grid((unsigned)hapmi_cdiv(n_kt, 4), (unsigned)n_kt, (unsigned)(b * H));
+    hipLaunchKernelGGL(attn_keep_bits_kernel, grid, dim3(256), 0, (hipStream_t)stream, keep_rows, keep_cols, (int)S, row_len, p,
+                       rng_state_dev, stream_id);
+    HAPMI_CHECK_LAUNCH("attention_keep_bits");
     return HAPMI_OK;
+}
+
+extern "C" int hapmi_attention_fwd_dropout(const void *qkv, const float *mask, int causal, void *out, float *lse, int64_t b,
+                                           int64_t S, int64_t H, float scale, const uint32_t *keep_rows, float p,
+                                           hapmi_stream_t stream) {
+    HAPMI_REQUIRE(keep_rows || b == 0, HAPMI_EINVAL, "attention_fwd_dropout: null keep words");
+    HAPMI_REQUIRE(p >= 0.f && p < 1.f, HAPMI_EINVAL, "attention_fwd_dropout: p = %g must lie in [0, 1)", (double)p);
+    return attention_fwd("attention_fwd_dropout", qkv, mask, causal, out, lse, b, S, H, scale, keep_rows, p, (hipStream_t)stream);
+}
+
+extern "C" int hapmi_attention_bwd_dropout(const void *qkv, const void *out, const void *dout, const float *lse,
+                                           const float *mask, int causal, void *dqkv, float *delta_ws, int64_t b, int64_t S,
+                                           int64_t H, float scale, const uint32_t *keep_rows, const uint32_t *keep_cols, float p,
+                                           hapmi_stream_t stream) {
+    HAPMI_REQUIRE((keep_rows && keep_cols) || b == 0, HAPMI_EINVAL, "attention_bwd_dropout: null keep words");
+    HAPMI_REQUIRE(p >= 0.f && p < 1.f, HAPMI_EINVAL, "attention_bwd_dropout: p = %g must lie in [0, 1)", (double)p);
+    return attention_bwd("attention_bwd_dropout", qkv, out, dout, lse, mask, causal, dqkv, delta_ws, b, S, H, scale, keep_rows, keep_cols, p,
+                         (hipStream_t)stream);
 }

@@ -993,8 +993,9 @@ class ShardExecutor:
                         p_drop: float = 0.0):
         """qkv = x W_in^T + b_in over Ea = H * head_dim attention columns (all heads, or this device's heads),
         softmax attention per head, out = ctx W_out^T (+ b_out).  x is [b, S, d]; W_in [3 Ea, d]; W_out [d_out, Ea].
-        ``p_drop`` > 0 (dropout of the probabilities, torch:nn/functional.py:6591): the probabilities are
-        materialised, as the reference's explicit path does, and the fused kernels are not used."""
+        ``p_drop`` > 0 (dropout of the probabilities, torch:nn/functional.py:6591): the fused kernels take the keep
+        decisions as bit words, written once per step by a kernel of their own; the path that materialises the
+        probabilities (float32, other head sizes) runs the dropout kernel over them.  Both take the same decisions."""
         for v in (w_in, b_in, w_out) + ((b_out,) if b_out is not None else ()):
             if v.kind != "param":
                 self._unsupported(node, "attention weights must be parameters")
@@ -1013,7 +1014,7 @@ class ShardExecutor:
                 self._unsupported(node, "attn_mask must be a float32 [L, S] additive mask")
             mask_t = mask.t
         scale = 1.0 / math.sqrt(hd)
-        fused = self.fused_attention and self.dtype == "bf16" and hd == 64 and p_drop == 0.0
+        fused = self.fused_attention and self.dtype == "bf16" and hd == 64 and p_drop < 1.0
         # a constant mask (a buffer of the module, not a gathered shard) that is exactly the causal one is
         # applied arithmetically by the fused kernels, which then also skip the key tiles above the diagonal
         causal = False
@@ -1034,7 +1035,14 @@ class ShardExecutor:
         if p_drop > 0.0:
             self._uses_rng = True
             out_bsd.meta["prob_dropout"] = (p_drop, sid, (b, H, S, Sp), S)
-            Pd = self._scratch("attn_Pd", (b, H, S, Sp))          # dropout(P): rebuilt from P wherever it is needed
+            if fused:
+                # the step's keep decisions in the two bit orders the kernels read; backward takes the forward's
+                n_words = ops.attention_keep_words(b, S, H)
+                keep_rows, keep_cols = self._new((n_words,), torch.int32), self._new((n_words,), torch.int32)
+            else:
+                Pd = self._scratch("attn_Pd", (b, H, S, Sp))      # dropout(P): rebuilt from P wherever it is needed
+        if not (fused and p_drop > 0.0):
+            keep_rows = keep_cols = None
         M = b * S
         sQ, sP = (S * 3 * Ea, hd), (H * S * Sp, S * Sp)
         bias_out = b_out.meta["master"] if b_out is not None else None
@@ -1042,7 +1050,9 @@ class ShardExecutor:
         def forward():
             ops.gemm(x.t, w_in.t, qkv, M, 3 * Ea, d, transB=True, bias=b_in.meta["master"])
             if fused:
-                ops.attention_fwd(qkv, fused_mask, ctx, lse, b, S, H, scale, causal)
+                if keep_rows is not None:
+                    ops.attention_keep_bits(keep_rows, keep_cols, b, S, H, Sp, p_drop, self.rng_state, sid)
+                ops.attention_fwd(qkv, fused_mask, ctx, lse, b, S, H, scale, causal, keep_rows, p_drop)
             else:
                 ops.gemm(qkv, qkv, P, S, S, hd, transB=True, lda=3 * Ea, ldb=3 * Ea, ldc=Sp, alpha=scale, batch1=b,
                          batch2=H, strideA=sQ, strideB=sQ, strideC=sP, offB=Ea)
@@ -1094,7 +1104,8 @@ class ShardExecutor:
             def backward():
                 ops.gemm(do, w_out.t, dctx, M, Ea, d_out)
                 if fused:
-                    ops.attention_bwd(qkv, ctx, dctx, lse, fused_mask, dqkv, delta, b, S, H, scale, causal)
+                    ops.attention_bwd(qkv, ctx, dctx, lse, fused_mask, dqkv, delta, b, S, H, scale, causal, keep_rows,
+                                      keep_cols, p_drop)
                 else:
                     # dP = dctx V^T ; dV = P^T dctx
                     ops.gemm(dctx, qkv, dP, S, S, hd, transB=True, lda=Ea, ldb=3 * Ea, ldc=Sp, batch1=b, batch2=H,

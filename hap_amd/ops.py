@@ -727,24 +727,63 @@ def _check_attn(qkv, out, lse, mask, b, S, H):
         raise TypeError("attention: float32 mask expected")
 
 
-def attention_fwd(qkv, mask, out, lse, b, S, H, scale, causal=False):
-    """``causal``: the mask is torch.triu(full(-inf), 1); pass ``mask=None`` with it."""
-    _dev(qkv, mask, out, lse)
+def attention_keep_words(b, S, H) -> int:
+    """Number of uint32 in each of the two keep-word buffers of attention with dropout."""
+    return b * H * S * 2 * ((S + 63) // 64)
+
+
+def _check_keep(t, b, S, H, what):
+    if t.dtype != torch.int32 or not t.is_contiguous():
+        raise TypeError(f"attention {what}: contiguous int32 words expected")
+    _need(t, attention_keep_words(b, S, H), f"attention {what}")
+
+
+def attention_keep_bits(keep_rows, keep_cols, b, S, H, row_len, p, rng_state, stream_id):
+    """The keep decisions of the probabilities' dropout as bit words (int32 tensors of attention_keep_words
+    elements): those ``dropout`` takes for a [b*H, S, row_len] tensor under the same (p, rng_state, stream_id)."""
+    _dev(keep_rows, keep_cols, rng_state)
+    _check_keep(keep_rows, b, S, H, "keep_rows")
+    _check_keep(keep_cols, b, S, H, "keep_cols")
+    if rng_state.dtype != torch.int64 or rng_state.numel() < 2:
+        raise TypeError("attention_keep_bits: rng_state must hold two int64")
+    check(lib().hapmi_attention_keep_bits(_ptr(keep_rows), _ptr(keep_cols), b, S, H, row_len, ctypes.c_float(p),
+                                          _ptr(rng_state), stream_id, _stream()))
+
+
+def attention_fwd(qkv, mask, out, lse, b, S, H, scale, causal=False, keep_rows=None, p=0.0):
+    """``causal``: the mask is torch.triu(full(-inf), 1); pass ``mask=None`` with it.  ``keep_rows`` (from
+    attention_keep_bits) with ``p``: dropout of the probabilities."""
+    _dev(qkv, mask, out, lse, keep_rows)
     _check_attn(qkv, out, lse, mask, b, S, H)
-    check(lib().hapmi_attention_fwd(_ptr(qkv), _ptr(mask), int(causal), _ptr(out), _ptr(lse), b, S, H,
-                                    ctypes.c_float(scale), _stream()))
+    if keep_rows is None:
+        check(lib().hapmi_attention_fwd(_ptr(qkv), _ptr(mask), int(causal), _ptr(out), _ptr(lse), b, S, H,
+                                        ctypes.c_float(scale), _stream()))
+        return
+    _check_keep(keep_rows, b, S, H, "keep_rows")
+    check(lib().hapmi_attention_fwd_dropout(_ptr(qkv), _ptr(mask), int(causal), _ptr(out), _ptr(lse), b, S, H,
+                                            ctypes.c_float(scale), _ptr(keep_rows), ctypes.c_float(p), _stream()))
 
 
-def attention_bwd(qkv, out, dout, lse, mask, dqkv, delta_ws, b, S, H, scale, causal=False):
-    _dev(qkv, out, dout, lse, mask, dqkv, delta_ws)
+def attention_bwd(qkv, out, dout, lse, mask, dqkv, delta_ws, b, S, H, scale, causal=False, keep_rows=None,
+                  keep_cols=None, p=0.0):
+    _dev(qkv, out, dout, lse, mask, dqkv, delta_ws, keep_rows, keep_cols)
     _check_attn(qkv, out, lse, mask, b, S, H)
     _need(dout, b * S * H * 64, "attention dout")
     _need(dqkv, b * S * 3 * H * 64, "attention dqkv")
     _need(delta_ws, b * H * S, "attention delta")
     if dout.dtype != torch.bfloat16 or dqkv.dtype != torch.bfloat16 or delta_ws.dtype != torch.float32:
         raise TypeError("attention_bwd: dtype mismatch")
-    check(lib().hapmi_attention_bwd(_ptr(qkv), _ptr(out), _ptr(dout), _ptr(lse), _ptr(mask), int(causal), _ptr(dqkv),
-                                    _ptr(delta_ws), b, S, H, ctypes.c_float(scale), _stream()))
+    if keep_rows is None and keep_cols is None:
+        check(lib().hapmi_attention_bwd(_ptr(qkv), _ptr(out), _ptr(dout), _ptr(lse), _ptr(mask), int(causal),
+                                        _ptr(dqkv), _ptr(delta_ws), b, S, H, ctypes.c_float(scale), _stream()))
+        return
+    if keep_rows is None or keep_cols is None:
+        raise ValueError("attention_bwd: keep_rows and keep_cols come together")
+    _check_keep(keep_rows, b, S, H, "keep_rows")
+    _check_keep(keep_cols, b, S, H, "keep_cols")
+    check(lib().hapmi_attention_bwd_dropout(_ptr(qkv), _ptr(out), _ptr(dout), _ptr(lse), _ptr(mask), int(causal),
+                                            _ptr(dqkv), _ptr(delta_ws), b, S, H, ctypes.c_float(scale),
+                                            _ptr(keep_rows), _ptr(keep_cols), ctypes.c_float(p), _stream()))
 
 
 def head_parallel_attention(x, w_in, b_in, w_out, num_heads, mask=None):

@@ -262,6 +262,27 @@ int hapmi_attention_bwd(const void *qkv, const void *out, const void *dout, cons
                         int causal, void *dqkv, float *delta_ws, int64_t b, int64_t S, int64_t H, float scale,
                         hapmi_stream_t stream);
 
+/* The same with dropout of the probabilities (dropout_p > 0 of F.multi_head_attention_forward, hap.rs:1257, 1307:
+ * out = dropout(softmax(scores)) V).  The keep decisions are those F.dropout's kernel (hapmi_dropout) takes for the
+ * elements of a [b*H, S, row_len] tensor of probabilities (row_len even, >= S) under the same p, RNG state and
+ * stream id, so this path and one that materialises the probabilities drop the same entries.
+ * hapmi_attention_keep_bits packs them into bit words in the two orders the kernels read them in:
+ *   keep_rows: b*H*S*2*ceil(S/64) uint32, read by forward and by backward
+ *              (per query: the tile's 64 keys in the lane's accumulator-register order);
+ *   keep_cols: the same count, read by backward (per key: one bit per query).
+ * Both are 8-byte aligned, written completely for the rows / columns below S, and belong to one (step, stream id):
+ * backward must be given the words its forward ran with.  p lies in [0, 1). */
+int hapmi_attention_keep_bits(uint32_t *keep_rows, uint32_t *keep_cols, int64_t b, int64_t S, int64_t H,
+                              int64_t row_len, float p, const int64_t *rng_state_dev, int64_t stream_id,
+                              hapmi_stream_t stream);
+int hapmi_attention_fwd_dropout(const void *qkv, const float *mask, int causal, void *out, float *lse, int64_t b,
+                                int64_t S, int64_t H, float scale, const uint32_t *keep_rows, float p,
+                                hapmi_stream_t stream);
+int hapmi_attention_bwd_dropout(const void *qkv, const void *out, const void *dout, const float *lse,
+                                const float *mask, int causal, void *dqkv, float *delta_ws, int64_t b, int64_t S,
+                                int64_t H, float scale, const uint32_t *keep_rows, const uint32_t *keep_cols, float p,
+                                hapmi_stream_t stream);
+
 /* torch.log_softmax + F.nll_loss(reduction='sum', ignore_index) (hap.rs:1829, 1881) and their
  * backward in one pass: row_loss[rows] float32, dlogits = (softmax - onehot) * grad_scale for
  * counted rows and 0 for ignored rows; dlogits may alias logits; rows of both are ld elements apart. */

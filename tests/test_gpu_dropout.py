@@ -93,14 +93,14 @@ def _masks_from_oracle(ex, step):
     return out
 
 
-@pytest.mark.parametrize("family,dtype", [("lm", "fp32"), ("lm", "bf16"), ("vit", "fp32")])
+@pytest.mark.parametrize("family,dtype", [("lm", "fp32"), ("lm", "bf16"), ("vit", "fp32"), ("vit", "bf16")])
 def test_program_with_dropout_against_the_oracle_given_the_masks(cuda, family, dtype):
     if family == "lm":
         model = make_lm(vocab=211, S=32, d=64, H=1 if dtype == "bf16" else 4, F=128, layers=2)
         x, y = lm_batch(8, 32, 211)
         kw = {}
     else:
-        model = make_vit(img=32, patch=8, d=64, F=128)
+        model = make_vit(img=32, patch=8, d=64, H=1 if dtype == "bf16" else 4, F=128)
         x, y = vit_batch(8, 32, 10)
         kw = dict(ffn="batch")
     model.dropout_p = 0.1

@@ -3,6 +3,8 @@ program calls in the reference: F.linear, F.layer_norm, softmax, log_softmax + n
 torch.optim).  Tolerances: float32 rtol 1e-4; bfloat16 rtol 2e-2 (inputs are rounded to bf16 on both sides)."""
 import math
 
+import numpy as np
+
 import pytest
 import torch
 import torch.nn.functional as F
@@ -535,6 +537,85 @@ def test_fused_attention_forward_backward(cuda, S, causal):
     dqkv = torch.full((b, S, 3 * E), float("nan"), dtype=torch.bfloat16, device=cuda)
     delta = torch.empty(b, H, S, dtype=torch.float32, device=cuda)
     ops.attention_bwd(dq, out, dout.to(cuda), lse, dmask, dqkv, delta, b, S, H, scale, causal=flag)
+    for name, got, ref in zip("qkv", dqkv.float().cpu().split(E, dim=2), x.grad.split(E, dim=2)):
+        assert rel_err(got, ref) < 2e-2, (name, rel_err(got, ref))
+
+
+def _keep_words_to_masks(keep_rows, keep_cols, b, H, S):
+    """Unpacks the two bit-word layouts of attention_keep_bits into bool [b*H, S(q), S(k)] tensors."""
+    n_kt = (S + 63) // 64
+    rows = keep_rows.cpu().numpy().astype(np.uint32).reshape(b * H, S, n_kt, 2)
+    cols = keep_cols.cpu().numpy().astype(np.uint32).reshape(b * H, S, 2 * n_kt)
+    k = np.arange(n_kt * 64)
+    kt, t, g, h, e = k // 64, (k // 32) % 2, (k // 8) % 4, (k // 4) % 2, k % 4
+    from_rows = ((rows[:, :, kt, h] >> (16 * t + 4 * g + e).astype(np.uint32)) & 1).astype(bool)[:, :, :S]
+    q = np.arange(S)
+    from_cols = ((cols[:, :, q // 32] >> (q % 32).astype(np.uint32)) & 1).astype(bool)       # [bh, k, q]
+    return torch.from_numpy(from_rows), torch.from_numpy(from_cols).transpose(1, 2)
+
+
+@pytest.mark.parametrize("S", [16, 64, 129, 197, 512])
+def test_attention_keep_words_are_the_dropout_kernels_decisions(cuda, S):
+    """Both bit layouts of attention_keep_bits hold exactly the decisions that the dropout kernel takes for a
+    [b*H, S, row_len] tensor of probabilities under the same state and stream id (bit-exact)."""
+    b, H, p, sid = 2, 3, 0.25, 11
+    Sp = (S + 7) // 8 * 8
+    state = torch.tensor([1234, 5], dtype=torch.int64, device=cuda)
+    n = ops.attention_keep_words(b, S, H)
+    kr = torch.full((n,), -1, dtype=torch.int32, device=cuda)
+    kc = torch.full((n,), -1, dtype=torch.int32, device=cuda)
+    ops.attention_keep_bits(kr, kc, b, S, H, Sp, p, state, sid)
+    want = ops.dropout_mask(b * H * S * Sp, p, state, sid).view(b * H, S, Sp)[:, :, :S].bool().cpu()
+    got_rows, got_cols = _keep_words_to_masks(kr, kc, b, H, S)
+    assert torch.equal(got_rows, want)
+    assert torch.equal(got_cols, want)
+    assert 0.70 < want.float().mean().item() < 0.80
+    # query bits beyond S inside a column's last word are zero
+    n_kt = (S + 63) // 64
+    cols = kc.cpu().numpy().astype(np.uint32).reshape(b * H, S, 2 * n_kt)
+    qq = np.arange(S, n_kt * 64)
+    if len(qq):
+        assert not ((cols[:, :, qq // 32] >> (qq % 32).astype(np.uint32)) & 1).any()
+
+
+@pytest.mark.parametrize("S,causal", [(16, False), (64, True), (129, "flag"), (197, False), (512, False), (512, "flag"),
+                                      (200, True)])
+def test_fused_attention_with_dropout_of_the_probabilities(cuda, S, causal):
+    """out = dropout(softmax(QK^T * scale + mask)) V (F.multi_head_attention_forward with dropout_p > 0) and its
+    gradients, in float64 from the same bf16 inputs with the keep decisions of the dropout kernel."""
+    g = torch.Generator().manual_seed(S + 1)
+    b, H, hd, p, sid = 2, 3, 64, 0.2, 7
+    E, Sp = H * hd, (S + 7) // 8 * 8
+    qkv = torch.randn(b, S, 3 * E, generator=g).bfloat16()
+    dout = torch.randn(b, S, E, generator=g).bfloat16()
+    mask = torch.triu(torch.full((S, S), float("-inf")), diagonal=1) if causal else None
+    scale = 1.0 / math.sqrt(hd)
+    state = torch.tensor([99, 3], dtype=torch.int64, device=cuda)
+    n = ops.attention_keep_words(b, S, H)
+    kr = torch.empty(n, dtype=torch.int32, device=cuda)
+    kc = torch.empty(n, dtype=torch.int32, device=cuda)
+    ops.attention_keep_bits(kr, kc, b, S, H, Sp, p, state, sid)
+    keep = ops.dropout_mask(b * H * S * Sp, p, state, sid).view(b, H, S, Sp)[..., :S].bool().cpu()
+    out = torch.empty(b, S, E, dtype=torch.bfloat16, device=cuda)
+    lse = torch.empty(b, H, S, dtype=torch.float32, device=cuda)
+    dq = qkv.to(cuda)
+    flag = causal == "flag"
+    dmask = mask.to(cuda) if causal is True else None
+    ops.attention_fwd(dq, dmask, out, lse, b, S, H, scale, causal=flag, keep_rows=kr, p=p)
+    x = qkv.double().requires_grad_(True)
+    q, k, v = [t.view(b, S, H, hd).transpose(1, 2) for t in x.split(E, dim=2)]
+    sc = q @ k.transpose(-1, -2) * scale
+    if causal:
+        sc = sc + mask.double()
+    P = torch.softmax(sc, -1) * keep.double() / (1.0 - p)
+    want = (P @ v).transpose(1, 2).reshape(b, S, E)
+    close(out, want.detach(), torch.bfloat16)
+    torch.testing.assert_close(lse.cpu(), torch.logsumexp(sc, -1).float().detach(), rtol=1e-3, atol=1e-3)
+    want.backward(dout.double())
+    dqkv = torch.full((b, S, 3 * E), float("nan"), dtype=torch.bfloat16, device=cuda)
+    delta = torch.empty(b, H, S, dtype=torch.float32, device=cuda)
+    ops.attention_bwd(dq, out, dout.to(cuda), lse, dmask, dqkv, delta, b, S, H, scale, causal=flag, keep_rows=kr,
+                      keep_cols=kc, p=p)
     for name, got, ref in zip("qkv", dqkv.float().cpu().split(E, dim=2), x.grad.split(E, dim=2)):
         assert rel_err(got, ref) < 2e-2, (name, rel_err(got, ref))
 
