@@ -1,6 +1,7 @@
 // Row-wise HBM-bound kernels: residual-add + LayerNorm (no affine), softmax with
 // additive mask, and log-softmax + NLL with its gradient.  Statistics are float32.
 #include "common.h"
+#include "dropout.h"
 
 namespace {
 
@@ -55,14 +56,45 @@ template <typename T, int EPV, int MAXE> struct RowRegs {
     }
 };
 
+// F.dropout on a row held in registers: element (row, column c) takes the decision of flat index row * width + c, as
+// the elementwise dropout kernel does for the whole tensor.  The vector layouts hold an element pair (even column,
+// next column) in one lane and have an even width, so one hash serves the pair; the scalar layout asks per element.
+// Kept elements are scaled and, for the 2-byte storage type, rounded as the stored dropout output would be.
 template <typename T, int EPV, int MAXE>
-__global__ __launch_bounds__(ROW_WAVES * 64) void add_layernorm_fwd_kernel(const T *x, const T *res, T *y, float *rstd,
-                                                                         int64_t rows, int width, float eps) {
+__device__ __forceinline__ void drop_row(RowRegs<T, EPV, MAXE> &a, const DropKey &key, int64_t row_first, int width, int lane) {
+    auto kept = [&](float v) {
+        v *= key.scale;
+        return sizeof(T) == 2 ? (float)(bf16_t)v : v;
+    };
+    if constexpr (EPV % 2 == 0) {
+#pragma unroll
+        for (int e = 0; e < MAXE; e += 2) {
+            const int c = RowRegs<T, EPV, MAXE>::col(e, lane);
+            if (c < width) {
+                const uint32_t bits = drop_pair_bits(key, (uint64_t)(row_first + c) >> 1);
+                a.v[e] = (bits & 0xffffU) >= key.thr ? kept(a.v[e]) : 0.f;
+                a.v[e + 1] = (bits >> 16) >= key.thr ? kept(a.v[e + 1]) : 0.f;
+            }
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < MAXE; ++e) {
+            const int c = RowRegs<T, EPV, MAXE>::col(e, lane);
+            if (c < width) a.v[e] = drop_keep(key, (uint64_t)(row_first + c)) ? kept(a.v[e]) : 0.f;
+        }
+    }
+}
+
+// y = LN(x + res), or with DROP y = LN(dropout(x) + res): F.dropout -> operator.add -> F.layer_norm in one pass
+template <typename T, int EPV, int MAXE, bool DROP>
+__device__ __forceinline__ void add_layernorm_fwd_row(const T *x, const T *res, T *y, float *rstd, int64_t rows, int width,
+                                                      float eps, float p, const int64_t *state, int64_t stream_id) {
     const int lane = threadIdx.x & 63;
     const int64_t r = (int64_t)blockIdx.x * ROW_WAVES + (threadIdx.x >> 6);
     if (r >= rows) return;
     RowRegs<T, EPV, MAXE> a;
     a.load(x + r * width, width, lane, 0.f);
+    if constexpr (DROP) drop_row(a, drop_key(state[0], state[1], stream_id, p), r * width, width, lane);
     if (res) {
         RowRegs<T, EPV, MAXE> b;
         b.load(res + r * width, width, lane, 0.f);
@@ -92,8 +124,23 @@ __global__ __launch_bounds__(ROW_WAVES * 64) void add_layernorm_fwd_kernel(const
 }
 
 template <typename T, int EPV, int MAXE>
-__global__ __launch_bounds__(ROW_WAVES * 64) void layernorm_bwd_kernel(const T *dy, const T *y, const float *rstd,
-                                                                     const T *dx_add, T *dx, int64_t rows, int width) {
+__global__ __launch_bounds__(ROW_WAVES * 64) void add_layernorm_fwd_kernel(const T *x, const T *res, T *y, float *rstd,
+                                                                         int64_t rows, int width, float eps) {
+    add_layernorm_fwd_row<T, EPV, MAXE, false>(x, res, y, rstd, rows, width, eps, 0.f, nullptr, 0);
+}
+
+template <typename T, int EPV, int MAXE>
+__global__ __launch_bounds__(ROW_WAVES * 64) void dropout_add_layernorm_fwd_kernel(const T *x, const T *res, T *y, float *rstd,
+                                                                                 int64_t rows, int width, float eps, float p,
+                                                                                 const int64_t *state, int64_t stream_id) {
+    add_layernorm_fwd_row<T, EPV, MAXE, true>(x, res, y, rstd, rows, width, eps, p, state, stream_id);
+}
+
+// dx = rstd * (dy - mean(dy) - y * mean(dy * y)) (+ dx_add); with DROP also dx_drop = dropout's backward of dx (the
+// gradient of the operand that went through F.dropout before the add), from the same decisions as forward
+template <typename T, int EPV, int MAXE, bool DROP>
+__device__ __forceinline__ void layernorm_bwd_row(const T *dy, const T *y, const float *rstd, const T *dx_add, T *dx, T *dx_drop,
+                                                  int64_t rows, int width, float p, const int64_t *state, int64_t stream_id) {
     const int lane = threadIdx.x & 63;
     const int64_t r = (int64_t)blockIdx.x * ROW_WAVES + (threadIdx.x >> 6);
     if (r >= rows) return;
@@ -116,6 +163,28 @@ __global__ __launch_bounds__(ROW_WAVES * 64) void layernorm_bwd_kernel(const T *
         for (int e = 0; e < MAXE; ++e) g.v[e] += o.v[e];
     }
     g.store(dx + r * width, width, lane);
+    if constexpr (DROP) {
+        if (sizeof(T) == 2) {                                      // dropout's backward reads the stored gradient
+#pragma unroll
+            for (int e = 0; e < MAXE; ++e) g.v[e] = (float)(bf16_t)g.v[e];
+        }
+        drop_row(g, drop_key(state[0], state[1], stream_id, p), r * width, width, lane);
+        g.store(dx_drop + r * width, width, lane);
+    }
+}
+
+template <typename T, int EPV, int MAXE>
+__global__ __launch_bounds__(ROW_WAVES * 64) void layernorm_bwd_kernel(const T *dy, const T *y, const float *rstd,
+                                                                     const T *dx_add, T *dx, int64_t rows, int width) {
+    layernorm_bwd_row<T, EPV, MAXE, false>(dy, y, rstd, dx_add, dx, nullptr, rows, width, 0.f, nullptr, 0);
+}
+
+template <typename T, int EPV, int MAXE>
+__global__ __launch_bounds__(ROW_WAVES * 64) void layernorm_bwd_dropout_kernel(const T *dy, const T *y, const float *rstd,
+                                                                             const T *dx_add, T *dx, T *dx_drop, int64_t rows,
+                                                                             int width, float p, const int64_t *state,
+                                                                             int64_t stream_id) {
+    layernorm_bwd_row<T, EPV, MAXE, true>(dy, y, rstd, dx_add, dx, dx_drop, rows, width, p, state, stream_id);
 }
 
 template <typename T, int EPV, int MAXE>
@@ -245,6 +314,57 @@ extern "C" int hapmi_layernorm_bwd(const void *dy, const void *y, const float *r
                            (const bf16_t *)y, rstd, (const bf16_t *)dx_add, (bf16_t *)dx, rows, (int)width);
     }
     HAPMI_CHECK_LAUNCH("layernorm_bwd");
+    return HAPMI_OK;
+}
+
+extern "C" int hapmi_dropout_add_layernorm_fwd(const void *x, const void *res, void *y, float *rstd, int64_t rows,
+                                               int64_t width, float eps, float p, const int64_t *rng_state_dev,
+                                               int64_t stream_id, int dtype, hapmi_stream_t stream) {
+    int rc = check_rows("dropout_add_layernorm_fwd", rows, width, dtype);
+    if (rc) return rc;
+    HAPMI_REQUIRE(p >= 0.f && p <= 1.f, HAPMI_EINVAL, "dropout_add_layernorm_fwd: bad probability %g", (double)p);
+    if (rows == 0) return HAPMI_OK;
+    HAPMI_REQUIRE(x && y && rstd && rng_state_dev, HAPMI_EINVAL, "dropout_add_layernorm_fwd: null pointer");
+    HAPMI_REQUIRE(((uintptr_t)rng_state_dev % 8) == 0, HAPMI_EALIGN, "dropout_add_layernorm_fwd: misaligned RNG state");
+    dim3 grid((unsigned)hapmi_cdiv(rows, ROW_WAVES));
+    const void *ptrs[3] = {x, y, res};
+    if (dtype == HAPMI_F32) {
+        int epv = row_epv<float>(ptrs, 3, width);
+        HAPMI_ROW_DISPATCH(dropout_add_layernorm_fwd_kernel, float, epv, width, grid, (hipStream_t)stream, (const float *)x,
+                           (const float *)res, (float *)y, rstd, rows, (int)width, eps, p, rng_state_dev, stream_id);
+    } else {
+        int epv = row_epv<bf16_t>(ptrs, 3, width);
+        HAPMI_ROW_DISPATCH(dropout_add_layernorm_fwd_kernel, bf16_t, epv, width, grid, (hipStream_t)stream, (const bf16_t *)x,
+                           (const bf16_t *)res, (bf16_t *)y, rstd, rows, (int)width, eps, p, rng_state_dev, stream_id);
+    }
+    HAPMI_CHECK_LAUNCH("dropout_add_layernorm_fwd");
+    return HAPMI_OK;
+}
+
+extern "C" int hapmi_layernorm_bwd_dropout(const void *dy, const void *y, const float *rstd, const void *dx_add, void *dx,
+                                           void *dx_drop, int64_t rows, int64_t width, float p,
+                                           const int64_t *rng_state_dev, int64_t stream_id, int dtype,
+                                           hapmi_stream_t stream) {
+    int rc = check_rows("layernorm_bwd_dropout", rows, width, dtype);
+    if (rc) return rc;
+    HAPMI_REQUIRE(p >= 0.f && p <= 1.f, HAPMI_EINVAL, "layernorm_bwd_dropout: bad probability %g", (double)p);
+    if (rows == 0) return HAPMI_OK;
+    HAPMI_REQUIRE(dy && y && rstd && dx && dx_drop && rng_state_dev, HAPMI_EINVAL, "layernorm_bwd_dropout: null pointer");
+    HAPMI_REQUIRE(((uintptr_t)rng_state_dev % 8) == 0, HAPMI_EALIGN, "layernorm_bwd_dropout: misaligned RNG state");
+    dim3 grid((unsigned)hapmi_cdiv(rows, ROW_WAVES));
+    const void *ptrs[5] = {dy, y, dx, dx_add, dx_drop};
+    if (dtype == HAPMI_F32) {
+        int epv = row_epv<float>(ptrs, 5, width);
+        HAPMI_ROW_DISPATCH(layernorm_bwd_dropout_kernel, float, epv, width, grid, (hipStream_t)stream, (const float *)dy,
+                           (const float *)y, rstd, (const float *)dx_add, (float *)dx, (float *)dx_drop, rows, (int)width, p,
+                           rng_state_dev, stream_id);
+    } else {
+        int epv = row_epv<bf16_t>(ptrs, 5, width);
+        HAPMI_ROW_DISPATCH(layernorm_bwd_dropout_kernel, bf16_t, epv, width, grid, (hipStream_t)stream, (const bf16_t *)dy,
+                           (const bf16_t *)y, rstd, (const bf16_t *)dx_add, (bf16_t *)dx, (bf16_t *)dx_drop, rows, (int)width, p,
+                           rng_state_dev, stream_id);
+    }
+    HAPMI_CHECK_LAUNCH("layernorm_bwd_dropout");
     return HAPMI_OK;
 }
 

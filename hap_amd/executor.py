@@ -62,7 +62,7 @@ class ShardExecutor:
                  overlap_wgrad: bool = False, launch_lists: bool = True, relu_mask_in_dgrad: bool = True,
                  overlap_optimizer: bool = False, optimizer_chunk_min: int = 1 << 20,
                  relu_bwd_in_split: bool = True, wgrad_group: int = 8, receive_in_place: bool = True,
-                 dropout_seed: int = 0, exchange_in_pieces: bool = True):
+                 dropout_seed: int = 0, exchange_in_pieces: bool = True, fuse_dropout: bool = True):
         """``example_inputs``: the program's inputs (global batch) as tensors or shapes; activations are
         sized from them.  ``rank`` / ``world_size`` are only needed by all_reduce / replicate, whose node
         forms do not carry them (collectives.py:86, 182)."""
@@ -102,6 +102,7 @@ class ShardExecutor:
         # relu's backward behind an all_to_all rides on the copying split of the backward exchange (one pass over
         # the gradient less per layer); False keeps the separate pass, for comparison
         self.relu_bwd_in_split = relu_bwd_in_split
+        self.fuse_dropout = fuse_dropout               # F.dropout inside the kernel next to it where one can take it
         # the backward all_to_all of the column-sharded FFN concatenates along dim 0: every peer's piece is a
         # contiguous row range of the result, so it is received there (Wire.recv(into=...)) instead of into a
         # buffer of its own that a copy kernel then moves; False keeps the copy
@@ -623,6 +624,9 @@ class ShardExecutor:
                 return self._append_cls_pos(node, ac, other)       # the position embedding's add (models.py:167)
             done = self._append_cls_pos(node, ac, None)             # some other add: the bare append first
             a, b = (done, b) if a is ac else (a, done)
+        if a.kind == "dropped" or b.kind == "dropped":
+            # _dropout has checked the form: the other operand is a tensor of this shape and layer_norm reads the sum
+            return Val("sum", None, shape=a.shape, a=a, b=b, needs_grad=True)
         if a.t is None or b.t is None:
             self._unsupported(node, "operands must be materialised tensors")
         if tuple(a.t.shape) == tuple(b.t.shape):
@@ -722,6 +726,10 @@ class ShardExecutor:
             self._unsupported(node, f"dropout of a {x.kind} value")
         self._uses_rng = True
         sid = self._node_ids[node]
+        if self.fuse_dropout and self._feeds_residual_layer_norm(node, x):
+            # dropout -> add -> layer_norm: the layer_norm kernels apply it to their operand (forward) and give its
+            # backward as a second result; nothing is materialised here
+            return Val("dropped", None, shape=x.t.shape, src=x, needs_grad=x.needs_grad, dropout=(p, sid))
         out = Val("tensor", self._new(x.t.shape), needs_grad=x.needs_grad, dropout=(p, sid))
         self.fwd.append(lambda: ops.dropout(x.t, out.t, p, self.rng_state, sid))
 
@@ -739,6 +747,22 @@ class ShardExecutor:
         self._tape.append(emit)
         return out
 
+    def _feeds_residual_layer_norm(self, node, x: Val) -> bool:
+        """node's only reader is an operator.add of it and an already materialised tensor of the same shape, whose
+        only reader is F.layer_norm (the form _add hands to _layer_norm as a lazy sum)."""
+        users = list(node.users)
+        if len(users) != 1 or users[0].target is not operator.add or len(users[0].args) != 2:
+            return False
+        add = users[0]
+        others = [a for a in add.args if a is not node]
+        if len(others) != 1 or not isinstance(others[0], torch.fx.Node):
+            return False
+        other = self.env.get(others[0])
+        if not isinstance(other, Val) or other.t is None or other.ld is not None or tuple(other.t.shape) != tuple(x.t.shape):
+            return False
+        ln = list(add.users)
+        return len(ln) == 1 and ln[0].target is F.layer_norm and len(ln[0].args) == 2 and not ln[0].kwargs
+
     def dropout_masks(self) -> Dict[str, torch.Tensor]:
         """The keep decisions of the step that ran last, by node name: for an F.dropout node a bool tensor of its
         input's shape, for an attention node with dropout_p > 0 a bool tensor [batch, heads, L, S] over its
@@ -749,7 +773,7 @@ class ShardExecutor:
                 continue
             if isinstance(v, Val) and v.meta.get("dropout") and node.target is F.dropout and float(node.args[1]) > 0:
                 p, sid = v.meta["dropout"]
-                out[node.name] = ops.dropout_mask(v.t.numel(), p, self.rng_state, sid).view(v.t.shape).bool()
+                out[node.name] = ops.dropout_mask(math.prod(v.shape), p, self.rng_state, sid).view(v.shape).bool()
             elif isinstance(v, Val) and v.kind == "mha" and v.meta.get("dropout"):
                 p, sid, shape, S = v.meta["dropout"]
                 n = 1
@@ -762,9 +786,17 @@ class ShardExecutor:
         v, shape = self._val(node.args[0]), tuple(node.args[1])
         if len(node.args) > 2 or node.kwargs:
             self._unsupported(node, "the program emits layer_norm without affine parameters")
+        drop = dropped = None
         if v.kind == "sum":
             a, b = v.meta["a"], v.meta["b"]
-            x, res, ref_shape = a.t, b.t, a.t.shape
+            if b.kind != "dropped" and a.kind == "dropped":
+                a, b = b, a
+            if b.kind == "dropped":            # LN(res + dropout(src)): the kernel's first operand is the dropped one
+                dropped, b = b, b.meta["src"]
+                drop = (dropped.meta["dropout"][0], self.rng_state, dropped.meta["dropout"][1])
+                x, res, ref_shape = b.t, a.t, a.t.shape
+            else:
+                x, res, ref_shape = a.t, b.t, a.t.shape
         else:
             a, b, x, res, ref_shape = v, None, v.t, None, v.t.shape
         if len(shape) != 1 or shape[0] != ref_shape[-1]:
@@ -772,7 +804,7 @@ class ShardExecutor:
         rows = x.numel() // shape[0]
         out = Val("tensor", self._placed_output(node, ref_shape), needs_grad=True)
         rstd = self._new((rows,), torch.float32)
-        self.fwd.append(lambda: ops.add_layernorm_fwd(x, res, out.t, rstd, _EPS))
+        self.fwd.append(lambda: ops.add_layernorm_fwd(x, res, out.t, rstd, _EPS, drop))
 
         def emit():
             if out.grad is None:
@@ -781,6 +813,13 @@ class ShardExecutor:
             if not targets:
                 return
             dx = self._new(ref_shape)
+            if dropped is not None and b.needs_grad:
+                dx_drop = self._new(ref_shape)
+                self.bwd.append(lambda: ops.layernorm_bwd(out.grad, out.t, rstd, None, dx, dx_drop, drop))
+                if a.needs_grad:
+                    self._accumulate_into(a, dx)
+                self._accumulate_into(b, dx_drop)
+                return
             self.bwd.append(lambda: ops.layernorm_bwd(out.grad, out.t, rstd, None, dx))
             for v in targets:                   # the residual add passes the same gradient to both operands
                 self._accumulate_into(v, dx)

@@ -670,7 +670,14 @@ def linear(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None
 # row-wise
 # ---------------------------------------------------------------------------
 
-def add_layernorm_fwd(x, res, y, rstd, eps=1e-5):
+def _check_rng(rng_state, what):
+    if rng_state is None or rng_state.dtype != torch.int64 or rng_state.numel() < 2:
+        raise TypeError(f"{what}: rng_state must hold two int64 (seed, step)")
+
+
+def add_layernorm_fwd(x, res, y, rstd, eps=1e-5, drop=None):
+    """y = LN(x + res); ``drop`` = (p, rng_state, stream_id): y = LN(dropout(x) + res) with the decisions that
+    ``dropout`` takes for x under the same three."""
     _dev(x, res, y, rstd)
     width = x.shape[-1]
     rows = x.numel() // width
@@ -679,21 +686,43 @@ def add_layernorm_fwd(x, res, y, rstd, eps=1e-5):
         if t_ is not None and t_.dtype != x.dtype:
             raise TypeError("add_layernorm_fwd: dtype mismatch")
     _need(rstd, rows, "add_layernorm_fwd rstd")
-    check(lib().hapmi_add_layernorm_fwd(_ptr(x), _ptr(res), _ptr(y), _ptr(rstd), rows, width,
-                                        ctypes.c_float(eps), dtype_code(x), _stream()))
+    if drop is None:
+        check(lib().hapmi_add_layernorm_fwd(_ptr(x), _ptr(res), _ptr(y), _ptr(rstd), rows, width,
+                                            ctypes.c_float(eps), dtype_code(x), _stream()))
+        return
+    p, rng_state, stream_id = drop
+    _dev(rng_state)
+    _check_rng(rng_state, "add_layernorm_fwd")
+    check(lib().hapmi_dropout_add_layernorm_fwd(_ptr(x), _ptr(res), _ptr(y), _ptr(rstd), rows, width,
+                                                ctypes.c_float(eps), ctypes.c_float(p), _ptr(rng_state),
+                                                int(stream_id), dtype_code(x), _stream()))
 
 
-def layernorm_bwd(dy, y, rstd, dx_add, dx):
-    _dev(dy, y, rstd, dx_add, dx)
+def layernorm_bwd(dy, y, rstd, dx_add, dx, dx_drop=None, drop=None):
+    """``dx_drop`` with ``drop`` = (p, rng_state, stream_id): also the gradient of the operand that went through
+    dropout before the add (dropout's backward of dx)."""
+    _dev(dy, y, rstd, dx_add, dx, dx_drop)
     width = y.shape[-1]
     rows = y.numel() // width
-    for t_ in (dy, y, dx_add, dx):
+    for t_ in (dy, y, dx_add, dx, dx_drop):
         _need(t_, rows * width, "layernorm_bwd")
         if t_ is not None and t_.dtype != y.dtype:
             raise TypeError("layernorm_bwd: dtype mismatch")
     _need(rstd, rows, "layernorm_bwd rstd")
-    check(lib().hapmi_layernorm_bwd(_ptr(dy), _ptr(y), _ptr(rstd), _ptr(dx_add), _ptr(dx), rows, width,
-                                    dtype_code(y), _stream()))
+    if (dx_drop is None) != (drop is None):
+        raise ValueError("layernorm_bwd: dx_drop and drop come together")
+    if drop is None:
+        check(lib().hapmi_layernorm_bwd(_ptr(dy), _ptr(y), _ptr(rstd), _ptr(dx_add), _ptr(dx), rows, width,
+                                        dtype_code(y), _stream()))
+        return
+    if dx_drop.data_ptr() == dx.data_ptr():
+        raise ValueError("layernorm_bwd: dx_drop must not alias dx")
+    p, rng_state, stream_id = drop
+    _dev(rng_state)
+    _check_rng(rng_state, "layernorm_bwd")
+    check(lib().hapmi_layernorm_bwd_dropout(_ptr(dy), _ptr(y), _ptr(rstd), _ptr(dx_add), _ptr(dx), _ptr(dx_drop),
+                                            rows, width, ctypes.c_float(p), _ptr(rng_state), int(stream_id),
+                                            dtype_code(y), _stream()))
 
 
 def softmax_fwd(x, mask, p, rows, width, ld, mask_rows=1):

@@ -238,6 +238,17 @@ int hapmi_add_layernorm_fwd(const void *x, const void *res, void *y, float *rstd
 /* dx = rstd * (dy - mean(dy) - y * mean(dy * y)) (+ dx_add if not NULL) */
 int hapmi_layernorm_bwd(const void *dy, const void *y, const float *rstd, const void *dx_add, void *dx,
                         int64_t rows, int64_t width, int dtype, hapmi_stream_t stream);
+/* F.dropout(x, p) -> operator.add(., res) -> F.layer_norm in one pass (hap.rs:1464, 1515, 1653: the residual
+ * connections of the encoder layer, models.py:112-117): y = LN(dropout(x) + res).  The keep decisions are those
+ * hapmi_dropout takes for x as a whole [rows, width] tensor under the same p, RNG state and stream id.  Backward
+ * gives dx (the gradient of the sum: res's) and dx_drop = dropout's backward of dx (x's), regenerating the mask;
+ * dx_drop must not alias dx. */
+int hapmi_dropout_add_layernorm_fwd(const void *x, const void *res, void *y, float *rstd, int64_t rows, int64_t width,
+                                    float eps, float p, const int64_t *rng_state_dev, int64_t stream_id, int dtype,
+                                    hapmi_stream_t stream);
+int hapmi_layernorm_bwd_dropout(const void *dy, const void *y, const float *rstd, const void *dx_add, void *dx,
+                                void *dx_drop, int64_t rows, int64_t width, float p, const int64_t *rng_state_dev,
+                                int64_t stream_id, int dtype, hapmi_stream_t stream);
 
 /* softmax over the last dimension of [rows, width] (row stride ld elements, the same for
  * input and output) with an optional additive float32 mask[mask_rows, width] (contiguous;

@@ -65,6 +65,36 @@ def test_dropout_kernel(cuda, dtype):
     assert not y.any()                                                         # p = 1: everything dropped
 
 
+@pytest.mark.parametrize("dtype,width", [(torch.float32, 96), (torch.bfloat16, 1024), (torch.bfloat16, 100), (torch.float32, 37)])
+def test_dropout_inside_the_residual_layer_norm(cuda, dtype, width):
+    """LN(dropout(x) + res) in one kernel and its two-result backward against the three separate kernels (dropout,
+    add + layer_norm, their backwards): the same decisions, and values equal to the last bit of the storage type
+    (both round where the separate kernels store)."""
+    rows, p, sid = 37, 0.3, 9
+    g = torch.Generator().manual_seed(width)
+    x = torch.randn(rows, width, generator=g).to(dtype).to(cuda)
+    res = torch.randn(rows, width, generator=g).to(dtype).to(cuda)
+    dy = torch.randn(rows, width, generator=g).to(dtype).to(cuda)
+    st = _state(cuda, 5, 2)
+    xd, y0, y1 = torch.empty_like(x), torch.empty_like(x), torch.empty_like(x)
+    r0, r1 = torch.empty(rows, device=cuda), torch.empty(rows, device=cuda)
+    ops.dropout(x, xd, p, st, sid)
+    ops.add_layernorm_fwd(xd, res, y0, r0)
+    ops.add_layernorm_fwd(x, res, y1, r1, drop=(p, st, sid))
+    # float32: the fused kernel may contract x * scale + res into one fused multiply-add
+    same = torch.equal if dtype == torch.bfloat16 else (lambda u, v: torch.allclose(u, v, rtol=1e-5, atol=1e-6))
+    assert same(y0, y1) and same(r0, r1)
+    dx0, dd0, dx1, dd1 = (torch.empty_like(x) for _ in range(4))
+    ops.layernorm_bwd(dy, y0, r0, None, dx0)
+    ops.dropout(dx0, dd0, p, st, sid)
+    ops.layernorm_bwd(dy, y1, r1, None, dx1, dd1, (p, st, sid))
+    assert same(dx0, dx1) and same(dd0, dd1)
+    keep = ops.dropout_mask(rows * width, p, st, sid).view(rows, width).bool()
+    assert torch.equal(dd1 != 0, keep & (dx1 != 0))
+    with pytest.raises(ValueError):
+        ops.layernorm_bwd(dy, y1, r1, None, dx1, dx1, (p, st, sid))
+
+
 def _masks_from_oracle(ex, step):
     """The decisions the CPU oracle is given: relu masks from the GPU (see test_gpu_full_size), dropout masks from
     the oracle's own restatement of the keep function for the executor's seed, the step count and the node ids."""
@@ -76,8 +106,8 @@ def _masks_from_oracle(ex, step):
         if node.op != "call_function":
             continue
         if node.target is F.dropout and float(node.args[1]) > 0:
-            shape = ex.env[node].t.shape
-            out[node.name] = ref.dropout_keep(seed, step, i, float(node.args[1]), ex.env[node].t.numel()).view(shape)
+            shape = ex.env[node].shape                     # a dropout inside a neighbouring kernel has no tensor
+            out[node.name] = ref.dropout_keep(seed, step, i, float(node.args[1]), math.prod(shape)).view(shape)
         elif node.target is F.multi_head_attention_forward and float(node.kwargs["dropout_p"]) > 0:
             p, sid, shape, S = ex.env[node].meta["dropout"]
             assert sid == i
@@ -149,7 +179,8 @@ def test_dropout_is_active_and_unbiased_in_a_program(cuda):
     base = plain.forward(x, y).item()
     losses = [ex.forward(x, y).item() for _ in range(20)]
     assert len(set(losses)) == 20 and all(abs(l - base) > 1e-6 * base for l in losses)
-    node = next(n for n in gm.graph.nodes if n.op == "call_function" and n.target is F.dropout)
+    # a dropout that has a tensor of its own (those in front of a residual layer_norm run inside its kernel)
+    node = next(n for n in gm.graph.nodes if n.op == "call_function" and n.target is F.dropout and ex.env[n].t is not None)
     src, out = ex.env[node.args[0]], ex.env[node]
     acc, acc_src = torch.zeros_like(out.t, dtype=torch.float64), torch.zeros_like(out.t, dtype=torch.float64)
     for _ in range(200):                                                       # the input varies too (attention dropout)
