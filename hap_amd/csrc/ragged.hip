@@ -2,6 +2,7 @@
 // concat as multi-segment strided copies, and the rank-ordered float32 sum.
 // All of these are HBM-bound; every thread moves 16-byte vectors, four in flight.
 #include "common.h"
+#include "dropout.h"
 
 namespace {
 
@@ -25,13 +26,13 @@ struct SegmentList {
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 template <typename V> struct ActNone {
-    static constexpr bool MASKED = false;
+    static constexpr bool MASKED = false, INDEXED = false;
     __device__ __forceinline__ V operator()(V v) const { return v; }
 };
 // relu's backward fused into a copy: the element is kept where the forward output, which lies `delta` bytes from
 // the source element, is > 0 (NaN counts as not positive, as `y > 0.f` does)
 struct ReluBwdBf16 {
-    static constexpr bool MASKED = true;
+    static constexpr bool MASKED = true, INDEXED = false;
     int64_t delta;
     __device__ __forceinline__ u32x4 operator()(u32x4 v, u32x4 y) const {
         u32x4 r;
@@ -46,7 +47,7 @@ struct ReluBwdBf16 {
     }
 };
 struct ReluBwdF32 {
-    static constexpr bool MASKED = true;
+    static constexpr bool MASKED = true, INDEXED = false;
     int64_t delta;
     __device__ __forceinline__ u32x4 operator()(u32x4 v, u32x4 y) const {
         u32x4 r;
@@ -56,7 +57,7 @@ struct ReluBwdF32 {
     }
 };
 struct ReluBf16 {
-    static constexpr bool MASKED = false;
+    static constexpr bool MASKED = false, INDEXED = false;
     __device__ __forceinline__ u32x4 operator()(u32x4 v) const {
         // a bf16 is negative iff its sign bit is set; -0.0 -> +0.0 matches relu's value
         u32x4 r;
@@ -70,12 +71,52 @@ struct ReluBf16 {
     }
 };
 struct ReluF32 {
-    static constexpr bool MASKED = false;
+    static constexpr bool MASKED = false, INDEXED = false;
     __device__ __forceinline__ u32x4 operator()(u32x4 v) const {
         u32x4 r;
 #pragma unroll
         for (int i = 0; i < 4; ++i) r[i] = (v[i] & 0x80000000u) ? 0u : v[i];
         return r;
+    }
+};
+
+// relu's backward times a constant: the backward of relu followed by dropout, given the DROPPED forward output (it is
+// positive exactly where relu passed the element and dropout kept it; the constant is dropout's 1 / (1 - p))
+template <typename T> struct ReluBwdScaled {
+    static constexpr bool MASKED = true, INDEXED = false;
+    int64_t delta;
+    float scale;
+    __device__ __forceinline__ u32x4 operator()(u32x4 v, u32x4 y) const {
+        union { u32x4 u; Vec16<T> e; } g, m;
+        g.u = v;
+        m.u = y;
+#pragma unroll
+        for (int i = 0; i < Vec16<T>::N; ++i) g.e.set(i, m.e.get(i) > 0.f ? g.e.get(i) * scale : 0.f);
+        return g.u;
+    }
+};
+// relu followed by dropout on the copied elements; the decision for an element is the one the elementwise dropout
+// kernel takes for its index in the destination tensor (which starts at dst_base)
+template <typename T> struct ReluDrop {
+    static constexpr bool MASKED = false, INDEXED = true;
+    const char *dst_base;
+    const int64_t *state;
+    int64_t stream_id;
+    float p;
+    __device__ __forceinline__ DropKey key() const { return drop_key(state[0], state[1], stream_id, p); }
+    // dst: where the 16 bytes go (an even element index: the vector is 16-byte aligned in an aligned tensor)
+    __device__ __forceinline__ u32x4 operator()(u32x4 v, const char *dst, const DropKey &k) const {
+        union { u32x4 u; Vec16<T> e; } x;
+        x.u = v;
+        const uint64_t first = (uint64_t)(dst - dst_base) / sizeof(T);
+#pragma unroll
+        for (int i = 0; i < Vec16<T>::N; i += 2) {
+            const uint32_t bits = drop_pair_bits(k, (first + i) >> 1);
+            const float a = x.e.get(i), b = x.e.get(i + 1);
+            x.e.set(i, (a > 0.f && (bits & 0xffffU) >= k.thr) ? a * k.scale : 0.f);
+            x.e.set(i + 1, (b > 0.f && (bits >> 16) >= k.thr) ? b * k.scale : 0.f);
+        }
+        return x.u;
     }
 };
 
@@ -88,6 +129,8 @@ __global__ __launch_bounds__(COPY_THREADS) void segment_copy_kernel(SegmentList 
     const uint64_t per_row = (uint64_t)s.row_bytes / sizeof(V);
     const uint64_t total = per_row * (uint64_t)s.rows;
     const uint64_t step = (uint64_t)gridDim.x * COPY_THREADS * COPY_UNROLL;
+    DropKey key;
+    if constexpr (Act::INDEXED) key = act.key();
     for (uint64_t base = (uint64_t)blockIdx.x * COPY_THREADS * COPY_UNROLL + threadIdx.x; base < total; base += step) {
         V v[COPY_UNROLL], y[Act::MASKED ? COPY_UNROLL : 1];
         uint64_t doff[COPY_UNROLL];
@@ -120,6 +163,7 @@ __global__ __launch_bounds__(COPY_THREADS) void segment_copy_kernel(SegmentList 
         for (int u = 0; u < COPY_UNROLL; ++u) {
             if (!ok[u]) continue;
             if constexpr (Act::MASKED) *(V *)(s.dst + doff[u]) = act(v[u], y[u]);
+            else if constexpr (Act::INDEXED) *(V *)(s.dst + doff[u]) = act(v[u], s.dst + doff[u], key);
             else *(V *)(s.dst + doff[u]) = act(v[u]);
         }
     }
@@ -127,9 +171,17 @@ __global__ __launch_bounds__(COPY_THREADS) void segment_copy_kernel(SegmentList 
 
 // act: HAPMI_ACT_NONE, HAPMI_ACT_RELU (applied to the copied elements), or ACT_RELU_BWD (elements kept where the
 // element `mask_delta` bytes after the source element is > 0)
-constexpr int ACT_RELU_BWD = -1;
+// ACT_RELU_BWD with scale != 1: the kept elements are multiplied by scale.  ACT_RELU_DROP: relu, then dropout as
+// DropSpec describes it.
+constexpr int ACT_RELU_BWD = -1, ACT_RELU_DROP = -2;
+struct DropSpec {
+    const void *dst_base;
+    const int64_t *state;
+    int64_t stream_id;
+    float p;
+};
 int launch_segments(const SegmentList &list, int act, int dtype, hipStream_t stream, const char *name,
-                    int64_t mask_delta = 0) {
+                    int64_t mask_delta = 0, float scale = 1.f, const DropSpec *drop = nullptr) {
     if (list.n == 0) return HAPMI_OK;
     // widest vector that divides every address, stride and row length
     uint64_t bits = 0;
@@ -154,10 +206,25 @@ int launch_segments(const SegmentList &list, int act, int dtype, hipStream_t str
     dim3 grid((unsigned)gx, (unsigned)list.n), block(COPY_THREADS);
     if (act == ACT_RELU_BWD) {
         HAPMI_REQUIRE(vec == 16 && mask_delta % 16 == 0, HAPMI_EALIGN, "%s: the fused relu backward needs 16-byte aligned pieces", name);
-        if (dtype == HAPMI_BF16)
+        if (scale != 1.f && dtype == HAPMI_BF16)
+            hipLaunchKernelGGL((segment_copy_kernel<u32x4, ReluBwdScaled<bf16_t>>), grid, block, 0, stream, list,
+                               ReluBwdScaled<bf16_t>{mask_delta, scale});
+        else if (scale != 1.f)
+            hipLaunchKernelGGL((segment_copy_kernel<u32x4, ReluBwdScaled<float>>), grid, block, 0, stream, list,
+                               ReluBwdScaled<float>{mask_delta, scale});
+        else if (dtype == HAPMI_BF16)
             hipLaunchKernelGGL((segment_copy_kernel<u32x4, ReluBwdBf16>), grid, block, 0, stream, list, ReluBwdBf16{mask_delta});
         else
             hipLaunchKernelGGL((segment_copy_kernel<u32x4, ReluBwdF32>), grid, block, 0, stream, list, ReluBwdF32{mask_delta});
+    } else if (act == ACT_RELU_DROP) {
+        HAPMI_REQUIRE(vec == 16 && drop && ((uintptr_t)drop->dst_base % 16) == 0, HAPMI_EALIGN,
+                      "%s: relu + dropout needs 16-byte aligned pieces", name);
+        if (dtype == HAPMI_BF16)
+            hipLaunchKernelGGL((segment_copy_kernel<u32x4, ReluDrop<bf16_t>>), grid, block, 0, stream, list,
+                               ReluDrop<bf16_t>{(const char *)drop->dst_base, drop->state, drop->stream_id, drop->p});
+        else
+            hipLaunchKernelGGL((segment_copy_kernel<u32x4, ReluDrop<float>>), grid, block, 0, stream, list,
+                               ReluDrop<float>{(const char *)drop->dst_base, drop->state, drop->stream_id, drop->p});
     } else if (act != HAPMI_ACT_NONE) {
         HAPMI_REQUIRE(act == HAPMI_ACT_RELU, HAPMI_EINVAL, "%s: only relu can be fused into a concat", name);
         HAPMI_REQUIRE(vec == 16, HAPMI_EALIGN, "%s: fused activation needs 16-byte aligned pieces", name);
@@ -309,9 +376,9 @@ extern "C" int hapmi_split_rows(const void *src, void *const *pieces, const int6
     return launch_segments(list, HAPMI_ACT_NONE, 0, (hipStream_t)stream, "split_rows");
 }
 
-extern "C" int hapmi_split_rows_relu_bwd(const void *src, const void *fwd_out, void *const *pieces,
-                                         const int64_t *lengths, int n_ranks, int64_t outer, int64_t inner_bytes,
-                                         int dtype, hapmi_stream_t stream) {
+namespace {
+int split_rows_relu_bwd(const void *src, const void *fwd_out, void *const *pieces, const int64_t *lengths, int n_ranks,
+                        int64_t outer, int64_t inner_bytes, float scale, int dtype, hapmi_stream_t stream) {
     int64_t total;
     int rc = check_lengths(lengths, n_ranks, &total, "split_rows_relu_bwd");
     if (rc) return rc;
@@ -329,11 +396,25 @@ extern "C" int hapmi_split_rows_relu_bwd(const void *src, const void *fwd_out, v
         off += lengths[i];
     }
     return launch_segments(list, ACT_RELU_BWD, dtype, (hipStream_t)stream, "split_rows_relu_bwd",
-                           (int64_t)((const char *)fwd_out - (const char *)src));
+                           (int64_t)((const char *)fwd_out - (const char *)src), scale);
+}
+}  // namespace
+
+extern "C" int hapmi_split_rows_relu_bwd(const void *src, const void *fwd_out, void *const *pieces,
+                                         const int64_t *lengths, int n_ranks, int64_t outer, int64_t inner_bytes,
+                                         int dtype, hapmi_stream_t stream) {
+    return split_rows_relu_bwd(src, fwd_out, pieces, lengths, n_ranks, outer, inner_bytes, 1.f, dtype, stream);
 }
 
-extern "C" int hapmi_concat_rows(const void *const *pieces, const int64_t *lengths, int n_ranks, void *dst,
-                                 int64_t outer, int64_t inner_bytes, int act, int dtype, hapmi_stream_t stream) {
+extern "C" int hapmi_split_rows_relu_bwd_scaled(const void *src, const void *fwd_out, void *const *pieces,
+                                                const int64_t *lengths, int n_ranks, int64_t outer, int64_t inner_bytes,
+                                                float scale, int dtype, hapmi_stream_t stream) {
+    return split_rows_relu_bwd(src, fwd_out, pieces, lengths, n_ranks, outer, inner_bytes, scale, dtype, stream);
+}
+
+namespace {
+int concat_rows(const void *const *pieces, const int64_t *lengths, int n_ranks, void *dst, int64_t outer, int64_t inner_bytes,
+                int act, int dtype, const DropSpec *drop, hapmi_stream_t stream) {
     int64_t total;
     int rc = check_lengths(lengths, n_ranks, &total, "concat_rows");
     if (rc) return rc;
@@ -354,7 +435,24 @@ extern "C" int hapmi_concat_rows(const void *const *pieces, const int64_t *lengt
         }
         off += lengths[i];
     }
-    return launch_segments(list, act, dtype, (hipStream_t)stream, "concat_rows");
+    return launch_segments(list, act, dtype, (hipStream_t)stream, "concat_rows", 0, 1.f, drop);
+}
+}  // namespace
+
+extern "C" int hapmi_concat_rows(const void *const *pieces, const int64_t *lengths, int n_ranks, void *dst,
+                                 int64_t outer, int64_t inner_bytes, int act, int dtype, hapmi_stream_t stream) {
+    HAPMI_REQUIRE(act == HAPMI_ACT_NONE || act == HAPMI_ACT_RELU, HAPMI_EINVAL, "concat_rows: only relu can be fused into a concat");
+    return concat_rows(pieces, lengths, n_ranks, dst, outer, inner_bytes, act, dtype, nullptr, stream);
+}
+
+extern "C" int hapmi_concat_rows_relu_dropout(const void *const *pieces, const int64_t *lengths, int n_ranks, void *dst,
+                                              int64_t outer, int64_t inner_bytes, float p, const int64_t *rng_state_dev,
+                                              int64_t stream_id, int dtype, hapmi_stream_t stream) {
+    HAPMI_REQUIRE(p >= 0.f && p <= 1.f && rng_state_dev && ((uintptr_t)rng_state_dev % 8) == 0, HAPMI_EINVAL,
+                  "concat_rows_relu_dropout: bad probability %g or RNG state", (double)p);
+    HAPMI_REQUIRE(hapmi_dtype_ok(dtype), HAPMI_EINVAL, "concat_rows_relu_dropout: bad dtype %d", dtype);
+    const DropSpec drop = {dst, rng_state_dev, stream_id, p};
+    return concat_rows(pieces, lengths, n_ranks, dst, outer, inner_bytes, ACT_RELU_DROP, dtype, &drop, stream);
 }
 
 // ---------------------------------------------------------------------------

@@ -726,6 +726,14 @@ class ShardExecutor:
             self._unsupported(node, f"dropout of a {x.kind} value")
         self._uses_rng = True
         sid = self._node_ids[node]
+        if (self.fuse_dropout and x.meta.get("fused_act") == "relu" and x.meta.get("can_fuse_drop") and p < 1.0
+                and "fused_drop" not in x.meta and self._only_reader(node, x)):
+            # relu -> dropout, both applied by the kernel that produces the value (it reads fused_drop when it runs).
+            # The stored value is the dropped one: positive exactly where relu passed and dropout kept, so every
+            # form of relu's backward serves as the backward of both once its result is scaled by 1 / (1 - p).
+            x.meta["fused_drop"] = (p, sid)
+            x.meta["dropout"] = (p, sid)
+            return x
         if self.fuse_dropout and self._feeds_residual_layer_norm(node, x):
             # dropout -> add -> layer_norm: the layer_norm kernels apply it to their operand (forward) and give its
             # backward as a second result; nothing is materialised here
@@ -925,8 +933,9 @@ class ShardExecutor:
                         and not x.meta.get("relu_bwd_done") and not x.meta.get("relu_bwd_in_split")):
                     mask = x.t
                     x.meta["relu_bwd_done"] = True
+                k = self._relu_grad_scale(x) if mask is not None else 1.0
                 self.bwd.append(lambda: ops.gemm(dy, w.t, g, M, K, N, lda=ldc, ldc=lda, accumulate=acc, relu_mask=mask,
-                                                 addend=addend))
+                                                 addend=addend, alpha=k))
         self._tape.append(emit)
         return out
 
@@ -980,20 +989,32 @@ class ShardExecutor:
         users = list(node.users)
         return len(users) == 1 and users[0].target is F.relu
 
+    @staticmethod
+    def _relu_grad_scale(out: Val) -> float:
+        """1 / (1 - p) of the dropout folded into the producer behind its relu (1 without one)."""
+        fd = out.meta.get("fused_drop")
+        return 1.0 / (1.0 - fd[0]) if fd else 1.0
+
     def _relu_backward_through(self, out: Val):
-        """For a producer that applied relu itself: d(pre-activation) = d(out) * (out > 0), in place."""
+        """For a producer that applied relu itself: d(pre-activation) = d(out) * (out > 0), in place (times the
+        factor of a dropout folded in behind the relu)."""
         if out.meta.get("relu_bwd_done"):
             return
         g = out.grad
+        k = self._relu_grad_scale(out)
         if len(self._grad_sharers.get(g.untyped_storage().data_ptr(), ())) > 1 or self._is_read_later(g):
             # the buffer is also another value's gradient (or a launch that is held back reads it): mask into a new one
             self.shared_gradient_copies += 1
             out.grad = self._new(g.shape, g.dtype)
             masked = out.grad
             self.bwd.append(lambda: ops.act_bwd(g, out.t, masked, "relu"))
+            if k != 1.0:
+                self.bwd.append(lambda: ops.scale(masked, k, masked))
             return
         self._guard_write(g)
         self.bwd.append(lambda: ops.act_bwd(g, out.t, g, "relu"))
+        if k != 1.0:
+            self.bwd.append(lambda: ops.scale(g, k, g))
 
     # ---- attention ------------------------------------------------------------------------------
     def _mha(self, node):
@@ -1479,14 +1500,18 @@ class ShardExecutor:
         return out
 
     def _emit_exchange(self, tag, direction, x_t, split_dim, cat_dim, split_L, cat_L, rank, sink, act=None,
-                       relu_of=None, receive_in_place=False, presplit=False):
+                       relu_of=None, receive_in_place=False, presplit=False, drop_from: Optional[Val] = None,
+                       relu_scale: float = 1.0):
         """The local half of an all_to_all.  ``act``: activation applied while concatenating.  ``relu_of``: forward
         output of a relu whose backward is applied to ``x_t`` while splitting (only for a split that copies).
         ``receive_in_place`` (concatenation along dim 0, no activation): the peers' pieces are received straight
         into their rows of the result, which nothing may write afterwards; no concat launch is left.
         ``presplit``: ``x_t`` is only a shape (a meta tensor); the caller writes the pieces itself (a GEMM whose result
         is laid out in pieces).  Returns (result, pieces, finish): nothing is launched until ``finish()`` appends
-        what is left of the exchange (the concat, the wire's send hooks)."""
+        what is left of the exchange (the concat, the wire's send hooks).
+        ``drop_from``: the value this exchange produces; if a dropout behind the fused relu has been folded into it
+        (meta fused_drop, set after this call), the concat applies it too.  ``relu_scale``: factor on ``relu_of``'s
+        masked gradient (that dropout's 1 / (1 - p))."""
         W = len(split_L)
         # pieces along the slowest dimension are contiguous ranges of the input: views, as torch.split gives the
         # reference (collectives.py:156); any other dimension needs the strided copy
@@ -1513,12 +1538,16 @@ class ShardExecutor:
                     self._wire_backed.add(out.untyped_storage().data_ptr())
                 parts.append(self.wire.recv(tag, direction, src, shape, self.cdt, self.dev, reduction=False, into=into))
 
+        def drop():
+            fd = drop_from.meta.get("fused_drop") if drop_from is not None else None
+            return (fd[0], self.rng_state, fd[1]) if fd else None
+
         def finish():
             if views or presplit:
-                sink.append(lambda: ops.concat_rows(parts, cat_dim, out, act))
+                sink.append(lambda: ops.concat_rows(parts, cat_dim, out, act, drop()))
             else:
-                sink.append(lambda: (ops.split_rows(x_t, split_L, split_dim, pieces, relu_of=relu_of),
-                                     ops.concat_rows(parts, cat_dim, out, act)))
+                sink.append(lambda: (ops.split_rows(x_t, split_L, split_dim, pieces, relu_of=relu_of, scale=relu_scale),
+                                     ops.concat_rows(parts, cat_dim, out, act, drop())))
             self._announce(tag, direction, rank, W, lambda dst: pieces[dst], sink)
         if presplit:
             return out, pieces, finish
@@ -1603,14 +1632,18 @@ class ShardExecutor:
                 and sum(1 for l in cL if l > 0) <= ops._lib.GEMM_MAX_SEGMENTS and sL[rank] > 0 and x.t.shape[-1] % 8 == 0):
             return self._exchange_in_pieces(node, x, sd, cd, sL, cL, rank)
         fuse = self._wants_fused_relu(node)
-        t = self._emit_exchange(node.name, "fwd", x.t, sd, cd, sL, cL, rank, self.fwd, "relu" if fuse else None)
-        out = Val("tensor", t, needs_grad=x.needs_grad)
+        out = Val("tensor", None, needs_grad=x.needs_grad)
+        out.t = self._emit_exchange(node.name, "fwd", x.t, sd, cd, sL, cL, rank, self.fwd, "relu" if fuse else None,
+                                    drop_from=out)
+        out.shape = tuple(out.t.shape)
         if fuse:
             out.meta["fused_act"] = "relu"
+            # a dropout behind the relu can ride on the same copy (16-byte vectors of the result)
+            out.meta["can_fuse_drop"] = self._split_can_mask(out.t, out.t, cd, cL)
             # the backward exchange splits along the forward's concat dimension; where that split copies, relu's
             # backward rides on the copy instead of a pass of its own over the gradient (or a mask read in the
             # next linear's data-gradient GEMM)
-            out.meta["relu_bwd_in_split"] = self.relu_bwd_in_split and cd != 0 and self._split_can_mask(t, t, cd, cL)
+            out.meta["relu_bwd_in_split"] = self.relu_bwd_in_split and cd != 0 and self._split_can_mask(out.t, out.t, cd, cL)
 
         def emit():
             if out.grad is None or not x.needs_grad:
@@ -1625,7 +1658,8 @@ class ShardExecutor:
             in_place = (self.receive_in_place and x.grad is None and isinstance(producer, torch.fx.Node)
                         and producer.target is F.linear and len(producer.users) == 1 and not x.meta.get("fused_act"))
             g = self._emit_exchange(node.name, "bwd", out.grad, cd, sd, cL, sL, rank, self.bwd,
-                                    relu_of=out.t if in_split else None, receive_in_place=in_place)
+                                    relu_of=out.t if in_split else None, receive_in_place=in_place,
+                                    relu_scale=self._relu_grad_scale(out) if in_split else 1.0)
             self._accumulate_into(x, g)
         self._tape.append(emit)
         return out

@@ -175,9 +175,10 @@ def place_rows(src: torch.Tensor, dst: torch.Tensor, dim: int, offset: int) -> t
 
 def split_rows(src: torch.Tensor, lengths: Sequence[int], dim: int,
                outs: Optional[Sequence[Optional[torch.Tensor]]] = None,
-               relu_of: Optional[torch.Tensor] = None) -> List[torch.Tensor]:
+               relu_of: Optional[torch.Tensor] = None, scale: float = 1.0) -> List[torch.Tensor]:
     """Pieces of ``src`` along ``dim``; with ``relu_of`` (a relu's forward output of src's shape) the pieces
-    are those of ``src * (relu_of > 0)``."""
+    are those of ``src * (relu_of > 0) * scale`` (scale != 1: relu followed by dropout, relu_of being the dropped
+    output and scale dropout's 1 / (1 - p))."""
     _dev(src)
     assert src.is_contiguous()
     outer, total, inner = _oli(src.shape, dim)
@@ -193,8 +194,13 @@ def split_rows(src: torch.Tensor, lengths: Sequence[int], dim: int,
     if relu_of is not None:
         _dev(relu_of)
         assert relu_of.is_contiguous() and relu_of.shape == src.shape and relu_of.dtype == src.dtype
-        check(lib().hapmi_split_rows_relu_bwd(_ptr(src), _ptr(relu_of), _ptrs(outs), _i64(lengths), len(lengths),
-                                              outer, inner * src.element_size(), dtype_code(src), _stream()))
+        if scale != 1.0:
+            check(lib().hapmi_split_rows_relu_bwd_scaled(_ptr(src), _ptr(relu_of), _ptrs(outs), _i64(lengths),
+                                                         len(lengths), outer, inner * src.element_size(),
+                                                         ctypes.c_float(scale), dtype_code(src), _stream()))
+        else:
+            check(lib().hapmi_split_rows_relu_bwd(_ptr(src), _ptr(relu_of), _ptrs(outs), _i64(lengths), len(lengths),
+                                                  outer, inner * src.element_size(), dtype_code(src), _stream()))
         return list(outs)
     check(lib().hapmi_split_rows(_ptr(src), _ptrs(outs), _i64(lengths), len(lengths), outer,
                                  inner * src.element_size(), _stream()))
@@ -202,7 +208,9 @@ def split_rows(src: torch.Tensor, lengths: Sequence[int], dim: int,
 
 
 def concat_rows(pieces: Sequence[torch.Tensor], dim: int, out: Optional[torch.Tensor] = None,
-                act: Optional[str] = None) -> torch.Tensor:
+                act: Optional[str] = None, drop=None) -> torch.Tensor:
+    """``drop`` = (p, rng_state, stream_id) with act = "relu": out = dropout(relu(cat(pieces))), the decisions
+    being those ``dropout`` takes for ``out`` under the same three."""
     _dev(*pieces, out)
     ref = pieces[0]
     lengths = [p.shape[dim] for p in pieces]
@@ -215,6 +223,16 @@ def concat_rows(pieces: Sequence[torch.Tensor], dim: int, out: Optional[torch.Te
             raise TypeError("concat_rows: dtype mismatch")
     _need(out, outer * sum(lengths) * inner, "concat_rows dst")
     if out.numel() == 0:
+        return out
+    if drop is not None:
+        if act != "relu":
+            raise ValueError("concat_rows: dropout rides on a fused relu only")
+        p, rng_state, stream_id = drop
+        _dev(rng_state)
+        _check_rng(rng_state, "concat_rows")
+        check(lib().hapmi_concat_rows_relu_dropout(_ptrs(pieces), _i64(lengths), len(lengths), _ptr(out), outer,
+                                                   inner * ref.element_size(), ctypes.c_float(p), _ptr(rng_state),
+                                                   int(stream_id), dtype_code(ref), _stream()))
         return out
     check(lib().hapmi_concat_rows(_ptrs(pieces), _i64(lengths), len(lengths), _ptr(out), outer,
                                   inner * ref.element_size(), _ACT[act], dtype_code(ref) if _ACT[act] else 0, _stream()))

@@ -93,6 +93,13 @@ int hapmi_split_rows(const void *src, void *const *pieces_host, const int64_t *l
 int hapmi_split_rows_relu_bwd(const void *src, const void *fwd_out, void *const *pieces_host,
                               const int64_t *lengths_host, int n_ranks, int64_t outer, int64_t inner_bytes,
                               int dtype, hapmi_stream_t stream);
+/* The same with the kept elements multiplied by `scale`: the backward of F.relu followed by F.dropout(p)
+ * (hap.rs:1417, 1464; the FFN's activation and the dropout behind it, models.py:116), given the DROPPED forward
+ * output as fwd_out -- it is positive exactly where relu passed the element and dropout kept it -- and
+ * scale = 1 / (1 - p); no random numbers are needed backward. */
+int hapmi_split_rows_relu_bwd_scaled(const void *src, const void *fwd_out, void *const *pieces_host,
+                                     const int64_t *lengths_host, int n_ranks, int64_t outer, int64_t inner_bytes,
+                                     float scale, int dtype, hapmi_stream_t stream);
 
 /* collectives.py:159 / :166: concatenate W contiguous pieces [outer, lengths[i], inner]
  * into dst[outer, sum(lengths), inner]; `act` != NONE applies the activation to
@@ -100,6 +107,12 @@ int hapmi_split_rows_relu_bwd(const void *src, const void *fwd_out, void *const 
  * (act = NONE, outer = 1 and pieces[i] == dst + offset of piece i) is left where it is. */
 int hapmi_concat_rows(const void *const *pieces_host, const int64_t *lengths_host, int n_ranks, void *dst,
                       int64_t outer, int64_t inner_bytes, int act, int dtype, hapmi_stream_t stream);
+/* hapmi_concat_rows with F.relu and then F.dropout(p) (hap.rs:1417, 1464) applied on the way: dst =
+ * dropout(relu(cat(pieces))), with the keep decisions hapmi_dropout takes for dst as a whole under the same p,
+ * RNG state and stream id.  Pieces and dst 16-byte aligned with inner_bytes * lengths a multiple of 16. */
+int hapmi_concat_rows_relu_dropout(const void *const *pieces_host, const int64_t *lengths_host, int n_ranks, void *dst,
+                                   int64_t outer, int64_t inner_bytes, float p, const int64_t *rng_state_dev,
+                                   int64_t stream_id, int dtype, hapmi_stream_t stream);
 
 /* the local sum of dist.reduce_scatter / dist.all_reduce (collectives.py:27, :95, :77):
  * dst[outer, len, inner] = sum_w contribs[w][outer, src_len, inner][:, offset:offset+len, :]

@@ -95,6 +95,40 @@ def test_dropout_inside_the_residual_layer_norm(cuda, dtype, width):
         ops.layernorm_bwd(dy, y1, r1, None, dx1, dx1, (p, st, sid))
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("dim", [0, 2])
+def test_relu_and_dropout_inside_the_concatenating_copy(cuda, dtype, dim):
+    """dropout(relu(cat(pieces))) in the copy of an all_to_all against concat, relu and dropout as separate kernels
+    (bit for bit), and its backward -- split of g * (dropped output > 0) / (1 - p) -- against dropout's and relu's
+    backward kernels followed by the split."""
+    p, sid = 0.3, 4
+    g = torch.Generator().manual_seed(3 + dim)
+    lengths = [8, 24, 0, 16]
+    shape = [6, 5, 48]
+    pieces = []
+    for l in lengths:
+        sh = list(shape)
+        sh[dim] = l
+        pieces.append(torch.randn(*sh, generator=g).to(dtype).to(cuda))
+    shape[dim] = sum(lengths)
+    st = _state(cuda, 21, 6)
+    want = torch.empty(*shape, dtype=dtype, device=cuda)
+    ops.concat_rows(pieces, dim, want, "relu")
+    ops.dropout(want, want, p, st, sid)
+    got = ops.concat_rows(pieces, dim, torch.empty_like(want), "relu", drop=(p, st, sid))
+    assert torch.equal(got, want)
+    keep = ops.dropout_mask(want.numel(), p, st, sid).view(want.shape).bool()
+    assert torch.equal(got != 0, keep & (torch.cat(pieces, dim) > 0))
+    dy = torch.randn(*shape, generator=g).to(dtype).to(cuda)
+    tmp = torch.empty_like(dy)
+    ops.dropout(dy, tmp, p, st, sid)
+    ops.act_bwd(tmp, want, tmp, "relu")
+    want_pieces = ops.split_rows(tmp, lengths, dim)
+    got_pieces = ops.split_rows(dy, lengths, dim, relu_of=got, scale=1.0 / (1.0 - p))
+    for a, b in zip(got_pieces, want_pieces):
+        assert torch.equal(a, b)
+
+
 def _masks_from_oracle(ex, step):
     """The decisions the CPU oracle is given: relu masks from the GPU (see test_gpu_full_size), dropout masks from
     the oracle's own restatement of the keep function for the executor's seed, the step count and the node ids."""
