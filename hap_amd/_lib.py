@@ -49,6 +49,7 @@ class GemmArgs(ctypes.Structure):
         ("A_segments", ctypes.c_void_p), ("B_segments", ctypes.c_void_p), ("C_segments", ctypes.c_void_p),
         ("c_mask_segments", ctypes.c_void_p), ("B_segments_list", ctypes.c_void_p),
         ("a_relu", ctypes.c_int), ("b_relu", ctypes.c_int),
+        ("drop_state", ctypes.c_void_p), ("drop_stream_id", ctypes.c_int64), ("drop_p", ctypes.c_float),
     ]
 
 

@@ -231,7 +231,8 @@ int launch_typed(GemmParams &p, int transA, int transB, int64_t batch, hipStream
     if (want_rs && (!workspace || ((uintptr_t)workspace % 16) != 0))
         return hapmi_set_error(HAPMI_EINVAL, "gemm: a_rowsum needs a 16-byte aligned workspace for its partial sums");
     const bool segmented = p.segA.n > 0 || p.segB.n > 0 || p.segC.n > 0;
-    const int64_t max_splits = (!segmented && workspace && ((uintptr_t)workspace % 16) == 0 && per_split > 0) ? split_bytes / per_split : 0;
+    // dropout in the epilogue is applied by the GEMM kernel itself, so the reduction is not split then
+    const int64_t max_splits = (!segmented && !p.drop_state && workspace && ((uintptr_t)workspace % 16) == 0 && per_split > 0) ? split_bytes / per_split : 0;
     Choice ch = choose(p.M, p.N, p.K, batch, bk, sizeof(TI) == 2, wide, max_splits, !transA && transB, need);
     if (ch.cfg < 0)
         return hapmi_set_error(HAPMI_EINVAL, "gemm: no tile configuration fits the pieces of the operands (boundaries along N "
@@ -403,6 +404,15 @@ extern "C" int hapmi_gemm(const hapmi_gemm_args *a, hapmi_stream_t stream) {
     p.relu_mask = a->c_relu_mask;
     HAPMI_REQUIRE(!a->c_relu_mask || (!lists && ((uintptr_t)a->c_relu_mask % 16) == 0), HAPMI_EINVAL,
                   "gemm: c_relu_mask needs a 16-byte aligned pointer and no pointer lists");
+    p.drop_state = a->drop_state;
+    p.drop_stream = a->drop_stream_id;
+    p.drop_p = a->drop_p;
+    if (a->drop_state) {
+        HAPMI_REQUIRE(!lists && batch == 1 && !a->transA && a->transB && !a->accumulate && a->ldc == a->N && (a->N % 2) == 0 && !a->C_segments &&
+                          ((uintptr_t)a->drop_state % 8) == 0 && a->drop_p >= 0.f && a->drop_p <= 1.f,
+                      HAPMI_EINVAL, "gemm: dropout in the epilogue takes one contiguous problem (transA = 0, transB = 1, ldc = N, N even), no accumulate, "
+                      "and a probability in [0, 1]");
+    }
 
     // operands / result in pieces
     SegNeeds need;

@@ -17,6 +17,7 @@
 // contiguous dimension of C.
 #pragma once
 #include "common.h"
+#include "dropout.h"
 #include "tile.h"
 #include <type_traits>
 
@@ -54,6 +55,9 @@ struct GemmParams {
     GemmSegs segA, segB, segC, segM;                          // A along K; B, C and the relu mask along N
     const void *listSegB[HAPMI_GEMM_MAX_LIST][HAPMI_GEMM_MAX_SEGMENTS];   // with pointer lists: the B pieces of problem z
     int a_relu, b_relu;                                       // relu on op(A) / op(B) fragments as they are read
+    const int64_t *drop_state;                                // optional: F.dropout behind the activation (RNG state on the device)
+    int64_t drop_stream;
+    float drop_p;
 };
 static_assert(sizeof(GemmParams) <= 3072, "the parameter block travels as a kernel argument (4 KiB at most)");
 
@@ -96,7 +100,8 @@ __device__ __forceinline__ f32x4 relu_frag(f32x4 v) {
 // fragments of op(A).  4: relu on the fragments of op(B) (TN layout: the weight gradient whose B operand is the
 // activation that a relu produced).  8: measurement build of the three-stage loop: every k-tile's operands are
 // loaded into LDS and waited for as usual, but no fragment is read and no MFMA issued (the result is zeros); it
-// tells how much of a launch's time is the movement of the operands from L2 into the CU.  The other kinds of pieces (B, C and the mask along N) only move this block's
+// tells how much of a launch's time is the movement of the operands from L2 into the CU.  16: F.dropout behind the
+// activation in the epilogue (NT layout: a linear's forward; p.drop_*).  The other kinds of pieces (B, C and the mask along N) only move this block's
 // base pointers and leading dimensions, which costs nothing, so they need no instantiation of their own.
 template <typename TI, typename TO, int BM, int BN, int WAVES_M, int WAVES_N, bool A_KMAJOR, bool B_KMAJOR, int NSTAGES, int OPMODE = 0>
 // the four-wave 128 x 128 tile is meant to run two blocks per CU: keep it within 256 registers
@@ -471,6 +476,32 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, ((WAVES_M * WAVES_N <= 4 && 
 #pragma unroll
                     for (int r = 0; r < 16; ++r) acc[i][j][r] = apply_act(acc[i][j][r], HAPMI_ACT_GELU);
         }
+        if constexpr ((OPMODE & 16) != 0) {
+            // F.dropout behind the activation: the decision for C[m][n] is the one the elementwise dropout kernel
+            // takes for element m * ldc + n (the host admits one contiguous problem only); registers 4 q + e of a
+            // lane are four neighbouring columns, so one hash serves two of them.  For a 2-byte result the value is
+            // rounded before it is scaled, as the stored activation would have been.
+            const DropKey key = drop_key(p.drop_state[0], p.drop_state[1], p.drop_stream, p.drop_p);
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+                const uint64_t row_first = (uint64_t)((m0 + wm + i * 32 + (lane & 31)) * ldc + n0 + wn + (lane >> 5) * 4);
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q)
+#pragma unroll
+                        for (int e = 0; e < 4; e += 2) {
+                            const uint32_t bits = drop_pair_bits(key, (row_first + j * 32 + q * 8 + e) >> 1);
+                            float lo = acc[i][j][q * 4 + e], hi = acc[i][j][q * 4 + e + 1];
+                            if (sizeof(TO) == 2) {
+                                lo = (float)(bf16_t)lo;
+                                hi = (float)(bf16_t)hi;
+                            }
+                            acc[i][j][q * 4 + e] = (bits & 0xffffU) >= key.thr ? lo * key.scale : 0.f;
+                            acc[i][j][q * 4 + e + 1] = (bits >> 16) >= key.thr ? hi * key.scale : 0.f;
+                        }
+            }
+        }
     }
 
     // bf16 output that is neither accumulated into nor a split-K partial: the band is staged as bf16 (half the
@@ -680,6 +711,11 @@ int launch_cfg(const GemmParams &p, int transA, int transB, int64_t batch, hipSt
             HAPMI_GEMM_LAUNCH_MODE(false, false, 4);
             return HAPMI_OK;
         }
+    }
+    if (p.drop_state) {
+        if (transA || !transB) return hapmi_set_error(HAPMI_EINVAL, "gemm: dropout in the epilogue needs transA = 0, transB = 1");
+        HAPMI_GEMM_LAUNCH_MODE(true, true, 16);
+        return HAPMI_OK;
     }
     if constexpr (PROBE != 0) {
         if (transA) return hapmi_set_error(HAPMI_EINVAL, "gemm: the measurement configuration takes transA = 0 only");

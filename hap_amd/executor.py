@@ -895,8 +895,13 @@ class ShardExecutor:
         fuse = self._wants_fused_relu(node) and ldc == N
         if fuse:
             out.meta["fused_act"] = "relu"
+            out.meta["can_fuse_drop"] = N % 2 == 0      # a dropout behind the relu rides on the epilogue as well
+
+        def drop():
+            fd = out.meta.get("fused_drop")
+            return (fd[0], self.rng_state, fd[1]) if fd else None
         self.fwd.append(lambda: ops.gemm(xt, w.t, store, M, N, K, transB=True, lda=lda, ldc=ldc, bias=bias,
-                                         act="relu" if fuse else None))
+                                         act="relu" if fuse else None, drop=drop()))
 
         def emit():
             if out.grad is None:

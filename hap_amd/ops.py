@@ -364,8 +364,10 @@ def gemm(A: Optional[torch.Tensor], B: Optional[torch.Tensor], C: Optional[torch
          offA=0, offB=0, offC=0, workspace: Optional[torch.Tensor] = None,
          a_rowsum: Optional[torch.Tensor] = None, relu_mask: Optional[torch.Tensor] = None,
          addend: Optional[torch.Tensor] = None, a_segments=None, b_segments=None, c_segments=None,
-         mask_segments=None, a_relu=False, b_relu=False):
-    """C = alpha * op(A) @ op(B) (+bias)(act)(+C).  Offsets and strides are in elements.  ``workspace`` (or
+         mask_segments=None, a_relu=False, b_relu=False, drop=None):
+    """C = alpha * op(A) @ op(B) (+bias)(act)(+C).  Offsets and strides are in elements.
+    ``drop`` = (p, rng_state, stream_id): dropout behind the activation, with the decisions ``dropout`` takes for C
+    (one contiguous problem).  ``workspace`` (or
     the buffer installed with ``set_gemm_workspace``) lets the library split a long reduction over K.
     ``a_rowsum`` (float32[M], transA only): the sums over k of op(A)'s rows are added into it.
     ``relu_mask`` ([M, ldc] like C): result elements whose mask is <= 0 are zero (relu backward).
@@ -374,6 +376,8 @@ def gemm(A: Optional[torch.Tensor], B: Optional[torch.Tensor], C: Optional[torch
     of pieces along K (A, stored [M, K]) or N (B stored [K, N], C, mask) instead of one tensor (pass None for it);
     ``a_relu`` / ``b_relu``: relu applied to that operand as it is loaded."""
     if a_segments is not None or b_segments is not None or c_segments is not None or a_relu or b_relu:
+        if drop is not None:
+            raise ValueError("gemm: dropout in the epilogue does not combine with operands in pieces")
         return _gemm_segmented(A, B, C, M, N, K, transA, transB, lda, ldb, ldc, bias, act, alpha, workspace, a_rowsum,
                                a_segments, b_segments, c_segments, mask_segments, a_relu, b_relu, accumulate)
     _dev(A, B, C, bias, a_rowsum, relu_mask, addend)
@@ -426,10 +430,15 @@ def gemm(A: Optional[torch.Tensor], B: Optional[torch.Tensor], C: Optional[torch
             raise TypeError("gemm addend: C's element type, accumulate and a single problem expected")
         _need(addend, _span(M, N, a.ldc), "gemm addend")
     a.c_addend = addend.data_ptr() if addend is not None else 0
+    if drop is not None:
+        p_, rng_state, stream_id = drop
+        _dev(rng_state)
+        _check_rng(rng_state, "gemm")
+        a.drop_state, a.drop_stream_id, a.drop_p = rng_state.data_ptr(), int(stream_id), float(p_)
     if min(strideA + strideB + strideC) < 0:
         raise _lib.HapmiError("gemm: negative batch stride")
     if _gemm_log is not None:
-        _gemm_log.append((a, (A, B, C, bias, ws, a_rowsum, relu_mask, addend)))  # the tensors keep the recorded pointers alive
+        _gemm_log.append((a, (A, B, C, bias, ws, a_rowsum, relu_mask, addend, drop)))  # the tensors keep the recorded pointers alive
     check(lib().hapmi_gemm(ctypes.byref(a), _stream()))
     return C
 

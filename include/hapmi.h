@@ -215,6 +215,13 @@ typedef struct {
     const hapmi_gemm_segments *A_segments, *B_segments, *C_segments, *c_mask_segments;
     const hapmi_gemm_segments *const *B_segments_list;
     int a_relu, b_relu;
+    /* F.dropout(., p) behind the activation (hap.rs:1464 after 1417: the dropout that follows the FFN's activation,
+     * models.py:116), applied by the epilogue with the decisions hapmi_dropout takes for C as a whole under the same
+     * p, RNG state and stream id.  One contiguous problem (transA = 0, transB = 1, batch 1, ldc = N, N even), no
+     * accumulate, no pieces; the reduction is not split.  drop_state = NULL: off */
+    const int64_t *drop_state;
+    int64_t drop_stream_id;
+    float drop_p;
 } hapmi_gemm_args;
 #define HAPMI_GEMM_MAX_LIST 16
 int hapmi_gemm(const hapmi_gemm_args *args_host, hapmi_stream_t stream);

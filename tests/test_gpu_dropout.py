@@ -129,6 +129,39 @@ def test_relu_and_dropout_inside_the_concatenating_copy(cuda, dtype, dim):
         assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("cfg,in_dtype,out_dtype", [(0, "bf16", "bf16"), (1, "bf16", "bf16"), (4, "bf16", "bf16"),
+                                                    (7, "bf16", "bf16"), (7, "bf16", "fp32"), (9, "bf16", "bf16"),
+                                                    (10, "fp32", "fp32"), (-1, "fp32", "fp32"), (-1, "bf16", "bf16")])
+def test_relu_and_dropout_in_the_gemm_epilogue(cuda, cfg, in_dtype, out_dtype):
+    """dropout(relu(x W^T + b)) from the GEMM's epilogue against the same GEMM with relu followed by the dropout
+    kernel: identical bits (the epilogue rounds a 2-byte result before scaling it, as the stored activation would
+    be), on a shape with partial tiles in M and N and a tile-aligned one, through several tile configurations."""
+    from hap_amd._lib import lib
+    tin = torch.bfloat16 if in_dtype == "bf16" else torch.float32
+    tout = torch.bfloat16 if out_dtype == "bf16" else torch.float32
+    p, sid = 0.25, 13
+    st = _state(cuda, 77, 1)
+    try:
+        lib().hapmi_gemm_tuning(cfg, 1 if cfg >= 0 else 0)
+        for (M, N, K) in [(424, 520, 192), (768, 512, 256)]:
+            g = torch.Generator().manual_seed(M)
+            A = torch.randn(M, K, generator=g).to(tin).to(cuda)
+            B = torch.randn(N, K, generator=g).to(tin).to(cuda)
+            bias = torch.randn(N, generator=g).to(cuda)
+            want = torch.empty(M, N, dtype=tout, device=cuda)
+            ops.gemm(A, B, want, M, N, K, transB=True, bias=bias, act="relu")
+            ops.dropout(want, want, p, st, sid)
+            got = torch.full((M, N), float("nan"), dtype=tout, device=cuda)
+            ops.gemm(A, B, got, M, N, K, transB=True, bias=bias, act="relu", drop=(p, st, sid))
+            assert torch.equal(got, want), (M, N, K)
+            assert 0.3 < (got != 0).float().mean().item() < 0.45      # half pass relu, three quarters of those are kept
+    finally:
+        lib().hapmi_gemm_tuning(-1, 0)
+    with pytest.raises(ops._lib.HapmiError):                           # a padded leading dimension has no flat index
+        ops.gemm(A, B, torch.empty(M, N + 8, dtype=tout, device=cuda), M, N, K, transB=True, ldc=N + 8, act="relu",
+                 drop=(p, st, sid))
+
+
 def _masks_from_oracle(ex, step):
     """The decisions the CPU oracle is given: relu masks from the GPU (see test_gpu_full_size), dropout masks from
     the oracle's own restatement of the keep function for the executor's seed, the step count and the node ids."""
