@@ -16,6 +16,9 @@ struct Segment {
     int64_t row_bytes;    // contiguous bytes per row
     int64_t src_stride;   // bytes between rows
     int64_t dst_stride;
+    // for functors that need to know which element of a tensor they hold (dropout): byte offset of the segment's
+    // first element in that tensor and the bytes between its rows there
+    int64_t index_first = 0, index_stride = 0;
 };
 
 struct SegmentList {
@@ -96,19 +99,18 @@ template <typename T> struct ReluBwdScaled {
     }
 };
 // relu followed by dropout on the copied elements; the decision for an element is the one the elementwise dropout
-// kernel takes for its index in the destination tensor (which starts at dst_base)
+// kernel takes for its index in the tensor that the segments' index_first / index_stride refer to
 template <typename T> struct ReluDrop {
     static constexpr bool MASKED = false, INDEXED = true;
-    const char *dst_base;
     const int64_t *state;
     int64_t stream_id;
     float p;
     __device__ __forceinline__ DropKey key() const { return drop_key(state[0], state[1], stream_id, p); }
-    // dst: where the 16 bytes go (an even element index: the vector is 16-byte aligned in an aligned tensor)
-    __device__ __forceinline__ u32x4 operator()(u32x4 v, const char *dst, const DropKey &k) const {
+    // at: byte offset of the 16 bytes in that tensor (a multiple of 16: an even element index)
+    __device__ __forceinline__ u32x4 operator()(u32x4 v, uint64_t at, const DropKey &k) const {
         union { u32x4 u; Vec16<T> e; } x;
         x.u = v;
-        const uint64_t first = (uint64_t)(dst - dst_base) / sizeof(T);
+        const uint64_t first = at / sizeof(T);
 #pragma unroll
         for (int i = 0; i < Vec16<T>::N; i += 2) {
             const uint32_t bits = drop_pair_bits(k, (first + i) >> 1);
@@ -133,7 +135,7 @@ __global__ __launch_bounds__(COPY_THREADS) void segment_copy_kernel(SegmentList 
     if constexpr (Act::INDEXED) key = act.key();
     for (uint64_t base = (uint64_t)blockIdx.x * COPY_THREADS * COPY_UNROLL + threadIdx.x; base < total; base += step) {
         V v[COPY_UNROLL], y[Act::MASKED ? COPY_UNROLL : 1];
-        uint64_t doff[COPY_UNROLL];
+        uint64_t doff[COPY_UNROLL], ioff[Act::INDEXED ? COPY_UNROLL : 1];
         bool ok[COPY_UNROLL];
 #pragma unroll
         for (int u = 0; u < COPY_UNROLL; ++u) {
@@ -151,6 +153,7 @@ __global__ __launch_bounds__(COPY_THREADS) void segment_copy_kernel(SegmentList 
                 col = c - row * per_row;
             }
             doff[u] = row * (uint64_t)s.dst_stride + col * sizeof(V);
+            if constexpr (Act::INDEXED) ioff[u] = (uint64_t)s.index_first + row * (uint64_t)s.index_stride + col * sizeof(V);
             const char *from = s.src + row * (uint64_t)s.src_stride + col * sizeof(V);
             if (ok[u]) {
                 if constexpr (NT) v[u] = __builtin_nontemporal_load((const V *)from);
@@ -163,7 +166,7 @@ __global__ __launch_bounds__(COPY_THREADS) void segment_copy_kernel(SegmentList 
         for (int u = 0; u < COPY_UNROLL; ++u) {
             if (!ok[u]) continue;
             if constexpr (Act::MASKED) *(V *)(s.dst + doff[u]) = act(v[u], y[u]);
-            else if constexpr (Act::INDEXED) *(V *)(s.dst + doff[u]) = act(v[u], s.dst + doff[u], key);
+            else if constexpr (Act::INDEXED) *(V *)(s.dst + doff[u]) = act(v[u], ioff[u], key);
             else *(V *)(s.dst + doff[u]) = act(v[u]);
         }
     }
@@ -175,7 +178,6 @@ __global__ __launch_bounds__(COPY_THREADS) void segment_copy_kernel(SegmentList 
 // DropSpec describes it.
 constexpr int ACT_RELU_BWD = -1, ACT_RELU_DROP = -2;
 struct DropSpec {
-    const void *dst_base;
     const int64_t *state;
     int64_t stream_id;
     float p;
@@ -217,14 +219,15 @@ int launch_segments(const SegmentList &list, int act, int dtype, hipStream_t str
         else
             hipLaunchKernelGGL((segment_copy_kernel<u32x4, ReluBwdF32>), grid, block, 0, stream, list, ReluBwdF32{mask_delta});
     } else if (act == ACT_RELU_DROP) {
-        HAPMI_REQUIRE(vec == 16 && drop && ((uintptr_t)drop->dst_base % 16) == 0, HAPMI_EALIGN,
-                      "%s: relu + dropout needs 16-byte aligned pieces", name);
+        bool idx_ok = drop != nullptr;
+        for (int i = 0; i < list.n; ++i) idx_ok = idx_ok && ((list.seg[i].index_first | list.seg[i].index_stride) & 15) == 0;
+        HAPMI_REQUIRE(vec == 16 && idx_ok, HAPMI_EALIGN, "%s: relu + dropout needs 16-byte aligned pieces", name);
         if (dtype == HAPMI_BF16)
             hipLaunchKernelGGL((segment_copy_kernel<u32x4, ReluDrop<bf16_t>>), grid, block, 0, stream, list,
-                               ReluDrop<bf16_t>{(const char *)drop->dst_base, drop->state, drop->stream_id, drop->p});
+                               ReluDrop<bf16_t>{drop->state, drop->stream_id, drop->p});
         else
             hipLaunchKernelGGL((segment_copy_kernel<u32x4, ReluDrop<float>>), grid, block, 0, stream, list,
-                               ReluDrop<float>{(const char *)drop->dst_base, drop->state, drop->stream_id, drop->p});
+                               ReluDrop<float>{drop->state, drop->stream_id, drop->p});
     } else if (act != HAPMI_ACT_NONE) {
         HAPMI_REQUIRE(act == HAPMI_ACT_RELU, HAPMI_EINVAL, "%s: only relu can be fused into a concat", name);
         HAPMI_REQUIRE(vec == 16, HAPMI_EALIGN, "%s: fused activation needs 16-byte aligned pieces", name);
@@ -429,9 +432,10 @@ int concat_rows(const void *const *pieces, const int64_t *lengths, int n_ranks, 
             // a piece that was produced at its place in dst (outer = 1: the place is one contiguous range) stays
             const bool in_place = act == HAPMI_ACT_NONE && outer == 1 &&
                                   (const char *)pieces[i] == (const char *)dst + off * inner_bytes;
-            if (!in_place)
+            if (!in_place)      // index_*: the piece's place in dst, for a dropout that rides on the copy
                 list.seg[list.n++] = {(const char *)pieces[i], (char *)dst + off * inner_bytes, outer,
-                                      lengths[i] * inner_bytes, lengths[i] * inner_bytes, total * inner_bytes};
+                                      lengths[i] * inner_bytes, lengths[i] * inner_bytes, total * inner_bytes,
+                                      off * inner_bytes, total * inner_bytes};
         }
         off += lengths[i];
     }
@@ -451,8 +455,33 @@ extern "C" int hapmi_concat_rows_relu_dropout(const void *const *pieces, const i
     HAPMI_REQUIRE(p >= 0.f && p <= 1.f && rng_state_dev && ((uintptr_t)rng_state_dev % 8) == 0, HAPMI_EINVAL,
                   "concat_rows_relu_dropout: bad probability %g or RNG state", (double)p);
     HAPMI_REQUIRE(hapmi_dtype_ok(dtype), HAPMI_EINVAL, "concat_rows_relu_dropout: bad dtype %d", dtype);
-    const DropSpec drop = {dst, rng_state_dev, stream_id, p};
+    const DropSpec drop = {rng_state_dev, stream_id, p};
     return concat_rows(pieces, lengths, n_ranks, dst, outer, inner_bytes, ACT_RELU_DROP, dtype, &drop, stream);
+}
+
+extern "C" int hapmi_relu_dropout_pieces(const void *const *src, void *const *dst, const int64_t *widths, int n_pieces,
+                                         int64_t rows, float p, const int64_t *rng_state_dev, int64_t stream_id,
+                                         int dtype, hapmi_stream_t stream) {
+    int64_t total;
+    int rc = check_lengths(widths, n_pieces, &total, "relu_dropout_pieces");
+    if (rc) return rc;
+    HAPMI_REQUIRE(rows >= 0 && src && dst && hapmi_dtype_ok(dtype), HAPMI_EINVAL, "relu_dropout_pieces: bad argument");
+    HAPMI_REQUIRE(p >= 0.f && p <= 1.f && rng_state_dev && ((uintptr_t)rng_state_dev % 8) == 0, HAPMI_EINVAL,
+                  "relu_dropout_pieces: bad probability %g or RNG state", (double)p);
+    const int64_t es = hapmi_elem_size(dtype);
+    SegmentList list;
+    list.n = 0;
+    int64_t off = 0;
+    for (int i = 0; i < n_pieces; ++i) {
+        if (widths[i] > 0 && rows > 0) {
+            HAPMI_REQUIRE(src[i] && dst[i], HAPMI_EINVAL, "relu_dropout_pieces: null pointer");
+            list.seg[list.n++] = {(const char *)src[i], (char *)dst[i], rows, widths[i] * es, widths[i] * es, widths[i] * es,
+                                  off * es, total * es};
+        }
+        off += widths[i];
+    }
+    const DropSpec drop = {rng_state_dev, stream_id, p};
+    return launch_segments(list, ACT_RELU_DROP, dtype, (hipStream_t)stream, "relu_dropout_pieces", 0, 1.f, &drop);
 }
 
 // ---------------------------------------------------------------------------

@@ -722,6 +722,8 @@ class ShardExecutor:
             return x
         if not 0.0 < p <= 1.0:
             self._unsupported(node, f"dropout probability {p}")
+        if x.kind == "pieces":
+            return self._dropout_on_pieces(node, x, p)
         if x.t is None or x.ld is not None:
             self._unsupported(node, f"dropout of a {x.kind} value")
         self._uses_rng = True
@@ -754,6 +756,23 @@ class ShardExecutor:
                 self.bwd.append(lambda: (ops.dropout(out.grad, tmp, p, self.rng_state, sid), ops.add(g, tmp, g)))
         self._tape.append(emit)
         return out
+
+    def _dropout_on_pieces(self, node, x: Val, p: float):
+        """relu -> dropout on the pieces of an all_to_all that a linear reads where they lie: one pass writes
+        dropout(relu(piece)) for every piece (decisions by the element's place in the concatenation, which never
+        exists); the linear then reads those, and its data gradient is masked with them and scaled by 1 / (1 - p),
+        which is the backward of both."""
+        if not (x.meta["relu"] and 0.0 < p < 1.0 and "mask_scale" not in x.meta):
+            self._unsupported(node, "on the pieces of an exchange only relu -> one dropout is handled")
+        self._uses_rng = True
+        sid = self._node_ids[node]
+        src = x.meta["pieces2d"]
+        dst = [self._new(t.shape) for t in src]
+        self.fwd.append(lambda: ops.relu_dropout_pieces(src, dst, p, self.rng_state, sid))
+        lead = tuple(x.shape[:-1])
+        return Val("pieces", None, shape=x.shape, needs_grad=x.needs_grad, relu=False, mask_scale=1.0 / (1.0 - p),
+                   pieces=[t.view(lead + (t.shape[-1],)) for t in dst], pieces2d=dst, dropout=(p, sid),
+                   backward_exchange=x.meta["backward_exchange"])
 
     def _feeds_residual_layer_norm(self, node, x: Val) -> bool:
         """node's only reader is an operator.add of it and an already materialised tensor of the same shape, whose
@@ -847,6 +866,8 @@ class ShardExecutor:
         out = Val("tensor", store, needs_grad=True)
         bias = b.meta["master"] if b is not None else None
         relu = bool(x.meta["relu"])
+        # pieces that already hold dropout(relu(.)): they are their own mask, and the masked gradient takes the factor
+        mask_scale = x.meta.get("mask_scale")
         self.fwd.append(lambda: ops.gemm(None, w.t, store, M, N, K, transB=True, bias=bias, a_segments=pieces, a_relu=relu))
 
         def emit():
@@ -858,8 +879,9 @@ class ShardExecutor:
             self._emit_wgrad(dy, list(pieces), gw, gb, N, K, M, N, K, accw, (w, b), x_relu=relu)
             if x.needs_grad:
                 back, finish = x.meta["backward_exchange"]()
-                mask = pieces if relu else None
-                self.bwd.append(lambda: ops.gemm(dy, w.t, None, M, K, N, c_segments=back, mask_segments=mask))
+                mask = pieces if (relu or mask_scale) else None
+                self.bwd.append(lambda: ops.gemm(dy, w.t, None, M, K, N, c_segments=back, mask_segments=mask,
+                                                 alpha=mask_scale or 1.0))
                 finish()
         self._tape.append(emit)
         return out
@@ -1597,17 +1619,23 @@ class ShardExecutor:
         return out
 
     def _feeds_only_relu_linear(self, node) -> bool:
-        """node -> F.relu -> [F.dropout(p = 0)]* -> F.linear (as its input), every link the only user."""
+        """node -> F.relu -> [F.dropout]* -> F.linear (as its input), every link the only user; of the dropouts at
+        most one has p > 0 (it gets a pass of its own over the pieces)."""
         users = list(node.users)
         if len(users) != 1 or users[0].target is not F.relu:
             return False
         n = users[0]
+        live = 0
         while True:
             users = list(n.users)
             if len(users) != 1:
                 return False
             u = users[0]
-            if u.target is F.dropout and float(u.args[1]) == 0.0 and u.args[0] is n:
+            if u.target is F.dropout and u.args[0] is n and len(u.args) == 2 and not u.kwargs:
+                p = float(u.args[1])
+                live += p > 0.0
+                if p >= 1.0 or live > 1 or (p > 0.0 and not self.fuse_dropout):
+                    return False
                 n = u
                 continue
             return u.target is F.linear and u.args[0] is n and u.args[1] is not n and u.args[2] is not n

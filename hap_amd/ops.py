@@ -239,6 +239,23 @@ def concat_rows(pieces: Sequence[torch.Tensor], dim: int, out: Optional[torch.Te
     return out
 
 
+def relu_dropout_pieces(src: Sequence[torch.Tensor], dst: Sequence[torch.Tensor], p: float, rng_state, stream_id: int):
+    """dst[i] = the columns of dropout(relu(cat(src, dim 1))) that piece i holds ([rows, width_i] each, contiguous),
+    with the decisions ``dropout`` takes for the concatenated [rows, sum(width)] tensor."""
+    _dev(*src, *dst, rng_state)
+    _check_rng(rng_state, "relu_dropout_pieces")
+    rows = src[0].shape[0]
+    widths = []
+    for a, b in zip(src, dst):
+        if a.dim() != 2 or a.shape != b.shape or a.dtype != src[0].dtype or b.dtype != a.dtype or a.shape[0] != rows:
+            raise ValueError("relu_dropout_pieces: pieces are [rows, width_i] tensors of one dtype, dst like src")
+        _need(a, a.numel(), "relu_dropout_pieces src")
+        _need(b, b.numel(), "relu_dropout_pieces dst")
+        widths.append(a.shape[1])
+    check(lib().hapmi_relu_dropout_pieces(_ptrs(src), _ptrs(dst), _i64(widths), len(widths), rows, ctypes.c_float(p),
+                                          _ptr(rng_state), int(stream_id), dtype_code(src[0]), _stream()))
+
+
 def ragged_reduce(contribs: Sequence[torch.Tensor], dim: int, offset: int, length: int,
                   out: Optional[torch.Tensor] = None, addend: Optional[torch.Tensor] = None) -> torch.Tensor:
     """out = sum_w contribs[w].narrow(dim, offset, length) in rank order, float32 accumulation; ``addend`` (out's

@@ -113,6 +113,13 @@ int hapmi_concat_rows(const void *const *pieces_host, const int64_t *lengths_hos
 int hapmi_concat_rows_relu_dropout(const void *const *pieces_host, const int64_t *lengths_host, int n_ranks, void *dst,
                                    int64_t outer, int64_t inner_bytes, float p, const int64_t *rng_state_dev,
                                    int64_t stream_id, int dtype, hapmi_stream_t stream);
+/* The same without concatenating, for a linear that reads the pieces of an all_to_all where they lie (A_segments of
+ * hapmi_gemm): dst[i][rows, widths[i]] = the columns of dropout(relu(cat(src, dim 1))) that piece i holds, every
+ * piece contiguous; the keep decisions are those hapmi_dropout takes for the [rows, sum(widths)] tensor as a whole.
+ * dst[i] may be src[i].  Pieces 16-byte aligned, widths * element size multiples of 16. */
+int hapmi_relu_dropout_pieces(const void *const *src_host, void *const *dst_host, const int64_t *widths_host,
+                              int n_pieces, int64_t rows, float p, const int64_t *rng_state_dev, int64_t stream_id,
+                              int dtype, hapmi_stream_t stream);
 
 /* the local sum of dist.reduce_scatter / dist.all_reduce (collectives.py:27, :95, :77):
  * dst[outer, len, inner] = sum_w contribs[w][outer, src_len, inner][:, offset:offset+len, :]

@@ -190,6 +190,70 @@ def _masks_from_oracle(ex, step):
     return out
 
 
+def test_relu_and_dropout_written_piece_by_piece(cuda):
+    """dropout(relu(.)) of the pieces of an all_to_all without concatenating them: every piece equals its columns of
+    the concatenated result that the separate kernels give (bit for bit), also in place."""
+    p, sid, rows = 0.3, 4, 45
+    g = torch.Generator().manual_seed(8)
+    widths = [128, 384, 64, 8]
+    src = [torch.randn(rows, w, generator=g).bfloat16().to(cuda) for w in widths]
+    st = _state(cuda, 2, 9)
+    want = torch.relu(torch.cat(src, 1))
+    ops.dropout(want, want, p, st, sid)
+    dst = [torch.full_like(t, float("nan")) for t in src]
+    ops.relu_dropout_pieces(src, dst, p, st, sid)
+    for d, w in zip(dst, torch.split(want, widths, 1)):
+        assert torch.equal(d, w)
+    ops.relu_dropout_pieces(src, src, p, st, sid)
+    for d, w in zip(src, torch.split(want, widths, 1)):
+        assert torch.equal(d, w)
+
+
+def test_program_with_dropout_on_exchange_pieces(cuda):
+    """all_to_all -> relu -> dropout -> linear with piece boundaries on multiples of 128: the linear reads dropped
+    pieces and its backward writes the pieces of the backward exchange.  The same program with the concatenating
+    copies takes the same decisions, so losses and gradients agree to bf16 rounding; and against the CPU oracle
+    given the masks."""
+    model = make_lm(vocab=211, S=32, d=64, H=1, F=1024, layers=2, causal=False)
+    model.dropout_p = 0.1
+    x, y = lm_batch(8, 32, 211, mlm=True)
+
+    def program():
+        return hap_amd.build_program(copy.deepcopy(model), hap_amd.ShardingPlan([RATIOS4], 0), 8)
+
+    def build(in_pieces):
+        return hap_amd.compile_program(program(), [x, y], dtype="bf16", wire=hap_amd.SyntheticWire(seed=3),
+                                       rank=0, world_size=4, exchange_in_pieces=in_pieces, dropout_seed=5)
+
+    a, b = build(True), build(False)
+    kinds = [v.kind for v in a.env.values() if hasattr(v, "kind")]
+    assert kinds.count("pieces") >= 4 and "pieces" not in [v.kind for v in b.env.values() if hasattr(v, "kind")]
+    for step in (1, 2):
+        la = a.forward(x, y).item()
+        a.backward()
+        lb = b.forward(x, y).item()
+        b.backward()
+        torch.cuda.synchronize()
+        ma, mb = a.dropout_masks(), b.dropout_masks()
+        assert set(ma) == set(mb) and all(torch.equal(ma[k], mb[k]) for k in ma)
+        assert abs(la - lb) <= 1e-3 * abs(lb)
+        for n, rec in a.params.items():
+            gb = b.params[n]["grad"]
+            if gb.norm().item() > 0:
+                assert rel_err(rec["grad"], gb) < 1e-2, n
+        decisions = _masks_from_oracle(a, step)
+        gm_ref = program()
+        run = SingleRankCPURun(gm_ref, 0, 4, hap_amd.SyntheticWire(seed=3), "fp32", wire_dtype=torch.bfloat16,
+                               decisions=decisions)
+        want = run.step(x, y)[0].item()
+        assert abs(la - want) <= 2e-2 * abs(want), (step, la, want)
+        ref_grads = {n: p_.grad for n, p_ in gm_ref.named_parameters() if p_.grad is not None}
+        scale = max(g.norm().item() for g in ref_grads.values())
+        for n, rec in a.params.items():
+            if ref_grads[n].norm().item() > 1e-4 * scale:
+                assert rel_err(rec["grad"], ref_grads[n]) < 2e-2, (step, n)
+
+
 @pytest.mark.parametrize("family,dtype", [("lm", "fp32"), ("lm", "bf16"), ("vit", "fp32"), ("vit", "bf16")])
 def test_program_with_dropout_against_the_oracle_given_the_masks(cuda, family, dtype):
     if family == "lm":
