@@ -153,7 +153,10 @@ def test_relu_and_dropout_in_the_gemm_epilogue(cuda, cfg, in_dtype, out_dtype):
             ops.dropout(want, want, p, st, sid)
             got = torch.full((M, N), float("nan"), dtype=tout, device=cuda)
             ops.gemm(A, B, got, M, N, K, transB=True, bias=bias, act="relu", drop=(p, st, sid))
-            assert torch.equal(got, want), (M, N, K)
+            if cfg >= 0:
+                assert torch.equal(got, want), (M, N, K)
+            else:       # left to itself the library may split the plain GEMM's reduction (another summation order)
+                assert torch.equal(got != 0, want != 0) and torch.allclose(got.float(), want.float(), rtol=1e-2 if tout == torch.bfloat16 else 1e-4, atol=1e-4)
             assert 0.3 < (got != 0).float().mean().item() < 0.45      # half pass relu, three quarters of those are kept
     finally:
         lib().hapmi_gemm_tuning(-1, 0)
