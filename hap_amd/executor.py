@@ -1101,7 +1101,8 @@ class ShardExecutor:
                 self._unsupported(node, "attn_mask must be a float32 [L, S] additive mask")
             mask_t = mask.t
         scale = 1.0 / math.sqrt(hd)
-        fused = self.fused_attention and self.dtype == "bf16" and hd == 64 and p_drop < 1.0
+        fused = (self.fused_attention and self.dtype == "bf16" and hd == 64
+                 and (p_drop == 0.0 or (self.fuse_dropout and p_drop < 1.0)))
         # a constant mask (a buffer of the module, not a gathered shard) that is exactly the causal one is
         # applied arithmetically by the fused kernels, which then also skip the key tiles above the diagonal
         causal = False

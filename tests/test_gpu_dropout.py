@@ -300,6 +300,45 @@ def test_program_with_dropout_against_the_oracle_given_the_masks(cuda, family, d
     assert any(not torch.equal(first[k], decisions[k]) for k in first if "dropout" in k)
 
 
+@pytest.mark.parametrize("family", ["lm", "vit"])
+def test_fused_and_separate_dropouts_take_the_same_decisions(cuda, family):
+    """The same bf16 program with every dropout inside a neighbouring kernel (the default) and with every dropout as
+    a pass of its own (fuse_dropout=False, attention through the materialised probabilities): the keep decisions
+    are identical, node by node, so losses and gradients agree to bf16 rounding."""
+    if family == "lm":
+        model = make_lm(vocab=211, S=32, d=64, H=1, F=1024, layers=2, causal=False)
+        x, y = lm_batch(8, 32, 211, mlm=True)
+        kw = {}
+    else:
+        model = make_vit(img=32, patch=8, d=64, H=1, F=128)
+        x, y = vit_batch(8, 32, 10)
+        kw = dict(ffn="batch")
+    model.dropout_p = 0.2
+
+    def build(fuse):
+        gm = hap_amd.build_program(copy.deepcopy(model), hap_amd.ShardingPlan([RATIOS4], 0, **kw), 8)
+        return hap_amd.compile_program(gm, [x, y], dtype="bf16", wire=hap_amd.SyntheticWire(seed=3), rank=0,
+                                       world_size=4, dropout_seed=11, fuse_dropout=fuse)
+
+    a, b = build(True), build(False)
+    assert len(a.fwd) < len(b.fwd)
+    for _ in range(2):
+        la = a.forward(x, y).item()
+        a.backward()
+        lb = b.forward(x, y).item()
+        b.backward()
+        torch.cuda.synchronize()
+        ma, mb = a.dropout_masks(), b.dropout_masks()
+        assert len(ma) >= 7 and set(ma) == set(mb)
+        for k in ma:
+            assert torch.equal(ma[k], mb[k]), k
+        assert abs(la - lb) <= 2e-3 * abs(lb)
+        for n, rec in a.params.items():
+            gb = b.params[n]["grad"]
+            if gb.norm().item() > 0:       # two bf16 computations with different rounding points: twice the bar each has against the oracle
+                assert rel_err(rec["grad"], gb) < 4e-2, n
+
+
 def test_dropout_is_active_and_unbiased_in_a_program(cuda):
     """Against the same program without dropout: the loss differs (dropout is on), and over many steps the mean of
     a dropped activation equals the undropped one (kept elements are scaled by 1 / (1 - p))."""
