@@ -982,7 +982,7 @@ class ShardExecutor:
             return x                                    # already applied by the producer
         if x.t is None or x.ld is not None:
             self._unsupported(node, f"activation on a {x.kind} value")
-        out = Val("tensor", self._new(x.t.shape), needs_grad=x.needs_grad)
+        out = Val(x.kind if x.kind == "expert" else "tensor", self._new(x.t.shape), shape=x.shape, needs_grad=x.needs_grad)
         self.fwd.append(lambda: ops.act_fwd(x.t, out.t, kind))
 
         def emit():
@@ -1713,6 +1713,8 @@ class ShardExecutor:
         if x.t is None or x.ld is not None:
             self._unsupported(node, f"all_reduce of a {x.kind} value")
         rank, W = self.rank_hint, self.world_hint
+        if x.kind == "expert":
+            return self._all_reduce_expert(node, x, rank, W)
         t = self._emit_sum(node.name, "fwd", x.t, rank, W, self.fwd)
         out = Val("tensor", t, needs_grad=x.needs_grad)
 
@@ -1720,6 +1722,39 @@ class ShardExecutor:
             if out.grad is None or not x.needs_grad:
                 return
             g = self._emit_sum(node.name, "bwd", out.grad, rank, W, self.bwd)
+            self._accumulate_into(x, g)
+        self._tape.append(emit)
+        return out
+
+    def _all_reduce_expert(self, node, x: Val, rank, W):
+        """all_reduce of expert-major activations (the partial sums of an expert product over a split model
+        dimension, hap.rs:3331-3335).  The program's tensor is [B, E, C, N] and that is what crosses the wire; the
+        storage here is [E, B, C, N], so the value is brought into the program's order before the sum and back
+        behind it (two strided copies per direction)."""
+        El, B, C, N = x.t.shape
+        each = [1] * El
+
+        def to_program_order(src, dst):          # [E, B, C, N] -> [B, E, C, N]
+            ops.concat_rows([src[e].view(B, 1, C * N) for e in range(El)], 1, dst.view(B, El, C * N))
+
+        def to_expert_major(src, dst):           # [B, E, C, N] -> [E, B, C, N]
+            ops.split_rows(src.view(B, El, C * N), each, 1, [dst[e].view(B, 1, C * N) for e in range(El)])
+
+        mine = self._new((B, El, C, N))
+        self.fwd.append(lambda: to_program_order(x.t, mine))
+        total = self._emit_sum(node.name, "fwd", mine, rank, W, self.fwd)
+        out = Val("expert", self._new(x.t.shape), shape=x.shape, needs_grad=x.needs_grad)
+        self.fwd.append(lambda: to_expert_major(total, out.t))
+
+        def emit():
+            if out.grad is None or not x.needs_grad:
+                return
+            g_mine = self._new((B, El, C, N))
+            dy = out.grad
+            self.bwd.append(lambda: to_program_order(dy, g_mine))
+            g_total = self._emit_sum(node.name, "bwd", g_mine, rank, W, self.bwd)
+            g = self._new(x.t.shape)
+            self.bwd.append(lambda: to_expert_major(g_total, g))
             self._accumulate_into(x, g)
         self._tape.append(emit)
         return out

@@ -31,7 +31,11 @@ Plans (each step is a legal Hoare triple of hap.rs:2786-3419):
                   the replicated rows, all_to_all, batch-sharded FFN2;
 ``ffn="batch"``   pure uneven data parallelism;
 MoE layers        gating on replicated tokens, experts sharded over the
-                  expert dimension, combine -> reduce_scatter / all_reduce.
+                  expert dimension, combine -> reduce_scatter / all_reduce
+                  (``moe="experts"``); ``moe="capacity"`` / ``"hidden"`` /
+                  ``"model"``: the capacity slots, the experts' hidden features
+                  or the tokens' model dimension are split instead (see
+                  ShardingPlan.moe).
 ``attn="heads"``  attention sharded over heads instead of samples (uneven head
                   counts: rows of the in-projection, columns of the
                   out-projection), all_gather before, reduce_scatter after;
@@ -235,14 +239,30 @@ def _moe_ffn(e: _Emitter, h1, prefix: str, emsize: int, n_expert: int, capacity:
         nhid = e._shape(prefix + "w1")[2]
         w1 = e.sharded(prefix + "w1", nhid, 2)
         w2 = e.sharded(prefix + "w2", nhid, 1)
+    elif e.plan.moe == "model":
+        # split of the model dimension: the tokens' columns (gather(0, 2), identity) -> gather(0, 3) for the dispatch,
+        # (gather(0, 1), gather(1, 3)) -> reduce for the first product, (gather(0, 2), identity) -> gather(0, 3) for
+        # the second, (gather(0, 3), identity) -> gather(0, 2) for the combine (hap.rs:3306-3310, 3331-3335,
+        # 3368-3372, 3405-3409); the gating sees whole token rows
+        L_D = e.plan.lengths(emsize)
+        w1 = e.sharded(prefix + "w1", emsize, 1)
+        w2 = e.sharded(prefix + "w2", emsize, 2)
     else:
         raise ValueError(f"unknown MoE split {e.plan.moe!r}")
-    x = e.call(torch.einsum, "bsd,bsec->becd", tokens, dispatch)
+    model_split = e.plan.moe == "model"
+    x = e.call(collectives.dynamic_slice, tokens, 2, L_D, e.rank) if model_split else tokens
+    x = e.call(torch.einsum, "bsd,bsec->becd", x, dispatch)
     x = e.call(torch.einsum, "edh,becd->bech", w1, x)
+    if model_split:
+        x = e.call(collectives.all_reduce, x)            # every device holds a partial sum over its columns of d
     x = e.g.call_function(F.relu, (x,), {"inplace": False})
     x = e.call(torch.einsum, "ehd,bech->becd", w2, x)
     partial = e.call(torch.einsum, "becd,bsec->bsd", x, combine)
-    if batch_sharded:
+    if model_split:
+        o = e.call(collectives.all_gather, partial, 2, L_D, e.rank)
+        if batch_sharded:
+            o = e.call(collectives.dynamic_slice, o, 0, L_B, e.rank)
+    elif batch_sharded:
         o = e.call(collectives.reduce_scatter, partial, 0, L_B, e.rank)
     else:
         o = e.call(collectives.all_reduce, partial)

@@ -83,7 +83,9 @@ class ShardingPlan:
                                  # tensors sliced on dim 2, expert weights on dim 0; "capacity": dispatch / combine
                                  # sliced on dim 3 (every device takes a range of every expert's slots), expert weights
                                  # whole; "hidden": routing whole, first expert weight sliced on dim 2 and the second on
-                                 # dim 1 (a feature split of the expert FFN; the second product is a partial sum)
+                                 # dim 1 (a feature split of the expert FFN; the second product is a partial sum);
+                                 # "model": the tokens' model dimension (dispatch input sliced on dim 2, first weight
+                                 # on dim 1 with its product all-reduced, second on dim 2, combine output gathered)
 
     @property
     def world_size(self) -> int:

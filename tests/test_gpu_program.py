@@ -169,16 +169,53 @@ def test_switch_moe(cuda, dtype, batch_sharded):
 
 @pytest.mark.parametrize("moe,dtype,batch_sharded", [("capacity", "fp32", True), ("capacity", "fp32", False),
                                                       ("capacity", "bf16", False), ("hidden", "fp32", True),
-                                                      ("hidden", "bf16", False)])
+                                                      ("hidden", "bf16", False), ("model", "fp32", True),
+                                                      ("model", "fp32", False)])
 def test_moe_capacity_and_hidden_splits(cuda, moe, dtype, batch_sharded):
     """The capacity split (dispatch / combine tensors sliced on dim 3, whole expert weights: every device works on
-    a range of every expert's slots) and the hidden-feature split of the expert FFN (hap.rs:3285-3419), uneven over
-    the devices, against the CPU run of all ranks."""
+    a range of every expert's slots), the hidden-feature split of the expert FFN and the split of the tokens' model
+    dimension (the first expert product is then a partial sum, all-reduced in the program's [B, E, C, H] order)
+    (hap.rs:3285-3419), uneven over the devices, against the CPU run of all ranks."""
     # hidden widths 40 / 40 / 24 / 24 of 128 (multiples of the 16-byte vector in either type), capacity slots 3 / 3 / 2 / 2
-    model = make_moe(C=10, F=128) if dtype == "fp32" else make_moe(d=64, F=128, C=10, std=0.3)
+    if moe == "model":      # model widths 20 / 20 / 12 / 12 of 64
+        model = make_moe(d=64, C=10)
+    else:
+        model = make_moe(C=10, F=128) if dtype == "fp32" else make_moe(d=64, F=128, C=10, std=0.3)
     B = 16 if batch_sharded else 4
     x, y = lm_batch(B, 16, 61)
     _compare(model, RATIOS_E, B, x, y, dtype, [0, 2], ADAM, ffn="batch", batch_sharded=batch_sharded, moe=moe)
+
+
+def test_moe_model_dimension_split_bf16_with_shared_decisions(cuda):
+    """The split of the tokens' model dimension in bf16 (widths 40 / 40 / 24 / 24 of 128).  Here routed tensors cross
+    the wire (the first expert product is all-reduced), and two bf16 computations of the gate differ on a few
+    near-ties, which moves whole rows between slots; so, as in the full-size tests, the GPU's discrete decisions
+    (chosen experts, relu masks; routing itself is checked bit for bit on the GPU's float32 logits) are handed to
+    the CPU oracle, which then has to give the same loss and gradients."""
+    from oracle.cpu_executor import SingleRankCPURun
+    from test_gpu_full_size import _check_grads, _gpu_decisions
+    # weights of std 0.05: with larger ones the attention scores of this width saturate the softmax, and its backward
+    # (p * (dp - sum(dp * p)) on probabilities stored in bf16: head size 32 takes the materialised path) loses its
+    # signal to cancellation, whatever the split
+    model = make_moe(d=128, F=64, C=10, std=0.05)
+    x, y = lm_batch(16, 16, 61)
+
+    def program():
+        return hap_amd.build_program(copy.deepcopy(model), hap_amd.ShardingPlan([RATIOS_E], 0, ffn="batch", moe="model"), 16)
+
+    wire = lambda: hap_amd.SyntheticWire(seed=3, grad_scale=1e-2)      # peers' gradients of the size of real ones
+    ex = hap_amd.compile_program(program(), [x, y], dtype="bf16", wire=wire(), rank=0, world_size=4)
+    loss = ex.forward(x, y).item()
+    ex.backward()
+    torch.cuda.synchronize()
+    decisions = _gpu_decisions(ex)
+    assert sum(1 for v in decisions.values() if v.dtype == torch.long) == 1          # one MoE layer's routing
+    gm_ref = program()
+    run = SingleRankCPURun(gm_ref, 0, 4, wire(), "fp32", wire_dtype=torch.bfloat16, decisions=decisions)
+    want = run.step(x, y)[0].item()
+    assert abs(loss - want) <= 2e-2 * abs(want), (loss, want)
+    _check_grads({n: rec["grad"].cpu() for n, rec in ex.params.items()},
+                 {n: p.grad for n, p in gm_ref.named_parameters() if p.grad is not None}, 2e-2)
 
 
 def test_moe_bf16_routing_matches(cuda):

@@ -214,11 +214,12 @@ def test_feature_sharded_embedding_table_spmd_equals_single_device(ffn):
     _check(model, run, x, y, sharded)
 
 
-@pytest.mark.parametrize("moe", ["capacity", "hidden"])
+@pytest.mark.parametrize("moe", ["capacity", "hidden", "model"])
 def test_moe_capacity_and_hidden_splits_spmd_equal_single_device(moe):
     """The other legal splits of the four MoE einsums (hap.rs:3285-3419): every device takes a range of every
     expert's capacity slots with whole expert weights, or every device holds a slice of the experts' hidden
-    features; batch-sharded attention around them as in the expert split."""
+    features, or of the tokens' model dimension (columns 10 / 10 / 6 / 6 of 32); batch-sharded attention around
+    them as in the expert split."""
     model = make_moe(C=10, F=48)                                # capacity slots 3 / 3 / 2 / 2, hidden widths 15 / 15 / 9 / 9
     B = 16
     x, y = lm_batch(B, 16, 61)
@@ -227,4 +228,7 @@ def test_moe_capacity_and_hidden_splits_spmd_equal_single_device(moe):
     if moe == "hidden":
         L_F = hap_amd.sharding_lengths(48, RATIOS_E)
         sharded = {"layers.1.w1": (2, L_F), "layers.1.w2": (1, L_F)}
+    if moe == "model":
+        L_D = hap_amd.sharding_lengths(32, RATIOS_E)
+        sharded = {"layers.1.w1": (1, L_D), "layers.1.w2": (2, L_D)}
     _check(model, run, x, y, sharded)
