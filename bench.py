@@ -189,6 +189,11 @@ def main():
         other = measure("bert", args, max(5, args.steps // 2), 3, share_shapes=not args.shared_peer_buffers)
         key = "bert_peer_buffers_per_layer" if args.shared_peer_buffers else "bert_peer_buffers_shared_by_shape"
         extra[key] = _brief(other)
+        if args.dropout == 0.0:
+            # the headline workload with the reference's default dropout probability (config.py:33): F.dropout in front
+            # of the residual LayerNorms and behind the FFN's relu, dropout_p on the attention probabilities
+            extra["bert_dropout_0.1"] = _brief(measure("bert", args, max(5, args.steps // 2), 3,
+                                                       share_shapes=args.shared_peer_buffers, dropout=0.1))
         for name in ("lm", "vit", "moe"):
             extra[name] = _brief(measure(name, args, max(5, args.steps // 2), 3, share_shapes=args.shared_peer_buffers))
         from hap_amd import ragged_bench
@@ -274,8 +279,9 @@ def _write_gemm_table(path, report, desc, vendor):
                 f"{total_flop / total_us / 1e6:.0f} TFLOP/s (cold single launches)\n")
 
 
-def measure(workload, args, steps, warmup, share_shapes=True):
-    """One workload: compile, autotune the GEMM plans (untimed), warm up, time `steps` steps, bracket the GEMMs."""
+def measure(workload, args, steps, warmup, share_shapes=True, dropout=None):
+    """One workload: compile, autotune the GEMM plans (untimed), warm up, time `steps` steps, bracket the GEMMs.
+    ``dropout``: the model's dropout probability (default: the command line's)."""
     import ctypes
     import gc
 
@@ -287,7 +293,7 @@ def measure(workload, args, steps, warmup, share_shapes=True):
     desc, dtype = WORKLOADS[workload]
     bert = workload == "bert"
     gm, x, y, meta = build_workload(workload, attn=args.attn if bert else "batch", zero=args.zero and bert,
-                                    dropout=args.dropout)
+                                    dropout=args.dropout if dropout is None else dropout)
     wire = hap_amd.SyntheticWire(seed=39, scale=1.0, grad_scale=1e-3, share_shapes=share_shapes)
     ex = hap_amd.compile_program(gm, [x, y], dtype=dtype, wire=wire, rank=0, world_size=len(meta["ratios"]),
                                  overlap_wgrad=args.overlap, relu_mask_in_dgrad=not args.no_relu_mask_in_dgrad,
@@ -377,7 +383,7 @@ def measure(workload, args, steps, warmup, share_shapes=True):
                    "exchange_read_and_written_in_pieces": ex.exchange_in_pieces,
                    "peer_buffers": "one set per message shape" if share_shapes else "one set per layer",
                    "attention_sharding": args.attn if bert else "batch",
-                   "zero_sharded_parameters": bool(args.zero and bert), "dropout": args.dropout,
+                   "zero_sharded_parameters": bool(args.zero and bert), "dropout": args.dropout if dropout is None else dropout,
                    "final_loss": loss},
         "roofline": {"bound": "mfma", "kernel": "gemm_kernel (all GEMM launches of the step)",
                      "achieved": achieved, "peak": peak, "unit": "TFLOP/s", "frac": achieved / peak,
