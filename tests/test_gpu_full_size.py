@@ -22,6 +22,8 @@ from a wrong result.  So each test
 Routing itself is integer work and bit-exact: the oracle's gating applied to the float32 logits the GPU computed
 gives the GPU's dispatch mask and combine weights.
 """
+import math
+
 import pytest
 import torch
 import torch.nn.functional as F
@@ -190,6 +192,48 @@ def test_lm_config1_full_size_fp32(cuda):
 
 def test_bert_large_shard_full_width_bf16(cuda):
     _full_check("bert", 2, "bf16")
+
+
+def test_bert_large_shard_full_width_bf16_with_dropout(cuda):
+    """Two layers of BASELINE config 2 with the reference's default dropout probability (config.py:33) at the real
+    shapes: F.dropout in front of both residual LayerNorms and behind the FFN's relu (on the exchange's pieces),
+    dropout_p on the probabilities of the fused attention (b 12, 16 heads, S 512).  The masks cannot be those of a
+    torch run (PARITY UNPINNED for the particular masks); the GPU's are checked against the CPU restatement of the
+    generator bit for bit and handed, with the relu masks, to the oracle, which must then give the GPU's loss and
+    gradients within the bf16 tolerance."""
+    p, seed = 0.1, 77
+    gm, x, y, meta = bench.build_workload("bert", layers_override=2, dropout=p)
+    W = len(meta["ratios"])
+    ex = hap_amd.compile_program(gm, [x, y], dtype="bf16", wire=hap_amd.SyntheticWire(seed=SEED), rank=0, world_size=W,
+                                 dropout_seed=seed)
+    kinds = [v.kind for v in ex.env.values() if hasattr(v, "kind")]
+    assert "pieces" in kinds and "dropped" in kinds                    # the dropouts run inside their neighbours
+    loss = ex.forward(x, y).item()
+    ex.backward()
+    torch.cuda.synchronize()
+    grads = {n: rec["grad"].clone() for n, rec in ex.params.items()}
+    decisions = _gpu_decisions(ex)
+    masks = {k: v.cpu() for k, v in ex.dropout_masks().items()}
+    assert len(masks) >= 8                                             # per layer: 3 F.dropout + the attention's
+    for i, node in enumerate(ex.gm.graph.nodes):                        # stream id = the node's index in the program
+        if node.name in masks:
+            m = masks[node.name]
+            if node.target is F.dropout:
+                want = ref_ops.dropout_keep(seed, 1, i, p, m.numel()).view(m.shape)
+            else:
+                _, _, shape, S = ex.env[node].meta["dropout"]
+                want = ref_ops.dropout_keep(seed, 1, i, p, math.prod(shape)).view(shape)[..., :S]
+            assert torch.equal(m, want), node.name
+            assert abs(m.float().mean().item() - (1 - p)) < 2e-3, node.name
+    decisions.update(masks)
+    gm_ref, _, _, _ = bench.build_workload("bert", layers_override=2, dropout=p)
+    run = SingleRankCPURun(gm_ref, 0, W, hap_amd.SyntheticWire(seed=SEED), "fp32", wire_dtype=torch.bfloat16,
+                           decisions=decisions)
+    torch.set_num_threads(16)
+    want = run.step(x, y)[0].item()
+    print(f"\n  bert with dropout {p}, 2 layers, bf16: loss {loss:.6f}, oracle with the GPU's masks {want:.6f}")
+    assert abs(loss - want) <= 2e-2 * abs(want), (loss, want)
+    _check_grads(grads, {n: q.grad for n, q in gm_ref.named_parameters() if q.grad is not None}, 2e-2)
 
 
 def test_bert_large_shard_full_depth_bf16_adam_step(cuda):
