@@ -132,11 +132,17 @@ template <typename T> struct RowVec {
     static constexpr int EPV = Vec16<T>::N;
 };
 
-// expert_in[e_loc, b, c, :] = x[b, token_of_slot[b, e_lo + e_loc, c], :] or 0
+// The device's share of the dense [B, S, E, C] routing tensors is a window in each of the three dimensions that the
+// einsums may be split along: experts [e_lo, e_lo + E_loc), capacity slots [c_lo, c_lo + C_loc) and positions
+// [s_lo, s_lo + S_loc).  Expert-major activations hold [E_loc, B, C_loc, d], token tensors [B, S_loc, d]; the routing
+// records always cover all S positions.
+//
+// expert_in[e_loc, b, c, :] = x[b, token_of_slot[b, e_lo + e_loc, c_lo + c] - s_lo, :], or 0 for an empty slot or a
+// token outside the window of positions
 template <typename T>
 __global__ __launch_bounds__(256) void moe_dispatch_kernel(const T *x, const int32_t *token_of_slot, T *expert_in, int B,
                                                          int S, int E, int C, int d, int e_lo, int E_loc, int c_lo,
-                                                         int C_loc) {
+                                                         int C_loc, int s_lo, int S_loc) {
     constexpr int EPV = Vec16<T>::N;
     const int lane = threadIdx.x & 63;
     const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -146,8 +152,8 @@ __global__ __launch_bounds__(256) void moe_dispatch_kernel(const T *x, const int
     const int el = (int)(row / ((int64_t)C_loc * B));
     const int tok = token_of_slot[((int64_t)b * E + e_lo + el) * C + c_lo + c];
     Vec16<T> *dst = (Vec16<T> *)(expert_in + row * d);
-    if (tok >= 0 && tok < S) {
-        const Vec16<T> *src = (const Vec16<T> *)(x + ((int64_t)b * S + tok) * d);
+    if (tok >= s_lo && tok < s_lo + S_loc) {
+        const Vec16<T> *src = (const Vec16<T> *)(x + ((int64_t)b * S_loc + tok - s_lo) * d);
         for (int i = lane; i < d / EPV; i += 64) dst[i] = src[i];
     } else {
         Vec16<T> z;
@@ -157,16 +163,17 @@ __global__ __launch_bounds__(256) void moe_dispatch_kernel(const T *x, const int
     }
 }
 
-// out[b, s, :] (+)= sum_k w_k * src[e_k - e_lo, b, slot_k, :] over kept local choices; w_k = gate_k or 1
+// out[b, s - s_lo, :] (+)= sum_k w_k * src[e_k - e_lo, b, slot_k - c_lo, :] over kept local choices; w_k = gate_k or 1
 template <typename T, bool WEIGHTED>
 __global__ __launch_bounds__(256) void moe_combine_kernel(const T *src, const int32_t *index, const int32_t *slot,
                                                         const float *gate, T *out, int B, int S, int C, int d, int e_lo,
-                                                        int E_loc, int c_lo, int C_loc, int accumulate) {
+                                                        int E_loc, int c_lo, int C_loc, int s_lo, int S_loc, int accumulate) {
     constexpr int EPV = Vec16<T>::N;
     const int lane = threadIdx.x & 63;
-    const int64_t tok = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (tok >= (int64_t)B * S) return;
-    const int b = (int)(tok / S);
+    const int64_t local = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);      // row of out: (b, s - s_lo)
+    if (local >= (int64_t)B * S_loc) return;
+    const int b = (int)(local / S_loc);
+    const int64_t tok = (int64_t)b * S + s_lo + (local - (int64_t)b * S_loc); // the token's row in the routing records
     const Vec16<T> *rows[2] = {nullptr, nullptr};
     float w[2] = {0.f, 0.f};
 #pragma unroll
@@ -177,7 +184,7 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const T *src, const in
             w[k] = WEIGHTED ? gate[tok * 2 + k] : 1.0f;
         }
     }
-    Vec16<T> *dst = (Vec16<T> *)(out + tok * d);
+    Vec16<T> *dst = (Vec16<T> *)(out + local * d);
     for (int i = lane; i < d / EPV; i += 64) {
         float acc[EPV];
 #pragma unroll
@@ -207,7 +214,7 @@ template <typename T>
 __global__ __launch_bounds__(256) void moe_combine_bwd_rows_kernel(const T *dout, const int32_t *index, const float *gate,
                                                                  const int32_t *token_of_slot, T *d_expert_out, int B,
                                                                  int S, int E, int C, int d, int e_lo, int E_loc,
-                                                                 int c_lo, int C_loc) {
+                                                                 int c_lo, int C_loc, int s_lo, int S_loc) {
     constexpr int EPV = Vec16<T>::N;
     const int lane = threadIdx.x & 63;
     const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -219,10 +226,10 @@ __global__ __launch_bounds__(256) void moe_combine_bwd_rows_kernel(const T *dout
     Vec16<T> *dst = (Vec16<T> *)(d_expert_out + row * d);
     float w = 0.f;
     const Vec16<T> *src = nullptr;
-    if (tok >= 0 && tok < S) {
+    if (tok >= s_lo && tok < s_lo + S_loc) {
         const int64_t t = (int64_t)b * S + tok;
         w = (index[t * 2] == e_lo + el) ? gate[t * 2] : gate[t * 2 + 1];
-        src = (const Vec16<T> *)(dout + t * d);
+        src = (const Vec16<T> *)(dout + ((int64_t)b * S_loc + tok - s_lo) * d);
     }
     for (int i = lane; i < d / EPV; i += 64) {
         Vec16<T> r;
@@ -238,22 +245,26 @@ __global__ __launch_bounds__(256) void moe_combine_bwd_rows_kernel(const T *dout
     }
 }
 
-// dgate[b, s, k] = <dout[b, s, :], expert_out[e_k - e_lo, b, slot_k, :]>
+// dgate[b, s, k] = <dout[b, s - s_lo, :], expert_out[e_k - e_lo, b, slot_k - c_lo, :]>, 0 for a token or a choice outside
+// the windows (dgate covers all S positions)
 template <typename T>
 __global__ __launch_bounds__(256) void moe_combine_bwd_gate_kernel(const T *dout, const T *expert_out, const int32_t *index,
                                                                  const int32_t *slot, float *dgate, int B, int S, int C,
-                                                                 int d, int e_lo, int E_loc, int c_lo, int C_loc) {
+                                                                 int d, int e_lo, int E_loc, int c_lo, int C_loc, int s_lo,
+                                                                 int S_loc) {
     constexpr int EPV = Vec16<T>::N;
     const int lane = threadIdx.x & 63;
     const int64_t tok = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (tok >= (int64_t)B * S) return;
     const int b = (int)(tok / S);
-    const Vec16<T> *g = (const Vec16<T> *)(dout + tok * d);
+    const int sp = (int)(tok - (int64_t)b * S) - s_lo;                         // position inside the window
+    const bool mine = sp >= 0 && sp < S_loc;
+    const Vec16<T> *g = (const Vec16<T> *)(dout + ((int64_t)b * S_loc + (mine ? sp : 0)) * d);
 #pragma unroll
     for (int k = 0; k < 2; ++k) {
         const int e = index[tok * 2 + k] - e_lo, sl = slot[tok * 2 + k];
         float acc = 0.f;
-        if (sl > 0 && sl < C && sl >= c_lo && sl < c_lo + C_loc && e >= 0 && e < E_loc) {
+        if (mine && sl > 0 && sl < C && sl >= c_lo && sl < c_lo + C_loc && e >= 0 && e < E_loc) {
             const Vec16<T> *r = (const Vec16<T> *)(expert_out + (((int64_t)e * B + b) * C_loc + sl - c_lo) * d);
             for (int i = lane; i < d / EPV; i += 64) {
                 const Vec16<T> a = g[i], v = r[i];
@@ -267,12 +278,14 @@ __global__ __launch_bounds__(256) void moe_combine_bwd_gate_kernel(const T *dout
 }
 
 int check_moe(const char *name, int64_t B, int64_t S, int64_t E, int64_t C, int64_t d, int64_t e_lo, int64_t E_loc,
-              int64_t c_lo, int64_t C_loc, int dtype) {
+              int64_t c_lo, int64_t C_loc, int64_t s_lo, int64_t S_loc, int dtype) {
     HAPMI_REQUIRE(hapmi_dtype_ok(dtype), HAPMI_EINVAL, "%s: bad dtype", name);
     HAPMI_REQUIRE(B >= 0 && S >= 1 && E >= 2 && C >= 1 && d >= 1 && e_lo >= 0 && E_loc >= 0 && e_lo + E_loc <= E,
                   HAPMI_EINVAL, "%s: bad shape", name);
     HAPMI_REQUIRE(c_lo >= 0 && C_loc >= 0 && c_lo + C_loc <= C, HAPMI_EINVAL, "%s: capacity range [%lld, %lld) outside [0, %lld)",
                   name, (long long)c_lo, (long long)(c_lo + C_loc), (long long)C);
+    HAPMI_REQUIRE(s_lo >= 0 && S_loc >= 0 && s_lo + S_loc <= S, HAPMI_EINVAL, "%s: range of positions [%lld, %lld) outside [0, %lld)",
+                  name, (long long)s_lo, (long long)(s_lo + S_loc), (long long)S);
     const int64_t epv = dtype == HAPMI_F32 ? 4 : 8;
     HAPMI_REQUIRE(d % epv == 0, HAPMI_EALIGN, "%s: d must be a multiple of %lld", name, (long long)epv);
     HAPMI_REQUIRE(B * S < (1ll << 31) && E_loc * B * C_loc < (1ll << 31), HAPMI_ELIMIT, "%s: too many rows", name);
@@ -337,50 +350,52 @@ extern "C" int hapmi_top2_densify(const int32_t *index, const int32_t *slot, con
 
 extern "C" int hapmi_moe_dispatch(const void *x, const int32_t *token_of_slot, void *expert_in, int64_t B, int64_t S,
                                   int64_t E, int64_t C, int64_t d, int64_t e_lo, int64_t E_loc, int64_t c_lo,
-                                  int64_t C_loc, int dtype, hapmi_stream_t stream) {
-    int rc = check_moe("moe_dispatch", B, S, E, C, d, e_lo, E_loc, c_lo, C_loc, dtype);
+                                  int64_t C_loc, int64_t s_lo, int64_t S_loc, int dtype, hapmi_stream_t stream) {
+    int rc = check_moe("moe_dispatch", B, S, E, C, d, e_lo, E_loc, c_lo, C_loc, s_lo, S_loc, dtype);
     if (rc) return rc;
     const int64_t rows = E_loc * B * C_loc;
     if (rows == 0) return HAPMI_OK;
-    HAPMI_REQUIRE(x && token_of_slot && expert_in, HAPMI_EINVAL, "moe_dispatch: null pointer");
+    HAPMI_REQUIRE((x || S_loc == 0) && token_of_slot && expert_in, HAPMI_EINVAL, "moe_dispatch: null pointer");
     dim3 grid((unsigned)hapmi_cdiv(rows, 4));
     if (dtype == HAPMI_F32)
-        hipLaunchKernelGGL((moe_dispatch_kernel<float>), grid, dim3(256), 0, (hipStream_t)stream, (const float *)x, token_of_slot, (float *)expert_in, (int)B, (int)S, (int)E, (int)C, (int)d, (int)e_lo, (int)E_loc, (int)c_lo, (int)C_loc);
+        hipLaunchKernelGGL((moe_dispatch_kernel<float>), grid, dim3(256), 0, (hipStream_t)stream, (const float *)x, token_of_slot, (float *)expert_in, (int)B, (int)S, (int)E, (int)C, (int)d, (int)e_lo, (int)E_loc, (int)c_lo, (int)C_loc, (int)s_lo, (int)S_loc);
     else
-        hipLaunchKernelGGL((moe_dispatch_kernel<bf16_t>), grid, dim3(256), 0, (hipStream_t)stream, (const bf16_t *)x, token_of_slot, (bf16_t *)expert_in, (int)B, (int)S, (int)E, (int)C, (int)d, (int)e_lo, (int)E_loc, (int)c_lo, (int)C_loc);
+        hipLaunchKernelGGL((moe_dispatch_kernel<bf16_t>), grid, dim3(256), 0, (hipStream_t)stream, (const bf16_t *)x, token_of_slot, (bf16_t *)expert_in, (int)B, (int)S, (int)E, (int)C, (int)d, (int)e_lo, (int)E_loc, (int)c_lo, (int)C_loc, (int)s_lo, (int)S_loc);
     HAPMI_CHECK_LAUNCH("moe_dispatch");
     return HAPMI_OK;
 }
 
 extern "C" int hapmi_moe_combine(const void *expert_out, const int32_t *index, const int32_t *slot, const float *gate,
                                  void *out, int64_t B, int64_t S, int64_t C, int64_t d, int64_t e_lo, int64_t E_loc,
-                                 int64_t c_lo, int64_t C_loc, int dtype, hapmi_stream_t stream) {
-    int rc = check_moe("moe_combine", B, S, e_lo + E_loc > 2 ? e_lo + E_loc : 2, C, d, e_lo, E_loc, c_lo, C_loc, dtype);
+                                 int64_t c_lo, int64_t C_loc, int64_t s_lo, int64_t S_loc, int dtype, hapmi_stream_t stream) {
+    int rc = check_moe("moe_combine", B, S, e_lo + E_loc > 2 ? e_lo + E_loc : 2, C, d, e_lo, E_loc, c_lo, C_loc, s_lo, S_loc, dtype);
     if (rc) return rc;
     if (B == 0) return HAPMI_OK;
+    if (S_loc == 0) return HAPMI_OK;
     HAPMI_REQUIRE(expert_out && index && slot && gate && out, HAPMI_EINVAL, "moe_combine: null pointer");
-    dim3 grid((unsigned)hapmi_cdiv(B * S, 4));
+    dim3 grid((unsigned)hapmi_cdiv(B * S_loc, 4));
     if (dtype == HAPMI_F32)
-        hipLaunchKernelGGL((moe_combine_kernel<float, true>), grid, dim3(256), 0, (hipStream_t)stream, (const float *)expert_out, index, slot, gate, (float *)out, (int)B, (int)S, (int)C, (int)d, (int)e_lo, (int)E_loc, (int)c_lo, (int)C_loc, 0);
+        hipLaunchKernelGGL((moe_combine_kernel<float, true>), grid, dim3(256), 0, (hipStream_t)stream, (const float *)expert_out, index, slot, gate, (float *)out, (int)B, (int)S, (int)C, (int)d, (int)e_lo, (int)E_loc, (int)c_lo, (int)C_loc, (int)s_lo, (int)S_loc, 0);
     else
-        hipLaunchKernelGGL((moe_combine_kernel<bf16_t, true>), grid, dim3(256), 0, (hipStream_t)stream, (const bf16_t *)expert_out, index, slot, gate, (bf16_t *)out, (int)B, (int)S, (int)C, (int)d, (int)e_lo, (int)E_loc, (int)c_lo, (int)C_loc, 0);
+        hipLaunchKernelGGL((moe_combine_kernel<bf16_t, true>), grid, dim3(256), 0, (hipStream_t)stream, (const bf16_t *)expert_out, index, slot, gate, (bf16_t *)out, (int)B, (int)S, (int)C, (int)d, (int)e_lo, (int)E_loc, (int)c_lo, (int)C_loc, (int)s_lo, (int)S_loc, 0);
     HAPMI_CHECK_LAUNCH("moe_combine");
     return HAPMI_OK;
 }
 
 extern "C" int hapmi_moe_dispatch_bwd(const void *d_expert_in, const int32_t *index, const int32_t *slot,
                                       const float *gate, void *dx, int64_t B, int64_t S, int64_t C, int64_t d,
-                                      int64_t e_lo, int64_t E_loc, int64_t c_lo, int64_t C_loc, int accumulate, int dtype,
-                                      hapmi_stream_t stream) {
-    int rc = check_moe("moe_dispatch_bwd", B, S, e_lo + E_loc > 2 ? e_lo + E_loc : 2, C, d, e_lo, E_loc, c_lo, C_loc, dtype);
+                                      int64_t e_lo, int64_t E_loc, int64_t c_lo, int64_t C_loc, int64_t s_lo, int64_t S_loc,
+                                      int accumulate, int dtype, hapmi_stream_t stream) {
+    int rc = check_moe("moe_dispatch_bwd", B, S, e_lo + E_loc > 2 ? e_lo + E_loc : 2, C, d, e_lo, E_loc, c_lo, C_loc, s_lo, S_loc, dtype);
     if (rc) return rc;
     if (B == 0) return HAPMI_OK;
+    if (S_loc == 0) return HAPMI_OK;
     HAPMI_REQUIRE(d_expert_in && index && slot && gate && dx, HAPMI_EINVAL, "moe_dispatch_bwd: null pointer");
-    dim3 grid((unsigned)hapmi_cdiv(B * S, 4));
+    dim3 grid((unsigned)hapmi_cdiv(B * S_loc, 4));
     if (dtype == HAPMI_F32)
-        hipLaunchKernelGGL((moe_combine_kernel<float, false>), grid, dim3(256), 0, (hipStream_t)stream, (const float *)d_expert_in, index, slot, gate, (float *)dx, (int)B, (int)S, (int)C, (int)d, (int)e_lo, (int)E_loc, (int)c_lo, (int)C_loc, accumulate);
+        hipLaunchKernelGGL((moe_combine_kernel<float, false>), grid, dim3(256), 0, (hipStream_t)stream, (const float *)d_expert_in, index, slot, gate, (float *)dx, (int)B, (int)S, (int)C, (int)d, (int)e_lo, (int)E_loc, (int)c_lo, (int)C_loc, (int)s_lo, (int)S_loc, accumulate);
     else
-        hipLaunchKernelGGL((moe_combine_kernel<bf16_t, false>), grid, dim3(256), 0, (hipStream_t)stream, (const bf16_t *)d_expert_in, index, slot, gate, (bf16_t *)dx, (int)B, (int)S, (int)C, (int)d, (int)e_lo, (int)E_loc, (int)c_lo, (int)C_loc, accumulate);
+        hipLaunchKernelGGL((moe_combine_kernel<bf16_t, false>), grid, dim3(256), 0, (hipStream_t)stream, (const bf16_t *)d_expert_in, index, slot, gate, (bf16_t *)dx, (int)B, (int)S, (int)C, (int)d, (int)e_lo, (int)E_loc, (int)c_lo, (int)C_loc, (int)s_lo, (int)S_loc, accumulate);
     HAPMI_CHECK_LAUNCH("moe_dispatch_bwd");
     return HAPMI_OK;
 }
@@ -388,22 +403,22 @@ extern "C" int hapmi_moe_dispatch_bwd(const void *d_expert_in, const int32_t *in
 extern "C" int hapmi_moe_combine_bwd(const void *dout, const void *expert_out, const int32_t *index,
                                      const int32_t *slot, const float *gate, const int32_t *token_of_slot,
                                      void *d_expert_out, float *dgate, int64_t B, int64_t S, int64_t E, int64_t C,
-                                     int64_t d, int64_t e_lo, int64_t E_loc, int64_t c_lo, int64_t C_loc, int dtype,
-                                     hapmi_stream_t stream) {
-    int rc = check_moe("moe_combine_bwd", B, S, E, C, d, e_lo, E_loc, c_lo, C_loc, dtype);
+                                     int64_t d, int64_t e_lo, int64_t E_loc, int64_t c_lo, int64_t C_loc, int64_t s_lo,
+                                     int64_t S_loc, int dtype, hapmi_stream_t stream) {
+    int rc = check_moe("moe_combine_bwd", B, S, E, C, d, e_lo, E_loc, c_lo, C_loc, s_lo, S_loc, dtype);
     if (rc) return rc;
     if (B == 0) return HAPMI_OK;
-    HAPMI_REQUIRE(dout && expert_out && index && slot && gate && token_of_slot && d_expert_out && dgate, HAPMI_EINVAL,
+    HAPMI_REQUIRE((dout || S_loc == 0) && expert_out && index && slot && gate && token_of_slot && d_expert_out && dgate, HAPMI_EINVAL,
                   "moe_combine_bwd: null pointer");
     hipStream_t st = (hipStream_t)stream;
     const int64_t rows = E_loc * B * C_loc;
     dim3 grid_rows((unsigned)hapmi_cdiv(rows > 0 ? rows : 1, 4)), grid_tok((unsigned)hapmi_cdiv(B * S, 4));
     if (dtype == HAPMI_F32) {
-        if (rows) hipLaunchKernelGGL((moe_combine_bwd_rows_kernel<float>), grid_rows, dim3(256), 0, st, (const float *)dout, index, gate, token_of_slot, (float *)d_expert_out, (int)B, (int)S, (int)E, (int)C, (int)d, (int)e_lo, (int)E_loc, (int)c_lo, (int)C_loc);
-        hipLaunchKernelGGL((moe_combine_bwd_gate_kernel<float>), grid_tok, dim3(256), 0, st, (const float *)dout, (const float *)expert_out, index, slot, dgate, (int)B, (int)S, (int)C, (int)d, (int)e_lo, (int)E_loc, (int)c_lo, (int)C_loc);
+        if (rows) hipLaunchKernelGGL((moe_combine_bwd_rows_kernel<float>), grid_rows, dim3(256), 0, st, (const float *)dout, index, gate, token_of_slot, (float *)d_expert_out, (int)B, (int)S, (int)E, (int)C, (int)d, (int)e_lo, (int)E_loc, (int)c_lo, (int)C_loc, (int)s_lo, (int)S_loc);
+        hipLaunchKernelGGL((moe_combine_bwd_gate_kernel<float>), grid_tok, dim3(256), 0, st, (const float *)dout, (const float *)expert_out, index, slot, dgate, (int)B, (int)S, (int)C, (int)d, (int)e_lo, (int)E_loc, (int)c_lo, (int)C_loc, (int)s_lo, (int)S_loc);
     } else {
-        if (rows) hipLaunchKernelGGL((moe_combine_bwd_rows_kernel<bf16_t>), grid_rows, dim3(256), 0, st, (const bf16_t *)dout, index, gate, token_of_slot, (bf16_t *)d_expert_out, (int)B, (int)S, (int)E, (int)C, (int)d, (int)e_lo, (int)E_loc, (int)c_lo, (int)C_loc);
-        hipLaunchKernelGGL((moe_combine_bwd_gate_kernel<bf16_t>), grid_tok, dim3(256), 0, st, (const bf16_t *)dout, (const bf16_t *)expert_out, index, slot, dgate, (int)B, (int)S, (int)C, (int)d, (int)e_lo, (int)E_loc, (int)c_lo, (int)C_loc);
+        if (rows) hipLaunchKernelGGL((moe_combine_bwd_rows_kernel<bf16_t>), grid_rows, dim3(256), 0, st, (const bf16_t *)dout, index, gate, token_of_slot, (bf16_t *)d_expert_out, (int)B, (int)S, (int)E, (int)C, (int)d, (int)e_lo, (int)E_loc, (int)c_lo, (int)C_loc, (int)s_lo, (int)S_loc);
+        hipLaunchKernelGGL((moe_combine_bwd_gate_kernel<bf16_t>), grid_tok, dim3(256), 0, st, (const bf16_t *)dout, (const bf16_t *)expert_out, index, slot, dgate, (int)B, (int)S, (int)C, (int)d, (int)e_lo, (int)E_loc, (int)c_lo, (int)C_loc, (int)s_lo, (int)S_loc);
     }
     HAPMI_CHECK_LAUNCH("moe_combine_bwd");
     return HAPMI_OK;

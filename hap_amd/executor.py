@@ -554,7 +554,7 @@ class ShardExecutor:
             return Val("dead", why="head-averaged attention probabilities are never consumed by the program")
         if src.kind == "gating":
             return Val("routing", which="dispatch" if idx == 0 else "combine", gating=src, e_lo=0, E_loc=src.meta["E"],
-                       c_lo=0, C_loc=src.meta["C"])
+                       c_lo=0, C_loc=src.meta["C"], s_lo=0, S_loc=src.meta["x"].t.shape[1])
         self._unsupported(node, f"getitem on a {src.kind} value")
 
     # ------------------------------------------------------------------ ops
@@ -1761,11 +1761,11 @@ class ShardExecutor:
 
     def _dynamic_slice(self, node):
         v, dim, L, rank = self._val(node.args[0]), node.args[1], list(node.args[2]), node.args[3]
-        if v.kind == "routing" and dim in (2, 3):
-            # the device's window of the dense [B, S, E, C] tensor: experts (dim 2) and / or capacity slots (dim 3)
+        if v.kind == "routing" and dim in (1, 2, 3):
+            # the device's window of the dense [B, S, E, C] tensor: positions (dim 1), experts (dim 2), capacity slots (dim 3)
             m = dict(which=v.meta["which"], gating=v.meta["gating"], e_lo=v.meta["e_lo"], E_loc=v.meta["E_loc"],
-                     c_lo=v.meta["c_lo"], C_loc=v.meta["C_loc"])
-            lo, n = ("e_lo", "E_loc") if dim == 2 else ("c_lo", "C_loc")
+                     c_lo=v.meta["c_lo"], C_loc=v.meta["C_loc"], s_lo=v.meta["s_lo"], S_loc=v.meta["S_loc"])
+            lo, n = {1: ("s_lo", "S_loc"), 2: ("e_lo", "E_loc"), 3: ("c_lo", "C_loc")}[dim]
             if sum(L) != m[n]:
                 self._unsupported(node, f"the lengths {L} do not add up to the extent {m[n]} of dimension {dim}")
             m[lo], m[n] = m[lo] + sum(L[:rank]), L[rank]
@@ -1839,15 +1839,18 @@ class ShardExecutor:
         gv = route.meta["gating"]
         r, E, C = gv.meta["r"], gv.meta["E"], gv.meta["C"]
         e_lo, E_loc, c_lo, C_loc = route.meta["e_lo"], route.meta["E_loc"], route.meta["c_lo"], route.meta["C_loc"]
+        s_lo, S_loc = route.meta["s_lo"], route.meta["S_loc"]
         B, S, d = x.t.shape
+        if S != S_loc:
+            self._unsupported(node, f"tokens of {S} positions against a dispatch tensor of {S_loc}")
         out = Val("expert", self._new((E_loc, B, C_loc, d)), shape=(B, E_loc, C_loc, d), needs_grad=True)
-        self.fwd.append(lambda: ops.moe_dispatch(x.t, r, out.t, E, C, e_lo, E_loc, c_lo, C_loc))
+        self.fwd.append(lambda: ops.moe_dispatch(x.t, r, out.t, E, C, e_lo, E_loc, c_lo, C_loc, s_lo))
 
         def emit():
             if out.grad is None or not x.needs_grad:
                 return
             gx, acc = self._grad_slot(x)
-            self.bwd.append(lambda: ops.moe_dispatch_bwd(out.grad, r, gx, C, e_lo, E_loc, acc, c_lo, C_loc))
+            self.bwd.append(lambda: ops.moe_dispatch_bwd(out.grad, r, gx, C, e_lo, E_loc, acc, c_lo, C_loc, s_lo))
         self._tape.append(emit)
         return out
 
@@ -1903,9 +1906,9 @@ class ShardExecutor:
         if (El, Cl) != (E_loc, C_loc):
             self._unsupported(node, f"expert outputs [{El} experts, {Cl} slots] do not match the combine tensor's "
                                     f"window [{E_loc}, {C_loc}]")
-        S = r["index"].shape[1]
-        out = Val("tensor", self._new((B, S, d)), needs_grad=True)
-        self.fwd.append(lambda: ops.moe_combine(eo.t, r, out.t, C, e_lo, E_loc, c_lo, C_loc))
+        s_lo, S_loc = route.meta["s_lo"], route.meta["S_loc"]       # the output covers the combine tensor's positions
+        out = Val("tensor", self._new((B, S_loc, d)), needs_grad=True)
+        self.fwd.append(lambda: ops.moe_combine(eo.t, r, out.t, C, e_lo, E_loc, c_lo, C_loc, s_lo))
 
         def emit():
             if out.grad is None:
@@ -1915,7 +1918,7 @@ class ShardExecutor:
             eo.grad = self._new(eo.t.shape)
             gv.meta["dgate_used"] = True
             g, dgate = eo.grad, gv.meta["dgate"]
-            self.bwd.append(lambda: ops.moe_combine_bwd(out.grad, eo.t, r, g, dgate, E, C, e_lo, E_loc, c_lo, C_loc))
+            self.bwd.append(lambda: ops.moe_combine_bwd(out.grad, eo.t, r, g, dgate, E, C, e_lo, E_loc, c_lo, C_loc, s_lo))
         self._tape.append(emit)
         return out
 

@@ -1244,10 +1244,25 @@ def _capacity_window(C, c_lo, C_loc):
     return c_lo, C_loc
 
 
-def moe_dispatch(x, r, expert_in, E, C, e_lo, E_loc, c_lo=None, C_loc=None):
-    """einsum "bsd,bsec->becd" on the experts [e_lo, e_lo + E_loc) and capacity slots [c_lo, c_lo + C_loc) of the
-    routing ``r``: expert_in[E_loc, B, C_loc, d]."""
-    B, S, d = x.shape
+def _position_window(r, tokens, s_lo):
+    """(B, S, S_loc, s_lo, d): the routing ``r`` covers S positions, the token tensor [B, S_loc, d] holds those from
+    s_lo on (None: it must hold all of them)."""
+    B, S_loc, d = tokens.shape
+    S = r["index"].shape[1]
+    if s_lo is None:
+        if S_loc != S:
+            raise _lib.HapmiError(f"a token tensor of {S_loc} positions next to a routing of {S} needs s_lo")
+        s_lo = 0
+    s_lo = int(s_lo)
+    if r["index"].shape[0] != B or s_lo < 0 or s_lo + S_loc > S:
+        raise _lib.HapmiError(f"positions [{s_lo}, {s_lo + S_loc}) outside [0, {S}), or batch {B} against {r['index'].shape[0]}")
+    return B, S, S_loc, s_lo, d
+
+
+def moe_dispatch(x, r, expert_in, E, C, e_lo, E_loc, c_lo=None, C_loc=None, s_lo=None):
+    """einsum "bsd,bsec->becd" on the experts [e_lo, e_lo + E_loc), capacity slots [c_lo, c_lo + C_loc) and positions
+    [s_lo, s_lo + x.shape[1]) of the routing ``r``: expert_in[E_loc, B, C_loc, d]."""
+    B, S, S_loc, s_lo, d = _position_window(r, x, s_lo)
     _dev(x, expert_in)
     _check_routing(r, B, S, E, C)
     c_lo, C_loc = _capacity_window(C, c_lo, C_loc)
@@ -1255,11 +1270,11 @@ def moe_dispatch(x, r, expert_in, E, C, e_lo, E_loc, c_lo=None, C_loc=None):
     if expert_in.dtype != x.dtype or not x.is_contiguous():
         raise TypeError("moe_dispatch: dtype / layout mismatch")
     check(lib().hapmi_moe_dispatch(_ptr(x), _ptr(r["token_of_slot"]), _ptr(expert_in), B, S, E, C, d, e_lo, E_loc,
-                                   c_lo, C_loc, dtype_code(x), _stream()))
+                                   c_lo, C_loc, s_lo, S_loc, dtype_code(x), _stream()))
 
 
-def moe_combine(expert_out, r, out, C, e_lo, E_loc, c_lo=None, C_loc=None):
-    B, S, d = out.shape
+def moe_combine(expert_out, r, out, C, e_lo, E_loc, c_lo=None, C_loc=None, s_lo=None):
+    B, S, S_loc, s_lo, d = _position_window(r, out, s_lo)
     _dev(expert_out, out)
     _check_routing(r, B, S)
     c_lo, C_loc = _capacity_window(C, c_lo, C_loc)
@@ -1267,11 +1282,13 @@ def moe_combine(expert_out, r, out, C, e_lo, E_loc, c_lo=None, C_loc=None):
     if expert_out.dtype != out.dtype or not out.is_contiguous():
         raise TypeError("moe_combine: dtype / layout mismatch")
     check(lib().hapmi_moe_combine(_ptr(expert_out), _ptr(r["index"]), _ptr(r["slot"]), _ptr(r["gate"]), _ptr(out),
-                                  B, S, C, d, e_lo, E_loc, c_lo, C_loc, dtype_code(out), _stream()))
+                                  B, S, C, d, e_lo, E_loc, c_lo, C_loc, s_lo, S_loc, dtype_code(out), _stream()))
 
 
-def moe_combine_bwd(dout, expert_out, r, d_expert_out, dgate, E, C, e_lo, E_loc, c_lo=None, C_loc=None):
-    B, S, d = dout.shape
+def moe_combine_bwd(dout, expert_out, r, d_expert_out, dgate, E, C, e_lo, E_loc, c_lo=None, C_loc=None, s_lo=None):
+    B, S, S_loc, s_lo, d = _position_window(r, dout, s_lo)
+    if not dout.is_contiguous():
+        raise TypeError("moe_combine_bwd: dout must be contiguous")
     _dev(dout, expert_out, d_expert_out, dgate)
     _check_routing(r, B, S, E, C)
     c_lo, C_loc = _capacity_window(C, c_lo, C_loc)
@@ -1282,11 +1299,11 @@ def moe_combine_bwd(dout, expert_out, r, d_expert_out, dgate, E, C, e_lo, E_loc,
         raise TypeError("moe_combine_bwd: dtype mismatch")
     check(lib().hapmi_moe_combine_bwd(_ptr(dout), _ptr(expert_out), _ptr(r["index"]), _ptr(r["slot"]), _ptr(r["gate"]),
                                       _ptr(r["token_of_slot"]), _ptr(d_expert_out), _ptr(dgate), B, S, E, C, d, e_lo,
-                                      E_loc, c_lo, C_loc, dtype_code(dout), _stream()))
+                                      E_loc, c_lo, C_loc, s_lo, S_loc, dtype_code(dout), _stream()))
 
 
-def moe_dispatch_bwd(d_expert_in, r, dx, C, e_lo, E_loc, accumulate, c_lo=None, C_loc=None):
-    B, S, d = dx.shape
+def moe_dispatch_bwd(d_expert_in, r, dx, C, e_lo, E_loc, accumulate, c_lo=None, C_loc=None, s_lo=None):
+    B, S, S_loc, s_lo, d = _position_window(r, dx, s_lo)
     _dev(d_expert_in, dx)
     _check_routing(r, B, S)
     c_lo, C_loc = _capacity_window(C, c_lo, C_loc)
@@ -1294,7 +1311,8 @@ def moe_dispatch_bwd(d_expert_in, r, dx, C, e_lo, E_loc, accumulate, c_lo=None, 
     if d_expert_in.dtype != dx.dtype or not dx.is_contiguous():
         raise TypeError("moe_dispatch_bwd: dtype / layout mismatch")
     check(lib().hapmi_moe_dispatch_bwd(_ptr(d_expert_in), _ptr(r["index"]), _ptr(r["slot"]), _ptr(r["gate"]), _ptr(dx),
-                                       B, S, C, d, e_lo, E_loc, c_lo, C_loc, int(accumulate), dtype_code(dx), _stream()))
+                                       B, S, C, d, e_lo, E_loc, c_lo, C_loc, s_lo, S_loc, int(accumulate), dtype_code(dx),
+                                       _stream()))
 
 
 # ---------------------------------------------------------------------------

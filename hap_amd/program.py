@@ -33,9 +33,9 @@ Plans (each step is a legal Hoare triple of hap.rs:2786-3419):
 MoE layers        gating on replicated tokens, experts sharded over the
                   expert dimension, combine -> reduce_scatter / all_reduce
                   (``moe="experts"``); ``moe="capacity"`` / ``"hidden"`` /
-                  ``"model"``: the capacity slots, the experts' hidden features
-                  or the tokens' model dimension are split instead (see
-                  ShardingPlan.moe).
+                  ``"model"`` / ``"sequence"``: the capacity slots, the experts'
+                  hidden features, the tokens' model dimension or their
+                  positions are split instead (see ShardingPlan.moe).
 ``attn="heads"``  attention sharded over heads instead of samples (uneven head
                   counts: rows of the in-projection, columns of the
                   out-projection), all_gather before, reduce_scatter after;
@@ -208,7 +208,7 @@ def _dense_ffn(e: _Emitter, h1, prefix: str, emsize: int, nhid: int, B: int, p: 
 
 
 def _moe_ffn(e: _Emitter, h1, prefix: str, emsize: int, n_expert: int, capacity: int, B: int,
-             batch_sharded: bool, gating=models.top_2_gating):
+             batch_sharded: bool, gating=models.top_2_gating, seqlen: Optional[int] = None):
     L_E = e.plan.lengths(n_expert)
     if batch_sharded:
         L_B = e.plan.lengths(B)
@@ -247,19 +247,36 @@ def _moe_ffn(e: _Emitter, h1, prefix: str, emsize: int, n_expert: int, capacity:
         L_D = e.plan.lengths(emsize)
         w1 = e.sharded(prefix + "w1", emsize, 1)
         w2 = e.sharded(prefix + "w2", emsize, 2)
+    elif e.plan.moe == "sequence":
+        # split along the sequence: tokens and dispatch tensor windowed over positions, (gather(0, 1), gather(1, 1)) ->
+        # reduce (hap.rs:3300-3304); the expert products on the reduced, whole tensor (identity); the combine tensor
+        # windowed over positions gives the output gathered on dim 1.  (The reference's fifth triple of the combine,
+        # hap.rs:3411-3415, names dim 2 of the combine tensor next to an output gathered on dim 1; positions are the
+        # only dimension of that operand which gives such an output, and that is what is emitted here.)
+        L_S = e.plan.lengths(seqlen)
+        dispatch = e.call(collectives.dynamic_slice, dispatch, 1, L_S, e.rank)
+        combine = e.call(collectives.dynamic_slice, combine, 1, L_S, e.rank)
+        w1 = e.replicated(prefix + "w1")
+        w2 = e.replicated(prefix + "w2")
     else:
         raise ValueError(f"unknown MoE split {e.plan.moe!r}")
-    model_split = e.plan.moe == "model"
-    x = e.call(collectives.dynamic_slice, tokens, 2, L_D, e.rank) if model_split else tokens
+    model_split, seq_split = e.plan.moe == "model", e.plan.moe == "sequence"
+    x = tokens
+    if model_split:
+        x = e.call(collectives.dynamic_slice, tokens, 2, L_D, e.rank)
+    if seq_split:
+        x = e.call(collectives.dynamic_slice, tokens, 1, L_S, e.rank)
     x = e.call(torch.einsum, "bsd,bsec->becd", x, dispatch)
+    if seq_split:
+        x = e.call(collectives.all_reduce, x)            # every device placed the tokens of its positions
     x = e.call(torch.einsum, "edh,becd->bech", w1, x)
     if model_split:
         x = e.call(collectives.all_reduce, x)            # every device holds a partial sum over its columns of d
     x = e.g.call_function(F.relu, (x,), {"inplace": False})
     x = e.call(torch.einsum, "ehd,bech->becd", w2, x)
     partial = e.call(torch.einsum, "becd,bsec->bsd", x, combine)
-    if model_split:
-        o = e.call(collectives.all_gather, partial, 2, L_D, e.rank)
+    if model_split or seq_split:
+        o = e.call(collectives.all_gather, partial, 2 if model_split else 1, L_D if model_split else L_S, e.rank)
         if batch_sharded:
             o = e.call(collectives.dynamic_slice, o, 0, L_B, e.rank)
     elif batch_sharded:
@@ -340,7 +357,8 @@ def build_program(model: nn.Module, plan: ShardingPlan, global_batch: int,
             # synthesizer has no handler for models.switch_gating; its models call it at models.py:421)
             gating = (models.switch_gating if isinstance(layer, models.SwitchTransformerEncoderLayer)
                       else models.top_2_gating)
-            h = _moe_ffn(e, h1, prefix, d, layer.n_expert, layer.capacity, B, batch_sharded, gating)
+            h = _moe_ffn(e, h1, prefix, d, layer.n_expert, layer.capacity, B, batch_sharded, gating,
+                         seqlen=model.seqlen + (1 if model.family == "vit" else 0))
         else:
             h = _dense_ffn(e, h1, prefix, d, model.nhid, B, p, activation, batch_sharded)
 

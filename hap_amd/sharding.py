@@ -85,7 +85,10 @@ class ShardingPlan:
                                  # whole; "hidden": routing whole, first expert weight sliced on dim 2 and the second on
                                  # dim 1 (a feature split of the expert FFN; the second product is a partial sum);
                                  # "model": the tokens' model dimension (dispatch input sliced on dim 2, first weight
-                                 # on dim 1 with its product all-reduced, second on dim 2, combine output gathered)
+                                 # on dim 1 with its product all-reduced, second on dim 2, combine output gathered);
+                                 # "sequence": tokens, dispatch and combine tensors sliced over positions (dim 1): the
+                                 # dispatched tokens are all-reduced, every device runs the whole expert FFN, the
+                                 # combine output is gathered on dim 1
 
     @property
     def world_size(self) -> int:

@@ -408,29 +408,35 @@ int hapmi_top2_densify(const int32_t *index, const int32_t *slot, const float *g
                        float *combine, int64_t B, int64_t S, int64_t E, int64_t C, hapmi_stream_t stream);
 /* The four MoE einsums (hap.rs:2273, models.py:356-364) on index-form routing.  The device's share of the dense
  * [B, S, E, C] dispatch / combine tensors is a window of experts [e_lo, e_lo + E_loc) (the expert split of the
- * einsums, hap.rs:3316-3320, 3333-3337, 3399-3403) and of capacity slots [c_lo, c_lo + C_loc) (the capacity split,
- * hap.rs:3322-3326, 3357-3361, 3405-3409): dynamic_slice of the gating outputs along dim 2 / dim 3.  Expert-major
- * activations are [E_loc, B, C_loc, d]; the whole tensor is e_lo = c_lo = 0, E_loc = E, C_loc = C.
+ * einsums, hap.rs:3312-3316, 3325-3329, 3356-3360, 3393-3397), of capacity slots [c_lo, c_lo + C_loc) (the capacity
+ * split, hap.rs:3318-3322, 3349-3353, 3380-3384, 3399-3403) and of positions [s_lo, s_lo + S_loc) (the split along the
+ * sequence, hap.rs:3300-3304 for the dispatch): dynamic_slice of the gating outputs along dim 2 / dim 3 / dim 1.
+ * Expert-major activations are [E_loc, B, C_loc, d], token tensors (x, out, dout, dx) [B, S_loc, d]; the routing
+ * records and dgate always cover all S positions.  The whole tensor is e_lo = c_lo = s_lo = 0, E_loc = E, C_loc = C,
+ * S_loc = S.
  *
- * einsum "bsd,bsec->becd" as a row gather into expert_in[E_loc, B, C_loc, d] */
+ * einsum "bsd,bsec->becd" as a row gather into expert_in[E_loc, B, C_loc, d] (zero rows for empty slots and for
+ * tokens outside the window of positions: the result is then a partial sum over the devices) */
 int hapmi_moe_dispatch(const void *x, const int32_t *token_of_slot, void *expert_in, int64_t B, int64_t S,
                        int64_t E, int64_t C, int64_t d, int64_t e_lo, int64_t E_loc, int64_t c_lo, int64_t C_loc,
-                       int dtype, hapmi_stream_t stream);
+                       int64_t s_lo, int64_t S_loc, int dtype, hapmi_stream_t stream);
 /* einsum "becd,bsec->bsd" (models.py:364) as a weighted row gather:
- * out[b, s, :] = sum_k gate_k * expert_out[e_k - e_lo, b, slot_k - c_lo, :] over kept choices inside the window */
+ * out[b, s - s_lo, :] = sum_k gate_k * expert_out[e_k - e_lo, b, slot_k - c_lo, :] over kept choices inside the windows */
 int hapmi_moe_combine(const void *expert_out, const int32_t *index, const int32_t *slot, const float *gate,
                       void *out, int64_t B, int64_t S, int64_t C, int64_t d, int64_t e_lo, int64_t E_loc,
-                      int64_t c_lo, int64_t C_loc, int dtype, hapmi_stream_t stream);
-/* backward of combine: d_expert_out[e, b, c, :] = gate * dout[b, token, :] (0 for empty slots);
- * dgate[b, s, k] = <dout[b, s, :], expert_out[e_k - e_lo, b, slot_k - c_lo, :]> (0 if not kept / outside the window) */
+                      int64_t c_lo, int64_t C_loc, int64_t s_lo, int64_t S_loc, int dtype, hapmi_stream_t stream);
+/* backward of combine: d_expert_out[e, b, c, :] = gate * dout[b, token - s_lo, :] (0 for empty slots and tokens outside
+ * the window); dgate[b, s, k] = <dout[b, s - s_lo, :], expert_out[e_k - e_lo, b, slot_k - c_lo, :]> (0 if not kept /
+ * outside the windows) */
 int hapmi_moe_combine_bwd(const void *dout, const void *expert_out, const int32_t *index, const int32_t *slot,
                           const float *gate, const int32_t *token_of_slot, void *d_expert_out, float *dgate,
                           int64_t B, int64_t S, int64_t E, int64_t C, int64_t d, int64_t e_lo, int64_t E_loc,
-                          int64_t c_lo, int64_t C_loc, int dtype, hapmi_stream_t stream);
-/* backward of dispatch: dx[b, s, :] (+)= sum_k d_expert_in[e_k - e_lo, b, slot_k - c_lo, :] */
+                          int64_t c_lo, int64_t C_loc, int64_t s_lo, int64_t S_loc, int dtype, hapmi_stream_t stream);
+/* backward of dispatch: dx[b, s - s_lo, :] (+)= sum_k d_expert_in[e_k - e_lo, b, slot_k - c_lo, :] */
 int hapmi_moe_dispatch_bwd(const void *d_expert_in, const int32_t *index, const int32_t *slot, const float *gate,
                            void *dx, int64_t B, int64_t S, int64_t C, int64_t d, int64_t e_lo, int64_t E_loc,
-                           int64_t c_lo, int64_t C_loc, int accumulate, int dtype, hapmi_stream_t stream);
+                           int64_t c_lo, int64_t C_loc, int64_t s_lo, int64_t S_loc, int accumulate, int dtype,
+                           hapmi_stream_t stream);
 
 /* ---- optimizer (worker.py:47, 74-76; profiler.py:18) --------------------
  * Flat float32 master parameters and gradients; `shadow` (bf16 copy of the

@@ -51,55 +51,68 @@ def test_routing_is_bit_exact(cuda, B, S, E, C):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("window", [(2, 3, 0, 10), (2, 3, 4, 3), (0, 8, 0, 5), (0, 8, 7, 3)])
+@pytest.mark.parametrize("window", [(2, 3, 0, 10, 0, 48), (2, 3, 4, 3, 0, 48), (0, 8, 0, 5, 0, 48), (0, 8, 7, 3, 0, 48),
+                                    (0, 8, 0, 10, 0, 17), (0, 8, 0, 10, 17, 19), (0, 8, 0, 10, 36, 12), (2, 3, 4, 3, 17, 19),
+                                    (0, 8, 0, 10, 20, 0)])
 def test_dispatch_combine_match_dense_einsums(cuda, dtype, window):
-    """The device's share of the dense [B, S, E, C] dispatch / combine tensors is a window of experts and of capacity
-    slots (dynamic_slice on dim 2 / dim 3): whole capacity, a capacity range, and a range that holds slot 0 (always
-    empty) next to the whole expert range."""
+    """The device's share of the dense [B, S, E, C] dispatch / combine tensors is a window of experts, of capacity
+    slots and of positions (dynamic_slice on dim 2 / dim 3 / dim 1): whole capacity, a capacity range, a range that
+    holds slot 0 (always empty) next to the whole expert range; the first, a middle and the last range of positions
+    (token tensors then hold those positions only), all three windows at once, and an empty range of positions."""
     B, S, E, C, d = 2, 48, 8, 10, 32
-    e_lo, E_loc, c_lo, C_loc = window
+    e_lo, E_loc, c_lo, C_loc, s_lo, S_loc = window
     g = torch.Generator().manual_seed(9)
     lg = torch.randn(B, S, E, generator=g)
     x = torch.randn(B, S, d, generator=g).to(dtype)
     r = ops.top2_gate(lg.to(cuda), C)
     dispatch, combine = ref.top_2_gating(lg, E, C, torch.eye(E))
-    dsl = dispatch[:, :, e_lo:e_lo + E_loc, c_lo:c_lo + C_loc]
-    csl = combine[:, :, e_lo:e_lo + E_loc, c_lo:c_lo + C_loc]
-    ei = torch.empty(E_loc, B, C_loc, d, dtype=dtype, device=cuda)
-    ops.moe_dispatch(x.to(cuda), r, ei, E, C, e_lo, E_loc, c_lo, C_loc)
-    want_ei = torch.einsum("bsd,bsec->becd", x.float(), dsl)
+    pos = slice(s_lo, s_lo + S_loc)
+    dsl = dispatch[:, pos, e_lo:e_lo + E_loc, c_lo:c_lo + C_loc]
+    csl = combine[:, pos, e_lo:e_lo + E_loc, c_lo:c_lo + C_loc]
+    xs = x[:, pos].contiguous()
+    ei = torch.full((E_loc, B, C_loc, d), float("nan"), dtype=dtype, device=cuda)
+    ops.moe_dispatch(xs.to(cuda), r, ei, E, C, e_lo, E_loc, c_lo, C_loc, s_lo)
+    want_ei = torch.einsum("bsd,bsec->becd", xs.float(), dsl)
     assert torch.equal(ei.float().cpu().permute(1, 0, 2, 3), want_ei)            # a gather: exact
     eo = torch.randn(E_loc, B, C_loc, d, generator=g).to(dtype)
-    out = torch.empty(B, S, d, dtype=dtype, device=cuda)
-    ops.moe_combine(eo.to(cuda), r, out, C, e_lo, E_loc, c_lo, C_loc)
+    out = torch.full((B, S_loc, d), float("nan"), dtype=dtype, device=cuda)
+    ops.moe_combine(eo.to(cuda), r, out, C, e_lo, E_loc, c_lo, C_loc, s_lo)
     want_out = torch.einsum("becd,bsec->bsd", eo.float().permute(1, 0, 2, 3), csl)
     tol = 1e-5 if dtype == torch.float32 else 1e-2
-    assert rel_err(out, want_out) < tol
+    if S_loc:
+        assert rel_err(out, want_out) < tol
     # backward of combine and dispatch against autograd on the dense einsums
-    dout = torch.randn(B, S, d, generator=g).to(dtype)
+    dout = torch.randn(B, S_loc, d, generator=g).to(dtype)
     eo_a = eo.float().permute(1, 0, 2, 3).clone().requires_grad_(True)
     c_a = csl.clone().requires_grad_(True)
     torch.einsum("becd,bsec->bsd", eo_a, c_a).backward(dout.float())
-    d_eo = torch.empty(E_loc, B, C_loc, d, dtype=dtype, device=cuda)
-    dgate = torch.empty(B, S, 2, dtype=torch.float32, device=cuda)
-    ops.moe_combine_bwd(dout.to(cuda), eo.to(cuda), r, d_eo, dgate, E, C, e_lo, E_loc, c_lo, C_loc)
-    assert rel_err(d_eo.float().cpu().permute(1, 0, 2, 3), eo_a.grad) < tol
+    d_eo = torch.full((E_loc, B, C_loc, d), float("nan"), dtype=dtype, device=cuda)
+    dgate = torch.full((B, S, 2), float("nan"), dtype=torch.float32, device=cuda)
+    ops.moe_combine_bwd(dout.to(cuda), eo.to(cuda), r, d_eo, dgate, E, C, e_lo, E_loc, c_lo, C_loc, s_lo)
+    if S_loc:
+        assert rel_err(d_eo.float().cpu().permute(1, 0, 2, 3), eo_a.grad) < tol
+    else:
+        assert not d_eo.any()
     idx, slot = r["index"].cpu().long(), r["slot"].cpu().long()
     want_dgate = torch.zeros(B, S, 2)
     for b in range(B):
-        for s in range(S):
+        for s in range(s_lo, s_lo + S_loc):
             for k in range(2):
                 e = idx[b, s, k].item() - e_lo
                 c = slot[b, s, k].item() - c_lo
                 if slot[b, s, k] > 0 and 0 <= e < E_loc and 0 <= c < C_loc:
-                    want_dgate[b, s, k] = c_a.grad[b, s, e, c]
-    assert rel_err(dgate, want_dgate) < tol
+                    want_dgate[b, s, k] = c_a.grad[b, s - s_lo, e, c]
+    if S_loc:
+        assert rel_err(dgate, want_dgate) < tol
+    assert torch.equal(dgate.cpu() == 0, want_dgate == 0) or dtype == torch.bfloat16     # exact zeros outside the windows
+    assert not dgate.cpu()[:, :s_lo].any() and not dgate.cpu()[:, s_lo + S_loc:].any()
     d_ei = torch.randn(E_loc, B, C_loc, d, generator=g).to(dtype)
-    x_a = x.float().clone().requires_grad_(True)
+    x_a = xs.float().clone().requires_grad_(True)
     torch.einsum("bsd,bsec->becd", x_a, dsl).backward(d_ei.float().permute(1, 0, 2, 3))
-    dx = torch.empty(B, S, d, dtype=dtype, device=cuda)
-    ops.moe_dispatch_bwd(d_ei.to(cuda), r, dx, C, e_lo, E_loc, False, c_lo, C_loc)
-    assert rel_err(dx, x_a.grad) < tol
+    dx = torch.full((B, S_loc, d), float("nan"), dtype=dtype, device=cuda)
+    ops.moe_dispatch_bwd(d_ei.to(cuda), r, dx, C, e_lo, E_loc, False, c_lo, C_loc, s_lo)
+    if S_loc:
+        assert rel_err(dx, x_a.grad) < tol
 
 
 def test_gate_backward_matches_autograd(cuda):

@@ -170,12 +170,14 @@ def test_switch_moe(cuda, dtype, batch_sharded):
 @pytest.mark.parametrize("moe,dtype,batch_sharded", [("capacity", "fp32", True), ("capacity", "fp32", False),
                                                       ("capacity", "bf16", False), ("hidden", "fp32", True),
                                                       ("hidden", "bf16", False), ("model", "fp32", True),
-                                                      ("model", "fp32", False)])
+                                                      ("model", "fp32", False), ("sequence", "fp32", True),
+                                                      ("sequence", "fp32", False), ("sequence", "bf16", False)])
 def test_moe_capacity_and_hidden_splits(cuda, moe, dtype, batch_sharded):
     """The capacity split (dispatch / combine tensors sliced on dim 3, whole expert weights: every device works on
     a range of every expert's slots), the hidden-feature split of the expert FFN and the split of the tokens' model
-    dimension (the first expert product is then a partial sum, all-reduced in the program's [B, E, C, H] order)
-    (hap.rs:3285-3419), uneven over the devices, against the CPU run of all ranks."""
+    dimension (the first expert product is then a partial sum, all-reduced in the program's [B, E, C, H] order),
+    and the split along the sequence (tokens and routing windowed over positions 5 / 5 / 3 / 3 of 16, the dispatched
+    tokens all-reduced) (hap.rs:3285-3419), uneven over the devices, against the CPU run of all ranks."""
     # hidden widths 40 / 40 / 24 / 24 of 128 (multiples of the 16-byte vector in either type), capacity slots 3 / 3 / 2 / 2
     if moe == "model":      # model widths 20 / 20 / 12 / 12 of 64
         model = make_moe(d=64, C=10)

@@ -35,6 +35,7 @@ CASES = {
     "moe-capacity": (lambda: make_moe(C=10), RATIOS_E, 16, lambda: lm_batch(16, 16, 61), dict(ffn="batch", moe="capacity")),
     "moe-hidden": (lambda: make_moe(C=10), RATIOS_E, 16, lambda: lm_batch(16, 16, 61), dict(ffn="batch", moe="hidden")),
     "moe-model": (lambda: make_moe(C=10), RATIOS_E, 16, lambda: lm_batch(16, 16, 61), dict(ffn="batch", moe="model")),
+    "moe-sequence": (lambda: make_moe(C=10), RATIOS_E, 16, lambda: lm_batch(16, 16, 61), dict(ffn="batch", moe="sequence")),
     "moe-replicated-batch": (lambda: make_moe(), RATIOS_E, 4, lambda: lm_batch(4, 16, 61),
                              dict(ffn="batch", batch_sharded=False)),
 }

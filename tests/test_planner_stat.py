@@ -30,6 +30,7 @@ CASES = {
     "moe_capacity": dict(make=lambda: helpers.make_moe(C=10), ratios=RATIOS_E, B=8, kw=dict(ffn="batch", moe="capacity"), batch="lm"),
     "moe_hidden": dict(make=lambda: helpers.make_moe(C=10), ratios=RATIOS_E, B=8, kw=dict(ffn="batch", moe="hidden"), batch="lm"),
     "moe_model": dict(make=lambda: helpers.make_moe(C=10), ratios=RATIOS_E, B=8, kw=dict(ffn="batch", moe="model"), batch="lm"),
+    "moe_sequence": dict(make=lambda: helpers.make_moe(C=10), ratios=RATIOS_E, B=8, kw=dict(ffn="batch", moe="sequence"), batch="lm"),
     "lm_sequence": dict(make=lambda: helpers.make_lm(), ratios=RATIOS4, B=4, kw=dict(ffn="batch", shard_dim="sequence"), batch="lm"),
     "lm_feature_embedding": dict(make=lambda: helpers.make_lm(), ratios=RATIOS4, B=8, kw=dict(ffn="column", embedding="features"), batch="lm"),
     "moe_whole_batch": dict(make=lambda: helpers.make_moe(), ratios=RATIOS_E, B=4,

@@ -214,12 +214,12 @@ def test_feature_sharded_embedding_table_spmd_equals_single_device(ffn):
     _check(model, run, x, y, sharded)
 
 
-@pytest.mark.parametrize("moe", ["capacity", "hidden", "model"])
+@pytest.mark.parametrize("moe", ["capacity", "hidden", "model", "sequence"])
 def test_moe_capacity_and_hidden_splits_spmd_equal_single_device(moe):
     """The other legal splits of the four MoE einsums (hap.rs:3285-3419): every device takes a range of every
     expert's capacity slots with whole expert weights, or every device holds a slice of the experts' hidden
-    features, or of the tokens' model dimension (columns 10 / 10 / 6 / 6 of 32); batch-sharded attention around
-    them as in the expert split."""
+    features, or of the tokens' model dimension (columns 10 / 10 / 6 / 6 of 32), or the tokens of a range of positions
+    (5 / 5 / 3 / 3 of 16); batch-sharded attention around them as in the expert split."""
     model = make_moe(C=10, F=48)                                # capacity slots 3 / 3 / 2 / 2, hidden widths 15 / 15 / 9 / 9
     B = 16
     x, y = lm_batch(B, 16, 61)
