@@ -186,7 +186,7 @@ def test_wire_requests_of_gpu_and_cpu_runs_match(cuda):
 
 
 def test_lm_config1_full_size_fp32(cuda):
-    """BASELINE config 1 whole (2 layers, float32): the GPU against the float64 CPU run at 1e-4."""
+    """benchmark configuration 1 (bench.py --workload lm) whole (2 layers, float32): the GPU against the float64 CPU run at 1e-4."""
     _full_check("lm", 2, "fp32")
 
 
@@ -195,7 +195,7 @@ def test_bert_large_shard_full_width_bf16(cuda):
 
 
 def test_bert_large_shard_full_width_bf16_with_dropout(cuda):
-    """Two layers of BASELINE config 2 with the reference's default dropout probability (config.py:33) at the real
+    """Two layers of benchmark configuration 2 (bench.py --workload bert) with the reference's default dropout probability (config.py:33) at the real
     shapes: F.dropout in front of both residual LayerNorms and behind the FFN's relu (on the exchange's pieces),
     dropout_p on the probabilities of the fused attention (b 12, 16 heads, S 512).  The masks cannot be those of a
     torch run (PARITY UNPINNED for the particular masks); the GPU's are checked against the CPU restatement of the
@@ -237,7 +237,7 @@ def test_bert_large_shard_full_width_bf16_with_dropout(cuda):
 
 
 def test_bert_large_shard_full_depth_bf16_adam_step(cuda):
-    """All 24 layers of BASELINE config 2 with one Adam step: loss, gradients and updated weights."""
+    """All 24 layers of benchmark configuration 2 (bench.py --workload bert) with one Adam step: loss, gradients and updated weights."""
     ex, run, gm_ref, grads, ref_grads, before, before_ref = _full_check("bert", 24, "bf16", opt=True)
     ref_after = dict(gm_ref.named_parameters())
     lr = 5e-4
@@ -282,6 +282,6 @@ def test_moe_shard_full_width_fp32(cuda):
 
 
 def test_moe_shard_full_width_bf16(cuda):
-    """BASELINE config 4 in its own element type (routing: bit-exact on the GPU's own float32 logits; against the
+    """Benchmark configuration 4 (bench.py --workload moe) in its own element type (routing: bit-exact on the GPU's own float32 logits; against the
     float32 oracle only tokens with a near-tie may differ, and they are counted)."""
     _full_check("moe", 2, "bf16")
