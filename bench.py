@@ -28,6 +28,11 @@ RATIOS_E = [.3125, .3125, .1875, .1875]
 PEAK = {"bf16": 2500.0, "fp32": 157.3}        # dense MFMA TFLOP/s, MI355X
 HBM_PEAK = 8000.0                              # GB/s
 
+# counted on the default workload with the commands of profiles/bert_large_shard_step.counters.md: 87 852 KiB fetched
+# (x 2.0) + 33 629 KiB written per GEMM launch; every operand read and every result written once: 19.3 GB per step
+PROFILED_GEMM_TRAFFIC_PER_LAUNCH = (2.0 * 87852 + 33629) * 1024
+PROFILED_GEMM_ALGORITHMIC_BYTES_PER_LAUNCH = 19.3e9 / 207
+
 WORKLOADS = {
     # name: (description, dtype)
     "bert": ("BERT-large uneven shard: 24L d1024 h16 FFN 1536/4096 seq512 batch 12/32 vocab30522 MLM Adam", "bf16"),
@@ -393,6 +398,15 @@ def measure(workload, args, steps, warmup, share_shapes=True, dropout=None):
                      "event_brackets_ms_per_step": ms.value / max(1, steps if graph is None else 3),
                      "empty_brackets_ms_per_step": empty.value / max(1, steps if graph is None else 3), "traffic": None},
     }
+    default_bert = (bert and args.attn == "batch" and not args.zero and (args.dropout if dropout is None else dropout) == 0.0
+                    and not args.no_exchange_in_pieces and not args.no_receive_in_place and args.wgrad_group == 8)
+    if default_bert:
+        # bytes per GEMM launch between the L2 caches and the memory fabric, counted offline with rocprofv3 --pmc
+        # (FETCH_SIZE scaled by the factor a copy of known size gives, plus WRITE_SIZE; mean over the step's launches)
+        r = result["roofline"]
+        r["traffic"] = PROFILED_GEMM_TRAFFIC_PER_LAUNCH
+        r["traffic_unit"] = "bytes per launch (mean over the step's GEMM launches), rocprofv3 --pmc FETCH_SIZE x 2.0 + WRITE_SIZE"
+        r["algorithmic_bytes"] = PROFILED_GEMM_ALGORITHMIC_BYTES_PER_LAUNCH
     # the reference calibrates its planner with hap.stat / (seconds of one training step) (profiler.py:33-39)
     shard_stat = planner.stat(gm, {"input_shape": {"x": tuple(x.shape), "y": tuple(y.shape)}})
     result["config"]["hap_stat_flops_of_shard"] = shard_stat
