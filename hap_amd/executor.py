@@ -1728,7 +1728,8 @@ class ShardExecutor:
 
     def _all_reduce_expert(self, node, x: Val, rank, W):
         """all_reduce of expert-major activations (the partial sums of an expert product over a split model
-        dimension, hap.rs:3331-3335).  The program's tensor is [B, E, C, N] and that is what crosses the wire; the
+        dimension, hap.rs:3331-3335, or the dispatched tokens of a split over positions, hap.rs:3300-3304).  The
+        program's tensor is [B, E, C, N] and that is what crosses the wire; the
         storage here is [E, B, C, N], so the value is brought into the program's order before the sum and back
         behind it (two strided copies per direction)."""
         El, B, C, N = x.t.shape
