@@ -554,7 +554,7 @@ def _keep_words_to_masks(keep_rows, keep_cols, b, H, S):
     return torch.from_numpy(from_rows), torch.from_numpy(from_cols).transpose(1, 2)
 
 
-@pytest.mark.parametrize("S", [16, 64, 129, 197, 512])
+@pytest.mark.parametrize("S", [1, 16, 64, 65, 129, 197, 512])
 def test_attention_keep_words_are_the_dropout_kernels_decisions(cuda, S):
     """Both bit layouts of attention_keep_bits hold exactly the decisions that the dropout kernel takes for a
     [b*H, S, row_len] tensor of probabilities under the same state and stream id (bit-exact)."""
@@ -569,7 +569,8 @@ def test_attention_keep_words_are_the_dropout_kernels_decisions(cuda, S):
     got_rows, got_cols = _keep_words_to_masks(kr, kc, b, H, S)
     assert torch.equal(got_rows, want)
     assert torch.equal(got_cols, want)
-    assert 0.70 < want.float().mean().item() < 0.80
+    if S >= 16:
+        assert 0.70 < want.float().mean().item() < 0.80
     # query bits beyond S inside a column's last word are zero
     n_kt = (S + 63) // 64
     cols = kc.cpu().numpy().astype(np.uint32).reshape(b * H, S, 2 * n_kt)
@@ -578,8 +579,8 @@ def test_attention_keep_words_are_the_dropout_kernels_decisions(cuda, S):
         assert not ((cols[:, :, qq // 32] >> (qq % 32).astype(np.uint32)) & 1).any()
 
 
-@pytest.mark.parametrize("S,causal", [(16, False), (64, True), (129, "flag"), (197, False), (512, False), (512, "flag"),
-                                      (200, True)])
+@pytest.mark.parametrize("S,causal", [(8, False), (16, False), (64, True), (65, "flag"), (129, "flag"), (197, False),
+                                      (512, False), (512, "flag"), (200, True)])
 def test_fused_attention_with_dropout_of_the_probabilities(cuda, S, causal):
     """out = dropout(softmax(QK^T * scale + mask)) V (F.multi_head_attention_forward with dropout_p > 0) and its
     gradients, in float64 from the same bf16 inputs with the keep decisions of the dropout kernel."""
