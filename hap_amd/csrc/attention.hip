@@ -444,10 +444,12 @@ __global__ __launch_bounds__(AT_THREADS, 2) void attn_bwd_dq_kernel(const bf16_t
             lv.load(V + (int64_t)nx * ld, S - nx);
             if constexpr (DROP) keep_next = keep_row[(nx / TILE) * 2];
         }
+        if (blk * 128 + wave * 32 >= S) continue;                  // a wave without queries only moves tiles and meets barriers
 
         // one 32-row kv block at a time keeps only one score / dP accumulator pair live
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
+            if (t == 1 && kv0 + 32 >= S) break;                    // the sequence ends in the tile's first half: no key here
             f32x16 st = zero16(), dp = zero16();
 #pragma unroll
             for (int s = 0; s < 4; ++s) {
@@ -568,11 +570,13 @@ __global__ __launch_bounds__(AT_THREADS, 2) void attn_bwd_dkv_kernel(const bf16_
             ldo.load(dO + (int64_t)nx * E, S - nx);
             if constexpr (DROP) keep2_next = keep_col[nx / TILE];
         }
+        if (blk * 128 + wave * 32 >= S) continue;                  // a wave without keys only moves tiles and meets barriers
 
         // one 32-row query block at a time keeps only one score / dP accumulator pair live; the loop is kept
         // rolled so that the scheduler cannot pull the second block's fragments ahead of the first one's math
 #pragma unroll 1
         for (int t = 0; t < 2; ++t) {
+            if (t == 1 && q0 + 32 >= S) break;                     // the sequence ends in the tile's first half: no query here
             f32x16 sc = zero16(), dp = zero16();
 #pragma unroll
             for (int s = 0; s < 4; ++s) {
