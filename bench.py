@@ -160,8 +160,6 @@ def main():
                     help="bert workload only: parameters stored as dim-0 shards and gathered at use")
     ap.add_argument("--gemm-table", default=None,
                     help="write a table of the step's distinct GEMM shapes (tile configuration, time of a cold launch) to this file")
-    ap.add_argument("--gemm-table-vendor", action="store_true",
-                    help="with --gemm-table: also time torch.mm on each bf16 shape, for orientation")
     ap.add_argument("--gemm-plan-file", default=None,
                     help="JSON file of pinned GEMM plans: loaded instead of autotuning when it exists, written after "
                          "autotuning otherwise (a profiler run can then repeat the plan of an unprofiled run)")
@@ -221,61 +219,21 @@ def _brief(r):
             "gemm_ms_per_step": r["roofline"]["gemm_ms_per_step"], "final_loss": r["config"]["final_loss"]}
 
 
-def _write_gemm_table(path, report, desc, vendor):
+def _write_gemm_table(path, report, desc):
     """One row per distinct GEMM signature of the step: the tile configuration that autotuning picked and the time of
     one launch on the program's own operands with cold caches (the median of three launches, each behind a write
-    over a buffer larger than the caches).  With `vendor`, two more measurements on buffers of the same shape and
-    layout under the same protocol: `operands only`, the measurement configuration of the library that moves every
-    k-tile of both operands from memory into LDS in 192 x 128 tiles but multiplies nothing (shapes with transA = 0,
-    bf16 results), next to the full launch of that tile configuration (7), and torch.mm (the vendor BLAS), bf16
-    output, no bias / row sums / pieces: for orientation only, nothing in the package calls it."""
-    import torch
-    from hap_amd import ops
-    from hap_amd._lib import lib
+    over a buffer larger than the caches)."""
     rows, total_us, total_flop = [], 0.0, 0.0
-    flush = torch.zeros(512 << 20, dtype=torch.int8, device="cuda:0") if vendor else None
-
-    def cold(fn):
-        ts = []
-        for _ in range(5):
-            flush.add_(1)
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record()
-            fn()
-            e1.record()
-            e1.synchronize()
-            ts.append(e0.elapsed_time(e1) * 1e3)
-        return sorted(ts)[2]
     for key, cfg, splits, us, launches, problems in report:
         M, N, K, batch, tA, tB, in_dt, out_dt, segA, segB, segC, a_relu, b_relu = key
         flop = 2.0 * M * N * K * batch
         total_us += us * launches
         total_flop += flop * launches
-        v = ""
-        if vendor and in_dt == 1:
-            A = torch.randn((K, M) if tA else (M, K), device="cuda:0").bfloat16()
-            B = torch.randn((N, K) if tB else (K, N), device="cuda:0").bfloat16()
-            C = torch.empty(M, N, device="cuda:0", dtype=torch.bfloat16)
-            opA, opB = (A.t() if tA else A), (B.t() if tB else B)
-            for _ in range(2):
-                torch.mm(opA, opB, out=C)
-            t = cold(lambda: torch.mm(opA, opB, out=C))
-            v = f"  vendor (one problem) {t:7.1f} us {2.0 * M * N * K / t / 1e6:5.0f} TFLOP/s"
-            if not tA and out_dt == 1 and K % 8 == 0 and N % 8 == 0:
-                try:
-                    times = []
-                    for cfg_probe in (7, ops.OPERAND_MOVEMENT_ONLY_CONFIG):
-                        lib().hapmi_gemm_tuning(cfg_probe, 1)
-                        ops.gemm(A, B, C, M, N, K, transB=bool(tB))
-                        times.append(cold(lambda: ops.gemm(A, B, C, M, N, K, transB=bool(tB))))
-                finally:
-                    lib().hapmi_gemm_tuning(-1, 0)
-                v += f"  | 192x128 tiles: {times[0]:6.1f} us, operands only {times[1]:6.1f} us"
         kind = "".join(c for c, on in (("A", segA), ("B", segB), ("C", segC)) if on)
         rows.append((us * launches, f"{us * launches / 1e3:6.2f} ms/step  x{launches:3d}  M{M:6d} N{N:6d} K{K:6d} batch{batch:4d} "
                      f"{'T' if tA else 'N'}{'T' if tB else 'N'} {'bf16' if in_dt == 1 else 'f32'}->{'bf16' if out_dt == 1 else 'f32'}"
                      f"  cfg{cfg:2d} split{splits:2d}  {us:7.1f} us {flop / us / 1e6:5.0f} TFLOP/s"
-                     f"{'  pieces ' + kind if kind else ''}{'  relu on A' if a_relu else ''}{'  relu on B' if b_relu else ''}{v}"))
+                     f"{'  pieces ' + kind if kind else ''}{'  relu on A' if a_relu else ''}{'  relu on B' if b_relu else ''}"))
     with open(path, "w") as f:
         f.write(f"{desc}\n")
         for _, line in sorted(rows, reverse=True):
@@ -322,7 +280,7 @@ def measure(workload, args, steps, warmup, share_shapes=True, dropout=None):
         if args.gemm_plan_file:
             ops.save_gemm_plans(args.gemm_plan_file)
         if args.gemm_table and workload == args.workload:
-            _write_gemm_table(args.gemm_table, report, desc, args.gemm_table_vendor)
+            _write_gemm_table(args.gemm_table, report, desc)
 
     graph = None
     for _ in range(warmup):

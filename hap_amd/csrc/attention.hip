@@ -189,7 +189,7 @@ template <bool CAUSAL> struct BlockOrder {
     __device__ __forceinline__ static int batch_head() { return CAUSAL ? linear() % (int)gridDim.y : work_item() / (int)gridDim.x; }
 };
 
-// CAUSAL: key j is visible to query i iff j <= i (the additive mask torch.triu(full(-inf), 1), models.py:76),
+// CAUSAL: key j is visible to query i iff j <= i (the additive mask torch.triu(full(-inf), 1), models.py:72, 97),
 // applied arithmetically; kv tiles that lie completely above the diagonal of the block's 128 queries are skipped.
 // DROP: dropout of the probabilities (F.multi_head_attention_forward with dropout_p > 0, hap.rs:1257, 1307).  The
 // keep decisions come as bit words (attn_keep_bits below): the row sums stay those of the undropped probabilities,

@@ -18,6 +18,7 @@ typedef float f32x2 __attribute__((ext_vector_type(2)));
 #define HAPMI_WAVE 64
 
 int hapmi_set_error(int code, const char *fmt, ...);
+int hapmi_sumsq_static_setup();   // elementwise.hip: per-device set-up that hapmi_init runs
 
 #define HAPMI_REQUIRE(cond, code, ...)                           \
     do {                                                         \

@@ -338,7 +338,10 @@ __global__ __launch_bounds__(256) void embedding_fwd_kernel(const int64_t *ids, 
 // dtable[id, :] += sum over the tokens t with ids[t] == id of dout[t, :] * scale, added in token order.  One wave per
 // token; the wave of the FIRST token of an id (no earlier token has the same id) gathers all of that id's rows in
 // registers and adds the sum to the table row, the other waves leave.  No atomics and one writer per table row, so
-// the same call gives the same bits every time.  Rows up to 64 * EB_COLS wide.
+// the same call gives the same bits every time.  A wave holds 64 * EB_COLS columns of a row; wider rows are cut into
+// column blocks over blockIdx.y.  Cost: every wave reads all earlier ids (n_tokens^2 / 2 id loads per call and column
+// block, 64 per instruction): 19 M for the 6144 tokens of a [12, 512] shard, negligible next to the rows moved; a batch
+// of far more tokens per call would want a sort by id first.
 constexpr int EB_COLS = 32;
 template <typename T>
 __global__ __launch_bounds__(256) void embedding_bwd_kernel(const int64_t *ids, const T *dout, float *dtable,
@@ -348,6 +351,7 @@ __global__ __launch_bounds__(256) void embedding_bwd_kernel(const int64_t *ids, 
     if (t >= n_tokens) return;
     const int64_t id = ids[t];
     if (id < 0 || id >= vocab) return;
+    const int64_t col0 = (int64_t)blockIdx.y * (64 * EB_COLS);   // this block's columns: col0 .. col0 + 64 * EB_COLS
     // is an earlier token of the same id?  (wave-uniform)
     for (int64_t u0 = 0; u0 < t; u0 += 64) {
         const int64_t u = u0 + lane;
@@ -366,8 +370,8 @@ __global__ __launch_bounds__(256) void embedding_bwd_kernel(const int64_t *ids, 
             const T *row = dout + (u0 + b) * d;
 #pragma unroll
             for (int j = 0; j < EB_COLS; ++j) {
-                const int64_t c = (int64_t)j * 64 + lane;
-                if ((int64_t)j * 64 < d && c < d) {
+                const int64_t c = col0 + (int64_t)j * 64 + lane;
+                if (col0 + (int64_t)j * 64 < d && c < d) {
                     float g = ld_f(row, c) * scale;
                     if (sizeof(T) == 2) g = (float)(bf16_t)g;
                     acc[j] += g;
@@ -377,8 +381,8 @@ __global__ __launch_bounds__(256) void embedding_bwd_kernel(const int64_t *ids, 
     }
 #pragma unroll
     for (int j = 0; j < EB_COLS; ++j) {
-        const int64_t c = (int64_t)j * 64 + lane;
-        if ((int64_t)j * 64 < d && c < d) dtable[id * d + c] += acc[j];
+        const int64_t c = col0 + (int64_t)j * 64 + lane;
+        if (col0 + (int64_t)j * 64 < d && c < d) dtable[id * d + c] += acc[j];
     }
 }
 
@@ -402,10 +406,10 @@ extern "C" int hapmi_embedding_fwd(const int64_t *ids, const void *table, const 
 extern "C" int hapmi_embedding_bwd(const int64_t *ids, const void *dout, float *dtable, int64_t n_tokens, int64_t d,
                                    int64_t vocab, float scale, int dtype, hapmi_stream_t stream) {
     HAPMI_REQUIRE(hapmi_dtype_ok(dtype) && n_tokens >= 0 && d >= 1 && vocab >= 1, HAPMI_EINVAL, "embedding_bwd: bad argument");
-    HAPMI_REQUIRE(d <= 64 * EB_COLS, HAPMI_ELIMIT, "embedding_bwd: rows of at most %d elements", 64 * EB_COLS);
+    HAPMI_REQUIRE(hapmi_cdiv(d, 64 * EB_COLS) <= 65535, HAPMI_ELIMIT, "embedding_bwd: rows of at most %d elements", 65535 * 64 * EB_COLS);
     if (n_tokens == 0) return HAPMI_OK;
     HAPMI_REQUIRE(ids && dout && dtable, HAPMI_EINVAL, "embedding_bwd: null pointer");
-    dim3 grid((unsigned)hapmi_cdiv(n_tokens, 4));
+    dim3 grid((unsigned)hapmi_cdiv(n_tokens, 4), (unsigned)hapmi_cdiv(d, 64 * EB_COLS));
     if (dtype == HAPMI_F32)
         hipLaunchKernelGGL((embedding_bwd_kernel<float>), grid, dim3(256), 0, (hipStream_t)stream, ids, (const float *)dout, dtable, n_tokens, d, vocab, scale);
     else
@@ -700,7 +704,19 @@ constexpr int kMaxDevices = 64;
 std::mutex g_scratch_mu;
 float *g_scratch_ptr[kMaxDevices] = {nullptr};
 
-int sumsq_scratch_of_current_device(float **ptr) {
+// the device a stream belongs to (the current device for the null stream)
+int device_of_stream(hipStream_t st, int *dev) {
+    hipError_t e = st ? hipStreamGetDevice(st, dev) : hipGetDevice(dev);
+    if (e != hipSuccess) return hapmi_set_error(HAPMI_ELAUNCH, "sumsq_static: device of the stream: %s", hipGetErrorString(e));
+    HAPMI_REQUIRE(*dev >= 0 && *dev < kMaxDevices, HAPMI_ELIMIT, "sumsq_static: device index %d beyond %d", *dev, kMaxDevices);
+    return HAPMI_OK;
+}
+}  // namespace
+
+// Looks up the address of the current device's copy of the scratch array (hapmi_init calls this, so that a later
+// hapmi_sumsq_static is a pure enqueue: no symbol lookup, no lazy module load, nothing a stream capture would record
+// or refuse).
+int hapmi_sumsq_static_setup() {
     int dev = -1;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return hapmi_set_error(HAPMI_ELAUNCH, "sumsq_static: hipGetDevice: %s", hipGetErrorString(e));
@@ -713,10 +729,8 @@ int sumsq_scratch_of_current_device(float **ptr) {
             return hapmi_set_error(HAPMI_ELAUNCH, "sumsq_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
         g_scratch_ptr[dev] = (float *)p;
     }
-    *ptr = g_scratch_ptr[dev];
     return HAPMI_OK;
 }
-}  // namespace
 
 extern "C" int hapmi_sumsq_static(const float *g, int64_t n, float *out, hapmi_stream_t stream) {
     HAPMI_REQUIRE(n >= 0 && out, HAPMI_EINVAL, "sumsq_static: bad argument");
@@ -729,9 +743,17 @@ extern "C" int hapmi_sumsq_static(const float *g, int64_t n, float *out, hapmi_s
     HAPMI_REQUIRE(hapmi_cdiv(n, SUMSQ_CHUNK) <= SUMSQ_STATIC_CHUNKS, HAPMI_ELIMIT,
                   "sumsq_static: %lld elements exceed the built-in scratch (at most %lld elements; use hapmi_sumsq "
                   "with a workspace)", (long long)n, (long long)(SUMSQ_STATIC_CHUNKS * SUMSQ_CHUNK));
-    float *scratch = nullptr;
-    const int rc = sumsq_scratch_of_current_device(&scratch);
+    int dev = -1;
+    const int rc = device_of_stream((hipStream_t)stream, &dev);
     if (rc) return rc;
+    float *scratch = nullptr;
+    {
+        std::lock_guard<std::mutex> lk(g_scratch_mu);
+        scratch = g_scratch_ptr[dev];
+    }
+    HAPMI_REQUIRE(scratch, HAPMI_EINVAL,
+                  "sumsq_static: hapmi_init() has not run with device %d current (it looks up that device's scratch "
+                  "array; this call only enqueues kernels)", dev);
     // every partial sum that the final kernel reads is written by the first kernel of this call: nothing in the
     // array has to start at zero, whatever an earlier call left there
     return sumsq_launch(g, n, out, scratch, (hipStream_t)stream);

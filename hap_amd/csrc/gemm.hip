@@ -32,7 +32,6 @@ HAPMI_GEMM_DECLARE_CFG(8);
 HAPMI_GEMM_DECLARE_CFG(9);
 HAPMI_GEMM_DECLARE_CFG(10);
 HAPMI_GEMM_DECLARE_CFG(11);
-HAPMI_GEMM_DECLARE_CFG(12);
 
 namespace {
 
@@ -42,9 +41,8 @@ struct TileCfg {
 };
 constexpr TileCfg kCfg[] = {{128, 128, 2, 2}, {256, 256, 2, 4}, {384, 192, 4, 2}, {192, 256, 2, 4}, {256, 192, 4, 2},
                              {256, 128, 4, 2}, {128, 256, 2, 4}, {192, 128, 2, 4}, {256, 128, 2, 2}, {128, 192, 4, 2},
-                             {64, 64, 2, 2}, {64, 128, 2, 2}, {192, 128, 2, 4}};
-constexpr int kNumCfg = 13;
-constexpr int kProbeCfg = 12;                    // operand movement only: a measurement build, never chosen automatically
+                             {64, 64, 2, 2}, {64, 128, 2, 2}};
+constexpr int kNumCfg = 12;
 constexpr bool is_f32_cfg(int c) { return c == 10 || c == 11; }   // small tiles for float32 operands only
 constexpr int kNumCU = 256;
 int g_force_cfg = -1;
@@ -93,13 +91,12 @@ struct SegNeeds {
     bool three_stage = false;
     int64_t n_align = 0;                       // 0: no constraint; else every piece boundary along N is a multiple of it
 };
-constexpr bool kThreeStage[] = {false, false, false, false, false, true, true, true, true, true, false, false, true};
+constexpr bool kThreeStage[] = {false, false, false, false, false, true, true, true, true, true, false, false};
 
 bool cfg_eligible(int c, bool bf16_in, bool wide, bool row_major_operands, bool forced, const SegNeeds &need = SegNeeds()) {
     if (need.three_stage && !kThreeStage[c]) return false;
     if (need.n_align > 0 && need.n_align % kCfg[c].bn != 0) return false;
     if (c == 0) return true;
-    if (c == kProbeCfg) return forced && bf16_in;
     if (is_f32_cfg(c)) return !bf16_in;
     if (!bf16_in || !wide) return false;
     if (c == 2 && !row_major_operands && !forced) return false;          // 384x192 with a transposing loader spills registers
@@ -277,7 +274,6 @@ int launch_typed(GemmParams &p, int transA, int transB, int64_t batch, hipStream
         case 9: rc = hapmi_gemm_launch_cfg9(p, in_dtype, out_dtype, transA, transB, batch, st); break;
         case 10: rc = hapmi_gemm_launch_cfg10(p, in_dtype, out_dtype, transA, transB, batch, st); break;
         case 11: rc = hapmi_gemm_launch_cfg11(p, in_dtype, out_dtype, transA, transB, batch, st); break;
-        case 12: rc = hapmi_gemm_launch_cfg12(p, in_dtype, out_dtype, transA, transB, batch, st); break;
         default: rc = hapmi_gemm_launch_cfg0(p, in_dtype, out_dtype, transA, transB, batch, st);
     }
     if (rc) return rc;
@@ -409,9 +405,10 @@ extern "C" int hapmi_gemm(const hapmi_gemm_args *a, hapmi_stream_t stream) {
     p.drop_p = a->drop_p;
     if (a->drop_state) {
         HAPMI_REQUIRE(!lists && batch == 1 && !a->transA && a->transB && !a->accumulate && a->ldc == a->N && (a->N % 2) == 0 && !a->C_segments &&
+                          !a->A_segments && !a->B_segments && !a->c_mask_segments && !a->B_segments_list && !a->a_relu && !a->b_relu &&
                           ((uintptr_t)a->drop_state % 8) == 0 && a->drop_p >= 0.f && a->drop_p <= 1.f,
                       HAPMI_EINVAL, "gemm: dropout in the epilogue takes one contiguous problem (transA = 0, transB = 1, ldc = N, N even), no accumulate, "
-                      "and a probability in [0, 1]");
+                      "no pieces, no relu on an operand, and a probability in [0, 1]");
     }
 
     // operands / result in pieces
@@ -520,7 +517,6 @@ extern "C" int hapmi_gemm_plan_set(int64_t M, int64_t N, int64_t K, int64_t batc
     HAPMI_REQUIRE(hapmi_dtype_ok(in_dtype) && hapmi_dtype_ok(out_dtype), HAPMI_EINVAL, "gemm_plan_set: bad dtype");
     HAPMI_REQUIRE(tile_config < kNumCfg && k_splits >= 1 && k_splits <= 64, HAPMI_EINVAL,
                   "gemm_plan_set: configuration %d / splits %d out of range", tile_config, k_splits);
-    HAPMI_REQUIRE(tile_config != kProbeCfg, HAPMI_EINVAL, "gemm_plan_set: configuration %d multiplies nothing (a measurement build) and cannot be pinned", kProbeCfg);
     const PlanKey key(M, N, K, batch, (int)(transA != 0), (int)(transB != 0), in_dtype, out_dtype);
     std::lock_guard<std::mutex> lk(g_plans_mu);
     if (tile_config < 0) g_plans.erase(key);

@@ -98,9 +98,7 @@ __device__ __forceinline__ f32x4 relu_frag(f32x4 v) {
 // OPMODE bits (compile-time, so that the main loop of every instantiation is free of branches).  1: A is read in
 // pieces along K (p.segA; NT layout, three stages, direct loads; a plain A travels as one piece).  2: relu on the
 // fragments of op(A).  4: relu on the fragments of op(B) (TN layout: the weight gradient whose B operand is the
-// activation that a relu produced).  8: measurement build of the three-stage loop: every k-tile's operands are
-// loaded into LDS and waited for as usual, but no fragment is read and no MFMA issued (the result is zeros); it
-// tells how much of a launch's time is the movement of the operands from L2 into the CU.  16: F.dropout behind the
+// activation that a relu produced).  16: F.dropout behind the
 // activation in the epilogue (NT layout: a linear's forward; p.drop_*).  The other kinds of pieces (B, C and the mask along N) only move this block's
 // base pointers and leading dimensions, which costs nothing, so they need no instantiation of their own.
 template <typename TI, typename TO, int BM, int BN, int WAVES_M, int WAVES_N, bool A_KMAJOR, bool B_KMAJOR, int NSTAGES, int OPMODE = 0>
@@ -345,7 +343,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, ((WAVES_M * WAVES_N <= 4 && 
                 const int nxt2 = cur == 0 ? 2 : cur - 1;          // (cur + 2) % 3: the buffer of tile kt - 1
                 if (kt + 2 < kt_end) issue_tile(kt + 2, nxt2);
                 if (do_rs && kt % p.tiles_n == tn) rs_add_lds(As + cur * A_BYTES);
-                if constexpr ((OPMODE & 8) == 0) compute_tile(As + cur * A_BYTES, Bs + cur * B_BYTES);
+                compute_tile(As + cur * A_BYTES, Bs + cur * B_BYTES);
                 cur = cur == 2 ? 0 : cur + 1;
             }
             __syncthreads();
@@ -672,7 +670,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, ((WAVES_M * WAVES_N <= 4 && 
     }
 }
 
-template <typename TI, typename TO, int BM, int BN, int WM, int WN, int NSTAGES = 2, int PROBE = 0>
+template <typename TI, typename TO, int BM, int BN, int WM, int WN, int NSTAGES = 2>
 int launch_cfg(const GemmParams &p, int transA, int transB, int64_t batch, hipStream_t st) {
     GemmParams q = p;
     q.tiles_m = (int)hapmi_cdiv(p.M, BM);
@@ -715,12 +713,6 @@ int launch_cfg(const GemmParams &p, int transA, int transB, int64_t batch, hipSt
     if (p.drop_state) {
         if (transA || !transB) return hapmi_set_error(HAPMI_EINVAL, "gemm: dropout in the epilogue needs transA = 0, transB = 1");
         HAPMI_GEMM_LAUNCH_MODE(true, true, 16);
-        return HAPMI_OK;
-    }
-    if constexpr (PROBE != 0) {
-        if (transA) return hapmi_set_error(HAPMI_EINVAL, "gemm: the measurement configuration takes transA = 0 only");
-        if (transB) HAPMI_GEMM_LAUNCH_MODE(true, true, PROBE);
-        else HAPMI_GEMM_LAUNCH_MODE(true, false, PROBE);
         return HAPMI_OK;
     }
     if (!transA && transB) HAPMI_GEMM_LAUNCH(true, true);

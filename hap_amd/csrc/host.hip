@@ -26,7 +26,7 @@ extern "C" int hapmi_init(void) {
     if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
         return hapmi_set_error(HAPMI_EARCH, "device %d is %s; this library holds gfx950 code only", dev,
                                prop.gcnArchName);
-    return HAPMI_OK;
+    return hapmi_sumsq_static_setup();
 }
 
 // Integer shard lengths.  full_length == 1 gives every rank one unit (the

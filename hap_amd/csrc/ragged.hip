@@ -6,8 +6,7 @@
 
 namespace {
 
-int g_grid_shift = 2;      // grid cap = 4096 << shift blocks (hapmi_ragged_tuning changes it for measurements)
-bool g_copy_nt = false;    // measurement hook: streaming loads in the plain 16-byte segment copy
+constexpr int kGridShift = 2;   // grid cap = 4096 << shift blocks
 
 struct Segment {
     const char *src;
@@ -202,7 +201,7 @@ int launch_segments(const SegmentList &list, int act, int dtype, hipStream_t str
     }
     if (max_chunks == 0) return HAPMI_OK;
     int64_t gx = hapmi_cdiv(max_chunks, (int64_t)COPY_THREADS * COPY_UNROLL);
-    const int64_t cap = hapmi_cdiv((int64_t)(256 * 16) << g_grid_shift, list.n);   // blocks over all segments
+    const int64_t cap = hapmi_cdiv((int64_t)(256 * 16) << kGridShift, list.n);   // blocks over all segments
     if (gx > cap) gx = cap;
     if (gx < 1) gx = 1;
     dim3 grid((unsigned)gx, (unsigned)list.n), block(COPY_THREADS);
@@ -235,8 +234,6 @@ int launch_segments(const SegmentList &list, int act, int dtype, hipStream_t str
             hipLaunchKernelGGL((segment_copy_kernel<u32x4, ReluBf16>), grid, block, 0, stream, list, ReluBf16());
         else
             hipLaunchKernelGGL((segment_copy_kernel<u32x4, ReluF32>), grid, block, 0, stream, list, ReluF32());
-    } else if (vec == 16 && g_copy_nt) {
-        hipLaunchKernelGGL((segment_copy_kernel<u32x4, ActNone<u32x4>, true>), grid, block, 0, stream, list, ActNone<u32x4>());
     } else if (vec == 16) {
         hipLaunchKernelGGL((segment_copy_kernel<u32x4, ActNone<u32x4>>), grid, block, 0, stream, list, ActNone<u32x4>());
     } else if (vec == 4) {
@@ -498,8 +495,7 @@ constexpr int RED_THREADS = 256;
 
 // bit0 nontemporal loads, bit1 nontemporal store, bit2 two vectors per thread.  Measured on eight contributions of
 // 131 MB: plain 5.2 TB/s, streaming loads 5.7-6.0, with two vectors per thread 6.1; streaming stores lose 0.2
-constexpr int RED_VARIANT_DEFAULT = 5;
-int g_red_variant = RED_VARIANT_DEFAULT;
+constexpr int RED_VARIANT = 5;
 
 struct ReduceOut {
     void *dst;
@@ -656,23 +652,14 @@ int launch_reduce(const ReduceArgs &a, const ReduceOuts &outs, int64_t outer, in
     }
     for (int w = 0; w < a.n; ++w) vec_ok = vec_ok && ((uintptr_t)a.src[w] % 16 == 0);
     if (vec_ok) {
-        const int u = (g_red_variant & 4) ? 2 : 1;
+        const int u = (RED_VARIANT & 4) ? 2 : 1;
         const int64_t total = outer * (max_len * inner / EPV);
         int64_t gx = hapmi_cdiv(total, (int64_t)RED_THREADS * u);
-        const int64_t cap = hapmi_cdiv((int64_t)(256 * 16) << g_grid_shift, outs.n);
+        const int64_t cap = hapmi_cdiv((int64_t)(256 * 16) << kGridShift, outs.n);
         if (gx > cap) gx = cap;
         if (gx < 1) gx = 1;
         dim3 grid((unsigned)gx, (unsigned)outs.n);
-        switch (g_red_variant & 7) {
-            case 1: launch_reduce_var<T, 1>(a, outs, outer, src_len, inner, grid, stream); break;
-            case 2: launch_reduce_var<T, 2>(a, outs, outer, src_len, inner, grid, stream); break;
-            case 3: launch_reduce_var<T, 3>(a, outs, outer, src_len, inner, grid, stream); break;
-            case 4: launch_reduce_var<T, 4>(a, outs, outer, src_len, inner, grid, stream); break;
-            case 5: launch_reduce_var<T, 5>(a, outs, outer, src_len, inner, grid, stream); break;
-            case 6: launch_reduce_var<T, 6>(a, outs, outer, src_len, inner, grid, stream); break;
-            case 7: launch_reduce_var<T, 7>(a, outs, outer, src_len, inner, grid, stream); break;
-            default: launch_reduce_var<T, 0>(a, outs, outer, src_len, inner, grid, stream);
-        }
+        launch_reduce_var<T, RED_VARIANT>(a, outs, outer, src_len, inner, grid, stream);
     } else {
         for (int r = 0; r < outs.n; ++r) {
             const ReduceOut &o = outs.out[r];
@@ -774,9 +761,3 @@ extern "C" int hapmi_pad_rows_multi(const void *const *srcs, void *const *dsts, 
     return launch_segments(list, HAPMI_ACT_NONE, 0, (hipStream_t)stream, "pad_rows_multi");
 }
 
-extern "C" int hapmi_ragged_tuning(int reduce_variant, int grid_shift) {
-    g_red_variant = reduce_variant < 0 ? RED_VARIANT_DEFAULT : (reduce_variant & 7);
-    g_copy_nt = reduce_variant >= 0 && (reduce_variant & 8);
-    g_grid_shift = grid_shift < 0 ? 2 : (grid_shift & 7);
-    return HAPMI_OK;
-}

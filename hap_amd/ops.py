@@ -601,7 +601,6 @@ _SPLIT_MENU = (1, 2, 3, 4, 5, 6, 7, 8, 10, 12, 16)
 _BF16_TILE_CONFIGS = tuple(range(10))
 _F32_TILE_CONFIGS = (0, 10, 11)
 _THREE_STAGE_CONFIGS = (5, 6, 7, 8, 9)
-OPERAND_MOVEMENT_ONLY_CONFIG = 12     # measurement build of configuration 7: loads every k-tile, multiplies nothing
 _TILE_N = {0: 128, 1: 256, 2: 192, 3: 256, 4: 192, 5: 128, 6: 256, 7: 128, 8: 128, 9: 192, 10: 64, 11: 128}
 
 

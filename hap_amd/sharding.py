@@ -83,7 +83,10 @@ class ShardingPlan:
                                  # tensors sliced on dim 2, expert weights on dim 0; "capacity": dispatch / combine
                                  # sliced on dim 3 (every device takes a range of every expert's slots), expert weights
                                  # whole; "hidden": routing whole, first expert weight sliced on dim 2 and the second on
-                                 # dim 1 (a feature split of the expert FFN; the second product is a partial sum);
+                                 # dim 1 (a feature split of the expert FFN; the second product is a partial sum, which is fed
+                                 # to the combine einsum as it is and reduced after it: [B, S, d] instead of [B, E, C, d]
+                                 # crosses the wire.  Equal by linearity, but not a program the reference's synthesizer
+                                 # emits: it would all_reduce in front of the combine, hap.rs:3369-3373, 3385-3415);
                                  # "model": the tokens' model dimension (dispatch input sliced on dim 2, first weight
                                  # on dim 1 with its product all-reduced, second on dim 2, combine output gathered);
                                  # "sequence": tokens, dispatch and combine tensors sliced over positions (dim 1): the

@@ -41,7 +41,9 @@ enum {
 };
 #define HAPMI_MAX_RANKS 64
 
-/* ---- host side ------------------------------------------------------- */
+/* ---- host side -------------------------------------------------------
+ * hapmi_init: once per process and per device, with that device current: checks that it is gfx950 and looks up the
+ * device's copy of the scratch array that hapmi_sumsq_static uses. */
 int hapmi_init(void);
 const char *hapmi_last_error(void);
 int hapmi_version(void);
@@ -94,7 +96,8 @@ int hapmi_split_rows_relu_bwd(const void *src, const void *fwd_out, void *const 
                               const int64_t *lengths_host, int n_ranks, int64_t outer, int64_t inner_bytes,
                               int dtype, hapmi_stream_t stream);
 /* The same with the kept elements multiplied by `scale`: the backward of F.relu followed by F.dropout(p)
- * (hap.rs:1417, 1464; the FFN's activation and the dropout behind it, models.py:116), given the DROPPED forward
+ * (hap.rs:1417, 1464; the FFN's activation and the dropout behind it: `self.dropout` in `_ff_block` of torch's
+ * nn.TransformerEncoderLayer, torch:nn/modules/transformer.py:981, which models.py:74, 100 build), given the DROPPED forward
  * output as fwd_out -- it is positive exactly where relu passed the element and dropout kept it -- and
  * scale = 1 / (1 - p); no random numbers are needed backward. */
 int hapmi_split_rows_relu_bwd_scaled(const void *src, const void *fwd_out, void *const *pieces_host,
@@ -143,11 +146,6 @@ int hapmi_ragged_reduce_multi(const void *const *contribs_host, int n_ranks, voi
 /* collectives.py:9-12 padded() for several shards in ONE launch: dsts[i][outer, padded_len, inner] <- srcs[i][outer, lengths[i], inner]. */
 int hapmi_pad_rows_multi(const void *const *srcs_host, void *const *dsts_host, const int64_t *lengths_host, int n_shards,
                          int64_t outer, int64_t padded_len, int64_t inner_bytes, hapmi_stream_t stream);
-
-/* Tuning hook for measurements of the kernels above: reduce_variant bit 0 / 1 = non-temporal loads / stores,
- * bit 2 = two vectors per thread, bit 3 = non-temporal loads in the plain 16-byte segment copy; grid_shift caps the
- * grid at 4096 << shift blocks; -1 = defaults (reduce: non-temporal loads, two vectors per thread; copy: plain; 2). */
-int hapmi_ragged_tuning(int reduce_variant, int grid_shift);
 
 /* ---- GEMM: F.linear (hap.rs:1032) and the expert einsums (hap.rs:2273) --
  * C[z] = op(A[z]) * op(B[z]) (+ bias[N]) (act) (+ C[z] if accumulate)
@@ -223,7 +221,7 @@ typedef struct {
     const hapmi_gemm_segments *const *B_segments_list;
     int a_relu, b_relu;
     /* F.dropout(., p) behind the activation (hap.rs:1464 after 1417: the dropout that follows the FFN's activation,
-     * models.py:116), applied by the epilogue with the decisions hapmi_dropout takes for C as a whole under the same
+     * torch:nn/modules/transformer.py:981 in the layers built at models.py:74, 100), applied by the epilogue with the decisions hapmi_dropout takes for C as a whole under the same
      * p, RNG state and stream id.  One contiguous problem (transA = 0, transB = 1, batch 1, ldc = N, N even), no
      * accumulate, no pieces; the reduction is not split.  drop_state = NULL: off */
     const int64_t *drop_state;
@@ -242,9 +240,7 @@ int hapmi_gemm(const hapmi_gemm_args *args_host, hapmi_stream_t stream);
  * Tuning hook for measurements: force tile configuration `tile_config` (block tile / waves: 0: 128x128 / 2x2,
  * 1: 256x256 / 2x4, 2: 384x192 / 4x2, 3: 192x256 / 2x4, 4: 256x192 / 4x2, 5: 256x128 / 4x2, 6: 128x256 / 2x4,
  * 7: 192x128 / 2x4, 8: 256x128 / 2x2, 9: 128x192 / 4x2, 10: 64x64 / 2x2, 11: 64x128 / 2x2; 5..9 keep three
- * k-tiles in LDS (two in flight); 1..9 take bf16 operands only, 10 and 11 float32 operands only; 12 is a measurement
- * build of 7 for bf16 operands and results with transA = 0: it moves the operands of every k-tile into LDS
- * but multiplies nothing (the result is zeros), so its time is the cost of the operand movement alone; a configuration
+ * k-tiles in LDS (two in flight); 1..9 take bf16 operands only, 10 and 11 float32 operands only; a configuration
  * that does not fit the call's operand type is ignored; -1 = automatic) and `k_splits` (0 = automatic). */
 int hapmi_gemm_tuning(int tile_config, int k_splits);
 
@@ -266,7 +262,8 @@ int hapmi_add_layernorm_fwd(const void *x, const void *res, void *y, float *rstd
 int hapmi_layernorm_bwd(const void *dy, const void *y, const float *rstd, const void *dx_add, void *dx,
                         int64_t rows, int64_t width, int dtype, hapmi_stream_t stream);
 /* F.dropout(x, p) -> operator.add(., res) -> F.layer_norm in one pass (hap.rs:1464, 1515, 1653: the residual
- * connections of the encoder layer, models.py:112-117): y = LN(dropout(x) + res).  The keep decisions are those
+ * connections of the encoder layer: dropout1 / dropout2 and norm1 / norm2 of torch's nn.TransformerEncoderLayer,
+ * torch:nn/modules/transformer.py:952-956, 977, 982, in the layers built at models.py:74, 100): y = LN(dropout(x) + res).  The keep decisions are those
  * hapmi_dropout takes for x as a whole [rows, width] tensor under the same p, RNG state and stream id.  Backward
  * gives dx (the gradient of the sum: res's) and dx_drop = dropout's backward of dx (x's), regenerating the mask;
  * dx_drop must not alias dx. */
@@ -291,7 +288,7 @@ int hapmi_softmax_bwd(const void *dp, const void *p, void *ds, int64_t rows, int
  * F.multi_head_attention_forward, hap.rs:1301-1327; bf16 only, head_dim 64):
  * qkv[b, S, 3*H*64] -> out[b, S, H*64]; lse[b, H, S] float32 (log-sum-exp of every score row) is kept for
  * backward; mask is NULL or an additive float32 [S, S].  causal != 0 (mask must then be NULL) stands for the
- * mask torch.triu(full(-inf), diagonal=1) that the language models register as src_mask (models.py:76): the
+ * mask torch.triu(full(-inf), diagonal=1) that the language models register as src_mask (models.py:72, 97): the
  * same result without reading a mask, and the key tiles above the diagonal are skipped.  Backward writes
  * dqkv[b, S, 3*H*64] completely; delta_ws is float32 scratch of b*H*S elements. */
 int hapmi_attention_fwd(const void *qkv, const float *mask, int causal, void *out, float *lse, int64_t b, int64_t S,
@@ -471,7 +468,9 @@ int hapmi_sumsq(const float *g, int64_t n, float *out, float *workspace, int64_t
  * forbid it.  The partial sums go to a 256 KiB array inside the library's device code (each GPU the library runs
  * on holds its copy until the process ends), so n is limited to 2^30 elements (HAPMI_ELIMIT beyond).  Calls that
  * overlap on one GPU (different streams) share that array and race; calls on one stream are ordered and give the
- * bits of hapmi_sumsq. */
+ * bits of hapmi_sumsq.  The array used is that of the stream's device (the current device for the null stream);
+ * hapmi_init() must have run with that device current (HAPMI_EINVAL otherwise), so that this call is nothing but
+ * kernel launches on `stream` and may be recorded by a stream capture. */
 int hapmi_sumsq_static(const float *g, int64_t n, float *out, hapmi_stream_t stream);
 /* torch.nn.utils.clip_grad_norm_ coefficient (worker.py:74): coef = min(1, max_norm / (sqrt(sumsq) + 1e-6)) */
 int hapmi_clip_coef(const float *sumsq, float max_norm, float *coef, hapmi_stream_t stream);
