@@ -40,9 +40,12 @@ WORKLOADS = {
     "vit": ("ViT-L/16: 24L d1024 h16 FFN4096 197 tokens batch 48/128 1000 classes Adam", "bf16"),
     "moe": ("MoE LM: 12L d768 h12 16 experts (5 local) top-2 C=80 seq512 batch 16 vocab33280 Adam", "bf16"),
 }
+# capacity slots per expert of the MoE workload: ceil(512 / 16 * 2.5) = 80 by the reference's rule (config.py:25-28
+# doubles the capacity factor 1.25 for models whose name ends in `moe`); 40 if the factor is taken as it stands
+MOE_CAPACITY = 80
 
 
-def build_workload(name, layers_override=None, attn="batch", zero=False, dropout=0.0):
+def build_workload(name, layers_override=None, attn="batch", zero=False, dropout=0.0, capacity=None):
     import torch
     import hap_amd
     from hap_amd import models
@@ -78,7 +81,7 @@ def build_workload(name, layers_override=None, attn="batch", zero=False, dropout
     elif name == "moe":
         L = layers_override or 12
         B, S, V = 16, 512, 33280
-        model = models.RMoE(V, S, 768, 12, 3072, 0.0, 16, 80, L, causal=True)
+        model = models.RMoE(V, S, 768, 12, 3072, 0.0, 16, capacity or MOE_CAPACITY, L, causal=True)
         ids = torch.randint(0, V, (B, S + 1), generator=g)
         x, y = ids[:, :-1].contiguous(), ids[:, 1:].contiguous()
         plan = hap_amd.ShardingPlan([RATIOS_E], 0, ffn="batch")
@@ -156,6 +159,9 @@ def main():
     ap.add_argument("--dropout", type=float, default=0.0,
                     help="dropout probability of the model (the reference's default is 0.1, config.py:33; the headline "
                          "configuration names none and runs with 0)")
+    ap.add_argument("--moe-capacity", type=int, default=MOE_CAPACITY,
+                    help="moe workload only: capacity slots per expert (80 = the reference's rule, config.py:25-28; "
+                         "40 = capacity factor 1.25 taken as it stands)")
     ap.add_argument("--zero", action="store_true",
                     help="bert workload only: parameters stored as dim-0 shards and gathered at use")
     ap.add_argument("--gemm-table", default=None,
@@ -199,6 +205,9 @@ def main():
                                                        share_shapes=args.shared_peer_buffers, dropout=0.1))
         for name in ("lm", "vit", "moe"):
             extra[name] = _brief(measure(name, args, max(5, args.steps // 2), 3, share_shapes=args.shared_peer_buffers))
+        # the MoE workload with the capacity factor 1.25 taken as it stands (C = 40) instead of the reference's doubled one
+        extra["moe_C40"] = _brief(measure("moe", args, max(5, args.steps // 2), 3, share_shapes=args.shared_peer_buffers,
+                                          capacity=40))
         from hap_amd import ragged_bench
         rg = ragged_bench.run(20, 5, False)
         extra["ragged"] = {"workload": rg["config"]["workload"], "GBps": rg["value"], "ms_per_pass": rg["ms_per_step"],
@@ -242,9 +251,10 @@ def _write_gemm_table(path, report, desc):
                 f"{total_flop / total_us / 1e6:.0f} TFLOP/s (cold single launches)\n")
 
 
-def measure(workload, args, steps, warmup, share_shapes=True, dropout=None):
+def measure(workload, args, steps, warmup, share_shapes=True, dropout=None, capacity=None):
     """One workload: compile, autotune the GEMM plans (untimed), warm up, time `steps` steps, bracket the GEMMs.
-    ``dropout``: the model's dropout probability (default: the command line's)."""
+    ``dropout``: the model's dropout probability (default: the command line's); ``capacity``: slots per expert of the
+    MoE workload (default: --moe-capacity)."""
     import ctypes
     import gc
 
@@ -255,8 +265,11 @@ def measure(workload, args, steps, warmup, share_shapes=True, dropout=None):
 
     desc, dtype = WORKLOADS[workload]
     bert = workload == "bert"
+    if workload == "moe":
+        capacity = capacity or args.moe_capacity
+        desc = desc.replace(f"C={MOE_CAPACITY}", f"C={capacity}")
     gm, x, y, meta = build_workload(workload, attn=args.attn if bert else "batch", zero=args.zero and bert,
-                                    dropout=args.dropout if dropout is None else dropout)
+                                    dropout=args.dropout if dropout is None else dropout, capacity=capacity)
     wire = hap_amd.SyntheticWire(seed=39, scale=1.0, grad_scale=1e-3, share_shapes=share_shapes)
     ex = hap_amd.compile_program(gm, [x, y], dtype=dtype, wire=wire, rank=0, world_size=len(meta["ratios"]),
                                  overlap_wgrad=args.overlap, relu_mask_in_dgrad=not args.no_relu_mask_in_dgrad,

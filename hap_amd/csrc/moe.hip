@@ -5,98 +5,76 @@
 namespace {
 
 constexpr int GATE_THREADS = 256;
-constexpr int GATE_WAVES = GATE_THREADS / 64;
 constexpr int GATE_MAX_E = 64;
 
-// One block per batch row.  Pass A: softmax, top-2 (ties -> lower expert index), 1-based position of every
-// first choice among the earlier first choices of the same expert.  Pass B: positions of the second choices,
-// offset per expert by the SUM of its first-choice positions (n(n+1)/2), as the reference adds
-// sum(position_in_expert[:, :, 0, :]) rather than the count.  A position >= C drops the choice (slot 0).
-// TOP_K = 1 is switch gating: pass A only; the second entry of every record is written as a dropped choice
+// Gating runs as two launches.  gate_choice_kernel, one thread per token: softmax over the experts, the two largest
+// probabilities (ties -> lower expert index) as index / gate records.  gate_position_kernel, one wave per (batch
+// row, expert): walks the row's S tokens in order, 64 at a time, and gives every token that chose this expert its
+// 1-based position among the row's earlier choices of the same expert (a ballot and a population count per 64
+// tokens); first the first choices, then the second choices, offset by the SUM of the expert's first-choice positions
+// (n(n+1)/2), as the reference adds sum(position_in_expert[:, :, 0, :]) rather than the count.  A position >= C drops
+// the choice (slot 0).  B * E waves work in parallel where the positions of a row are a serial count.
+// TOP_K = 1 is switch gating: first choices only; the second entry of every record is written as a dropped choice
 // (gate 0, slot 0), so the dispatch / combine kernels and the gate backward serve both kinds of record.
 template <int TOP_K>
-__global__ __launch_bounds__(GATE_THREADS) void top2_gate_kernel(const float *logits, float *probs, int32_t *index,
-                                                               int32_t *slot, float *gate, int32_t *token_of_slot,
-                                                               int S, int E, int C) {
-    __shared__ int wave_cnt[GATE_WAVES][GATE_MAX_E];
-    __shared__ long long run[GATE_MAX_E];
-    __shared__ long long offset1[GATE_MAX_E];
-    const int b = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+__global__ __launch_bounds__(GATE_THREADS) void gate_choice_kernel(const float *logits, float *probs, int32_t *index,
+                                                                 int32_t *slot, float *gate, int64_t n_tok, int E) {
+    const int64_t tok = (int64_t)blockIdx.x * GATE_THREADS + threadIdx.x;
+    if (tok >= n_tok) return;
+    const float *lg = logits + tok * E;
+    float m = -INFINITY;
+    for (int e = 0; e < E; ++e) m = fmaxf(m, lg[e]);
+    float sum = 0.f;
+    for (int e = 0; e < E; ++e) sum += expf(lg[e] - m);
+    const float inv = 1.0f / sum;
+    int i0 = 0, i1 = -1;
+    float p0 = -1.f, p1 = -1.f;
+    for (int e = 0; e < E; ++e) {
+        const float pe = expf(lg[e] - m) * inv;
+        probs[tok * E + e] = pe;
+        if (pe > p0) {
+            p1 = p0; i1 = i0;
+            p0 = pe; i0 = e;
+        } else if (pe > p1) {
+            p1 = pe; i1 = e;
+        }
+    }
+    if (i1 < 0) i1 = (i0 + 1) % E;      // only with NaN logits; gate stays -1, so the choice is dropped
+    index[tok * 2 + 0] = i0;
+    index[tok * 2 + 1] = i1;
+    gate[tok * 2 + 0] = p0;
+    gate[tok * 2 + 1] = TOP_K == 2 ? p1 : 0.f;
+    if (TOP_K == 1) slot[tok * 2 + 1] = 0;
+}
+
+template <int TOP_K>
+__global__ __launch_bounds__(GATE_THREADS) void gate_position_kernel(const int32_t *index, const float *gate, int32_t *slot,
+                                                                   int32_t *token_of_slot, int B, int S, int E, int C) {
+    const int lane = threadIdx.x & 63;
+    const int64_t pair = (int64_t)blockIdx.x * (GATE_THREADS / 64) + (threadIdx.x >> 6);      // (b, e), wave-uniform
+    if (pair >= (int64_t)B * E) return;
+    const int b = (int)(pair / E), e = (int)(pair % E);
     const unsigned long long lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
-
-    for (int i = tid; i < E * C; i += GATE_THREADS) token_of_slot[(int64_t)b * E * C + i] = -1;
-    for (int e = tid; e < E; e += GATE_THREADS) run[e] = 0;
-    __syncthreads();
-
+    int32_t *tos = token_of_slot + ((int64_t)b * E + e) * C;
+    for (int c = lane; c < C; c += 64) tos[c] = -1;
+    long long run = 0, offset = 0;
+#pragma unroll
     for (int pass = 0; pass < TOP_K; ++pass) {
-        for (int s0 = 0; s0 < S; s0 += GATE_THREADS) {
-            const int s = s0 + tid;
-            const bool valid = s < S;
-            const int64_t tok = (int64_t)b * S + s;
-            int my = -1;
-            if (valid) {
-                if (pass == 0) {
-                    const float *lg = logits + tok * E;
-                    float m = -INFINITY;
-                    for (int e = 0; e < E; ++e) m = fmaxf(m, lg[e]);
-                    float sum = 0.f;
-                    for (int e = 0; e < E; ++e) sum += expf(lg[e] - m);
-                    const float inv = 1.0f / sum;
-                    int i0 = 0, i1 = -1;
-                    float p0 = -1.f, p1 = -1.f;
-                    for (int e = 0; e < E; ++e) {
-                        const float pe = expf(lg[e] - m) * inv;
-                        probs[tok * E + e] = pe;
-                        if (pe > p0) {
-                            p1 = p0; i1 = i0;
-                            p0 = pe; i0 = e;
-                        } else if (pe > p1) {
-                            p1 = pe; i1 = e;
-                        }
-                    }
-                    if (i1 < 0) i1 = (i0 + 1) % E;      // only with NaN logits; gate stays -1, so the choice is dropped
-                    index[tok * 2 + 0] = i0;
-                    index[tok * 2 + 1] = i1;
-                    gate[tok * 2 + 0] = p0;
-                    gate[tok * 2 + 1] = TOP_K == 2 ? p1 : 0.f;
-                    if (TOP_K == 1) slot[tok * 2 + 1] = 0;
-                    my = i0;
-                } else {
-                    my = index[tok * 2 + 1];
-                }
+        for (int s0 = 0; s0 < S; s0 += 64) {
+            const int s = s0 + lane;
+            const int64_t rec = ((int64_t)b * S + s) * 2 + pass;
+            const bool mine = s < S && index[rec] == e;
+            const unsigned long long bal = __ballot(mine);
+            if (mine) {
+                const long long pos = run + __popcll(bal & lt_mask) + 1 + offset;
+                const int sl = (pos < C && gate[rec] > 0.f) ? (int)pos : 0;
+                slot[rec] = sl;
+                if (sl > 0) tos[sl] = s;             // slots 1 .. C - 1 of this wave's own (b, e): behind its own fill
             }
-            int in_wave = 0;
-            for (int e = 0; e < E; ++e) {
-                const unsigned long long bal = __ballot(my == e);
-                if (my == e) in_wave = __popcll(bal & lt_mask);
-                if (lane == 0) wave_cnt[wave][e] = __popcll(bal);
-            }
-            __syncthreads();
-            if (valid) {
-                long long pos = run[my] + in_wave + 1;
-                for (int w = 0; w < wave; ++w) pos += wave_cnt[w][my];
-                if (pass == 1) pos += offset1[my];
-                const float gv = gate[tok * 2 + pass];
-                const int sl = (pos < C && gv > 0.f) ? (int)pos : 0;
-                slot[tok * 2 + pass] = sl;
-                if (sl > 0) token_of_slot[((int64_t)b * E + my) * C + sl] = s;
-            }
-            __syncthreads();
-            for (int e = tid; e < E; e += GATE_THREADS) {
-                long long add = 0;
-                for (int w = 0; w < GATE_WAVES; ++w) add += wave_cnt[w][e];
-                run[e] += add;
-            }
-            __syncthreads();
+            run += __popcll(bal);
         }
-        if (pass == 0) {
-            for (int e = tid; e < E; e += GATE_THREADS) {
-                const long long n = run[e];
-                offset1[e] = n * (n + 1) / 2;
-                run[e] = 0;
-            }
-            __syncthreads();
-        }
+        offset = run * (run + 1) / 2;
+        run = 0;
     }
 }
 
@@ -302,8 +280,10 @@ extern "C" int hapmi_top2_gate(const float *logits, float *probs, int32_t *index
     HAPMI_REQUIRE(S < (1ll << 30) && B < (1ll << 31) && E * C < (1ll << 31), HAPMI_ELIMIT, "top2_gate: shape too large");
     if (B == 0) return HAPMI_OK;
     HAPMI_REQUIRE(logits && probs && index && slot && gate && token_of_slot, HAPMI_EINVAL, "top2_gate: null pointer");
-    hipLaunchKernelGGL(top2_gate_kernel<2>, dim3((unsigned)B), dim3(GATE_THREADS), 0, (hipStream_t)stream, logits, probs,
-                       index, slot, gate, token_of_slot, (int)S, (int)E, (int)C);
+    hipLaunchKernelGGL(gate_choice_kernel<2>, dim3((unsigned)hapmi_cdiv(B * S, GATE_THREADS)), dim3(GATE_THREADS), 0,
+                       (hipStream_t)stream, logits, probs, index, slot, gate, B * S, (int)E);
+    hipLaunchKernelGGL(gate_position_kernel<2>, dim3((unsigned)hapmi_cdiv(B * E, GATE_THREADS / 64)), dim3(GATE_THREADS), 0,
+                       (hipStream_t)stream, index, gate, slot, token_of_slot, (int)B, (int)S, (int)E, (int)C);
     HAPMI_CHECK_LAUNCH("top2_gate");
     return HAPMI_OK;
 }
@@ -316,8 +296,10 @@ extern "C" int hapmi_switch_gate(const float *logits, float *probs, int32_t *ind
     HAPMI_REQUIRE(S < (1ll << 30) && B < (1ll << 31) && E * C < (1ll << 31), HAPMI_ELIMIT, "switch_gate: shape too large");
     if (B == 0) return HAPMI_OK;
     HAPMI_REQUIRE(logits && probs && index && slot && gate && token_of_slot, HAPMI_EINVAL, "switch_gate: null pointer");
-    hipLaunchKernelGGL(top2_gate_kernel<1>, dim3((unsigned)B), dim3(GATE_THREADS), 0, (hipStream_t)stream, logits, probs,
-                       index, slot, gate, token_of_slot, (int)S, (int)E, (int)C);
+    hipLaunchKernelGGL(gate_choice_kernel<1>, dim3((unsigned)hapmi_cdiv(B * S, GATE_THREADS)), dim3(GATE_THREADS), 0,
+                       (hipStream_t)stream, logits, probs, index, slot, gate, B * S, (int)E);
+    hipLaunchKernelGGL(gate_position_kernel<1>, dim3((unsigned)hapmi_cdiv(B * E, GATE_THREADS / 64)), dim3(GATE_THREADS), 0,
+                       (hipStream_t)stream, index, gate, slot, token_of_slot, (int)B, (int)S, (int)E, (int)C);
     HAPMI_CHECK_LAUNCH("switch_gate");
     return HAPMI_OK;
 }

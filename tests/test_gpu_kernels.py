@@ -45,7 +45,7 @@ def test_gemm_layouts_and_ragged_edges(cuda, dtype, tA, tB, M, N, K):
     opA = A.double().t() if tA else A.double()
     opB = B.double().t() if tB else B.double()
     want = opA @ opB + bias.double()
-    close(C[:, :N], want, dtype, scale=2.0)
+    close(C[:, :N], want, dtype)
     assert (C[:, N:] == 0).all()
 
 
@@ -59,11 +59,11 @@ def test_gemm_epilogue_accumulate_alpha_act_batch(cuda, dtype):
     C = C0.clone().to(cuda)                                   # float32 output from either input type
     ops.gemm(A.to(cuda), B.to(cuda), C, M, N, K, alpha=0.5, accumulate=True, batch1=b1, batch2=b2,
              strideA=(b2 * M * K, M * K), strideB=(b2 * K * N, K * N), strideC=(b2 * M * N, M * N))
-    close(C, C0.double() + 0.5 * (A.double() @ B.double()), dtype, scale=2.0)
+    close(C, C0.double() + 0.5 * (A.double() @ B.double()), dtype)
     for act, fn in (("relu", torch.relu), ("gelu", F.gelu)):
         out = torch.empty(M, N, dtype=dtype, device=cuda)
         ops.gemm(A[0, 0].to(cuda), B[0, 0].to(cuda), out, M, N, K, act=act)
-        close(out, fn(A[0, 0].double() @ B[0, 0].double()), dtype, scale=2.0)
+        close(out, fn(A[0, 0].double() @ B[0, 0].double()), dtype)
 
 
 def test_gemm_refuses_misaligned(cuda):
@@ -88,10 +88,10 @@ def test_add_layernorm_forward_backward(cuda, dtype, rows, width):
     dx = torch.empty_like(y)
     ops.layernorm_bwd(dy.to(cuda), y, rstd, None, dx)
     want.backward(dy.double())
-    close(dx, s.grad, dtype, scale=2.0)
+    close(dx, s.grad, dtype)
     dx2 = torch.empty_like(y)
     ops.layernorm_bwd(dy.to(cuda), y, rstd, dy.to(cuda), dx2)
-    close(dx2, s.grad + dy.double(), dtype, scale=2.0)
+    close(dx2, s.grad + dy.double(), dtype)
     # without a residual
     ops.add_layernorm_fwd(x.to(cuda), None, y, rstd)
     close(y, F.layer_norm(x.double(), (width,)), dtype)
@@ -115,7 +115,7 @@ def test_softmax_with_mask_forward_backward(cuda, dtype, S, ld):
     ops.softmax_bwd(ds, p, ds, rows, S, ld)
     pw = p[:, :S].double().cpu()
     wantd = pw * (dp[:, :S].double() - (dp[:, :S].double() * pw).sum(-1, keepdim=True))
-    close(ds[:, :S], wantd, dtype, scale=2.0)
+    close(ds[:, :S], wantd, dtype)
 
 
 @pytest.mark.parametrize("dtype", DT)
@@ -283,11 +283,11 @@ def test_gemm_every_tile_configuration_and_layout(cuda, cfg, tA, tB):
             for out_dtype in (torch.bfloat16, torch.float32):
                 C = torch.full((M, N), float("nan"), dtype=out_dtype, device=cuda)
                 ops.gemm(A.to(cuda), B.to(cuda), C, M, N, K, transA=bool(tA), transB=bool(tB), bias=bias.to(cuda))
-                close(C, want, torch.bfloat16, scale=2.0)
+                close(C, want, torch.bfloat16)
             start = torch.randn(M, N, generator=g)
             C = start.clone().to(cuda)
             ops.gemm(A.to(cuda), B.to(cuda), C, M, N, K, transA=bool(tA), transB=bool(tB), accumulate=True)
-            close(C, want - bias.double() + start.double(), torch.bfloat16, scale=2.0)
+            close(C, want - bias.double() + start.double(), torch.bfloat16)
     finally:
         lib().hapmi_gemm_tuning(-1, 0)
 
@@ -316,7 +316,7 @@ def test_gemm_scale_bias_activation_in_every_epilogue(cuda, cfg, act):
                         C = torch.full((M, N), float("nan"), dtype=out_dtype, device=cuda)
                         ops.gemm(A.to(cuda), B.to(cuda), C, M, N, K, transB=True, alpha=alpha,
                                  bias=bias.to(cuda) if with_bias else None, act=act if act != "none" else None)
-                        close(C, want, torch.bfloat16, scale=2.0)
+                        close(C, want, torch.bfloat16)
     finally:
         lib().hapmi_gemm_tuning(-1, 0)
 
@@ -339,11 +339,11 @@ def test_gemm_float32_tile_configurations_and_layouts(cuda, cfg, tA, tB):
             for out_dtype in (torch.float32, torch.bfloat16):
                 C = torch.full((M, N), float("nan"), dtype=out_dtype, device=cuda)
                 ops.gemm(A.to(cuda), B.to(cuda), C, M, N, K, transA=bool(tA), transB=bool(tB), bias=bias.to(cuda))
-                close(C, want, out_dtype, scale=2.0)
+                close(C, want, out_dtype)
             start = torch.randn(M, N, generator=g)
             C = start.clone().to(cuda)
             ops.gemm(A.to(cuda), B.to(cuda), C, M, N, K, transA=bool(tA), transB=bool(tB), accumulate=True)
-            close(C, want - bias.double() + start.double(), torch.float32, scale=2.0)
+            close(C, want - bias.double() + start.double(), torch.float32)
     finally:
         lib().hapmi_gemm_tuning(-1, 0)
 
@@ -366,10 +366,10 @@ def test_gemm_split_k_and_tile_configs(cuda, dtype, cfg):
             lib().hapmi_gemm_tuning(cfg, splits)
             C = C0.clone().to(cuda)
             ops.gemm(A.to(cuda), B.to(cuda), C, M, N, K, transA=True, bias=bias.to(cuda), accumulate=True, workspace=ws)
-            close(C, want + C0.double(), dtype, scale=2.0)
+            close(C, want + C0.double(), dtype)
             out = torch.empty(M, N, dtype=dtype, device=cuda)
             ops.gemm(A.to(cuda), B.to(cuda), out, M, N, K, transA=True, bias=bias.to(cuda), act="relu", workspace=ws)
-            close(out, torch.relu(want), dtype, scale=2.0)
+            close(out, torch.relu(want), dtype)
     finally:
         lib().hapmi_gemm_tuning(-1, 0)
 
@@ -396,7 +396,7 @@ def test_gemm_row_sums_of_a_transposed_operand(cuda, dtype, cfg, tB):
             C = torch.empty(M, N, dtype=torch.float32, device=cuda)
             rs = start.clone().to(cuda)
             ops.gemm(A.to(cuda), B.to(cuda), C, M, N, K, transA=True, transB=tB, workspace=ws, a_rowsum=rs)
-            close(C, want_c, dtype, scale=2.0)
+            close(C, want_c, dtype)
             tol = 1e-5 if dtype == torch.float32 else 1e-4       # float32 sums of exactly represented inputs
             torch.testing.assert_close(rs.cpu().double(), want_rs, rtol=tol, atol=tol * K ** 0.5)
     finally:
@@ -429,7 +429,7 @@ def test_gemm_relu_mask_on_the_result(cuda, dtype, out_dtype, cfg, splits, accum
         lib().hapmi_gemm_tuning(cfg, splits)
         C = start.clone().to(cuda)
         ops.gemm(A.to(cuda), B.to(cuda), C, M, N, K, workspace=ws, accumulate=accumulate, relu_mask=mask.to(cuda))
-        close(C, want, dtype if out_dtype == torch.float32 else out_dtype, scale=2.0)
+        close(C, want, dtype if out_dtype == torch.float32 else out_dtype)
         assert (C.cpu()[mask == 0] == (start[mask == 0] if accumulate else 0)).all()
     finally:
         lib().hapmi_gemm_tuning(-1, 0)
@@ -448,7 +448,7 @@ def test_gemm_relu_mask_with_a_batch(cuda, dtype):
     ops.gemm(A.to(cuda), B.to(cuda), C, M, N, K, transB=True, batch1=E, strideA=(M * K, 0), strideB=(N * K, 0),
              strideC=(M * N, 0), relu_mask=mask.to(cuda))
     want = torch.einsum("emk,enk->emn", A.double(), B.double()) * (mask > 0)
-    close(C, want, dtype, scale=2.0)
+    close(C, want, dtype)
     assert (C.cpu()[mask == 0] == 0).all()
 
 
@@ -474,7 +474,7 @@ def test_gemm_accumulates_onto_a_separate_addend(cuda, dtype, out_dtype, cfg, sp
         C = torch.full((M, N), 7.0, dtype=out_dtype, device=cuda)
         ops.gemm(A, B, C, M, N, K, workspace=ws, accumulate=True, addend=R)
         assert torch.equal(C, in_place) and torch.equal(R, keep)
-        close(C, A.double().cpu() @ B.double().cpu() + keep.double().cpu(), dtype if out_dtype == torch.float32 else out_dtype, scale=2.0)
+        close(C, A.double().cpu() @ B.double().cpu() + keep.double().cpu(), dtype if out_dtype == torch.float32 else out_dtype)
     finally:
         lib().hapmi_gemm_tuning(-1, 0)
     with pytest.raises(TypeError):
@@ -504,7 +504,7 @@ def test_gemm_group_of_weight_gradients_behind_pointer_lists(cuda, cfg, n, accum
     for z in range(n):
         assert torch.equal(W[z], single[z]), z
         want = dY[z].double().t() @ X[z].double() + (start[z].double() if accumulate else 0)
-        close(W[z], want.cpu(), torch.bfloat16, scale=2.0)
+        close(W[z], want.cpu(), torch.bfloat16)
         if b[z] is not None:
             torch.testing.assert_close(b[z].cpu(), dY[z].float().sum(0).cpu(), rtol=1e-4, atol=1e-3)
     with pytest.raises(ValueError):
@@ -780,11 +780,11 @@ def test_gemm_a_in_pieces_along_k_with_relu(cuda, cfg):
             want = src @ W.double().t() + bias.double()
             C = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=cuda)
             ops.gemm(None, W.to(cuda), C, M, N, K, transB=True, bias=bias.to(cuda), a_segments=pieces, a_relu=relu)
-            close(C, want, torch.bfloat16, scale=2.0)
+            close(C, want, torch.bfloat16)
         # relu on a plain operand
         C = torch.full((M, N), float("nan"), dtype=torch.float32, device=cuda)
         ops.gemm(act.to(cuda), W.to(cuda), C, M, N, K, transB=True, a_relu=True)
-        close(C, torch.relu(act.double()) @ W.double().t(), torch.bfloat16, scale=2.0)
+        close(C, torch.relu(act.double()) @ W.double().t(), torch.bfloat16)
     finally:
         lib().hapmi_gemm_tuning(-1, 0)
 
@@ -810,16 +810,16 @@ def test_gemm_result_and_operand_in_pieces_along_n(cuda, cfg, lengths):
     try:
         lib().hapmi_gemm_tuning(cfg, 1)
         ops.gemm(dy.to(cuda), W.to(cuda), None, rows, F_, d_out, c_segments=outs, mask_segments=fwd_pieces)
-        close(torch.cat(outs, 1), want_dx, torch.bfloat16, scale=2.0)
+        close(torch.cat(outs, 1), want_dx, torch.bfloat16)
         outs2 = [torch.full((rows, l), float("nan"), dtype=torch.bfloat16, device=cuda) for l in lengths]
         ops.gemm(dy.to(cuda), W.to(cuda), None, rows, F_, d_out, c_segments=outs2)
-        close(torch.cat(outs2, 1), dy.double() @ W.double(), torch.bfloat16, scale=2.0)
+        close(torch.cat(outs2, 1), dy.double() @ W.double(), torch.bfloat16)
         # weight gradient [d_out, F] = dY^T relu(pre), bias gradient = column sums of dY
         want_dw = dy.double().t() @ torch.relu(pre.double())
         gw = torch.full((d_out, F_), float("nan"), device=cuda)
         gb = torch.zeros(d_out, device=cuda)
         ops.gemm(dy.to(cuda), None, gw, d_out, F_, rows, transA=True, b_segments=fwd_pieces, b_relu=True, a_rowsum=gb)
-        close(gw, want_dw, torch.bfloat16, scale=2.0)
+        close(gw, want_dw, torch.bfloat16)
         torch.testing.assert_close(gb.cpu().double(), dy.double().sum(0), rtol=1e-4, atol=1e-3)
         # three layers in one launch
         pres = [torch.randn(rows, F_, generator=g).bfloat16() for _ in range(3)]
@@ -828,7 +828,7 @@ def test_gemm_result_and_operand_in_pieces_along_n(cuda, cfg, lengths):
         ops.gemm_group([t.to(cuda) for t in dys], [_pieces(t, lengths, cuda) for t in pres],
                        gws, d_out, F_, rows, transA=True, b_relu=True)
         for z in range(3):
-            close(gws[z], dys[z].double().t() @ torch.relu(pres[z].double()), torch.bfloat16, scale=2.0)
+            close(gws[z], dys[z].double().t() @ torch.relu(pres[z].double()), torch.bfloat16)
     finally:
         lib().hapmi_gemm_tuning(-1, 0)
 

@@ -196,14 +196,16 @@ def test_config5_shapes_round_trip_and_reduce(cuda):
     for a, x, s in zip(again, shards, S):
         assert torch.equal(a[:s], x)
     # reduce-scatter layout: 8 virtual ranks each hold a full [total, 4096] tensor
-    fulls = [torch.randn(total, 4096, generator=g).bfloat16().to(cuda) for _ in range(8)]
+    fulls_cpu = [torch.randn(total, 4096, generator=g).bfloat16() for _ in range(8)]
+    fulls = [f.to(cuda) for f in fulls_cpu]
     off = 0
-    acc = torch.zeros(total, 4096, dtype=torch.float32, device=cuda)
-    for f in fulls:
+    acc = torch.zeros(total, 4096, dtype=torch.float32)                         # the reference sum: on the CPU
+    for f in fulls_cpu:
         acc += f.float()                                                        # same rank order, float32
+    want = acc.bfloat16()
     for r, s in enumerate(S):
         out = ops.ragged_reduce(fulls, 0, off, s)
-        assert torch.equal(out, acc[off:off + s].bfloat16())
+        assert torch.equal(out.cpu(), want[off:off + s])
         off += s
 
 
