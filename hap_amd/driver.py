@@ -9,7 +9,9 @@ gradients (worker.py:74) -> Adam(lr 5e-4) step (worker.py:47, config.py:48), wit
 * every iteration its wall-clock duration and mean / standard deviation over the last ``avg_iter`` iterations
   (worker.py:78-83, config.py:50-52).
 
-``report`` receives the formatted lines (default: stderr, as the reference's eprint).
+``report`` receives the formatted lines (default: stderr, as the reference's eprint); ``after_backward(it,
+executor)``, if given, is called between backward and the optimizer step (the reference has no such hook; it lets a
+caller log or record the step's gradients).
 """
 from __future__ import annotations
 
@@ -36,7 +38,8 @@ def mean_std(values: List[float]):
 def train_loop(executor, x: torch.Tensor, y: torch.Tensor, *, batch_size: int, seqlen: int, run_iter: int = RUN_ITER,
                log_iter: int = LOG_ITER, avg_iter: int = AVG_ITER, lr: float = LR, clip_grad_norm: Optional[float] = CLIP,
                optimizer: str = "adam", report_per_iter_time: bool = True,
-               report: Callable[[str], None] = _eprint) -> dict:
+               report: Callable[[str], None] = _eprint,
+               after_backward: Optional[Callable[[int, object], None]] = None) -> dict:
     executor.configure_optimizer(kind=optimizer, lr=lr, clip_grad_norm=clip_grad_norm)
     executor.load_inputs(x, y)
     times: List[float] = []
@@ -52,6 +55,8 @@ def train_loop(executor, x: torch.Tensor, y: torch.Tensor, *, batch_size: int, s
             report(f"loss (log ppl) {it}: {total / log_iter:.3f}, wall clock: {time.time() - start:.3f}")
             total = 0.0
         executor.backward()
+        if after_backward is not None:                 # an observer of the step's gradients (before clipping)
+            after_backward(it, executor)
         executor.step()
         if report_per_iter_time:
             torch.cuda.synchronize()
