@@ -28,10 +28,24 @@ RATIOS_E = [.3125, .3125, .1875, .1875]
 PEAK = {"bf16": 2500.0, "fp32": 157.3}        # dense MFMA TFLOP/s, MI355X
 HBM_PEAK = 8000.0                              # GB/s
 
-# counted on the default workload with the commands of profiles/bert_large_shard_step.counters.md: 87 852 KiB fetched
-# (x 2.0) + 33 629 KiB written per GEMM launch; every operand read and every result written once: 19.3 GB per step
+# OFFLINE constants, not measured by a bench run: counted on the default workload with the commands of
+# profiles/bert_large_shard_step.counters.md: 87 852 KiB fetched (x 2.0) + 33 629 KiB written per GEMM launch; every
+# operand read and every result written once: 19.3 GB per step in 207 launches.  They belong to the GEMM plan below
+# (signature (M, N, K, batch, transA, transB, in, out) -> (tile configuration, K splits): the plan file that the
+# profile's commands name); a run whose autotuned plan or launch count differs reports no traffic.
 PROFILED_GEMM_TRAFFIC_PER_LAUNCH = (2.0 * 87852 + 33629) * 1024
-PROFILED_GEMM_ALGORITHMIC_BYTES_PER_LAUNCH = 19.3e9 / 207
+PROFILED_GEMM_LAUNCHES_PER_STEP = 207
+PROFILED_GEMM_ALGORITHMIC_BYTES_PER_LAUNCH = 19.3e9 / PROFILED_GEMM_LAUNCHES_PER_STEP
+PROFILED_GEMM_PLAN = {
+    (1024, 1024, 6144, 8, 1, 0, 1, 0): (6, 1), (1024, 4096, 6144, 8, 1, 0, 1, 0): (1, 1),
+    (1536, 1024, 16384, 8, 1, 0, 1, 0): (3, 1), (3072, 1024, 6144, 8, 1, 0, 1, 0): (3, 1),
+    (6144, 1024, 1024, 1, 0, 0, 1, 1): (7, 1), (6144, 1024, 1024, 1, 0, 1, 1, 1): (7, 1),
+    (6144, 1024, 3072, 1, 0, 0, 1, 1): (7, 1), (6144, 1024, 4096, 1, 0, 1, 1, 1): (7, 1),
+    (6144, 1024, 30522, 1, 0, 0, 1, 1): (3, 2), (6144, 3072, 1024, 1, 0, 1, 1, 1): (9, 1),
+    (6144, 4096, 1024, 1, 0, 0, 1, 1): (6, 1), (6144, 30522, 1024, 1, 0, 1, 1, 1): (4, 1),
+    (16384, 1024, 1536, 1, 0, 0, 1, 1): (1, 1), (16384, 1536, 1024, 1, 0, 1, 1, 1): (6, 1),
+    (30522, 1024, 6144, 1, 1, 0, 1, 0): (1, 1),
+}
 
 WORKLOADS = {
     # name: (description, dtype)
@@ -372,12 +386,20 @@ def measure(workload, args, steps, warmup, share_shapes=True, dropout=None, capa
     default_bert = (bert and args.attn == "batch" and not args.zero and (args.dropout if dropout is None else dropout) == 0.0
                     and not args.no_exchange_in_pieces and not args.no_receive_in_place and args.wgrad_group == 8)
     if default_bert:
-        # bytes per GEMM launch between the L2 caches and the memory fabric, counted offline with rocprofv3 --pmc
-        # (FETCH_SIZE scaled by the factor a copy of known size gives, plus WRITE_SIZE; mean over the step's launches)
+        # bytes per GEMM launch between the L2 caches and the memory fabric, counted OFFLINE with rocprofv3 --pmc
+        # (FETCH_SIZE scaled by the factor a copy of known size gives, plus WRITE_SIZE; mean over the step's launches):
+        # a property of the tile plan that was profiled, so it is reported only for a run that uses that plan
         r = result["roofline"]
-        r["traffic"] = PROFILED_GEMM_TRAFFIC_PER_LAUNCH
-        r["traffic_unit"] = "bytes per launch (mean over the step's GEMM launches), rocprofv3 --pmc FETCH_SIZE x 2.0 + WRITE_SIZE"
-        r["algorithmic_bytes"] = PROFILED_GEMM_ALGORITHMIC_BYTES_PER_LAUNCH
+        plan_now = ops.pinned_gemm_plans()
+        same_plan = all(plan_now.get(k) == v for k, v in PROFILED_GEMM_PLAN.items())
+        same_launches = round(r["launches_per_step"]) == PROFILED_GEMM_LAUNCHES_PER_STEP
+        r["traffic"] = PROFILED_GEMM_TRAFFIC_PER_LAUNCH if same_plan and same_launches else None
+        r["traffic_source"] = ("offline profile, not measured in this run: rocprofv3 --pmc FETCH_SIZE x 2.0 + WRITE_SIZE per "
+                               "launch, mean over the step's GEMM launches (profiles/bert_large_shard_step.counters.md); "
+                               "reported only when this run's GEMM plan and launch count are the profiled ones")
+        r["traffic_plan_is_the_profiled_one"] = bool(same_plan and same_launches)
+        r["traffic_unit"] = "bytes per launch"
+        r["algorithmic_bytes"] = PROFILED_GEMM_ALGORITHMIC_BYTES_PER_LAUNCH if same_launches else None
     # the reference calibrates its planner with hap.stat / (seconds of one training step) (profiler.py:33-39)
     shard_stat = planner.stat(gm, {"input_shape": {"x": tuple(x.shape), "y": tuple(y.shape)}})
     result["config"]["hap_stat_flops_of_shard"] = shard_stat

@@ -1658,6 +1658,12 @@ class ShardExecutor:
         sL, cL, rank = list(node.args[3]), list(node.args[4]), node.args[5]
         if x.t is None or x.ld is not None:
             self._unsupported(node, f"all_to_all of a {x.kind} value")
+        if any(u.target is torch.log_softmax for u in node.users):
+            # ShardingPlan(decoder="vocabulary"): the generator emits it and the CPU tests pin it against the
+            # single-device model; the logits' exchange (pieces whose widths are no multiple of the 16-byte vector,
+            # e.g. 11446 of 30522 columns) has no GPU parity test yet, so the executor does not run it
+            self._unsupported(node, "an all_to_all in front of log_softmax (the vocabulary-split output projection) is "
+                                    "not built in this executor")
         # piece boundaries: multiples of 64 for the k-tiles of the forward GEMM and of 128, the narrowest bf16 tile,
         # for the N tiles of the two backward GEMMs
         bounds = [sum(cL[:i]) for i in range(1, len(cL))]

@@ -678,6 +678,11 @@ def clear_gemm_plans():
     _pinned_plans.clear()
 
 
+def pinned_gemm_plans() -> dict:
+    """The plans pinned in this process: (M, N, K, batch, transA, transB, in, out) -> (tile configuration, K splits)."""
+    return dict(_pinned_plans)
+
+
 def save_gemm_plans(path: str) -> int:
     """Write the plans pinned by autotuning in this process as JSON; returns their number."""
     import json

@@ -333,14 +333,32 @@ def build_program(model: nn.Module, plan: ShardingPlan, global_batch: int,
             h = e.call(operator.add, h, e.g.get_attr("pe"))      # [1,S,d]: size-1 dim, never split
         mask = e.replicated("src_mask") if getattr(model, "src_mask", None) is not None else None
     elif model.family == "vit":
-        x = e.sharded_input("x", B)
+        if plan.patch_embed not in ("batch", "features"):
+            raise ValueError("ShardingPlan: patch_embed is 'batch' or 'features'")
+        x = e.whole_input("x") if plan.patch_embed == "features" else e.sharded_input("x", B)
         y = e.sharded_input("y", B)
         pe = model.patch_embed
-        c = e.call(F.conv2d, x, e.replicated("patch_embed.proj.weight"), e.replicated("patch_embed.proj.bias"),
-                   tuple(pe.patch_size), (0, 0), (1, 1), 1)
-        c = e.call(torch.flatten, c, 2, -1)
-        c = e.call(torch.transpose, c, 1, 2)
-        c = e.call(models.append_cls_token, c, e.replicated("cls_token"))
+        if plan.patch_embed == "features":
+            # the convolution's kernel and bias sliced over the output channels, whole images: output gathered on
+            # dim 1 (hap.rs:3083-3087); flatten keeps it (a communicatable tensor, hap.rs:1794), the all_gather makes it
+            # whole; transpose and the class token run on the whole batch, whose rows are then cut to the device's
+            # images (append_cls_token's output is communicatable, hap.rs:2107)
+            if not batch_sharded or plan.zero:
+                raise ValueError("patch_embed='features' is a plan of the batch-sharded ViT with whole parameters")
+            L_d = plan.lengths(d)
+            c = e.call(F.conv2d, x, e.sharded("patch_embed.proj.weight", d, 0), e.sharded("patch_embed.proj.bias", d, 0),
+                       tuple(pe.patch_size), (0, 0), (1, 1), 1)
+            c = e.call(torch.flatten, c, 2, -1)
+            c = e.call(collectives.all_gather, c, 1, L_d, e.rank)
+            c = e.call(torch.transpose, c, 1, 2)
+            c = e.call(models.append_cls_token, c, e.replicated("cls_token"))
+            c = e.call(collectives.dynamic_slice, c, 0, plan.lengths(B), e.rank)
+        else:
+            c = e.call(F.conv2d, x, e.replicated("patch_embed.proj.weight"), e.replicated("patch_embed.proj.bias"),
+                       tuple(pe.patch_size), (0, 0), (1, 1), 1)
+            c = e.call(torch.flatten, c, 2, -1)
+            c = e.call(torch.transpose, c, 1, 2)
+            c = e.call(models.append_cls_token, c, e.replicated("cls_token"))
         h = e.call(operator.add, c, e.replicated("pos_embed"))
         mask = None
     else:
@@ -362,13 +380,32 @@ def build_program(model: nn.Module, plan: ShardingPlan, global_batch: int,
         else:
             h = _dense_ffn(e, h1, prefix, d, model.nhid, B, p, activation, batch_sharded)
 
+    if plan.decoder not in ("whole", "vocabulary"):
+        raise ValueError("ShardingPlan: decoder is 'whole' or 'vocabulary'")
+    vocab_split = plan.decoder == "vocabulary"
+    if vocab_split and (not batch_sharded or plan.shard_dim != "batch" or plan.zero):
+        raise ValueError("decoder='vocabulary' is a plan of the batch-sharded programs with whole parameters")
+
+    def decode(t, cat_dim):
+        """The output projection; ``cat_dim``: the logits' class dimension.  Vocabulary split: the feature partition of a linear (hap.rs:2807-2816) needs its
+        input whole, so the activations are gathered over the batch, every device computes its columns of the logits
+        for all samples, and one all_to_all (split along the batch, concatenated along the classes: the exchange of
+        the column-sharded FFN, hap.rs:2713-2744) gives the device's samples their whole rows for log_softmax."""
+        if not vocab_split:
+            return e.call(F.linear, t, e.replicated("decoder.weight"), e.replicated("decoder.bias"))
+        V = e._shape("decoder.weight")[0]
+        L_B, L_V = plan.lengths(B), plan.lengths(V)
+        full = e.call(collectives.all_gather, t, 0, L_B, e.rank)
+        u = e.call(F.linear, full, e.sharded("decoder.weight", V, 0), e.sharded("decoder.bias", V, 0))
+        return e.call(collectives.all_to_all, u, 0, cat_dim, L_B, L_V, e.rank)
+
     if model.family == "lm":
-        logits = e.call(F.linear, h, e.replicated("decoder.weight"), e.replicated("decoder.bias"))
+        logits = decode(h, 2)
         lp = e.call(torch.log_softmax, logits, 2)
         lp = e.call(torch.transpose, lp, 1, 2)
     else:
         c = e.call(models.get_cls_token, h)
-        logits = e.call(F.linear, c, e.replicated("decoder.weight"), e.replicated("decoder.bias"))
+        logits = decode(c, 1)
         lp = e.call(torch.log_softmax, logits, 1)
     loss = e.g.call_function(F.nll_loss, (lp, y), {"reduction": "sum"})
     e.g.output(loss)

@@ -79,6 +79,14 @@ class ShardingPlan:
                                  # hap.rs:2795, 3061, 3214-3218, 2996; attention needs the whole sequence)
     embedding: str = "rows"      # "rows": ids sharded, table whole; "features": ids whole, table sharded on dim 1,
                                  # output gathered on dim 2 (hap.rs:3220-3224), then all_gather + dynamic_slice
+    decoder: str = "whole"       # "whole": the output projection on the device's samples with the whole weight;
+                                 # "vocabulary": its weight and bias sliced on dim 0 (the feature partition of a linear,
+                                 # hap.rs:2807-2816): all_gather of the activations, the device's columns of the logits
+                                 # for every sample, all_to_all back to whole rows of the device's samples
+    patch_embed: str = "batch"   # ViT: "batch": the patch convolution on the device's images with the whole kernel;
+                                 # "features": kernel and bias sliced on dim 0 and whole images (hap.rs:3083-3087),
+                                 # output channels gathered behind the flatten, cut to the device's images behind the
+                                 # class token
     moe: str = "experts"         # how the four MoE einsums are split (hap.rs:3285-3419): "experts": dispatch / combine
                                  # tensors sliced on dim 2, expert weights on dim 0; "capacity": dispatch / combine
                                  # sliced on dim 3 (every device takes a range of every expert's slots), expert weights

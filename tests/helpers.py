@@ -59,7 +59,8 @@ def rank_programs(model, ratios, B, **kw):
         m = copy.deepcopy(model)
         plan = hap_amd.ShardingPlan([list(ratios)], r, ffn=kw.get("ffn", "column"), zero=kw.get("zero", False),
                                      attn=kw.get("attn", "batch"), shard_dim=kw.get("shard_dim", "batch"),
-                                     embedding=kw.get("embedding", "rows"), moe=kw.get("moe", "experts"))
+                                     embedding=kw.get("embedding", "rows"), moe=kw.get("moe", "experts"),
+                                     decoder=kw.get("decoder", "whole"), patch_embed=kw.get("patch_embed", "batch"))
         progs.append(hap_amd.build_program(m, plan, B, activation=kw.get("activation", "relu"),
                                            batch_sharded=kw.get("batch_sharded", True)))
     return progs

@@ -30,7 +30,10 @@ CASES = {
     "lm-sequence": (lambda: make_lm(S=19), RATIOS4, 6, lambda: lm_batch(6, 19, 97), dict(ffn="batch", shard_dim="sequence")),
     "lm-feature-embedding": (lambda: make_lm(d=40, H=4), RATIOS4, 8, lambda: lm_batch(8, 16, 97),
                              dict(ffn="column", embedding="features")),
+    "lm-vocabulary-decoder": (lambda: make_lm(), RATIOS4, 8, lambda: lm_batch(8, 16, 97), dict(ffn="column", decoder="vocabulary")),
     "vit": (lambda: make_vit(), RATIOS4, 8, lambda: vit_batch(8, 16, 10), dict(ffn="batch")),
+    "vit-weight-split-patches": (lambda: make_vit(), RATIOS4, 8, lambda: vit_batch(8, 16, 10),
+                                 dict(ffn="batch", patch_embed="features", decoder="vocabulary")),
     "moe": (lambda: make_moe(), RATIOS_E, 16, lambda: lm_batch(16, 16, 61), dict(ffn="batch")),
     "moe-capacity": (lambda: make_moe(C=10), RATIOS_E, 16, lambda: lm_batch(16, 16, 61), dict(ffn="batch", moe="capacity")),
     "moe-hidden": (lambda: make_moe(C=10), RATIOS_E, 16, lambda: lm_batch(16, 16, 61), dict(ffn="batch", moe="hidden")),

@@ -26,6 +26,9 @@ CASES = {
     "lm_zero": dict(make=lambda: helpers.make_lm(), ratios=RATIOS4, B=16, kw=dict(ffn="column", zero=True), batch="lm"),
     "lm_heads": dict(make=lambda: helpers.make_lm(H=8), ratios=RATIOS4, B=16, kw=dict(ffn="batch", attn="heads"), batch="lm"),
     "vit": dict(make=lambda: helpers.make_vit(), ratios=RATIOS4, B=8, kw=dict(ffn="column"), batch="vit"),
+    "vit_weight_split_patches": dict(make=lambda: helpers.make_vit(), ratios=RATIOS4, B=8,
+                                     kw=dict(ffn="batch", patch_embed="features", decoder="vocabulary"), batch="vit"),
+    "lm_vocabulary_decoder": dict(make=lambda: helpers.make_lm(), ratios=RATIOS4, B=16, kw=dict(ffn="column", decoder="vocabulary"), batch="lm"),
     "moe": dict(make=lambda: helpers.make_moe(), ratios=RATIOS_E, B=8, kw=dict(ffn="batch"), batch="lm"),
     "moe_capacity": dict(make=lambda: helpers.make_moe(C=10), ratios=RATIOS_E, B=8, kw=dict(ffn="batch", moe="capacity"), batch="lm"),
     "moe_hidden": dict(make=lambda: helpers.make_moe(C=10), ratios=RATIOS_E, B=8, kw=dict(ffn="batch", moe="hidden"), batch="lm"),

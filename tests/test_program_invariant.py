@@ -5,11 +5,13 @@ import copy
 
 import pytest
 import torch
+import torch.nn.functional as F
 
 from helpers import (RATIOS4, RATIOS_E, joint_cpu, lm_batch, make_lm, make_moe, make_switch, make_vit, rel_err,
                      vit_batch)
 from oracle import single_device
 import hap_amd
+from hap_amd import collectives, models
 
 
 def _single(model, x, y):
@@ -261,3 +263,50 @@ def test_moe_hidden_split_with_deferred_reduction_in_bf16():
     deferred = gradient_errors("hidden", {"layers.1.w1": 2, "layers.1.w2": 1})
     for name in legal:
         assert deferred[name] <= 1.25 * legal[name] + 2e-2, (name, deferred[name], legal[name])
+
+
+@pytest.mark.parametrize("ffn", ["column", "batch"])
+def test_lm_vocabulary_split_decoder_spmd_equals_single_device(ffn):
+    """The feature partition of a linear (hap.rs:2807-2816) applied to the output projection: decoder weight and bias
+    sliced over the vocabulary (36 / 37 / 12 / 12 of 97), activations gathered over the batch, every rank's columns
+    of the logits exchanged by one all_to_all into whole rows of its own samples (hap.rs:2713-2744), log_softmax and
+    nll_loss on those."""
+    model = make_lm()
+    B = 8
+    x, y = lm_batch(B, 16, 97)
+    run = joint_cpu(model, RATIOS4, B, ffn=ffn, decoder="vocabulary")
+    L_V = hap_amd.sharding_lengths(97, RATIOS4)
+    # floors 36, 36, 12, 12 leave one unit: the largest deficit .375 - 36/97 is shared by ranks 0 and 1, the tie goes to the last
+    assert L_V == [36, 37, 12, 12]
+    sharded = {"decoder.weight": (0, L_V), "decoder.bias": (0, L_V)}
+    if ffn == "column":
+        L_F = hap_amd.sharding_lengths(64, RATIOS4)
+        for i in range(2):
+            sharded[f"layers.{i}.linear1.weight"] = (0, L_F)
+            sharded[f"layers.{i}.linear1.bias"] = (0, L_F)
+    _check(model, run, x, y, sharded)
+    targets = [n.target for n in run.programs[0].graph.nodes if n.op == "call_function" and n.target is not collectives.replicate]
+    assert targets[-4:] == [collectives.all_to_all, torch.log_softmax, torch.transpose, F.nll_loss]
+
+
+@pytest.mark.parametrize("decoder", ["whole", "vocabulary"])
+def test_vit_weight_split_patch_embedding_spmd_equals_single_device(decoder):
+    """The convolution's weight-split triple (hap.rs:3083-3087): kernel and bias sliced over the 32 output channels
+    (12 / 12 / 4 / 4), whole images in, output gathered on dim 1; the flattened output is all_gather-ed on dim 1, the
+    class token is appended on the whole batch and the rows are then cut to the rank's images.  With the class head
+    split over the 10 classes as well (4 / 4 / 1 / 1)."""
+    model = make_vit()
+    x, y = vit_batch(8, 16, 10)
+    run = joint_cpu(model, RATIOS4, 8, ffn="batch", patch_embed="features", decoder=decoder)
+    L_d = hap_amd.sharding_lengths(32, RATIOS4)
+    sharded = {"patch_embed.proj.weight": (0, L_d), "patch_embed.proj.bias": (0, L_d)}
+    if decoder == "vocabulary":
+        L_C = hap_amd.sharding_lengths(10, RATIOS4)
+        sharded.update({"decoder.weight": (0, L_C), "decoder.bias": (0, L_C)})
+    _check(model, run, x, y, sharded)
+    nodes = [n for n in run.programs[0].graph.nodes if n.op == "call_function" and n.target is not collectives.replicate]
+    conv = next(n for n in nodes if n.target is F.conv2d)
+    assert conv.args[0].op == "placeholder"                       # whole images
+    follow = [n.target for n in nodes[nodes.index(conv) + 1: nodes.index(conv) + 6]]
+    assert follow == [torch.flatten, collectives.all_gather, torch.transpose, models.append_cls_token,
+                      collectives.dynamic_slice]
