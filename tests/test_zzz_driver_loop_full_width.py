@@ -22,7 +22,7 @@ def test_loop_on_bert_width_bf16_shard_matches_cpu_oracle(cuda):
 
     * every step's loss against the CPU oracle running the same loop, at the bf16 tolerance 2e-2;
     * the loop's optimizer mechanics exactly: torch.nn.utils.clip_grad_norm_(0.5) + torch.optim.Adam on the CPU, fed
-      with the gradients the GPU computed in each step, must reproduce the GPU's final float32 masters (1e-5);
+      with the gradients the GPU computed in each step, must reproduce the GPU's final float32 masters (rtol 1e-5, atol 1e-7);
     * the final weights against the oracle's at 2e-2 (norm-wise per tensor).  Tensors that start at zero (the biases)
       hold nothing but four of Adam's normalised steps, which follow the gradient's sign and amplify the bf16
       difference between the two runs' gradients where a gradient is small: for them, and for the accumulated update
@@ -74,7 +74,9 @@ def test_loop_on_bert_width_bf16_shard_matches_cpu_oracle(cuda):
     for n in names:
         rec = ex.params[n]
         got, exp = rec["master"].cpu(), ref[n].detach()
-        torch.testing.assert_close(got, twins[n].detach(), rtol=1e-5, atol=1e-8, msg=lambda m: f"{n}: {m}")
+        # (absolute part: a 5000th of one step of lr 5e-4; the two norms behind the clipping coefficient are float32 sums
+        # of 9e7 squares taken in different orders)
+        torch.testing.assert_close(got, twins[n].detach(), rtol=1e-5, atol=1e-7, msg=lambda m: f"{n}: {m}")
         assert torch.equal(rec["shadow"].cpu(), got.to(torch.bfloat16)), n
         c = clear[n]
         if start[n].abs().max() > 0:                       # weights that start away from zero: the stated tolerance
