@@ -58,7 +58,7 @@ from __future__ import annotations
 
 import math
 import operator
-from typing import List, Optional
+from typing import Optional
 
 import torch
 import torch.fx

@@ -11,7 +11,7 @@ list with the integer lengths).  The arithmetic runs in the native library
 from __future__ import annotations
 
 import ctypes
-from dataclasses import dataclass, field
+from dataclasses import dataclass
 from typing import List, Sequence
 
 import torch

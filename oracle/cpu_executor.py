@@ -17,7 +17,6 @@ before rounding the result to bfloat16.
 """
 from __future__ import annotations
 
-import operator
 from typing import Dict, List, Optional
 
 import torch
