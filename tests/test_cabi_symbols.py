@@ -64,3 +64,31 @@ def test_gemm_argument_checks_run_before_any_launch():
     for needle, a in cases.items():
         rc = lib.hapmi_gemm(ctypes.byref(a), None)
         assert rc != 0 and needle in lib.hapmi_last_error(), (needle, rc, lib.hapmi_last_error())
+
+
+def test_more_host_side_checks_without_a_gpu():
+    """Argument checks that return before any device is touched: dropout in the GEMM epilogue refuses operands in
+    pieces or with relu on load (it used to launch the piece-reading kernel without the dropout), the plan table knows
+    twelve tile configurations, and the embedding backward accepts rows wider than one wave's 2048 columns."""
+    from hap_amd._lib import GemmArgs, _load, BF16
+    lib = _load()
+    a = GemmArgs()
+    a.M, a.N, a.K, a.lda, a.ldb, a.ldc = 64, 64, 64, 64, 64, 64
+    a.in_dtype, a.out_dtype, a.alpha, a.batch1, a.batch2 = BF16, BF16, 1.0, 1, 1
+    a.A, a.B, a.C, a.transA, a.transB = 0x1000, 0x1000, 0x1000, 0, 1
+    a.drop_state, a.drop_stream_id, a.drop_p = 0x1000, 3, 0.1
+    a.a_relu = 1
+    rc = lib.hapmi_gemm(ctypes.byref(a), None)
+    assert rc != 0 and b"no relu on an operand" in lib.hapmi_last_error(), lib.hapmi_last_error()
+
+    i64 = ctypes.c_int64
+    lib.hapmi_gemm_plan_set.argtypes = [i64, i64, i64, i64] + [ctypes.c_int] * 6
+    assert lib.hapmi_gemm_plan_set(64, 64, 64, 1, 0, 1, 1, 1, 11, 1) == 0
+    assert lib.hapmi_gemm_plan_set(64, 64, 64, 1, 0, 1, 1, 1, 12, 1) != 0          # no thirteenth configuration
+    assert b"out of range" in lib.hapmi_last_error()
+    assert lib.hapmi_gemm_plan_clear() == 0
+
+    vp = ctypes.c_void_p
+    lib.hapmi_embedding_bwd.argtypes = [vp, vp, vp, i64, i64, i64, ctypes.c_float, ctypes.c_int, vp]
+    assert lib.hapmi_embedding_bwd(None, None, None, 0, 3 * 2048 + 8, 100, 1.0, 1, None) == 0    # nothing to do, no limit hit
+    assert lib.hapmi_embedding_bwd(None, None, None, 0, 65536 * 2048, 100, 1.0, 1, None) == -5   # HAPMI_ELIMIT
