@@ -10,6 +10,8 @@ Functions and the reference lines they follow:
 * ``positional_encoding``  -- /root/reference/models.py:504-509.
 * ``top_2_gating``         -- /root/reference/models.py:477-502.
 * ``switch_gating``        -- /root/reference/models.py:452-475.
+* ``gating_slots``         -- the integer part of both (models.py:483-491, 458-466) in index form, in C
+  (oracle/gating_slots.c).
 * ``attention_with_dropped_probabilities`` -- F.multi_head_attention_forward's explicit path
   (torch:nn/functional.py:6435-6612, the call emitted at hap.rs:1301-1321) with a given dropout mask.
 * ``head_parallel_attention`` -- no reference counterpart (the reference shards
@@ -57,6 +59,9 @@ def _lib():
         _liboracle.oracle_sharding_round.argtypes = [
             ctypes.c_int64, ctypes.POINTER(ctypes.c_double), ctypes.c_int64,
             ctypes.POINTER(ctypes.c_int64)]
+        i64p = ctypes.POINTER(ctypes.c_int64)
+        _liboracle.oracle_gating_slots.restype = ctypes.c_int
+        _liboracle.oracle_gating_slots.argtypes = [i64p] + [ctypes.c_int64] * 5 + [i64p, i64p]
     return _liboracle
 
 
@@ -81,6 +86,16 @@ def positional_encoding(seqlen: int, emsize: int) -> np.ndarray:
     out[:, 0::2] = np.sin(angle[:, 0::2])
     out[:, 1::2] = np.cos(angle[:, 1::2])
     return out
+
+
+def densify_vectorised(index, slot, gate, n_expert: int, capacity: int):
+    """``densify`` without Python loops (any number of choices per token): combine[b, s, index_k, slot_k] = gate_k
+    for every kept choice, dispatch = combine > 0."""
+    B, S, k = index.shape
+    combine = torch.zeros(B, S, n_expert, capacity, dtype=gate.dtype)
+    b, s, j = (slot > 0).nonzero(as_tuple=True)
+    combine.index_put_((b, s, index[b, s, j], slot[b, s, j]), gate[b, s, j], accumulate=True)
+    return (combine > 0).to(torch.float32), combine
 
 
 # --------------------------------------------------------------------------
@@ -111,6 +126,22 @@ def top_2_gating(gate_input, n_expert: int, capacity: int, gate_weight, train: b
                * F.one_hot(pos, capacity)).sum(dim=2)                  # :498
     dispatch = (combine > 0).to(torch.float32)                         # :500
     return dispatch, combine
+
+
+def gating_slots(index: torch.Tensor, n_expert: int, capacity: int):
+    """The integer part of models.py:483-491 (top-2) / 458-466 (switch) in index form, in C
+    (oracle/gating_slots.c): ``index`` [B, S, k] int64 -> (slot [B, S, k] with 0 = dropped, token_of_slot [B, E, C]
+    with -1 = empty)."""
+    index = index.to(torch.int64).contiguous()
+    B, S, k = index.shape
+    slot = torch.zeros(B, S, k, dtype=torch.int64)
+    tos = torch.empty(B, n_expert, capacity, dtype=torch.int64)
+    i64p = ctypes.POINTER(ctypes.c_int64)
+    rc = _lib().oracle_gating_slots(ctypes.cast(index.data_ptr(), i64p), B, S, n_expert, capacity, k,
+                                    ctypes.cast(slot.data_ptr(), i64p), ctypes.cast(tos.data_ptr(), i64p))
+    if rc != 0:
+        raise ValueError("gating_slots: an expert index lies outside [0, n_expert)")
+    return slot, tos
 
 
 def head_parallel_attention(x, in_proj_weight, in_proj_bias, out_proj_weight, num_heads: int, attn_mask=None):

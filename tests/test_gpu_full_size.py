@@ -304,7 +304,9 @@ def test_moe_shard_full_depth_bf16_adam_step(cuda):
 def test_moe_shard_capacity_40(cuda, dtype):
     """Benchmark configuration 4 with the capacity factor 1.25 read literally: C = ceil(512 / 16 * 1.25) = 40 slots
     per expert (the reference's config.py:25-28 doubles the factor for models whose name ends in `moe`, which gives the
-    80 of the other tests); two layers at full width, so about half of the second choices are dropped for lack of a slot."""
+    80 of the other tests); two layers at full width.  At this shape nearly every second choice is dropped at either
+    capacity (the reference queues them behind the sum of the expert's first-choice positions, models.py:486: 528 for 32
+    first choices); at C = 40 some first choices of the busiest experts are dropped as well."""
     _full_check("moe", 2, dtype, capacity=40)
 
 
